@@ -1,0 +1,223 @@
+"""ctypes binding of libhspmm.so (include/hspmm.h).
+
+Every function here calls the C ABI; there is no Python or CPU fallback for the
+device operator: if the library is missing, or no gfx950 device is present,
+`Plan` raises.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+FP16 = 0            # HSPMM_FP16, reference -DUSE_FP16 (src/common.h:14-19)
+TF32 = 1            # HSPMM_TF32, reference -DUSE_TF32 (src/common.h:26-43), fp32 storage
+IDX_MAX = 0xFFFFFFFF
+ROW_WINDOW = 8
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "libhspmm.so")
+_lib = None
+
+
+class HspmmError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__("hspmm error %d: %s" % (code, text))
+        self.code = code
+
+
+def library_path():
+    return _LIB
+
+
+def build_library(force=True):
+    """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU)."""
+    cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j4"]
+    if force:
+        cmd.insert(1, "-B")
+    subprocess.check_call(cmd, stdout=subprocess.DEVNULL)
+    return _LIB
+
+
+class _Csr(C.Structure):
+    _fields_ = [("rows", C.c_uint32), ("cols", C.c_uint32), ("nnzs", C.c_uint32),
+                ("row_ptr", C.POINTER(C.c_uint32)), ("col_idx", C.POINTER(C.c_uint32)),
+                ("values", C.c_void_p)]
+
+
+class PlanInfo(C.Structure):
+    _fields_ = [("rows", C.c_uint32), ("cols", C.c_uint32), ("eff_row_windows", C.c_uint32),
+                ("total_tiles", C.c_uint32), ("dtype", C.c_int32), ("n_ranges", C.c_uint32),
+                ("n_split_windows", C.c_uint32), ("n_partial_slots", C.c_uint32),
+                ("compute_units", C.c_uint32), ("device_bytes", C.c_uint64)]
+
+
+def load_library():
+    """Load libhspmm.so; build it first only if it is not there."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB):
+        build_library(force=False)
+    L = C.CDLL(_LIB)
+    u32, vp, i = C.c_uint32, C.c_void_p, C.c_int
+    L.hspmm_last_error.restype = C.c_char_p
+    L.hspmm_create.argtypes = [C.POINTER(vp), i, u32, u32, u32, u32, vp, vp, vp, vp]
+    L.hspmm_run.argtypes = [vp, vp, vp, u32, vp]
+    L.hspmm_bench.argtypes = [vp, vp, vp, u32, i, i, vp, C.POINTER(C.c_float)]
+    L.hspmm_destroy.argtypes = [vp]
+    L.hspmm_destroy.restype = None
+    L.hspmm_configure.argtypes = [i, i, i, i]
+    L.hspmm_get_config.argtypes = [C.POINTER(i)] * 4
+    L.hspmm_get_config.restype = None
+    L.hspmm_set_kernel_mode.argtypes = [i]
+    L.hspmm_get_plan_info.argtypes = [vp, C.POINTER(PlanInfo)]
+    L.hspmm_get_partition.argtypes = [vp, vp, u32]
+    L.hspmm_partition_preview.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
+    L.hspmm_mtx_load.argtypes = [C.c_char_p, i, C.POINTER(_Csr)]
+    L.hspmm_csr_free.argtypes = [C.POINTER(_Csr)]
+    L.hspmm_csr_free.restype = None
+    L.hspmm_btcf_sizes.argtypes = [i, u32, vp, vp, C.POINTER(u32), C.POINTER(u32)]
+    L.hspmm_btcf_fill.argtypes = [i, u32, vp, vp, vp, i, vp, vp, vp, vp]
+    _lib = L
+    return L
+
+
+def _check(rc):
+    if rc != 0:
+        raise HspmmError(rc, load_library().hspmm_last_error().decode("utf-8", "replace"))
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None and a.size else None
+
+
+def _val_dtype(dtype):
+    if dtype == FP16:
+        return np.uint16
+    if dtype == TF32:
+        return np.float32
+    raise ValueError("dtype must be FP16 or TF32")
+
+
+def configure(buffer_stage=0, consumer_warp_num=0, producer_warp_group_num=0, sm_num=0):
+    """Scheduler::configure of the reference (src/scheduler.h:33-38)."""
+    _check(load_library().hspmm_configure(buffer_stage, consumer_warp_num, producer_warp_group_num, sm_num))
+
+
+def get_config():
+    v = [C.c_int() for _ in range(4)]
+    load_library().hspmm_get_config(*[C.byref(x) for x in v])
+    return tuple(x.value for x in v)
+
+
+def set_kernel_mode(mode):
+    _check(load_library().hspmm_set_kernel_mode(mode))
+
+
+def mtx_load(path, dtype):
+    """load_matrix of the reference (src/utils/load.h:152): .mtx -> CSR dict.
+    fp16 values are returned as uint16 bit patterns."""
+    L = load_library()
+    m = _Csr()
+    _check(L.hspmm_mtx_load(os.fsencode(path), dtype, C.byref(m)))
+    try:
+        n = m.nnzs
+        vt = _val_dtype(dtype)
+        row_ptr = np.ctypeslib.as_array(m.row_ptr, (m.rows + 1,)).copy()
+        col_idx = np.ctypeslib.as_array(m.col_idx, (max(n, 1),))[:n].copy()
+        vals = np.ctypeslib.as_array(C.cast(m.values, C.POINTER(np.ctypeslib.as_ctypes_type(vt))),
+                                     (max(n, 1),))[:n].copy()
+        return dict(rows=m.rows, cols=m.cols, nnzs=n, row_ptr=row_ptr, col_idx=col_idx, values=vals)
+    finally:
+        L.hspmm_csr_free(C.byref(m))
+
+
+def csr_to_btcf(rows, cols, row_ptr, col_idx, values, dtype, transpose=False):
+    """CSR2BTCFNOBITMAP of the reference (src/utils/convert.h:146): returns the
+    BTCF_MTX_NO_BITMAP fields (src/utils/class.h:74-85) as a dict of numpy arrays."""
+    L = load_library()
+    vt = _val_dtype(dtype)
+    cw = 16 if dtype == FP16 else 8
+    row_ptr = np.ascontiguousarray(row_ptr, np.uint32)
+    col_idx = np.ascontiguousarray(col_idx, np.uint32)
+    values = np.ascontiguousarray(values, vt)
+    if row_ptr.size != rows + 1:
+        raise ValueError("row_ptr must have rows + 1 entries")
+    W, T = C.c_uint32(), C.c_uint32()
+    _check(L.hspmm_btcf_sizes(dtype, rows, _p(row_ptr), _p(col_idx), C.byref(W), C.byref(T)))
+    W, T = W.value, T.value
+    rowOffset = np.zeros(W + 1, np.uint32)
+    tcA2B = np.empty(T * cw, np.uint32)
+    data = np.empty(T * ROW_WINDOW * cw, vt)
+    rowIdx = np.empty(W, np.uint32)
+    _check(L.hspmm_btcf_fill(dtype, rows, _p(row_ptr), _p(col_idx), _p(values), int(transpose),
+                             _p(rowOffset), _p(tcA2B), _p(data), _p(rowIdx)))
+    return dict(rows=rows, cols=cols, nnzs=int(col_idx.size), dtype=dtype, cw=cw,
+                total_row_windows=(rows + ROW_WINDOW - 1) // ROW_WINDOW, eff_row_windows=W,
+                total_tiles=T, rowOffset=rowOffset, tcA2B=tcA2B, data=data, rowIdx=rowIdx)
+
+
+def partition_preview(rowOffset, target_ranges):
+    """The work partition hspmm_create would build (host only)."""
+    L = load_library()
+    rowOffset = np.ascontiguousarray(rowOffset, np.uint32)
+    W = rowOffset.size - 1
+    n, ns, nslots = C.c_uint32(), C.c_uint32(), C.c_uint32()
+    _check(L.hspmm_partition_preview(W, _p(rowOffset), target_ranges, None, 0, C.byref(n), C.byref(ns),
+                                     C.byref(nslots)))
+    ranges = np.zeros((n.value, 5), np.uint32)
+    _check(L.hspmm_partition_preview(W, _p(rowOffset), target_ranges, _p(ranges), n.value, None, None, None))
+    return dict(ranges=ranges, n_split_windows=ns.value, n_partial_slots=nslots.value)
+
+
+class Plan:
+    """Device-resident A plus its work partition (hspmm_create / hspmm_destroy)."""
+
+    def __init__(self, btcf):
+        L = load_library()
+        self._h = C.c_void_p()
+        self.dtype = btcf["dtype"]
+        self.rows, self.cols = int(btcf["rows"]), int(btcf["cols"])
+        vt = _val_dtype(self.dtype)
+        ro = np.ascontiguousarray(btcf["rowOffset"], np.uint32)
+        a2b = np.ascontiguousarray(btcf["tcA2B"], np.uint32)
+        data = np.ascontiguousarray(btcf["data"], vt)
+        ri = np.ascontiguousarray(btcf["rowIdx"], np.uint32)
+        _check(L.hspmm_create(C.byref(self._h), self.dtype, self.rows, self.cols,
+                              int(btcf["eff_row_windows"]), int(btcf["total_tiles"]),
+                              _p(ro), _p(a2b), _p(data), _p(ri)))
+
+    def run(self, dB_ptr, dC_ptr, N, stream=0):
+        """dB_ptr / dC_ptr: integer device addresses (e.g. torch tensor .data_ptr())."""
+        _check(load_library().hspmm_run(self._h, C.c_void_p(dB_ptr), C.c_void_p(dC_ptr), N, C.c_void_p(stream)))
+
+    def bench(self, dB_ptr, dC_ptr, N, warmup=3, runs=5, stream=0):
+        """Total milliseconds of `runs` launches (WARMUP_RUNS / RUNS, src/common.h:48-49)."""
+        ms = C.c_float()
+        _check(load_library().hspmm_bench(self._h, C.c_void_p(dB_ptr), C.c_void_p(dC_ptr), N, warmup, runs,
+                                          C.c_void_p(stream), C.byref(ms)))
+        return ms.value
+
+    def info(self):
+        inf = PlanInfo()
+        _check(load_library().hspmm_get_plan_info(self._h, C.byref(inf)))
+        return {k: getattr(inf, k) for k, _ in PlanInfo._fields_}
+
+    def partition(self):
+        n = self.info()["n_ranges"]
+        ranges = np.zeros((n, 5), np.uint32)
+        if n:
+            _check(load_library().hspmm_get_partition(self._h, _p(ranges), n))
+        return ranges
+
+    def close(self):
+        if self._h:
+            load_library().hspmm_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

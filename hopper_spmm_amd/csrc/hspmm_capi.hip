@@ -1,0 +1,426 @@
+// C ABI of the SpMM operator (include/hspmm.h): plan creation (validation,
+// upload, work partition), launch, timing.  Host code only; the kernels live in
+// hspmm_kernels.hip.  Mirrors the host half of the reference's fp16_spmm
+// (reference src/fp16.cu:221-281) split into create / run / bench / destroy so
+// that a caller can keep A on the device across launches.
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+#include <cstdarg>
+#include <cstring>
+#include <string>
+#include <vector>
+#include <mutex>
+#include <new>
+
+#include "../../include/hspmm.h"
+#include "hspmm_device.h"
+#include "partition.hpp"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+#define HSPMM_HIP(call)                                                                      \
+    do {                                                                                     \
+        hipError_t e_ = (call);                                                              \
+        if (e_ != hipSuccess)                                                                \
+            return fail(HSPMM_ERR_DEVICE, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), \
+                        __FILE__, __LINE__);                                                 \
+    } while (0)
+
+// The knobs of the reference's Scheduler singleton (reference src/scheduler.h:7-10),
+// re-read as: prefetch depth, waves per workgroup, waves per SIMD, compute units.
+struct Config {
+    int buffer_stage = 0;
+    int consumer_warp_num = 0;
+    int producer_warp_group_num = 0;
+    int sm_num = 0;
+    int kernel_mode = 0;
+};
+std::mutex g_cfg_mutex;
+Config g_cfg;
+
+constexpr uint32_t kMinTilesPerRange = 24;
+
+}  // namespace
+
+namespace hspmm_host {
+void set_error(const std::string &msg) { g_last_error = msg; }
+}
+
+struct hspmm_plan {
+    int dtype = 0;
+    int device = 0;
+    uint32_t rows = 0, cols = 0, W = 0, T = 0;
+    uint32_t cw = 16, elem = 2;
+    int compute_units = 0;
+    Config cfg;
+    // device copies of the format arrays
+    uint32_t *d_rowOffset = nullptr, *d_rowIdx = nullptr;
+    uint32_t *d_a2b_raw = nullptr;      // as given (padding = IDX_MAX): scalar kernel
+    uint32_t *d_a2b = nullptr;          // padding renamed to the id in front of it: MFMA kernels
+    void *d_data = nullptr;
+    // partition
+    hspmm::Partition part;
+    uint32_t *d_ranges = nullptr, *d_split = nullptr, *d_fix_slots = nullptr;
+    float *d_scratch = nullptr;
+    size_t scratch_bytes = 0;
+    size_t fixed_bytes = 0;
+};
+
+namespace {
+
+template <typename T>
+int upload(T **dst, const T *src, size_t n, size_t *acc_bytes)
+{
+    const size_t bytes = (n ? n : 1) * sizeof(T);
+    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(dst), bytes));
+    if (n) HSPMM_HIP(hipMemcpy(*dst, src, n * sizeof(T), hipMemcpyHostToDevice));
+    *acc_bytes += bytes;
+    return HSPMM_OK;
+}
+
+int validate_format(uint32_t rows, uint32_t cols, uint32_t W, uint32_t T, uint32_t cw,
+                    const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data, const uint32_t *rowIdx)
+{
+    if (W == 0) {
+        if (T != 0) return fail(HSPMM_ERR_INVALID, "total_tiles = %u with no effective row window", T);
+        return HSPMM_OK;
+    }
+    if (!rowOffset || !tcA2B || !data || !rowIdx) return fail(HSPMM_ERR_INVALID, "null format array");
+    if (rows == 0 || cols == 0) return fail(HSPMM_ERR_INVALID, "empty matrix with %u effective windows", W);
+    if (uint64_t(W) > (uint64_t(rows) + 7u) / 8u)
+        return fail(HSPMM_ERR_INVALID, "eff_row_windows = %u exceeds the %u windows of %u rows", W, (rows + 7u) / 8u, rows);
+    if (rowOffset[0] != 0) return fail(HSPMM_ERR_INVALID, "rowOffset[0] = %u, expected 0", rowOffset[0]);
+    for (uint32_t w = 0; w < W; ++w) {
+        if (rowOffset[w + 1] <= rowOffset[w])
+            return fail(HSPMM_ERR_INVALID, "rowOffset not strictly increasing at window %u", w);
+        if (rowIdx[w] % HSPMM_ROW_WINDOW != 0 || rowIdx[w] >= rows)
+            return fail(HSPMM_ERR_INVALID, "rowIdx[%u] = %u is not a window start inside %u rows", w, rowIdx[w], rows);
+        if (w && rowIdx[w] <= rowIdx[w - 1])
+            return fail(HSPMM_ERR_INVALID, "rowIdx not strictly increasing at window %u", w);
+    }
+    if (rowOffset[W] != T)
+        return fail(HSPMM_ERR_INVALID, "rowOffset[%u] = %u differs from total_tiles = %u", W, rowOffset[W], T);
+    for (uint32_t t = 0; t < T; ++t) {
+        const uint32_t *ids = tcA2B + size_t(t) * cw;
+        if (ids[0] == HSPMM_IDX_MAX) return fail(HSPMM_ERR_INVALID, "tile %u starts with a padding column", t);
+        bool pad = false;
+        for (uint32_t k = 0; k < cw; ++k) {
+            if (ids[k] == HSPMM_IDX_MAX) { pad = true; continue; }
+            if (pad) return fail(HSPMM_ERR_INVALID, "tile %u: column id after padding", t);
+            if (ids[k] >= cols) return fail(HSPMM_ERR_INVALID, "tile %u: column id %u >= cols %u", t, ids[k], cols);
+        }
+    }
+    return HSPMM_OK;
+}
+
+int choose_ranges(const hspmm_plan *p)
+{
+    const int waves_per_simd = p->cfg.producer_warp_group_num > 0 ? p->cfg.producer_warp_group_num : 4;
+    uint64_t g = uint64_t(p->compute_units) * 4u * uint64_t(waves_per_simd);
+    const uint64_t cap = (uint64_t(p->T) + kMinTilesPerRange - 1) / kMinTilesPerRange;
+    if (g > cap) g = cap;
+    if (g < 1) g = 1;
+    return int(g);
+}
+
+int build_and_upload_partition(hspmm_plan *p, const uint32_t *rowOffset)
+{
+    if (p->W == 0) return HSPMM_OK;
+    p->part = hspmm::build_partition(p->W, rowOffset, uint32_t(choose_ranges(p)));
+    const auto &part = p->part;
+    std::vector<uint32_t> rw(part.ranges.size() * hspmm::kRangeWords, 0u);
+    for (size_t i = 0; i < part.ranges.size(); ++i) {
+        uint32_t *d = rw.data() + i * hspmm::kRangeWords;
+        d[0] = part.ranges[i].tile_begin; d[1] = part.ranges[i].tile_end; d[2] = part.ranges[i].first_window;
+        d[3] = part.ranges[i].head_slot; d[4] = part.ranges[i].tail_slot;
+    }
+    std::vector<uint32_t> sw(part.split.size() * hspmm::kFixWords, 0u);
+    for (size_t i = 0; i < part.split.size(); ++i) {
+        uint32_t *d = sw.data() + i * hspmm::kFixWords;
+        d[0] = part.split[i].window; d[1] = part.split[i].slot_begin; d[2] = part.split[i].slot_count;
+    }
+    int rc;
+    if ((rc = upload(&p->d_ranges, rw.data(), rw.size(), &p->fixed_bytes))) return rc;
+    if ((rc = upload(&p->d_split, sw.data(), sw.size(), &p->fixed_bytes))) return rc;
+    if ((rc = upload(&p->d_fix_slots, part.fix_slots.data(), part.fix_slots.size(), &p->fixed_bytes))) return rc;
+    return HSPMM_OK;
+}
+
+struct Choice {
+    bool scalar;
+    int layout, V, block_feat;
+    bool narrow;
+};
+
+Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32_t N)
+{
+    Choice c{};
+    const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
+    const uint64_t row_bytes = uint64_t(N) * p->elem;
+    c.narrow = p->cols < (1u << 24) && row_bytes < (1u << 24) && uint64_t(p->cols) * row_bytes <= (1ull << 32);
+    const int mode = p->cfg.kernel_mode;
+    if (mode == 1) { c.scalar = true; return c; }
+    if (p->dtype == HSPMM_FP16) {
+        if (N % 2 != 0 || (align & 3u)) { c.scalar = true; return c; }
+        const bool dw_ok = (N % 64 == 0);
+        if (mode != 2 && (dw_ok || mode == 3) && N % 32 == 0) {
+            c.layout = hspmm::kLayoutDW;
+            c.V = (N % 128 == 0) ? 4 : (N % 64 == 0) ? 2 : 1;
+            c.block_feat = 32 * c.V;
+            return c;
+        }
+        c.layout = hspmm::kLayoutX4;
+        if (N % 8 == 0 && !(align & 15u) && N > 32) c.V = 4;
+        else if (N % 4 == 0 && !(align & 7u) && N > 16) c.V = 2;
+        else c.V = 1;
+        c.block_feat = 32 * c.V;
+        return c;
+    }
+    if (align & 3u) { c.scalar = true; return c; }
+    c.layout = hspmm::kLayoutX4;
+    if (N % 4 == 0 && !(align & 15u) && N > 16) c.V = 4;
+    else if (N % 2 == 0 && !(align & 7u) && N > 8) c.V = 2;
+    else c.V = 1;
+    c.block_feat = 16 * c.V;
+    return c;
+}
+
+int ensure_scratch(hspmm_plan *p, size_t bytes)
+{
+    if (bytes <= p->scratch_bytes) return HSPMM_OK;
+    if (p->d_scratch) { HSPMM_HIP(hipFree(p->d_scratch)); p->d_scratch = nullptr; p->scratch_bytes = 0; }
+    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->d_scratch), bytes));
+    p->scratch_bytes = bytes;
+    return HSPMM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *hspmm_last_error(void) { return g_last_error.c_str(); }
+
+int hspmm_configure(int buffer_stage, int consumer_warp_num, int producer_warp_group_num, int sm_num)
+{
+    if (buffer_stage < 0 || buffer_stage > 8 || buffer_stage == 5 || buffer_stage == 7)
+        return fail(HSPMM_ERR_INVALID, "buffer_stage %d: supported depths are 1, 2, 3, 4, 6, 8 (0 = default)", buffer_stage);
+    if (consumer_warp_num < 0 || consumer_warp_num > hspmm::kMaxWavesPerGroup)
+        return fail(HSPMM_ERR_INVALID, "consumer_warp_num %d outside 0..%d", consumer_warp_num, hspmm::kMaxWavesPerGroup);
+    if (producer_warp_group_num < 0 || producer_warp_group_num > 16)
+        return fail(HSPMM_ERR_INVALID, "producer_warp_group_num %d outside 0..16", producer_warp_group_num);
+    if (sm_num < 0 || sm_num > 4096) return fail(HSPMM_ERR_INVALID, "sm_num %d outside 0..4096", sm_num);
+    std::lock_guard<std::mutex> lk(g_cfg_mutex);
+    g_cfg.buffer_stage = buffer_stage;
+    g_cfg.consumer_warp_num = consumer_warp_num;
+    g_cfg.producer_warp_group_num = producer_warp_group_num;
+    g_cfg.sm_num = sm_num;
+    return HSPMM_OK;
+}
+
+void hspmm_get_config(int *buffer_stage, int *consumer_warp_num, int *producer_warp_group_num, int *sm_num)
+{
+    std::lock_guard<std::mutex> lk(g_cfg_mutex);
+    if (buffer_stage) *buffer_stage = g_cfg.buffer_stage;
+    if (consumer_warp_num) *consumer_warp_num = g_cfg.consumer_warp_num;
+    if (producer_warp_group_num) *producer_warp_group_num = g_cfg.producer_warp_group_num;
+    if (sm_num) *sm_num = g_cfg.sm_num;
+}
+
+int hspmm_set_kernel_mode(int mode)
+{
+    if (mode < 0 || mode > 3) return fail(HSPMM_ERR_INVALID, "kernel mode %d outside 0..3", mode);
+    std::lock_guard<std::mutex> lk(g_cfg_mutex);
+    g_cfg.kernel_mode = mode;
+    return HSPMM_OK;
+}
+
+int hspmm_partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
+                            uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges,
+                            uint32_t *n_split_windows, uint32_t *n_partial_slots)
+{
+    if (eff_row_windows && !rowOffset) return fail(HSPMM_ERR_INVALID, "null rowOffset");
+    for (uint32_t w = 0; w < eff_row_windows; ++w)
+        if (rowOffset[w + 1] <= rowOffset[w] || rowOffset[0] != 0)
+            return fail(HSPMM_ERR_INVALID, "rowOffset must start at 0 and increase strictly");
+    const hspmm::Partition part = hspmm::build_partition(eff_row_windows, rowOffset, target_ranges);
+    if (n_ranges) *n_ranges = uint32_t(part.ranges.size());
+    if (n_split_windows) *n_split_windows = uint32_t(part.split.size());
+    if (n_partial_slots) *n_partial_slots = part.n_slots;
+    if (ranges) {
+        const size_t n = part.ranges.size() < capacity_ranges ? part.ranges.size() : capacity_ranges;
+        for (size_t i = 0; i < n; ++i) {
+            ranges[5 * i + 0] = part.ranges[i].tile_begin; ranges[5 * i + 1] = part.ranges[i].tile_end;
+            ranges[5 * i + 2] = part.ranges[i].first_window;
+            ranges[5 * i + 3] = part.ranges[i].head_slot; ranges[5 * i + 4] = part.ranges[i].tail_slot;
+        }
+    }
+    return HSPMM_OK;
+}
+
+int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
+                 uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
+                 const uint32_t *rowIdx)
+{
+    if (!out) return fail(HSPMM_ERR_INVALID, "null plan pointer");
+    *out = nullptr;
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32) return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
+    const uint32_t cw = dtype == HSPMM_FP16 ? 16u : 8u;
+    const uint32_t elem = dtype == HSPMM_FP16 ? 2u : 4u;
+    int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx);
+    if (rc) return rc;
+
+    hspmm_plan *p = new (std::nothrow) hspmm_plan;
+    if (!p) return fail(HSPMM_ERR_ALLOC, "out of host memory");
+    p->dtype = dtype; p->rows = rows; p->cols = cols; p->W = eff_row_windows; p->T = total_tiles;
+    p->cw = cw; p->elem = elem;
+    { std::lock_guard<std::mutex> lk(g_cfg_mutex); p->cfg = g_cfg; }
+
+    auto bail = [&](int code) { hspmm_destroy(p); return code; };
+    hipError_t e = hipGetDevice(&p->device);
+    if (e != hipSuccess) return bail(fail(HSPMM_ERR_DEVICE, "hipGetDevice failed: %s", hipGetErrorString(e)));
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, p->device);
+    if (e != hipSuccess) return bail(fail(HSPMM_ERR_DEVICE, "hipGetDeviceProperties failed: %s", hipGetErrorString(e)));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return bail(fail(HSPMM_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only", p->device,
+                         prop.gcnArchName));
+    p->compute_units = p->cfg.sm_num > 0 ? p->cfg.sm_num : prop.multiProcessorCount;
+
+    if (p->W) {
+        const size_t n_ids = size_t(total_tiles) * cw;
+        if ((rc = upload(&p->d_rowOffset, rowOffset, size_t(p->W) + 1, &p->fixed_bytes))) return bail(rc);
+        if ((rc = upload(&p->d_rowIdx, rowIdx, size_t(p->W), &p->fixed_bytes))) return bail(rc);
+        if ((rc = upload(&p->d_a2b_raw, tcA2B, n_ids, &p->fixed_bytes))) return bail(rc);
+        {
+            // padding ids -> the real id in front of them (the tile column is all zero)
+            std::vector<uint32_t> clean(tcA2B, tcA2B + n_ids);
+            for (size_t i = 1; i < n_ids; ++i)
+                if (clean[i] == HSPMM_IDX_MAX) clean[i] = clean[i - 1];
+            if ((rc = upload(&p->d_a2b, clean.data(), n_ids, &p->fixed_bytes))) return bail(rc);
+        }
+        {
+            uint8_t *dd = nullptr;
+            if ((rc = upload(&dd, static_cast<const uint8_t *>(data), size_t(total_tiles) * 8u * cw * elem,
+                             &p->fixed_bytes)))
+                return bail(rc);
+            p->d_data = dd;
+        }
+        if ((rc = build_and_upload_partition(p, rowOffset))) return bail(rc);
+    }
+    *out = p;
+    return HSPMM_OK;
+}
+
+void hspmm_destroy(hspmm_plan *p)
+{
+    if (!p) return;
+    (void)hipFree(p->d_rowOffset); (void)hipFree(p->d_rowIdx); (void)hipFree(p->d_a2b_raw); (void)hipFree(p->d_a2b);
+    (void)hipFree(p->d_data); (void)hipFree(p->d_ranges); (void)hipFree(p->d_split); (void)hipFree(p->d_fix_slots);
+    (void)hipFree(p->d_scratch);
+    delete p;
+}
+
+int hspmm_run(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream)
+{
+    if (!p) return fail(HSPMM_ERR_INVALID, "null plan");
+    if (N == 0) return fail(HSPMM_ERR_INVALID, "feature dimension N = 0");
+    if (p->rows == 0) return HSPMM_OK;
+    if (!dC) return fail(HSPMM_ERR_INVALID, "null C");
+    if (!dB && p->W) return fail(HSPMM_ERR_INVALID, "null B");
+    if (reinterpret_cast<uintptr_t>(dC) % p->elem || reinterpret_cast<uintptr_t>(dB) % p->elem)
+        return fail(HSPMM_ERR_INVALID, "B and C must be aligned to the element size");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (p->W == 0) {
+        HSPMM_HIP(hspmm::launch_fill_zero(dC, size_t(p->rows) * N * p->elem, s));
+        return HSPMM_OK;
+    }
+    const Choice c = choose_kernel(p, dB, dC, N);
+    hspmm::KernelArgs ka{};
+    ka.rowOffset = p->d_rowOffset; ka.data = p->d_data; ka.rowIdx = p->d_rowIdx;
+    ka.B = dB; ka.C = dC;
+    ka.eff_windows = p->W; ka.rows = p->rows; ka.N = N;
+    if (c.scalar) {
+        ka.tcA2B = p->d_a2b_raw;
+        HSPMM_HIP(hspmm::launch_spmm_scalar(p->dtype, ka, s));
+        return HSPMM_OK;
+    }
+    ka.tcA2B = p->d_a2b;
+    ka.ranges = p->d_ranges; ka.split = p->d_split; ka.fix_slots = p->d_fix_slots;
+    ka.n_ranges = uint32_t(p->part.ranges.size());
+    ka.n_split = uint32_t(p->part.split.size());
+    ka.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
+    if (uint64_t(ka.n_ranges) * ka.n_feat_blocks > 0x7FFFFFFFull)
+        return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many work items", N);
+    const size_t need = size_t(p->part.n_slots) * ka.n_feat_blocks * size_t(c.V) * 64u * 16u;
+    int rc = ensure_scratch(p, need);
+    if (rc) return rc;
+    ka.scratch = p->d_scratch;
+    const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage : (p->dtype == HSPMM_FP16 ? 3 : 4);
+    const int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
+    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, c.layout, ka, c.V, prefetch, c.narrow, wpg, s));
+    return HSPMM_OK;
+}
+
+int hspmm_bench(hspmm_plan *p, const void *dB, void *dC, uint32_t N, int warmup, int runs, void *stream,
+                float *total_ms)
+{
+    if (!total_ms) return fail(HSPMM_ERR_INVALID, "null total_ms");
+    if (warmup < 0 || runs < 1) return fail(HSPMM_ERR_INVALID, "warmup %d / runs %d", warmup, runs);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rc;
+    for (int i = 0; i < warmup; ++i)
+        if ((rc = hspmm_run(p, dB, dC, N, stream))) return rc;
+    hipEvent_t a, b;
+    HSPMM_HIP(hipEventCreate(&a));
+    HSPMM_HIP(hipEventCreate(&b));
+    HSPMM_HIP(hipEventRecord(a, s));
+    for (int i = 0; i < runs; ++i)
+        if ((rc = hspmm_run(p, dB, dC, N, stream))) { (void)hipEventDestroy(a); (void)hipEventDestroy(b); return rc; }
+    HSPMM_HIP(hipEventRecord(b, s));
+    HSPMM_HIP(hipEventSynchronize(b));
+    HSPMM_HIP(hipEventElapsedTime(total_ms, a, b));
+    HSPMM_HIP(hipEventDestroy(a));
+    HSPMM_HIP(hipEventDestroy(b));
+    return HSPMM_OK;
+}
+
+int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
+{
+    if (!p || !info) return fail(HSPMM_ERR_INVALID, "null argument");
+    info->rows = p->rows; info->cols = p->cols; info->eff_row_windows = p->W; info->total_tiles = p->T;
+    info->dtype = p->dtype;
+    info->n_ranges = uint32_t(p->part.ranges.size());
+    info->n_split_windows = uint32_t(p->part.split.size());
+    info->n_partial_slots = p->part.n_slots;
+    info->compute_units = uint32_t(p->compute_units);
+    info->device_bytes = uint64_t(p->fixed_bytes) + uint64_t(p->scratch_bytes);
+    return HSPMM_OK;
+}
+
+int hspmm_get_partition(const hspmm_plan *p, uint32_t *ranges, uint32_t capacity_ranges)
+{
+    if (!p || !ranges) return fail(HSPMM_ERR_INVALID, "null argument");
+    const size_t n = p->part.ranges.size() < capacity_ranges ? p->part.ranges.size() : capacity_ranges;
+    for (size_t i = 0; i < n; ++i) {
+        ranges[5 * i + 0] = p->part.ranges[i].tile_begin; ranges[5 * i + 1] = p->part.ranges[i].tile_end;
+        ranges[5 * i + 2] = p->part.ranges[i].first_window;
+        ranges[5 * i + 3] = p->part.ranges[i].head_slot; ranges[5 * i + 4] = p->part.ranges[i].tail_slot;
+    }
+    return HSPMM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,44 @@
+// Shared between the kernels and the C ABI layer: kernel argument block and
+// launch entry points.  Internal; the public interface is include/hspmm.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+namespace hspmm {
+
+constexpr uint32_t kIdxMax = 0xFFFFFFFFu;      // reference src/common.h:47
+constexpr uint32_t kRowWindow = 8u;            // reference src/common.h:17
+constexpr uint32_t kRangeWordsDev = 8u;
+constexpr uint32_t kRangeWords = kRangeWordsDev;
+constexpr uint32_t kFixWords = 4u;
+constexpr int kMaxWavesPerGroup = 4;
+
+struct KernelArgs {
+    // the four format arrays (device copies), reference src/fp16.cu:38-41
+    const uint32_t *rowOffset;
+    const uint32_t *tcA2B;       // MFMA kernels: padding ids renamed; scalar kernel: as given
+    const void     *data;
+    const uint32_t *rowIdx;
+    // partition
+    const uint32_t *ranges;      // n_ranges x kRangeWords
+    const uint32_t *split;       // n_split x kFixWords {window, slot_begin, slot_count, 0}
+    const uint32_t *fix_slots;
+    float          *scratch;     // partial sums: [slot][feature block][acc reg][lane] x 4 floats
+    const void     *B;           // cols x N
+    void           *C;           // rows x N
+    uint32_t n_ranges, n_split, eff_windows, rows, N, n_feat_blocks;
+};
+
+// dtype: 0 = fp16 tiles 8x16, 1 = fp32 tiles 8x8.  V = 32-bit words a lane loads
+// per B row (1, 2 or 4).
+// layout (fp16 only): kLayoutX4 = wide loads, contiguous features per lane, N % (2V) == 0;
+// kLayoutDW = word loads, features strided by 32 per lane, N % (32V) == 0.
+constexpr int kLayoutX4 = 0, kLayoutDW = 1;
+// narrow: B < 4 GiB and cols < 2^24 (32-bit gather offsets).
+hipError_t launch_spmm_mfma(int dtype, int layout, const KernelArgs &ka, int V, int prefetch, bool narrow,
+                            int waves_per_group, hipStream_t s);
+hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s);
+hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
+
+}  // namespace hspmm

@@ -1,0 +1,316 @@
+// Host-side format functions of the C ABI (include/hspmm.h): MatrixMarket
+// loading and the CSR -> condensed-tile conversion.  They produce the same arrays
+// as the reference's load_matrix (reference src/utils/load.h:152-322) and
+// CSR2BTCFNOBITMAP (reference src/utils/convert.h:146-225), built differently:
+// whole-file parsing with strtoul/strtof, a counting sort by row, and a
+// two-pass, multi-threaded window conversion without hash maps.
+#include <algorithm>
+#include <cerrno>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "../../include/hspmm.h"
+
+namespace hspmm_host {
+
+// Stores the text hspmm_last_error() returns on this thread (defined beside it).
+void set_error(const std::string &msg);
+
+// IEEE binary32 -> binary16, round to nearest even (what __float2half does on
+// the host, reference src/utils/load.h:226).
+static uint16_t float_to_half_bits(float f)
+{
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    x &= 0x7FFFFFFFu;
+    if (x > 0x7F800000u) return uint16_t(sign | 0x7E00u | ((x >> 13) & 0x1FFu));   // NaN (quiet)
+    if (x >= 0x477FF000u) return uint16_t(sign | 0x7C00u);                         // overflow -> inf
+    if (x >= 0x38800000u) {                                                        // normal half
+        const uint32_t mant = x & 0x1FFFu;                                         // 13 dropped bits
+        uint32_t h = (x - 0x38000000u) >> 13;                                      // rebias 127 -> 15
+        if (mant > 0x1000u || (mant == 0x1000u && (h & 1u))) ++h;
+        return uint16_t(sign | h);
+    }
+    if (x < 0x33000001u) return uint16_t(sign);                                    // underflow -> 0
+    // subnormal half: value = m * 2^(e-150) with 24-bit m; unit of the result is 2^-24
+    const int e = int(x >> 23);
+    const uint32_t m = (x & 0x7FFFFFu) | 0x800000u;
+    const int shift = 126 - e;                                                     // 14..24
+    uint32_t h = m >> shift;
+    const uint32_t rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (h & 1u))) ++h;
+    return uint16_t(sign | h);
+}
+
+static unsigned worker_count(size_t work_items, size_t min_per_worker)
+{
+    unsigned hw = std::thread::hardware_concurrency();
+    if (hw == 0) hw = 1;
+    if (hw > 16) hw = 16;
+    size_t by_work = work_items / (min_per_worker ? min_per_worker : 1);
+    if (by_work < 1) by_work = 1;
+    return unsigned(std::min<size_t>(hw, by_work));
+}
+
+template <class F>
+static void parallel_blocks(size_t n, size_t min_per_worker, F &&fn)
+{
+    const unsigned nw = worker_count(n, min_per_worker);
+    if (nw <= 1) { fn(size_t(0), n); return; }
+    std::vector<std::thread> th;
+    th.reserve(nw);
+    for (unsigned i = 0; i < nw; ++i) {
+        const size_t b = n * i / nw, e = n * (i + 1) / nw;
+        th.emplace_back([&fn, b, e] { fn(b, e); });
+    }
+    for (auto &t : th) t.join();
+}
+
+// One parsed text line in the manner of sscanf(line, "%u %u %f") == 3
+// (reference src/utils/load.h:219).
+static bool parse_triple(const char *p, uint32_t &r, uint32_t &c, float &v)
+{
+    char *end;
+    auto parse_u = [&](uint32_t &out) -> bool {
+        while (*p == ' ' || *p == '\t' || *p == '\n' || *p == '\v' || *p == '\f' || *p == '\r') ++p;
+        const char *q = p;
+        if (*q == '+' || *q == '-') ++q;
+        if (*q < '0' || *q > '9') return false;
+        errno = 0;
+        const unsigned long val = std::strtoul(p, &end, 10);
+        out = uint32_t(val);
+        p = end;
+        return true;
+    };
+    if (!parse_u(r) || !parse_u(c)) return false;
+    errno = 0;
+    const float f = std::strtof(p, &end);
+    if (end == p) return false;
+    v = f;
+    return true;
+}
+
+struct Triples {
+    uint32_t rows = 0, cols = 0, declared = 0;
+    std::vector<uint32_t> r, c;
+    std::vector<float> v;
+};
+
+// Reads the file the way the reference's fgets loop sees it: pieces of at most
+// 1023 characters ending at a newline (reference src/utils/load.h:155, 183, 215).
+static int read_triples(const char *path, Triples &t, std::string &err)
+{
+    FILE *f = std::fopen(path, "rb");
+    if (!f) { err = std::string("cannot open file ") + path; return HSPMM_ERR_IO; }
+    std::string text;
+    {
+        char buf[1 << 16];
+        size_t n;
+        while ((n = std::fread(buf, 1, sizeof buf, f)) > 0) text.append(buf, n);
+    }
+    std::fclose(f);
+    size_t pos = 0;
+    std::string line;
+    auto next_line = [&]() -> bool {
+        if (pos >= text.size()) return false;
+        size_t e = pos;
+        const size_t limit = std::min(text.size(), pos + 1023);
+        while (e < limit && text[e] != '\n') ++e;
+        if (e < limit) ++e;                         // keep the newline, like fgets
+        line.assign(text, pos, e - pos);
+        pos = e;
+        return true;
+    };
+    bool have = false;
+    while (next_line()) { have = true; if (line[0] != '%') break; }     // load.h:183-187
+    unsigned rows, cols, nnz;
+    if (!have || std::sscanf(line.c_str(), "%u %u %u", &rows, &cols, &nnz) != 3) {   // load.h:190
+        err = std::string("cannot parse the size line of ") + path;
+        return HSPMM_ERR_IO;
+    }
+    t.rows = rows; t.cols = cols; t.declared = nnz;
+    t.r.reserve(nnz); t.c.reserve(nnz); t.v.reserve(nnz);
+    while (t.r.size() < nnz && next_line()) {                           // load.h:215
+        uint32_t r, c; float v;
+        if (parse_triple(line.c_str(), r, c, v)) {
+            t.r.push_back(r - 1u); t.c.push_back(c - 1u); t.v.push_back(v);   // load.h:221-222
+        }
+    }
+    return HSPMM_OK;
+}
+
+}  // namespace hspmm_host
+
+using namespace hspmm_host;
+
+extern "C" {
+
+int hspmm_mtx_load(const char *path, int dtype, hspmm_csr *out)
+{
+    if (!path || !out) { set_error("null argument"); return HSPMM_ERR_INVALID; }
+    std::memset(out, 0, sizeof *out);
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    Triples t;
+    std::string err;
+    int rc = read_triples(path, t, err);
+    if (rc) { set_error(err); return rc; }
+    const size_t nnz = t.r.size();
+    if (nnz != t.declared)                                              // load.h:234-238
+        std::fprintf(stderr, "warning: %s declares %u entries, %zu were read\n", path, t.declared, nnz);
+    for (size_t i = 0; i < nnz; ++i)
+        if (t.r[i] >= t.rows || t.c[i] >= t.cols) {
+            set_error("entry " + std::to_string(i) + " of " + path + " lies outside the declared shape");
+            return HSPMM_ERR_IO;
+        }
+    const size_t es = dtype == HSPMM_FP16 ? 2 : 4;
+    uint32_t *row_ptr = static_cast<uint32_t *>(std::calloc(size_t(t.rows) + 1, 4));
+    uint32_t *col_idx = static_cast<uint32_t *>(std::malloc((nnz ? nnz : 1) * 4));
+    void *values = std::malloc((nnz ? nnz : 1) * es);
+    if (!row_ptr || !col_idx || !values) {
+        std::free(row_ptr); std::free(col_idx); std::free(values);
+        set_error("out of host memory");
+        return HSPMM_ERR_ALLOC;
+    }
+    // counting sort by row (stable), then a stable sort by column inside each row:
+    // the (row, column) order of load.h:137-145, with file order kept for equal keys
+    for (size_t i = 0; i < nnz; ++i) row_ptr[t.r[i] + 1]++;
+    for (uint32_t r = 0; r < t.rows; ++r) row_ptr[r + 1] += row_ptr[r];
+    std::vector<uint32_t> order(nnz), cursor(row_ptr, row_ptr + t.rows);
+    for (size_t i = 0; i < nnz; ++i) order[cursor[t.r[i]]++] = uint32_t(i);
+    parallel_blocks(t.rows, 4096, [&](size_t rb, size_t re) {
+        for (size_t r = rb; r < re; ++r)
+            std::stable_sort(order.begin() + row_ptr[r], order.begin() + row_ptr[r + 1],
+                             [&](uint32_t a, uint32_t b) { return t.c[a] < t.c[b]; });
+    });
+    for (size_t i = 0; i < nnz; ++i) {
+        const uint32_t s = order[i];
+        col_idx[i] = t.c[s];
+        if (es == 2) static_cast<uint16_t *>(values)[i] = float_to_half_bits(t.v[s]);
+        else static_cast<float *>(values)[i] = t.v[s];
+    }
+    out->rows = t.rows; out->cols = t.cols; out->nnzs = uint32_t(nnz);
+    out->row_ptr = row_ptr; out->col_idx = col_idx; out->values = values;
+    return HSPMM_OK;
+}
+
+void hspmm_csr_free(hspmm_csr *m)
+{
+    if (!m) return;
+    std::free(m->row_ptr); std::free(m->col_idx); std::free(m->values);
+    std::memset(m, 0, sizeof *m);
+}
+
+}  // extern "C"
+
+namespace hspmm_host {
+
+// Distinct sorted column ids of rows [r0, r1) into `uniq`; returns their number.
+static uint32_t window_columns(const uint32_t *row_ptr, const uint32_t *col_idx, uint32_t r0, uint32_t r1,
+                               std::vector<uint32_t> &uniq)
+{
+    const uint32_t b = row_ptr[r0], e = row_ptr[r1];
+    uniq.assign(col_idx + b, col_idx + e);
+    std::sort(uniq.begin(), uniq.end());
+    uniq.erase(std::unique(uniq.begin(), uniq.end()), uniq.end());
+    return uint32_t(uniq.size());
+}
+
+// tiles[w] = number of tiles of window w (0 for a window without entries).
+static void count_tiles(uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx, uint32_t cw,
+                        std::vector<uint32_t> &tiles)
+{
+    const size_t nwin = (size_t(rows) + HSPMM_ROW_WINDOW - 1) / HSPMM_ROW_WINDOW;
+    tiles.assign(nwin, 0u);
+    parallel_blocks(nwin, 2048, [&](size_t wb, size_t we) {
+        std::vector<uint32_t> uniq;
+        for (size_t w = wb; w < we; ++w) {
+            const uint32_t r0 = uint32_t(w * HSPMM_ROW_WINDOW);
+            const uint32_t r1 = std::min<uint64_t>(uint64_t(r0) + HSPMM_ROW_WINDOW, rows);
+            if (row_ptr[r1] == row_ptr[r0]) continue;                       // convert.h:162
+            const uint32_t u = window_columns(row_ptr, col_idx, r0, r1, uniq);
+            tiles[w] = (u + cw - 1) / cw;                                   // convert.h:178-185
+        }
+    });
+}
+
+}  // namespace hspmm_host
+
+extern "C" {
+
+int hspmm_btcf_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                     uint32_t *eff_row_windows, uint32_t *total_tiles)
+{
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    if (!row_ptr || !eff_row_windows || !total_tiles || (!col_idx && row_ptr[rows])) {
+        set_error("null argument");
+        return HSPMM_ERR_INVALID;
+    }
+    const uint32_t cw = dtype == HSPMM_FP16 ? 16u : 8u;
+    std::vector<uint32_t> tiles;
+    count_tiles(rows, row_ptr, col_idx, cw, tiles);
+    uint64_t W = 0, T = 0;
+    for (uint32_t t : tiles) { W += t != 0; T += t; }
+    if (T > 0xFFFFFFFFull) { set_error("tile count exceeds 32 bits"); return HSPMM_ERR_UNSUPPORTED; }
+    *eff_row_windows = uint32_t(W);
+    *total_tiles = uint32_t(T);
+    return HSPMM_OK;
+}
+
+int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                    const void *values, int transpose, uint32_t *rowOffset, uint32_t *tcA2B, void *data,
+                    uint32_t *rowIdx)
+{
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    if (!row_ptr || !rowOffset) { set_error("null argument"); return HSPMM_ERR_INVALID; }
+    const uint32_t cw = dtype == HSPMM_FP16 ? 16u : 8u;
+    const size_t es = dtype == HSPMM_FP16 ? 2 : 4;
+    const size_t tile_elems = size_t(HSPMM_ROW_WINDOW) * cw;
+    std::vector<uint32_t> tiles;
+    count_tiles(rows, row_ptr, col_idx, cw, tiles);
+    const size_t nwin = tiles.size();
+    // exclusive scans: effective-window index and first tile of every window
+    std::vector<uint32_t> eff_index(nwin + 1, 0u), first_tile(nwin + 1, 0u);
+    for (size_t w = 0; w < nwin; ++w) {
+        eff_index[w + 1] = eff_index[w] + (tiles[w] != 0);
+        first_tile[w + 1] = first_tile[w] + tiles[w];
+    }
+    rowOffset[0] = 0;                                                        // convert.h:152
+    if (first_tile[nwin] && (!tcA2B || !data || !rowIdx || !col_idx || !values)) {
+        set_error("null argument");
+        return HSPMM_ERR_INVALID;
+    }
+    parallel_blocks(nwin, 2048, [&](size_t wb, size_t we) {
+        std::vector<uint32_t> uniq;
+        for (size_t w = wb; w < we; ++w) {
+            if (!tiles[w]) continue;
+            const uint32_t r0 = uint32_t(w * HSPMM_ROW_WINDOW);
+            const uint32_t r1 = std::min<uint64_t>(uint64_t(r0) + HSPMM_ROW_WINDOW, rows);
+            const uint32_t u = window_columns(row_ptr, col_idx, r0, r1, uniq);
+            const uint32_t ew = eff_index[w], ft = first_tile[w], nt = tiles[w];
+            rowOffset[ew + 1] = ft + nt;                                     // convert.h:186
+            rowIdx[ew] = r0;                                                 // convert.h:187
+            uint32_t *ids = tcA2B + size_t(ft) * cw;
+            for (uint32_t i = 0; i < nt * cw; ++i) ids[i] = i < u ? uniq[i] : HSPMM_IDX_MAX;   // convert.h:178-184
+            unsigned char *win = static_cast<unsigned char *>(data) + size_t(ft) * tile_elems * es;
+            std::memset(win, 0, size_t(nt) * tile_elems * es);               // convert.h:191-193
+            for (uint32_t r = r0; r < r1; ++r)
+                for (uint32_t id = row_ptr[r]; id < row_ptr[r + 1]; ++id) {  // stored order: a later duplicate wins
+                    const uint32_t rank = uint32_t(std::lower_bound(uniq.begin(), uniq.end(), col_idx[id]) - uniq.begin());
+                    const uint32_t tc = rank / cw, lc = rank % cw, lr = r % HSPMM_ROW_WINDOW;
+                    const size_t off = transpose ? size_t(lc) * HSPMM_ROW_WINDOW + lr       // convert.h:209
+                                                 : size_t(lr) * cw + lc;                    // convert.h:212
+                    std::memcpy(win + (size_t(tc) * tile_elems + off) * es,
+                                static_cast<const unsigned char *>(values) + size_t(id) * es, es);
+                }
+        }
+    });
+    return HSPMM_OK;
+}
+
+}  // extern "C"

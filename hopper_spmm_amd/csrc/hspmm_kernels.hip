@@ -1,0 +1,693 @@
+// gfx950 (MI355X) kernels for C = A * B with A in the condensed 8-row-window
+// tile format (reference src/utils/class.h:74-85).  They replace the reference's
+// fp16_spmm_kernel (reference src/fp16.cu:36-175) and supply the fp32-storage
+// ("tf32") variant the reference only sketches (src/common.h:26-43).
+//
+// Design (one wave = one independent pipeline, no LDS, no barriers):
+//   * A wave owns a contiguous range of tiles (a few hundred) of the flat tile
+//     sequence and, for feature dimensions wider than one block, one feature
+//     block.  Windows are contiguous in the tile sequence, so the loads stream
+//     through the range without regard to window boundaries; only the MFMA
+//     stage looks at them (to store a finished window and clear accumulators).
+//   * Per fp16 tile a lane issues one 16-byte load of four column ids, one
+//     8-byte load of its part of the sparse tile and four loads of 4*V bytes
+//     from the four B rows those ids name; the 16 lanes of a quarter-wave cover
+//     one B row contiguously, a whole wave four rows per instruction.
+//   * fp16 contraction without any transposition of B: an MFMA operand register
+//     holds two k-slots.  A B register as loaded holds features (2c, 2c+1) of one
+//     gathered row, i.e. "k-slot pair" = (even feature, odd feature).  The sparse
+//     operand is built so that MFMA row 2r holds a[r][k] in the even slot and 0 in
+//     the odd one, MFMA row 2r+1 the reverse.  Output row 2r then is window row r
+//     for the even features, row 2r+1 for the odd ones: all 16 MFMA rows and all
+//     32 k-slots do useful work for an 8-row window, and a lane ends up with
+//     contiguous features of two window rows, which it stores with wide stores.
+//   * fp32 ("tf32") contraction uses v_mfma_f32_16x16x4_f32; one B register per
+//     lane per k, no packing issue; MFMA rows 8..15 are zero padding.
+//   * Loads for tile t+P are issued before the MFMAs of tile t (P = prefetch
+//     depth, registers as the ring buffer); hardware returns vector loads in
+//     order, so the wait before the MFMAs of tile t leaves P-1 tiles in flight.
+//   * Padding columns (id 0xFFFFFFFF) are renamed, in the plan's device copy of the
+//     ids, to the real column in front of them; their tile column is all zero.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "hspmm_device.h"
+
+namespace hspmm {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float    f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int V> struct Vec;
+template <> struct Vec<1> { typedef uint32_t type; };
+template <> struct Vec<2> { typedef u32x2 type; };
+template <> struct Vec<4> { typedef u32x4 type; };
+
+template <int V>
+__device__ __forceinline__ void load_words(const void *p, uint32_t (&dst)[V])
+{
+    typename Vec<V>::type v = *reinterpret_cast<const typename Vec<V>::type *>(p);
+    if constexpr (V == 1) dst[0] = v;
+    else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) dst[i] = v[i];
+    }
+}
+
+template <int V>
+__device__ __forceinline__ void store_words(void *p, const uint32_t (&src)[V])
+{
+    typename Vec<V>::type v;
+    if constexpr (V == 1) v = src[0];
+    else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) v[i] = src[i];
+    }
+    *reinterpret_cast<typename Vec<V>::type *>(p) = v;
+}
+
+template <int V>
+__device__ __forceinline__ void unpack(const typename Vec<V>::type v, uint32_t (&dst)[V])
+{
+    if constexpr (V == 1) dst[0] = v;
+    else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) dst[i] = v[i];
+    }
+}
+
+__device__ __forceinline__ uint32_t pack_half2_rn(float lo, float hi)
+{
+    // float -> half conversion in the default rounding mode (nearest even), as the
+    // reference's store does (src/fp16.cu:167, cvt.rn.f16.f32).
+    _Float16 l = (_Float16)lo, h = (_Float16)hi;
+    uint16_t lb = __builtin_bit_cast(uint16_t, l), hb = __builtin_bit_cast(uint16_t, h);
+    return uint32_t(lb) | (uint32_t(hb) << 16);
+}
+
+__device__ __forceinline__ uint32_t umin32(uint32_t a, uint32_t b) { return a < b ? a : b; }
+
+// ---------------------------------------------------------------------------
+// Element-type traits: how one tile is loaded, multiplied and stored.
+// ---------------------------------------------------------------------------
+// Uniform (per-wave) reads of the small index arrays go through the constant
+// address space so that they become scalar loads, which do not share the
+// in-order return queue of the vector loads that stream the tiles.
+typedef const uint32_t __attribute__((address_space(4))) *const_u32_ptr;
+__device__ __forceinline__ const_u32_ptr as_const(const uint32_t *p)
+{
+    return (const_u32_ptr)(uintptr_t)p;
+}
+
+// Where a lane reads its 4*V bytes of B row c.  The column ids the MFMA kernels see
+// are the plan's device copy in which every padding id has been replaced by the
+// id in front of it (a real column of the same tile): the sparse tile holds zeros
+// in a padding column, so the product is the same, and no lane ever needs a
+// bounds test or a second base pointer.  NARROW: B is smaller than 4 GiB and has
+// fewer than 2^24 rows, so one 24-bit multiply-add gives a 32-bit offset from a
+// scalar base.
+template <bool NARROW>
+struct Gather {
+    const char *base;        // B (uniform)
+    uint32_t row_bytes;      // N * element size
+    uint32_t lane_off;       // byte offset of the lane's first feature inside a row
+    __device__ __forceinline__ const char *row(uint32_t c) const
+    {
+        if constexpr (NARROW) {
+            const uint32_t off = __umul24(c, row_bytes) + lane_off;
+            return base + size_t(off);
+        } else {
+            return base + (size_t(c) * row_bytes + lane_off);
+        }
+    }
+};
+
+// Common part of the two fp16 layouts: the sparse operand.
+struct Fp16Lane {
+    uint32_t g, j;                             // quarter-wave, lane in quarter
+    uint32_t sel_lo, sel_hi;                   // byte selectors for the sparse operand
+    const uint32_t *a_src;                     // lane's words inside tile 0
+    const uint32_t *idx_src;                   // lane's ids inside tile 0
+    __device__ __forceinline__ void init(uint32_t lane, const void *data, const uint32_t *tcA2B)
+    {
+        g = lane >> 4; j = lane & 15u;
+        const uint32_t r = j >> 1, parity = j & 1u;
+        // v_perm_b32 selectors: bytes 0-3 come from the second source, 0x0c gives 0x00.
+        //   even MFMA row: value in the low half  -> {lo: b0 b1 0 0}, {hi: b2 b3 0 0}
+        //   odd  MFMA row: value in the high half -> {lo: 0 0 b0 b1}, {hi: 0 0 b2 b3}
+        sel_lo = parity ? 0x01000c0cu : 0x0c0c0100u;
+        sel_hi = parity ? 0x03020c0cu : 0x0c0c0302u;
+        a_src = reinterpret_cast<const uint32_t *>(data) + r * 8u + g * 2u;
+        idx_src = tcA2B + g * 4u;
+    }
+    // MFMA row 2r carries a[r][k] in the even k-slot of each pair, row 2r+1 in the odd one.
+    __device__ __forceinline__ half8_t sparse_operand(const u32x2 &a) const
+    {
+        u32x4 aw;
+        aw[0] = __builtin_amdgcn_perm(0u, a[0], sel_lo);
+        aw[1] = __builtin_amdgcn_perm(0u, a[0], sel_hi);
+        aw[2] = __builtin_amdgcn_perm(0u, a[1], sel_lo);
+        aw[3] = __builtin_amdgcn_perm(0u, a[1], sel_hi);
+        return __builtin_bit_cast(half8_t, aw);
+    }
+};
+
+// fp16, layout "X4": a lane reads 4*V contiguous bytes of each of its four B rows
+// (one wide load per row) and owns 2*V contiguous features.  Any N that is a
+// multiple of 2*V.  The B operand of MFMA p is word p of the four loads, which
+// costs register moves.
+template <int V>
+struct Fp16Tile {
+    static constexpr int kCW = 16;                 // tile columns (src/common.h:18)
+    static constexpr int kBlockFeat = 32 * V;      // features one wave covers
+    static constexpr int kLaneFeat = 2 * V;        // lane's first feature = j * kLaneFeat
+    static constexpr int kElem = 2;
+    static constexpr int kAcc = V;                 // f32x4 accumulators per lane
+    typedef typename Vec<V>::type BVec;
+    typedef u32x4 Idx;                             // four column ids per lane per tile
+    typedef Fp16Lane Lane;
+
+    __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t tile)
+    {
+        return *reinterpret_cast<const u32x4 *>(L.idx_src + size_t(tile) * 16u);
+    }
+    // The registers of one tile in flight are separate variables of the caller
+    // (b0..b3: the lane's words of four B rows, a: its two words of the sparse tile).
+    template <class G>
+    __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t tile, const Idx idx, const G &gat,
+                                                     BVec &b0, BVec &b1, BVec &b2, BVec &b3, u32x2 &a)
+    {
+        b0 = *reinterpret_cast<const BVec *>(gat.row(idx[0]));
+        b1 = *reinterpret_cast<const BVec *>(gat.row(idx[1]));
+        b2 = *reinterpret_cast<const BVec *>(gat.row(idx[2]));
+        b3 = *reinterpret_cast<const BVec *>(gat.row(idx[3]));
+        a = *reinterpret_cast<const u32x2 *>(L.a_src + size_t(tile) * 64u);
+    }
+    template <int p> __device__ static __forceinline__ uint32_t word(const BVec &v)
+    {
+        if constexpr (V == 1) return v; else return v[p];
+    }
+    template <int p>
+    __device__ static __forceinline__ void mma_one(const half8_t av, const BVec &b0, const BVec &b1, const BVec &b2,
+                                                   const BVec &b3, f32x4 (&acc)[kAcc])
+    {
+        if constexpr (p < V) {
+            u32x4 bw;
+            bw[0] = word<p>(b0); bw[1] = word<p>(b1); bw[2] = word<p>(b2); bw[3] = word<p>(b3);
+            acc[p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, bw), acc[p], 0, 0, 0);
+        }
+    }
+    __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
+                                               const BVec &b3, const u32x2 &a, f32x4 (&acc)[kAcc])
+    {
+        const half8_t av = L.sparse_operand(a);
+        mma_one<0>(av, b0, b1, b2, b3, acc); mma_one<1>(av, b0, b1, b2, b3, acc);
+        mma_one<2>(av, b0, b1, b2, b3, acc); mma_one<3>(av, b0, b1, b2, b3, acc);
+    }
+    // acc[p][e]: MFMA row 4g+e = window row 2g + e/2, feature lane_feat + 2p + (e & 1).
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[kAcc], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+            const uint32_t row = row0 + 2u * L.g + rr;
+            uint32_t out[V];
+#pragma unroll
+            for (int p = 0; p < V; ++p) out[p] = pack_half2_rn(acc[p][2 * rr], acc[p][2 * rr + 1]);
+            if (active && row < rows) store_words<V>(c_lane + size_t(row) * row_bytes, out);
+        }
+    }
+    // Zero rows [r_begin, r_end) of this lane's features.
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        uint32_t z[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) z[i] = 0u;
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) store_words<V>(c_lane + size_t(r) * row_bytes, z);
+    }
+};
+
+// fp16, layout "DW": a lane reads single words, word p of a row at feature
+// 32p + 2j, so that the 16 lanes of a quarter-wave still read 64 contiguous
+// bytes, and the four words that form the B operand of MFMA p (one per B row)
+// are loaded straight into four consecutive registers: no moves.  Needs N to be
+// a multiple of 32*V.
+template <int V>
+struct Fp16TileDW {
+    static constexpr int kCW = 16;
+    static constexpr int kBlockFeat = 32 * V;
+    static constexpr int kLaneFeat = 2;            // lane's first feature = 2j, then +32 per word
+    static constexpr int kElem = 2;
+    static constexpr int kAcc = V;
+    typedef u32x4 BVec;                            // b_p = word p of the four B rows
+    typedef u32x4 Idx;
+    typedef Fp16Lane Lane;
+
+    __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t tile)
+    {
+        return *reinterpret_cast<const u32x4 *>(L.idx_src + size_t(tile) * 16u);
+    }
+    template <class G>
+    __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t tile, const Idx idx, const G &gat,
+                                                     BVec &b0, BVec &b1, BVec &b2, BVec &b3, u32x2 &a)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(gat.row(idx[q]));
+            b0[q] = src[0];
+            if constexpr (V > 1) b1[q] = src[16];
+            if constexpr (V > 2) b2[q] = src[32];
+            if constexpr (V > 3) b3[q] = src[48];
+        }
+        a = *reinterpret_cast<const u32x2 *>(L.a_src + size_t(tile) * 64u);
+    }
+    __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
+                                               const BVec &b3, const u32x2 &a, f32x4 (&acc)[kAcc])
+    {
+        const half8_t av = L.sparse_operand(a);
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, b0), acc[0], 0, 0, 0);
+        if constexpr (V > 1) acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, b1), acc[1], 0, 0, 0);
+        if constexpr (V > 2) acc[2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, b2), acc[2], 0, 0, 0);
+        if constexpr (V > 3) acc[3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, b3), acc[3], 0, 0, 0);
+    }
+    // acc[p][e]: MFMA row 4g+e = window row 2g + e/2, feature 32p + 2j + (e & 1).
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[kAcc], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+            const uint32_t row = row0 + 2u * L.g + rr;
+            if (active && row < rows) {
+                uint32_t *dst = reinterpret_cast<uint32_t *>(c_lane + size_t(row) * row_bytes);
+#pragma unroll
+                for (int p = 0; p < V; ++p) dst[16 * p] = pack_half2_rn(acc[p][2 * rr], acc[p][2 * rr + 1]);
+            }
+        }
+    }
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) {
+            uint32_t *dst = reinterpret_cast<uint32_t *>(c_lane + size_t(r) * row_bytes);
+#pragma unroll
+            for (int p = 0; p < V; ++p) dst[16 * p] = 0u;
+        }
+    }
+};
+
+// fp32 storage ("tf32" build of the reference): 8x8 tiles, v_mfma_f32_16x16x4_f32.
+// MFMA rows 0..7 are the window rows, rows 8..15 zero; lane (g, j) supplies k = g
+// and k = g + 4 of a tile and V contiguous features.
+template <int V>
+struct Fp32Tile {
+    static constexpr int kCW = 8;                  // src/common.h:41
+    static constexpr int kBlockFeat = 16 * V;
+    static constexpr int kLaneFeat = V;
+    static constexpr int kElem = 4;
+    static constexpr int kAcc = V;
+    typedef typename Vec<V>::type BVec;
+    typedef u32x2 Idx;                             // two column ids per lane per tile
+
+    struct Lane {
+        uint32_t g, j;
+        uint32_t a_mask;                           // all ones for MFMA rows 0..7, else 0
+        const uint32_t *a_src;
+        const uint32_t *idx_src;
+        __device__ __forceinline__ void init(uint32_t lane, const void *data, const uint32_t *tcA2B)
+        {
+            g = lane >> 4; j = lane & 15u;
+            a_mask = j < 8u ? 0xFFFFFFFFu : 0u;
+            a_src = reinterpret_cast<const uint32_t *>(data) + (j & 7u) * 8u + g;
+            idx_src = tcA2B + g;
+        }
+    };
+    __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t tile)
+    {
+        const uint32_t *p = L.idx_src + size_t(tile) * 8u;
+        Idx r; r[0] = p[0]; r[1] = p[4];
+        return r;
+    }
+    template <class G>
+    __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t tile, const Idx idx, const G &gat,
+                                                     BVec &b0, BVec &b1, BVec &, BVec &, u32x2 &a)
+    {
+        b0 = *reinterpret_cast<const BVec *>(gat.row(idx[0]));
+        b1 = *reinterpret_cast<const BVec *>(gat.row(idx[1]));
+        const uint32_t *p = L.a_src + size_t(tile) * 64u;
+        a[0] = p[0]; a[1] = p[4];
+    }
+    template <int p> __device__ static __forceinline__ float word(const BVec &v)
+    {
+        if constexpr (V == 1) return __builtin_bit_cast(float, v); else return __builtin_bit_cast(float, v[p]);
+    }
+    template <int p>
+    __device__ static __forceinline__ void mma_one(const float a0, const float a1, const BVec &b0, const BVec &b1,
+                                                   f32x4 (&acc)[kAcc])
+    {
+        if constexpr (p < V) {
+            acc[p] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, word<p>(b0), acc[p], 0, 0, 0);
+            acc[p] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, word<p>(b1), acc[p], 0, 0, 0);
+        }
+    }
+    __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &,
+                                               const BVec &, const u32x2 &a, f32x4 (&acc)[kAcc])
+    {
+        const float a0 = __builtin_bit_cast(float, a[0] & L.a_mask);
+        const float a1 = __builtin_bit_cast(float, a[1] & L.a_mask);
+        mma_one<0>(a0, a1, b0, b1, acc); mma_one<1>(a0, a1, b0, b1, acc);
+        mma_one<2>(a0, a1, b0, b1, acc); mma_one<3>(a0, a1, b0, b1, acc);
+    }
+    // acc[p][e]: MFMA row 4g+e (a window row when g < 2), feature lane_feat + p.
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[kAcc], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t row = row0 + 4u * L.g + e;
+            uint32_t out[V];
+#pragma unroll
+            for (int p = 0; p < V; ++p) out[p] = __builtin_bit_cast(uint32_t, acc[p][e]);
+            if (active && L.g < 2u && row < rows) store_words<V>(c_lane + size_t(row) * row_bytes, out);
+        }
+    }
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        uint32_t z[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) z[i] = 0u;
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) store_words<V>(c_lane + size_t(r) * row_bytes, z);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Main kernel: one wave per (tile range, feature block).
+// ---------------------------------------------------------------------------
+// State of the window walk (all wave-uniform, kept in scalar registers).
+struct WindowWalk {
+    uint32_t w;            // current effective window
+    uint32_t wstart, wend; // its tile span
+    uint32_t row0;         // its first matrix row
+    uint32_t next_row;     // first row of the next effective window (or rows)
+    uint32_t seg_start, seg_end;   // part of the span inside this wave's range
+};
+
+template <class TT, int V, int P, bool NARROW>
+__global__ __launch_bounds__(kMaxWavesPerGroup * 64, (P <= 4 ? 4 : 2))
+void spmm_mfma_kernel(const KernelArgs ka)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t item = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    if (item >= ka.n_ranges * ka.n_feat_blocks) return;
+    const uint32_t range = item / ka.n_feat_blocks;
+    const uint32_t fb = item - range * ka.n_feat_blocks;
+    const const_u32_ptr rd = as_const(ka.ranges) + size_t(range) * kRangeWords;
+    const const_u32_ptr rowOffset = as_const(ka.rowOffset);
+    const const_u32_ptr rowIdx = as_const(ka.rowIdx);
+    const uint32_t t0 = rd[0], t1 = rd[1];
+    const uint32_t head_slot = rd[3], tail_slot = rd[4];
+    const uint32_t W = ka.eff_windows, rows = ka.rows;
+
+    typename TT::Lane L;
+    L.init(lane, ka.data, ka.tcA2B);
+    const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
+    const bool active = feat < ka.N;
+    const size_t row_bytes = size_t(ka.N) * TT::kElem;
+    char *c_lane = reinterpret_cast<char *>(ka.C) + size_t(feat) * TT::kElem;
+    Gather<NARROW> gat;
+    gat.base = reinterpret_cast<const char *>(ka.B);
+    gat.row_bytes = uint32_t(row_bytes);
+    gat.lane_off = active ? feat * TT::kElem : 0u;     // lanes past N read (and drop) the row start
+
+    WindowWalk ww;
+    ww.w = rd[2];
+    ww.wstart = rowOffset[ww.w];
+    ww.wend = rowOffset[ww.w + 1u];
+    ww.row0 = rowIdx[ww.w];
+    ww.next_row = (ww.w + 1u < W) ? rowIdx[ww.w + 1u] : rows;
+    ww.seg_start = t0;
+    ww.seg_end = umin32(ww.wend, t1);
+
+    // Rows before the first effective window belong to the wave that starts at tile 0.
+    if (t0 == 0u) TT::zero_rows(L, c_lane, row_bytes, 0u, rowIdx[0], active);
+
+    f32x4 acc[TT::kAcc];
+#pragma unroll
+    for (int p = 0; p < TT::kAcc; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t tlast = t1 - 1u;
+    typedef typename TT::BVec BVec;
+#define HSPMM_DECL(k) BVec b0_##k, b1_##k, b2_##k, b3_##k; u32x2 a_##k; typename TT::Idx I##k;
+#define HSPMM_REGS(k) b0_##k, b1_##k, b2_##k, b3_##k, a_##k
+
+#define HSPMM_FOR_STAGES(X) \
+    X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7)
+    HSPMM_FOR_STAGES(HSPMM_DECL)
+#define HSPMM_PRO_IDX(k) if constexpr (P > k) I##k = TT::load_idx(L, umin32(t0 + k, tlast));
+#define HSPMM_PRO_TILE(k) if constexpr (P > k) { \
+        TT::load_tile(L, umin32(t0 + k, tlast), I##k, gat, HSPMM_REGS(k)); \
+        I##k = TT::load_idx(L, umin32(t0 + P + k, tlast)); \
+        __builtin_amdgcn_sched_barrier(0); }
+    // The order of the loads below must be the order of the steady state (the
+    // compiler derives the steady state's wait counts from both ways into the
+    // loop), hence the scheduling barriers.
+    HSPMM_FOR_STAGES(HSPMM_PRO_IDX)
+    __builtin_amdgcn_sched_barrier(0);
+    HSPMM_FOR_STAGES(HSPMM_PRO_TILE)
+
+    // MFMAs of `tile` from its registers, then the window bookkeeping.
+    auto compute = [&](const BVec &b0, const BVec &b1, const BVec &b2, const BVec &b3, const u32x2 &a,
+                       const uint32_t tile) __attribute__((always_inline)) {
+        TT::mma(L, b0, b1, b2, b3, a, acc);
+        if (tile + 1u == ww.seg_end) {
+            const bool complete = (ww.seg_start == ww.wstart) && (ww.seg_end == ww.wend);
+            if (complete) {
+                TT::store_window(L, acc, c_lane, row_bytes, ww.row0, rows, active);
+            } else {
+                const uint32_t slot = (ww.seg_start == t0) ? head_slot : tail_slot;
+                if (slot != kIdxMax) {
+                    f32x4 *dst = reinterpret_cast<f32x4 *>(ka.scratch) +
+                                 (size_t(slot) * ka.n_feat_blocks + fb) * (TT::kAcc * 64u) + lane;
+#pragma unroll
+                    for (int p = 0; p < TT::kAcc; ++p) dst[p * 64] = acc[p];
+                }
+            }
+            if (ww.seg_end == ww.wend) {
+                // this wave holds the window's last tile: it also clears the empty
+                // windows that follow (rows up to the next effective window)
+                const uint32_t gap_begin = ww.row0 + kRowWindow;
+                if (gap_begin < ww.next_row) TT::zero_rows(L, c_lane, row_bytes, gap_begin, ww.next_row, active);
+            }
+#pragma unroll
+            for (int p = 0; p < TT::kAcc; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+            // next window (the reads are clamped; values past the end are not used)
+            ++ww.w;
+            ww.wstart = ww.wend;
+            ww.wend = rowOffset[umin32(ww.w + 1u, W)];
+            ww.row0 = ww.next_row;
+            ww.next_row = (ww.w + 1u < W) ? rowIdx[ww.w + 1u] : rows;
+            ww.seg_start = ww.seg_end;
+            ww.seg_end = umin32(ww.wend, t1);
+        }
+    };
+
+    // Steady state: every stage computes its tile and reloads its registers with
+    // the tile P further on, without conditions, so that the wait in front of a
+    // stage's MFMAs leaves the loads of the P-1 younger stages in flight.
+    uint32_t t = t0;
+    for (; t + 2u * P <= t1; t += P) {
+#define HSPMM_STEADY(k) if constexpr (P > k) { \
+        compute(HSPMM_REGS(k), t + k); \
+        TT::load_tile(L, t + k + P, I##k, gat, HSPMM_REGS(k)); \
+        I##k = TT::load_idx(L, umin32(t + k + 2u * P, tlast)); \
+        __builtin_amdgcn_sched_barrier(0); }
+        HSPMM_FOR_STAGES(HSPMM_STEADY)
+    }
+    // Drain: fewer than 2P tiles are left; loads stop at the end of the range.
+    for (; t < t1; t += P) {
+#define HSPMM_DRAIN(k) if constexpr (P > k) { \
+        if (t + k < t1) compute(HSPMM_REGS(k), t + k); \
+        if (t + k + P < t1) { \
+            TT::load_tile(L, t + k + P, I##k, gat, HSPMM_REGS(k)); \
+            I##k = TT::load_idx(L, umin32(t + k + 2u * P, tlast)); } }
+        HSPMM_FOR_STAGES(HSPMM_DRAIN)
+    }
+#undef HSPMM_DRAIN
+#undef HSPMM_STEADY
+#undef HSPMM_PRO_TILE
+#undef HSPMM_PRO_IDX
+#undef HSPMM_REGS
+#undef HSPMM_DECL
+#undef HSPMM_FOR_STAGES
+}
+
+// ---------------------------------------------------------------------------
+// Second kernel: adds, in range order, the fp32 partial sums of every window
+// whose tiles were cut across ranges, and stores the window.
+// ---------------------------------------------------------------------------
+template <class TT, int V>
+__global__ __launch_bounds__(kMaxWavesPerGroup * 64)
+void spmm_fixup_kernel(const KernelArgs ka)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t item = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    if (item >= ka.n_split * ka.n_feat_blocks) return;
+    const uint32_t entry = item / ka.n_feat_blocks;
+    const uint32_t fb = item - entry * ka.n_feat_blocks;
+    const uint32_t *fx = ka.split + size_t(entry) * kFixWords;
+    const uint32_t w = fx[0], sb = fx[1], sc = fx[2];
+
+    typename TT::Lane L;
+    L.init(lane, ka.data, ka.tcA2B);
+    const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
+    const bool active = feat < ka.N;
+    const size_t row_bytes = size_t(ka.N) * TT::kElem;
+    char *c_lane = reinterpret_cast<char *>(ka.C) + size_t(feat) * TT::kElem;
+
+    f32x4 acc[TT::kAcc];
+#pragma unroll
+    for (int p = 0; p < TT::kAcc; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (uint32_t i = 0; i < sc; ++i) {
+        const uint32_t slot = ka.fix_slots[sb + i];
+        const f32x4 *src = reinterpret_cast<const f32x4 *>(ka.scratch) +
+                           (size_t(slot) * ka.n_feat_blocks + fb) * (TT::kAcc * 64u) + lane;
+#pragma unroll
+        for (int p = 0; p < TT::kAcc; ++p) acc[p] += src[p * 64];
+    }
+    TT::store_window(L, acc, c_lane, row_bytes, ka.rowIdx[w], ka.rows, active);
+}
+
+// ---------------------------------------------------------------------------
+// All-shapes kernel (any N, any alignment): one workgroup per effective window
+// and 256-feature slab, one thread per feature, plain fp32 multiply-add.  Used
+// when the feature dimension rules out the vector loads above (odd N in fp16),
+// and as an independent second implementation in tests.
+// ---------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<_Float16>(_Float16 v) { return (float)v; }
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ _Float16 from_f32<_Float16>(float v) { return (_Float16)v; }
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+
+template <typename T, int CW>
+__global__ __launch_bounds__(256)
+void spmm_scalar_kernel(const KernelArgs ka)
+{
+    const uint32_t w = blockIdx.x;
+    const uint32_t f = blockIdx.y * 256u + threadIdx.x;
+    const uint32_t N = ka.N, rows = ka.rows, W = ka.eff_windows;
+    const bool active = f < N;
+    const T *B = reinterpret_cast<const T *>(ka.B);
+    T *C = reinterpret_cast<T *>(ka.C);
+    const T *data = reinterpret_cast<const T *>(ka.data);
+    float acc[kRowWindow];
+#pragma unroll
+    for (uint32_t r = 0; r < kRowWindow; ++r) acc[r] = 0.f;
+    const uint32_t tb = ka.rowOffset[w], te = ka.rowOffset[w + 1];
+    for (uint32_t t = tb; t < te; ++t) {
+        for (uint32_t k = 0; k < CW; ++k) {
+            const uint32_t c = ka.tcA2B[size_t(t) * CW + k];
+            if (c == kIdxMax) continue;
+            const float b = active ? to_f32<T>(B[size_t(c) * N + f]) : 0.f;
+#pragma unroll
+            for (uint32_t r = 0; r < kRowWindow; ++r)
+                acc[r] = __builtin_fmaf(to_f32<T>(data[(size_t(t) * kRowWindow + r) * CW + k]), b, acc[r]);
+        }
+    }
+    if (!active) return;
+    const uint32_t row0 = ka.rowIdx[w];
+#pragma unroll
+    for (uint32_t r = 0; r < kRowWindow; ++r)
+        if (row0 + r < rows) C[size_t(row0 + r) * N + f] = from_f32<T>(acc[r]);
+    const uint32_t next_row = (w + 1u < W) ? ka.rowIdx[w + 1] : rows;
+    for (uint32_t r = row0 + kRowWindow; r < next_row; ++r) C[size_t(r) * N + f] = from_f32<T>(0.f);
+    if (w == 0u)
+        for (uint32_t r = 0; r < row0; ++r) C[size_t(r) * N + f] = from_f32<T>(0.f);
+}
+
+// Whole-matrix clear for a matrix without any stored entry (every row of C is 0).
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t *dst, size_t n_words, uint16_t *tail, int tail_halves)
+{
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n_words; i += stride) dst[i] = 0u;
+    if (blockIdx.x == 0 && threadIdx.x < (unsigned)tail_halves) tail[threadIdx.x] = 0;
+}
+
+// ---------------------------------------------------------------------------
+// Launch helpers (host).
+// ---------------------------------------------------------------------------
+template <class TT, int V, bool NARROW>
+static hipError_t launch_main_p(const KernelArgs &ka, int prefetch, dim3 grid, dim3 block, hipStream_t s)
+{
+    switch (prefetch) {
+    case 1: spmm_mfma_kernel<TT, V, 1, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 2: spmm_mfma_kernel<TT, V, 2, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 3: spmm_mfma_kernel<TT, V, 3, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 6: spmm_mfma_kernel<TT, V, 6, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 8: spmm_mfma_kernel<TT, V, 8, NARROW><<<grid, block, 0, s>>>(ka); break;
+    default: spmm_mfma_kernel<TT, V, 4, NARROW><<<grid, block, 0, s>>>(ka); break;
+    }
+    return hipGetLastError();
+}
+template <class TT, int V>
+static hipError_t launch_main_n(const KernelArgs &ka, int prefetch, bool narrow, dim3 grid, dim3 block, hipStream_t s)
+{
+    return narrow ? launch_main_p<TT, V, true>(ka, prefetch, grid, block, s)
+                  : launch_main_p<TT, V, false>(ka, prefetch, grid, block, s);
+}
+
+template <template <int> class TTV>
+static hipError_t launch_mfma(const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, hipStream_t s)
+{
+    const uint32_t items = ka.n_ranges * ka.n_feat_blocks;
+    const dim3 block(64u * waves_per_group);
+    const dim3 grid((items + waves_per_group - 1) / waves_per_group);
+    hipError_t e;
+    if (V == 4) e = launch_main_n<TTV<4>, 4>(ka, prefetch, narrow, grid, block, s);
+    else if (V == 2) e = launch_main_n<TTV<2>, 2>(ka, prefetch, narrow, grid, block, s);
+    else e = launch_main_n<TTV<1>, 1>(ka, prefetch, narrow, grid, block, s);
+    if (e != hipSuccess || ka.n_split == 0) return e;
+    const uint32_t fitems = ka.n_split * ka.n_feat_blocks;
+    const dim3 fgrid((fitems + waves_per_group - 1) / waves_per_group);
+    if (V == 4) spmm_fixup_kernel<TTV<4>, 4><<<fgrid, block, 0, s>>>(ka);
+    else if (V == 2) spmm_fixup_kernel<TTV<2>, 2><<<fgrid, block, 0, s>>>(ka);
+    else spmm_fixup_kernel<TTV<1>, 1><<<fgrid, block, 0, s>>>(ka);
+    return hipGetLastError();
+}
+
+hipError_t launch_spmm_mfma(int dtype, int layout, const KernelArgs &ka, int V, int prefetch, bool narrow,
+                            int waves_per_group, hipStream_t s)
+{
+    if (dtype != 0) return launch_mfma<Fp32Tile>(ka, V, prefetch, narrow, waves_per_group, s);
+    return layout == kLayoutDW ? launch_mfma<Fp16TileDW>(ka, V, prefetch, narrow, waves_per_group, s)
+                               : launch_mfma<Fp16Tile>(ka, V, prefetch, narrow, waves_per_group, s);
+}
+
+hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s)
+{
+    const dim3 grid(ka.eff_windows, (ka.N + 255u) / 256u);
+    if (dtype == 0) spmm_scalar_kernel<_Float16, 16><<<grid, 256, 0, s>>>(ka);
+    else spmm_scalar_kernel<float, 8><<<grid, 256, 0, s>>>(ka);
+    return hipGetLastError();
+}
+
+hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s)
+{
+    // bytes is a multiple of 2 (fp16) or 4 (fp32); dst is at least 4-byte aligned.
+    const size_t words = bytes / 4;
+    const int tail = int((bytes % 4) / 2);
+    size_t blocks = (words + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (blocks == 0) blocks = 1;
+    fill_zero_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(reinterpret_cast<uint32_t *>(dst), words,
+                                                          reinterpret_cast<uint16_t *>(dst) + words * 2, tail);
+    return hipGetLastError();
+}
+
+}  // namespace hspmm

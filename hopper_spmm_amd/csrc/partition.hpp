@@ -1,0 +1,131 @@
+// Host-side work partition for the persistent SpMM waves.
+//
+// The reference walks effective row windows round-robin over its thread blocks
+// (reference src/fp16.cu:86, 138) and each window's tiles in order
+// (src/fp16.cu:90, 140).  Here the flat tile sequence 0..T-1 (windows are
+// contiguous in it) is cut into ranges of about equal cost; one wave walks one
+// range.  A cut that falls near a window boundary snaps to it; a window that is
+// still cut (a heavy window) has its per-range partial sums kept in fp32 slots
+// and added in range order by a second small kernel, so the result does not
+// depend on timing.
+#pragma once
+#include <cstdint>
+#include <vector>
+#include <algorithm>
+
+namespace hspmm {
+
+constexpr uint32_t kNoSlot = 0xFFFFFFFFu;
+
+
+
+struct Range {
+    uint32_t tile_begin, tile_end;    // [begin, end) in the flat tile sequence
+    uint32_t first_window;            // effective window holding tile_begin
+    uint32_t head_slot, tail_slot;    // partial-sum slots (kNoSlot = none)
+};
+
+struct SplitWindow {
+    uint32_t window;                  // effective window index
+    uint32_t slot_begin, slot_count;  // into Partition::fix_slots, in range order
+};
+
+struct Partition {
+    std::vector<Range> ranges;
+    std::vector<SplitWindow> split;
+    std::vector<uint32_t> fix_slots;
+    uint32_t n_slots = 0;
+};
+
+// rowOffset has W+1 entries, rowOffset[0] == 0, strictly increasing.
+// target_ranges: wanted number of ranges (>= 1).
+// window_cost: cost of finishing one window, in units of one tile.
+// slack: a cut closer than slack * (mean tiles per range) to a window boundary
+// moves onto the boundary.
+inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t target_ranges,
+                                 double window_cost = 0.5, double slack = 0.35)
+{
+    Partition P;
+    if (W == 0) return P;
+    const uint32_t T = rowOffset[W];
+    if (T == 0) return P;
+    if (target_ranges < 1) target_ranges = 1;
+    const double total = double(T) + window_cost * double(W);
+    const double per = total / double(target_ranges);
+    const double snap = slack * double(T) / double(target_ranges);
+
+    std::vector<uint32_t> cuts;
+    cuts.reserve(target_ranges + 1);
+    cuts.push_back(0);
+    uint32_t w = 0;                    // window holding the current cut (monotone)
+    for (uint32_t i = 1; i < target_ranges; ++i) {
+        const double c = per * double(i);
+        // advance to the last window boundary whose prefix cost is <= c
+        while (w + 1 <= W && double(rowOffset[w + 1]) + window_cost * double(w + 1) <= c) ++w;
+        if (w >= W) break;
+        const double base = double(rowOffset[w]) + window_cost * double(w);
+        const uint32_t ws = rowOffset[w], we = rowOffset[w + 1];
+        double into = c - base;
+        if (into < 0) into = 0;
+        uint32_t tau = ws + uint32_t(into);
+        if (tau > we) tau = we;
+        if (double(tau - ws) <= snap) tau = ws;
+        else if (double(we - tau) <= snap) tau = we;
+        if (tau > cuts.back() && tau < T) cuts.push_back(tau);
+    }
+    cuts.push_back(T);
+
+    const size_t R = cuts.size() - 1;
+    P.ranges.resize(R);
+    uint32_t win = 0;
+    for (size_t r = 0; r < R; ++r) {
+        Range &g = P.ranges[r];
+        g.tile_begin = cuts[r];
+        g.tile_end = cuts[r + 1];
+        while (rowOffset[win + 1] <= g.tile_begin) ++win;
+        g.first_window = win;
+        g.head_slot = g.tail_slot = kNoSlot;
+    }
+    // Partial segments: only the first and the last window segment of a range can
+    // be incomplete.  The kernel's rule: an incomplete segment that starts at the
+    // range's first tile uses head_slot, any other incomplete segment tail_slot.
+    uint32_t cur_split = kNoSlot;     // window of the open split entry
+    for (size_t r = 0; r < R; ++r) {
+        Range &g = P.ranges[r];
+        uint32_t wv = g.first_window;
+        uint32_t t = g.tile_begin;
+        while (t < g.tile_end) {
+            const uint32_t ws = rowOffset[wv], we = rowOffset[wv + 1];
+            const uint32_t se = std::min(we, g.tile_end);
+            const bool complete = (t == ws) && (se == we);
+            if (!complete) {
+                const uint32_t slot = P.n_slots++;
+                if (t == g.tile_begin) g.head_slot = slot; else g.tail_slot = slot;
+                if (cur_split != wv) {
+                    P.split.push_back(SplitWindow{wv, uint32_t(P.fix_slots.size()), 0});
+                    cur_split = wv;
+                }
+                P.fix_slots.push_back(slot);
+                P.split.back().slot_count++;
+            }
+            // jump over the complete windows in the middle of the range
+            if (se == we) {
+                ++wv;
+                t = se;
+                if (t < g.tile_end) {
+                    // skip whole windows until the last one of the range
+                    const uint32_t *lo = rowOffset + wv;
+                    const uint32_t *hi = std::upper_bound(lo, rowOffset + W + 1, g.tile_end);
+                    // windows wv .. (hi - rowOffset - 2) end at or before tile_end
+                    const uint32_t last_full = uint32_t(hi - rowOffset) - 1;   // rowOffset[last_full] <= tile_end
+                    if (last_full > wv) { wv = last_full; t = rowOffset[wv]; }
+                }
+            } else {
+                t = se;
+            }
+        }
+    }
+    return P;
+}
+
+}  // namespace hspmm

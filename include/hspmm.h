@@ -1,0 +1,156 @@
+/*
+ * hspmm.h - C ABI of the MI355X (gfx950) SpMM operator  C = A * B
+ *
+ * A is sparse in the condensed row-window tile format without bitmap
+ * (BTCF_MTX_NO_BITMAP, reference src/utils/class.h:74-85, produced by
+ * CSR2BTCFNOBITMAP, reference src/utils/convert.h:146-225):
+ *   rowOffset[W+1]  first tile of each effective 8-row window
+ *   tcA2B[T*CW]     column id of every tile column, IDX_MAX (0xFFFFFFFF) = padding
+ *   data[T*8*CW]    dense 8 x CW tiles, row-major inside a tile
+ *   rowIdx[W]       first matrix row of each effective window (multiple of 8)
+ * with CW = 16 and 2-byte IEEE half values for HSPMM_FP16, CW = 8 and 4-byte
+ * float values for HSPMM_TF32 (reference src/common.h:14-43).
+ * B is dense cols x N, C is dense rows x N, both row-major, same element type
+ * as `data` (reference src/fp16.cu:36-46, 163-170).  Accumulation is fp32; the
+ * fp16 path rounds once to nearest-even on store.
+ *
+ * All functions return 0 (HSPMM_OK) or a positive error code; the text of the
+ * last error on the calling thread is available from hspmm_last_error().
+ * Nothing here calls exit() or throws across the boundary.
+ */
+#ifndef HSPMM_H
+#define HSPMM_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HSPMM_FP16 0            /* reference -DUSE_FP16 build, src/common.h:14-19 */
+#define HSPMM_TF32 1            /* reference -DUSE_TF32 build, src/common.h:26-43 (fp32 storage) */
+#define HSPMM_IDX_MAX 0xFFFFFFFFu   /* reference src/common.h:47 */
+#define HSPMM_ROW_WINDOW 8u         /* reference src/common.h:17 */
+
+enum {
+    HSPMM_OK = 0,
+    HSPMM_ERR_INVALID = 1,      /* bad argument or malformed format arrays */
+    HSPMM_ERR_DEVICE = 2,       /* a HIP runtime call failed */
+    HSPMM_ERR_ALLOC = 3,        /* host or device allocation failed */
+    HSPMM_ERR_IO = 4,           /* file cannot be opened / parsed */
+    HSPMM_ERR_UNSUPPORTED = 5
+};
+
+typedef struct hspmm_plan hspmm_plan;
+
+/* ---- device operator ---------------------------------------------------- */
+
+/* Replaces the allocation + host-to-device part of fp16_spmm (reference
+ * src/fp16.cu:228-249) and create_tma_desc_A (src/fp16.cu:177-219): validates
+ * the four format arrays (host pointers), copies them to the current HIP
+ * device and builds the work partition the kernels walk.  `dtype` is
+ * HSPMM_FP16 or HSPMM_TF32. */
+int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
+                 uint32_t eff_row_windows, uint32_t total_tiles,
+                 const uint32_t *rowOffset, const uint32_t *tcA2B,
+                 const void *data, const uint32_t *rowIdx);
+
+/* Replaces one launch of fp16_spmm_kernel (reference src/fp16.cu:256): computes
+ * all of C = A*B for feature dimension N.  dB (cols x N) and dC (rows x N) are
+ * DEVICE pointers, row-major, 4-byte aligned; every element of C is written
+ * (rows without nonzeros become 0).  Asynchronous on `stream` (a hipStream_t,
+ * NULL = default stream).  A plan owns scratch memory, so launches of one plan
+ * must not overlap in time; different plans may run concurrently. */
+int hspmm_run(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stream);
+
+/* Replaces the warm-up + timed loop of fp16_spmm (reference src/fp16.cu:254-268,
+ * WARMUP_RUNS / RUNS of src/common.h:48-49): `warmup` untimed launches, then
+ * `runs` back-to-back launches between two device events on `stream`;
+ * *total_ms receives the time of the `runs` launches together. */
+int hspmm_bench(hspmm_plan *plan, const void *dB, void *dC, uint32_t N,
+                int warmup, int runs, void *stream, float *total_ms);
+
+/* Replaces the cudaFree block of fp16_spmm (reference src/fp16.cu:274-279). */
+void hspmm_destroy(hspmm_plan *plan);
+
+/* Replaces checkCudaErrors' message (reference src/utils/utils.h:9-21) without
+ * exiting: text of the last failure on this thread ("" if none). */
+const char *hspmm_last_error(void);
+
+/* Replaces Scheduler::configure (reference src/scheduler.h:33-38).  Values are
+ * read by the next hspmm_create on any thread; 0 keeps the built-in default.
+ *   buffer_stage             tiles each wave keeps in flight (prefetch depth): 1, 2, 3, 4, 6 or 8
+ *   consumer_warp_num        waves per workgroup, 1..4
+ *   producer_warp_group_num  tile ranges (waves) per SIMD the partition aims at, 1..16
+ *   sm_num                   compute units to balance over (default: the device's) */
+int hspmm_configure(int buffer_stage, int consumer_warp_num,
+                    int producer_warp_group_num, int sm_num);
+/* Getter side of the same singleton (reference src/scheduler.h:26-30, 41). */
+void hspmm_get_config(int *buffer_stage, int *consumer_warp_num,
+                      int *producer_warp_group_num, int *sm_num);
+
+/* Kernel selection, read by the next hspmm_create: 0 = automatic (MFMA kernels
+ * whenever the feature dimension allows), 1 = always the scalar all-shapes
+ * kernel, 2 = fp16 MFMA kernel with wide loads only, 3 = fp16 MFMA kernel with
+ * word loads whenever N is a multiple of 32. */
+int hspmm_set_kernel_mode(int mode);
+
+typedef struct {
+    uint32_t rows, cols, eff_row_windows, total_tiles;
+    int32_t  dtype;
+    uint32_t n_ranges;          /* tile ranges (one wave each per feature block) */
+    uint32_t n_split_windows;   /* windows whose tiles span more than one range */
+    uint32_t n_partial_slots;   /* fp32 partial accumulators the split windows use */
+    uint32_t compute_units;
+    uint64_t device_bytes;      /* bytes of device memory the plan holds right now */
+} hspmm_plan_info;
+
+/* No reference counterpart (the reference prints its statistics from main,
+ * src/fp16.cu:295-301): reports the shape of the plan and of its partition. */
+int hspmm_get_plan_info(const hspmm_plan *plan, hspmm_plan_info *info);
+
+/* No reference counterpart: copies the partition for inspection (tests).
+ * ranges: n_ranges x 5 words {tile_begin, tile_end, first_window, head_slot,
+ * tail_slot} (slot 0xFFFFFFFF = none). */
+int hspmm_get_partition(const hspmm_plan *plan, uint32_t *ranges, uint32_t capacity_ranges);
+
+/* No reference counterpart: the partition hspmm_create would build for a
+ * rowOffset array and a wanted number of ranges, computed on the host alone
+ * (no device needed).  ranges as in hspmm_get_partition; any output may be NULL. */
+int hspmm_partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
+                            uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges,
+                            uint32_t *n_split_windows, uint32_t *n_partial_slots);
+
+/* ---- host format functions ---------------------------------------------- */
+
+typedef struct {
+    uint32_t rows, cols, nnzs;  /* CSR_MTX, reference src/utils/class.h:30-37 */
+    uint32_t *row_ptr;          /* rows + 1 */
+    uint32_t *col_idx;          /* nnzs */
+    void     *values;           /* nnzs halves (HSPMM_FP16) or floats (HSPMM_TF32) */
+} hspmm_csr;
+
+/* Replaces load_matrix (reference src/utils/load.h:152-322): MatrixMarket
+ * coordinate text -> CSR sorted by (row, column), 1-based -> 0-based, values
+ * rounded to half for HSPMM_FP16.  Arrays are owned by the library until
+ * hspmm_csr_free.  Returns HSPMM_ERR_IO where the reference prints an error
+ * and returns an empty matrix. */
+int hspmm_mtx_load(const char *path, int dtype, hspmm_csr *out);
+/* Replaces free_csr_matrix (reference src/utils/load.h:337-355). */
+void hspmm_csr_free(hspmm_csr *m);
+
+/* Replaces CSR2BTCFNOBITMAP (reference src/utils/convert.h:146-225) in two
+ * calls so that the caller owns the arrays: first the sizes, then the fill.
+ * `transpose` != 0 gives the SPARSE_A_TRANSPOSE tile order (convert.h:207-209),
+ * which the device operator does not accept. */
+int hspmm_btcf_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                     uint32_t *eff_row_windows, uint32_t *total_tiles);
+int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                    const void *values, int transpose,
+                    uint32_t *rowOffset, uint32_t *tcA2B, void *data, uint32_t *rowIdx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSPMM_H */

@@ -1,0 +1,456 @@
+/*
+ * CPU oracle for the condensed-tile SpMM path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain C, the host-side algorithms and the intended
+ * arithmetic of the reference SpMM path so that the HIP implementation can be
+ * checked against it.  It is linked only by the test-suite, by the smoke check
+ * and by the `cpu_baseline` leg of the benchmark; the product library never
+ * links, loads or calls anything in this directory.
+ *
+ * Each function cites the reference lines it follows (paths relative to the
+ * reference checkout).
+ *
+ * Parity status of each function (what pins it):
+ *   orc_f32_to_f16 / orc_f16_to_f32  exhaustive comparison with numpy float16
+ *   orc_mtx_read                     reference-produced golden vectors (tiny.mtx,
+ *                                    gap.mtx), scipy COO->CSR cross-check
+ *   orc_btcf_count / orc_btcf_fill   the same golden vectors, round-trip to CSR,
+ *                                    brute force on small dense matrices
+ *   orc_spmm_csr_* / orc_spmm_btcf_* dense numpy float64 product on the same
+ *                                    rounded inputs, closed forms, CSR-order vs
+ *                                    tile-order agreement
+ *   orc_tile_mma_* / orc_tile_accum  closed forms of the reference's micro-tests
+ *                                    (256*i+136 and the 1+0.01*i pattern)
+ *   orc_verdict_*                    hand-computed cases
+ * The reference holds no end-to-end SpMM fixture (its kernel is unfinished), so
+ * SpMM-level parity is pinned by the mathematics above, not by reference output.
+ */
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <math.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_IDX_MAX 0xFFFFFFFFu   /* src/common.h:47  IDX_MAX = UINT32_MAX */
+#define ORC_ROW_WINDOW 8u         /* src/common.h:17,23,33,40  ROW_WINDOW = 8 */
+
+/* ------------------------------------------------------------------------- */
+/* half <-> float, bit level (round to nearest even), as __float2half /      */
+/* __half2float do on the host (src/utils/load.h:226, src/test_fp16.cu:295). */
+/* ------------------------------------------------------------------------- */
+uint16_t orc_f32_to_f16(float f)
+{
+    uint32_t x; memcpy(&x, &f, 4);
+    uint32_t sign = (x >> 16) & 0x8000u;
+    uint32_t ax = x & 0x7FFFFFFFu;
+    if (ax >= 0x7F800000u)                       /* inf / nan */
+        return (uint16_t)(sign | 0x7C00u | (ax > 0x7F800000u ? (0x0200u | ((ax >> 13) & 0x3FFu)) : 0u));
+    if (ax >= 0x477FF000u)                       /* rounds to >= 65520 -> inf */
+        return (uint16_t)(sign | 0x7C00u);
+    if (ax < 0x33000001u)                        /* <= 2^-25 : rounds to zero */
+        return (uint16_t)sign;
+    int32_t e = (int32_t)(ax >> 23) - 127;
+    uint32_t m = (ax & 0x7FFFFFu) | 0x800000u;   /* 24-bit significand */
+    uint32_t shift, half;
+    if (e < -14) {                               /* subnormal half */
+        shift = (uint32_t)(13 + (-14 - e));      /* 14..24 */
+        half = m >> shift;
+    } else {
+        shift = 13;
+        half = ((uint32_t)(e + 15) << 10) + ((m >> 13) & 0x3FFu);
+    }
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (half & 1u))) half++;   /* carry may bump exponent: correct */
+    return (uint16_t)(sign | half);
+}
+
+float orc_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1Fu;
+    uint32_t m = h & 0x3FFu;
+    uint32_t x;
+    if (e == 0) {
+        if (m == 0) x = sign;
+        else {                                   /* subnormal: normalise */
+            int s = 0;
+            while (!(m & 0x400u)) { m <<= 1; s++; }
+            m &= 0x3FFu;
+            x = sign | ((uint32_t)(127 - 15 - s + 1) << 23) | (m << 13);
+        }
+    } else if (e == 31) x = sign | 0x7F800000u | (m << 13);
+    else x = sign | ((e - 15 + 127) << 23) | (m << 13);
+    float f; memcpy(&f, &x, 4);
+    return f;
+}
+
+void orc_f32_to_f16_array(const float *src, uint16_t *dst, size_t n)
+{ for (size_t i = 0; i < n; ++i) dst[i] = orc_f32_to_f16(src[i]); }
+
+void orc_f16_to_f32_array(const uint16_t *src, float *dst, size_t n)
+{ for (size_t i = 0; i < n; ++i) dst[i] = orc_f16_to_f32(src[i]); }
+
+/* ------------------------------------------------------------------------- */
+/* MatrixMarket coordinate text -> CSR.  Follows src/utils/load.h:152-322.   */
+/* ------------------------------------------------------------------------- */
+typedef struct {
+    uint32_t rows, cols, nnzs;      /* CSR_MTX, src/utils/class.h:30-37 */
+    uint32_t declared_nnz;          /* the header's count before the shrink at load.h:234-238 */
+    uint32_t *row_ptr;              /* rows + 1 */
+    uint32_t *col_idx;              /* nnzs */
+    void     *values;               /* nnzs x (2 bytes fp16 | 4 bytes fp32) */
+    int       status;               /* 0 ok, 1 cannot open, 2 bad size line, 3 alloc, 4 index out of range */
+} orc_csr;
+
+typedef struct { uint32_t r, c, seq; } orc_key;
+
+static int orc_key_cmp(const void *a, const void *b)
+{
+    const orc_key *x = (const orc_key *)a, *y = (const orc_key *)b;
+    if (x->r != y->r) return x->r < y->r ? -1 : 1;      /* load.h:141-142 row first */
+    if (x->c != y->c) return x->c < y->c ? -1 : 1;      /* load.h:144 then column   */
+    /* The reference's qsort is unstable for equal (row,col); file order is kept here
+       so that the oracle is deterministic.  Inputs with duplicates are ill-defined
+       in the reference. */
+    return x->seq < y->seq ? -1 : (x->seq > y->seq);
+}
+
+/* elem_size: 2 = fp16 build (USE_FP16, value rounded with RN, load.h:226),
+ *            4 = fp32 storage (USE_TF32, value kept as parsed, load.h:224). */
+orc_csr *orc_mtx_read(const char *path, int elem_size)
+{
+    orc_csr *m = (orc_csr *)calloc(1, sizeof(orc_csr));
+    if (!m) return NULL;
+    FILE *f = fopen(path, "r");
+    if (!f) { m->status = 1; return m; }                               /* load.h:176-180 */
+    char line[1024];                                                   /* load.h:155 */
+    int have = 0;
+    while (fgets(line, sizeof line, f)) {                              /* load.h:183-187 */
+        have = 1;
+        if (line[0] != '%') break;
+    }
+    uint32_t rows, cols, nnz;
+    if (!have || sscanf(line, "%u %u %u", &rows, &cols, &nnz) != 3) {  /* load.h:190-194 */
+        fclose(f); m->status = 2; return m;
+    }
+    uint32_t *ri = (uint32_t *)malloc((size_t)(nnz ? nnz : 1) * 4);
+    uint32_t *ci = (uint32_t *)malloc((size_t)(nnz ? nnz : 1) * 4);
+    float    *vf = (float *)malloc((size_t)(nnz ? nnz : 1) * 4);
+    if (!ri || !ci || !vf) { fclose(f); free(ri); free(ci); free(vf); m->status = 3; return m; }
+    uint32_t count = 0;
+    while (count < nnz && fgets(line, sizeof line, f)) {               /* load.h:215 */
+        uint32_t r, c; float v;
+        if (sscanf(line, "%u %u %f", &r, &c, &v) == 3) {               /* load.h:219 */
+            ri[count] = r - 1; ci[count] = c - 1; vf[count] = v;       /* load.h:221-222 */
+            count++;
+        }                                                              /* other lines are skipped */
+    }
+    fclose(f);
+    m->declared_nnz = nnz;
+    nnz = count;                                                       /* load.h:234-238 */
+    for (uint32_t i = 0; i < nnz; ++i)
+        if (ri[i] >= rows || ci[i] >= cols) { free(ri); free(ci); free(vf); m->status = 4; return m; }
+
+    orc_key *keys = (orc_key *)malloc((size_t)(nnz ? nnz : 1) * sizeof(orc_key));
+    m->row_ptr = (uint32_t *)calloc((size_t)rows + 1, 4);
+    m->col_idx = (uint32_t *)malloc((size_t)(nnz ? nnz : 1) * 4);
+    m->values  = malloc((size_t)(nnz ? nnz : 1) * (size_t)elem_size);
+    if (!keys || !m->row_ptr || !m->col_idx || !m->values) {
+        free(keys); free(ri); free(ci); free(vf); m->status = 3; return m;
+    }
+    for (uint32_t i = 0; i < nnz; ++i) { keys[i].r = ri[i]; keys[i].c = ci[i]; keys[i].seq = i; }
+    qsort(keys, nnz, sizeof(orc_key), orc_key_cmp);                    /* load.h:256-257 */
+    for (uint32_t i = 0; i < nnz; ++i) {                               /* load.h:284-300 */
+        uint32_t s = keys[i].seq;
+        m->col_idx[i] = ci[s];
+        if (elem_size == 2) ((uint16_t *)m->values)[i] = orc_f32_to_f16(vf[s]);
+        else                ((float *)m->values)[i] = vf[s];
+        m->row_ptr[ri[s] + 1]++;
+    }
+    for (uint32_t r = 0; r < rows; ++r) m->row_ptr[r + 1] += m->row_ptr[r];
+    m->rows = rows; m->cols = cols; m->nnzs = nnz;
+    free(keys); free(ri); free(ci); free(vf);
+    return m;
+}
+
+void orc_csr_free(orc_csr *m)
+{
+    if (!m) return;
+    free(m->row_ptr); free(m->col_idx); free(m->values); free(m);
+}
+
+/* Structural checks of src/utils/load.h:44-73 (validate_csr_from_coo, parts 1-2).
+ * Returns the number of violations. */
+int orc_csr_validate(uint32_t rows, uint32_t cols, uint32_t nnz,
+                     const uint32_t *row_ptr, const uint32_t *col_idx)
+{
+    int bad = 0;
+    if (row_ptr[0] != 0) bad++;                                        /* load.h:44-47 */
+    if (row_ptr[rows] != nnz) bad++;                                   /* load.h:49-53 */
+    for (uint32_t i = 0; i < rows; ++i) if (row_ptr[i] > row_ptr[i + 1]) bad++;   /* load.h:56-62 */
+    for (uint32_t i = 0; i < nnz; ++i) if (col_idx[i] >= cols) bad++;  /* load.h:66-73 */
+    return bad;
+}
+
+/* ------------------------------------------------------------------------- */
+/* CSR -> condensed tiles without bitmap.  Follows src/utils/convert.h:146-225 */
+/* ------------------------------------------------------------------------- */
+static int orc_u32_cmp(const void *a, const void *b)
+{
+    uint32_t x = *(const uint32_t *)a, y = *(const uint32_t *)b;
+    return x < y ? -1 : (x > y);
+}
+
+/* Pass 1: sizes.  eff_windows = windows holding at least one stored entry
+ * (convert.h:161-163); total_tiles = sum over them of ceil(distinct cols / CW)
+ * (convert.h:178-186). */
+void orc_btcf_count(uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                    uint32_t cw, uint32_t *eff_windows, uint32_t *total_tiles)
+{
+    uint32_t W = 0, T = 0, cap = 0; uint32_t *tmp = NULL;
+    for (uint32_t r0 = 0; r0 < rows; r0 += ORC_ROW_WINDOW) {
+        uint32_t r1 = r0 + ORC_ROW_WINDOW < rows ? r0 + ORC_ROW_WINDOW : rows;   /* convert.h:158 */
+        uint32_t b = row_ptr[r0], e = row_ptr[r1], n = e - b;
+        if (n == 0) continue;                                                     /* convert.h:162 */
+        if (n > cap) { cap = n; tmp = (uint32_t *)realloc(tmp, (size_t)cap * 4); }
+        memcpy(tmp, col_idx + b, (size_t)n * 4);
+        qsort(tmp, n, 4, orc_u32_cmp);                                            /* convert.h:167 */
+        uint32_t u = 1;
+        for (uint32_t i = 1; i < n; ++i) if (tmp[i] != tmp[i - 1]) u++;          /* convert.h:169 */
+        W++; T += (u + cw - 1) / cw;
+    }
+    free(tmp);
+    *eff_windows = W; *total_tiles = T;
+}
+
+/* Pass 2: fill caller-provided arrays.
+ *   rowOffset[W+1], tcA2B[T*cw], data[T*8*cw*elem_size] (zeroed here), rowIdx[W].
+ * transpose != 0 selects the SPARSE_A_TRANSPOSE element order (convert.h:207-209). */
+void orc_btcf_fill(uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                   const void *values, uint32_t elem_size, uint32_t cw, int transpose,
+                   uint32_t *rowOffset, uint32_t *tcA2B, void *data, uint32_t *rowIdx)
+{
+    uint32_t W = 0, T = 0, cap = 0; uint32_t *uniq = NULL;
+    rowOffset[0] = 0;                                                             /* convert.h:152 */
+    const size_t tile_elems = (size_t)ORC_ROW_WINDOW * cw;
+    for (uint32_t r0 = 0; r0 < rows; r0 += ORC_ROW_WINDOW) {
+        uint32_t r1 = r0 + ORC_ROW_WINDOW < rows ? r0 + ORC_ROW_WINDOW : rows;
+        uint32_t b = row_ptr[r0], e = row_ptr[r1], n = e - b;
+        if (n == 0) continue;
+        if (n > cap) { cap = n; uniq = (uint32_t *)realloc(uniq, (size_t)cap * 4); }
+        memcpy(uniq, col_idx + b, (size_t)n * 4);
+        qsort(uniq, n, 4, orc_u32_cmp);
+        uint32_t u = 1;
+        for (uint32_t i = 1; i < n; ++i) if (uniq[i] != uniq[i - 1]) uniq[u++] = uniq[i];
+        uint32_t tiles = (u + cw - 1) / cw;
+        uint32_t *a2b = tcA2B + (size_t)T * cw;
+        for (uint32_t i = 0; i < tiles * cw; ++i) a2b[i] = i < u ? uniq[i] : ORC_IDX_MAX;   /* convert.h:178-184 */
+        rowOffset[W + 1] = rowOffset[W] + tiles;                                  /* convert.h:186 */
+        rowIdx[W] = r0;                                                           /* convert.h:187 */
+        unsigned char *win = (unsigned char *)data + (size_t)T * tile_elems * elem_size;
+        memset(win, 0, (size_t)tiles * tile_elems * elem_size);                   /* convert.h:191-193 */
+        for (uint32_t r = r0; r < r1; ++r) {                                      /* convert.h:196 */
+            for (uint32_t id = row_ptr[r]; id < row_ptr[r + 1]; ++id) {           /* convert.h:197 */
+                uint32_t c = col_idx[id], lo = 0, hi = u;                         /* rank of c, convert.h:198 */
+                while (hi - lo > 1) { uint32_t mid = (lo + hi) / 2; if (uniq[mid] <= c) lo = mid; else hi = mid; }
+                uint32_t tc = lo / cw, lc = lo % cw, lr = r % ORC_ROW_WINDOW;     /* convert.h:199-201 */
+                size_t off = transpose ? (size_t)lc * ORC_ROW_WINDOW + lr         /* convert.h:209 */
+                                       : (size_t)lr * cw + lc;                    /* convert.h:212 */
+                memcpy(win + ((size_t)tc * tile_elems + off) * elem_size,         /* convert.h:215 (later id overwrites) */
+                       (const unsigned char *)values + (size_t)id * elem_size, elem_size);
+            }
+        }
+        W++; T += tiles;
+    }
+    free(uniq);
+}
+
+/* ------------------------------------------------------------------------- */
+/* SpMM oracles.  Arithmetic of src/test_fp16.cu:292-297 applied to C = A*B: */
+/* products of half->float values accumulated in fp32, k (column) ascending, */
+/* result rounded once to fp16 with RN (src/fp16.cu:131,167: float acc,      */
+/* implicit float->__half store).                                            */
+/* ------------------------------------------------------------------------- */
+static int orc_threads(int req)
+{
+#ifdef _OPENMP
+    return req > 0 ? req : omp_get_max_threads();
+#else
+    (void)req; return 1;
+#endif
+}
+
+int orc_max_threads(void) { return orc_threads(0); }
+
+/* C[rows x N] (fp16) = A_csr (fp16) * B[cols x N] (fp16).  absdot, when not NULL,
+ * receives sum_k |a||b| per output (fp32) for error bounds in tests. */
+void orc_spmm_csr_f16(uint32_t rows, uint32_t N, const uint32_t *row_ptr, const uint32_t *col_idx,
+                      const uint16_t *vals, const uint16_t *B, uint16_t *C, float *absdot, int nthreads)
+{
+    int nt = orc_threads(nthreads); (void)nt;
+    #pragma omp parallel num_threads(nt)
+    {
+        float *acc = (float *)malloc((size_t)N * 4 * 2);
+        float *mag = acc + N;
+        #pragma omp for schedule(dynamic, 64)
+        for (int64_t r = 0; r < (int64_t)rows; ++r) {
+            for (uint32_t j = 0; j < N; ++j) { acc[j] = 0.0f; mag[j] = 0.0f; }
+            for (uint32_t id = row_ptr[r]; id < row_ptr[r + 1]; ++id) {
+                float a = orc_f16_to_f32(vals[id]);
+                const uint16_t *b = B + (size_t)col_idx[id] * N;
+                if (absdot) for (uint32_t j = 0; j < N; ++j) {
+                    float p = a * orc_f16_to_f32(b[j]); acc[j] += p; mag[j] += fabsf(p);
+                } else for (uint32_t j = 0; j < N; ++j) acc[j] += a * orc_f16_to_f32(b[j]);
+            }
+            uint16_t *c = C + (size_t)r * N;
+            for (uint32_t j = 0; j < N; ++j) c[j] = orc_f32_to_f16(acc[j]);
+            if (absdot) memcpy(absdot + (size_t)r * N, mag, (size_t)N * 4);
+        }
+        free(acc);
+    }
+}
+
+/* fp32 storage variant (USE_TF32 build: MAT_VAL_TYPE float, src/common.h:27).
+ * trunc_tf32 != 0 masks the low 13 mantissa bits of both inputs before the
+ * product, which is what a tensor core does with raw fp32 bits; the reference's
+ * conversion helper does not write back (src/ptx/ptx_utils.h:32-37). */
+static inline float orc_tf32_trunc(float f)
+{ uint32_t x; memcpy(&x, &f, 4); x &= 0xFFFFE000u; memcpy(&f, &x, 4); return f; }
+
+void orc_spmm_csr_f32(uint32_t rows, uint32_t N, const uint32_t *row_ptr, const uint32_t *col_idx,
+                      const float *vals, const float *B, float *C, float *absdot,
+                      int trunc_tf32, int nthreads)
+{
+    int nt = orc_threads(nthreads); (void)nt;
+    #pragma omp parallel for schedule(dynamic, 64) num_threads(nt)
+    for (int64_t r = 0; r < (int64_t)rows; ++r) {
+        float *c = C + (size_t)r * N;
+        float *mg = absdot ? absdot + (size_t)r * N : NULL;
+        for (uint32_t j = 0; j < N; ++j) c[j] = 0.0f;
+        if (mg) for (uint32_t j = 0; j < N; ++j) mg[j] = 0.0f;
+        for (uint32_t id = row_ptr[r]; id < row_ptr[r + 1]; ++id) {
+            float a = trunc_tf32 ? orc_tf32_trunc(vals[id]) : vals[id];
+            const float *b = B + (size_t)col_idx[id] * N;
+            for (uint32_t j = 0; j < N; ++j) {
+                float bv = trunc_tf32 ? orc_tf32_trunc(b[j]) : b[j];
+                float p = a * bv; c[j] += p; if (mg) mg[j] += fabsf(p);
+            }
+        }
+    }
+}
+
+/* Tile-order SpMM: the walk the reference kernel intends (src/fp16.cu:86-90,
+ * 138-170): for each effective window, for each of its tiles, for each k whose
+ * tcA2B entry is not IDX_MAX, every window row accumulates
+ * data[t][r][k] * B[tcA2B[t][k]][:] in fp32; C[rowIdx[w]+r][:] = RN16(acc).
+ * Rows outside every effective window, and nothing beyond `rows`, are written
+ * as zero (the reference leaves them uninitialised; zero is the SpMM value). */
+void orc_spmm_btcf_f16(uint32_t rows, uint32_t N, uint32_t eff_windows,
+                       const uint32_t *rowOffset, const uint32_t *tcA2B, const uint16_t *data,
+                       const uint32_t *rowIdx, const uint16_t *B, uint16_t *C)
+{
+    const uint32_t cw = 16;
+    memset(C, 0, (size_t)rows * N * 2);
+    float *acc = (float *)malloc((size_t)ORC_ROW_WINDOW * N * 4);
+    for (uint32_t w = 0; w < eff_windows; ++w) {
+        memset(acc, 0, (size_t)ORC_ROW_WINDOW * N * 4);
+        for (uint32_t t = rowOffset[w]; t < rowOffset[w + 1]; ++t)
+            for (uint32_t k = 0; k < cw; ++k) {
+                uint32_t col = tcA2B[(size_t)t * cw + k];
+                if (col == ORC_IDX_MAX) continue;
+                const uint16_t *b = B + (size_t)col * N;
+                for (uint32_t r = 0; r < ORC_ROW_WINDOW; ++r) {
+                    float a = orc_f16_to_f32(data[((size_t)t * ORC_ROW_WINDOW + r) * cw + k]);
+                    float *ar = acc + (size_t)r * N;
+                    for (uint32_t j = 0; j < N; ++j) ar[j] += a * orc_f16_to_f32(b[j]);
+                }
+            }
+        for (uint32_t r = 0; r < ORC_ROW_WINDOW && rowIdx[w] + r < rows; ++r)
+            for (uint32_t j = 0; j < N; ++j)
+                C[(size_t)(rowIdx[w] + r) * N + j] = orc_f32_to_f16(acc[(size_t)r * N + j]);
+    }
+    free(acc);
+}
+
+void orc_spmm_btcf_f32(uint32_t rows, uint32_t N, uint32_t eff_windows, uint32_t cw,
+                       const uint32_t *rowOffset, const uint32_t *tcA2B, const float *data,
+                       const uint32_t *rowIdx, const float *B, float *C)
+{
+    memset(C, 0, (size_t)rows * N * 4);
+    float *acc = (float *)malloc((size_t)ORC_ROW_WINDOW * N * 4);
+    for (uint32_t w = 0; w < eff_windows; ++w) {
+        memset(acc, 0, (size_t)ORC_ROW_WINDOW * N * 4);
+        for (uint32_t t = rowOffset[w]; t < rowOffset[w + 1]; ++t)
+            for (uint32_t k = 0; k < cw; ++k) {
+                uint32_t col = tcA2B[(size_t)t * cw + k];
+                if (col == ORC_IDX_MAX) continue;
+                const float *b = B + (size_t)col * N;
+                for (uint32_t r = 0; r < ORC_ROW_WINDOW; ++r) {
+                    float a = data[((size_t)t * ORC_ROW_WINDOW + r) * cw + k];
+                    float *ar = acc + (size_t)r * N;
+                    for (uint32_t j = 0; j < N; ++j) ar[j] += a * b[j];
+                }
+            }
+        for (uint32_t r = 0; r < ORC_ROW_WINDOW && rowIdx[w] + r < rows; ++r)
+            memcpy(C + (size_t)(rowIdx[w] + r) * N, acc + (size_t)r * N, (size_t)N * 4);
+    }
+    free(acc);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Tile-level check arithmetic of the reference's micro-tests.               */
+/* ------------------------------------------------------------------------- */
+/* src/test_fp16.cu:284-297: C[i][j] = sum_k h2f(A[i*K+k]) * h2f(B[j*K+k]), both K-major. */
+void orc_tile_mma_f16(const uint16_t *A, const uint16_t *B, float *C, int M, int N, int K)
+{
+    for (int i = 0; i < M; ++i) for (int j = 0; j < N; ++j) {
+        float s = 0.0f;
+        for (int k = 0; k < K; ++k) s += orc_f16_to_f32(A[i * K + k]) * orc_f16_to_f32(B[j * K + k]);
+        C[i * N + j] = s;
+    }
+}
+/* test/02.tma_and_wgmma/tma_wgmma.cu:217-230: same with fp32 inputs. */
+void orc_tile_mma_f32(const float *A, const float *B, float *C, int M, int N, int K)
+{
+    for (int i = 0; i < M; ++i) for (int j = 0; j < N; ++j) {
+        float s = 0.0f;
+        for (int k = 0; k < K; ++k) s += A[i * K + k] * B[j * K + k];
+        C[i * N + j] = s;
+    }
+}
+/* src/tf32.cu:16-28 (== test/03.warp_specialized/utils.h:31-43):
+ * C[r][c] += A[r*K*T + i*K + k] * B[c*K*T + i*K + k], tiles outermost. */
+void orc_tile_accum_f32(const float *A, const float *B, float *C, int M, int N, int K, int T)
+{
+    for (int i = 0; i < M * N; ++i) C[i] = 0.0f;
+    for (int i = 0; i < T; ++i)
+        for (int r = 0; r < M; ++r) for (int c = 0; c < N; ++c) for (int k = 0; k < K; ++k)
+            C[r * N + c] += A[r * K * T + k + i * K] * B[c * K * T + k + i * K];
+}
+
+/* Verdict of src/test_fp16.cu:302-309: fails where |e-a| / (|e| + 1e-8) > tol. */
+size_t orc_verdict_rel(const float *expected, const float *actual, size_t n, float tol)
+{
+    size_t bad = 0;
+    for (size_t i = 0; i < n; ++i) {
+        float rel = fabsf(expected[i] - actual[i]) / (fabsf(expected[i]) + 1e-8f);
+        if (!(rel <= tol)) bad++;
+    }
+    return bad;
+}
+/* Verdict of src/tf32.cu:37-70: relative if |ref| > 1e-6, else absolute 1e-5. */
+size_t orc_verdict_rel_abs(const float *actual, const float *ref, size_t n, double tol)
+{
+    size_t bad = 0;
+    for (size_t i = 0; i < n; ++i) {
+        double err = fabs((double)actual[i] - (double)ref[i]);
+        double rv = fabs((double)ref[i]);
+        if (rv > 1e-6) { if (!(err / rv <= tol)) bad++; }
+        else if (!(err <= 1e-5)) bad++;
+    }
+    return bad;
+}

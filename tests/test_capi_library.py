@@ -1,0 +1,86 @@
+"""The C-ABI library loads without a GPU and exports every symbol that
+include/hspmm.h declares; host-only entry points behave (no device calls here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hspmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hspmm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(hs):
+    lib = ctypes.CDLL(hs.library_path())
+    names = declared_symbols()
+    assert len(names) >= 14 and "hspmm_create" in names and "hspmm_run" in names
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_no_torch_types_in_the_header():
+    text = open(os.path.join(ROOT, "include", "hspmm.h")).read()
+    assert "torch" not in text and "at::" not in text and 'extern "C"' in text
+
+
+def test_scheduler_knobs_round_trip(hs):
+    # Scheduler::configure / getters of the reference (src/scheduler.h:26-41)
+    assert hs.get_config() == (0, 0, 0, 0)
+    hs.configure(4, 2, 3, 128)
+    assert hs.get_config() == (4, 2, 3, 128)
+    for bad in ((5, 0, 0, 0), (9, 0, 0, 0), (0, 5, 0, 0), (0, 0, 17, 0), (-1, 0, 0, 0), (0, 0, 0, -3)):
+        with pytest.raises(hs.HspmmError):
+            hs.configure(*bad)
+    assert hs.get_config() == (4, 2, 3, 128)
+    hs.configure()
+    assert hs.get_config() == (0, 0, 0, 0)
+    with pytest.raises(hs.HspmmError):
+        hs.set_kernel_mode(9)
+    hs.set_kernel_mode(0)
+
+
+def test_create_rejects_malformed_formats_before_touching_the_device(hs):
+    ok = dict(rows=16, cols=40, dtype=0, eff_row_windows=2, total_tiles=2,
+              rowOffset=np.array([0, 1, 2], np.uint32), rowIdx=np.array([0, 8], np.uint32),
+              tcA2B=np.concatenate([np.arange(16), np.arange(16) + 3]).astype(np.uint32),
+              data=np.zeros(2 * 128, np.uint16))
+    def broken(**kw):
+        d = dict(ok); d.update(kw); return d
+    cases = [
+        broken(rowOffset=np.array([1, 2, 3], np.uint32)),
+        broken(rowOffset=np.array([0, 1, 1], np.uint32)),
+        broken(rowOffset=np.array([0, 1, 3], np.uint32)),
+        broken(rowIdx=np.array([0, 4], np.uint32)),
+        broken(rowIdx=np.array([8, 0], np.uint32)),
+        broken(rowIdx=np.array([0, 16], np.uint32)),
+        broken(tcA2B=np.concatenate([np.arange(16), np.arange(16) + 30]).astype(np.uint32)),
+        broken(tcA2B=np.concatenate([[0xFFFFFFFF], np.arange(31)]).astype(np.uint32)),
+        broken(tcA2B=np.concatenate([[0, 0xFFFFFFFF, 5], np.arange(29)]).astype(np.uint32)),
+        broken(eff_row_windows=3, rowOffset=np.array([0, 1, 2, 3], np.uint32), rowIdx=np.array([0, 8, 16], np.uint32), total_tiles=3),
+    ]
+    for c in cases:
+        with pytest.raises(hs.HspmmError) as e:
+            hs.Plan(c)
+        assert e.value.code in (1,), str(e.value)        # HSPMM_ERR_INVALID, raised by host-side validation
+    L = hs.load_library()
+    h = ctypes.c_void_p()
+    assert L.hspmm_create(ctypes.byref(h), 3, 8, 8, 0, 0, None, None, None, None) == 1   # unknown dtype
+    assert b"dtype" in L.hspmm_last_error() and not h.value
+
+
+def test_operator_fails_loudly_without_a_gfx950_device(hs):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    ok = dict(rows=8, cols=16, dtype=0, eff_row_windows=1, total_tiles=1,
+              rowOffset=np.array([0, 1], np.uint32), rowIdx=np.array([0], np.uint32),
+              tcA2B=np.arange(16).astype(np.uint32), data=np.zeros(128, np.uint16))
+    with pytest.raises(hs.HspmmError) as e:
+        hs.Plan(ok)
+    assert e.value.code == 2                              # HSPMM_ERR_DEVICE: no CPU fallback exists

@@ -1,0 +1,145 @@
+"""The product's host format functions (hspmm_mtx_load, hspmm_btcf_sizes/fill in
+libhspmm.so) against the pinned oracle and the reference-produced golden vectors.
+Bit-exact: this is integer / byte work."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from util import random_csr
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DT = {0: "fp16", 1: "tf32"}
+
+
+def _same_btcf(a, b):
+    for k in ("eff_row_windows", "total_tiles", "total_row_windows"):
+        assert a[k] == b[k], k
+    for k in ("rowOffset", "tcA2B", "rowIdx"):
+        assert np.array_equal(a[k], b[k]), k
+    assert a["data"].tobytes() == b["data"].tobytes()
+
+
+def test_golden_vectors_through_the_library(hs):
+    with open(os.path.join(GOLD, "expected.json")) as f:
+        G = json.load(f)
+    for name in ("tiny", "gap"):
+        g = G[name]
+        dt = 0 if g["dtype"] == "fp16" else 1
+        m = hs.mtx_load(os.path.join(GOLD, g["file"]), dt)
+        assert (m["rows"], m["cols"], m["nnzs"]) == (g["rows"], g["cols"], g["nnzs"])
+        b = hs.csr_to_btcf(m["rows"], m["cols"], m["row_ptr"], m["col_idx"], m["values"], dt)
+        assert b["total_row_windows"] == g["total_row_windows"]
+        assert b["eff_row_windows"] == g["eff_row_windows"] and b["total_tiles"] == g["total_tiles"]
+        assert b["data"].size == g["data_size"]
+        assert b["rowOffset"].tolist() == g["rowOffset"]
+        assert b["rowIdx"].tolist() == g["rowIdx"]
+        assert b["tcA2B"].tolist() == g["tcA2B"]
+        if "tile_nonzeros" in g:
+            want = np.zeros((g["total_tiles"], 8, b["cw"]), np.float32)
+            for t, r, k, v in g["tile_nonzeros"]:
+                want[t, r, k] = v
+            assert np.array_equal(b["data"].view(np.float16).astype(np.float32).reshape(want.shape), want)
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_loader_equals_oracle(hs, oracle, tmp_path, dtype):
+    rng = np.random.default_rng(100 + dtype)
+    for case in range(6):
+        rows, cols = int(rng.integers(1, 200)), int(rng.integers(1, 200))
+        nnz = int(rng.integers(0, min(rows * cols, 3000) + 1))
+        flat = rng.choice(rows * cols, size=nnz, replace=False)
+        r, c = flat // cols, flat % cols
+        v = rng.normal(size=nnz) * 10.0 ** rng.integers(-9, 6, nnz)
+        p = tmp_path / ("m%d.mtx" % case)
+        with open(p, "w") as f:
+            f.write("%%MatrixMarket matrix coordinate real general\n%comment line\n%\n")
+            f.write("%d %d %d\n" % (rows, cols, nnz))
+            for i in range(nnz):
+                if case == 1 and i % 17 == 3:
+                    f.write("this line is skipped\n")
+                sep = "\t" if case == 2 else " "
+                f.write("%d%s%d%s%.9g\n" % (r[i] + 1, sep, c[i] + 1, sep, v[i]))
+        a = hs.mtx_load(str(p), dtype)
+        o = oracle.mtx_read(str(p), DT[dtype])
+        assert (a["rows"], a["cols"], a["nnzs"]) == (o["rows"], o["cols"], o["nnzs"])
+        assert np.array_equal(a["row_ptr"], o["row_ptr"])
+        assert np.array_equal(a["col_idx"], o["col_idx"])
+        assert a["values"].tobytes() == o["values"].tobytes()
+
+
+def test_loader_special_values_and_short_files(hs, oracle, tmp_path):
+    p = tmp_path / "s.mtx"
+    p.write_text("%%MatrixMarket\n4 4 9\n1 1 65520\n1 2 1e-8\n2 2 -6.1e-5\n2 3 5.96e-8\n"
+                 "3 1 inf\n3 3 0x1.8p1\n4 4 2.98e-8\n4 1 1e39\n")
+    for dt in (0, 1):
+        a = hs.mtx_load(str(p), dt)
+        o = oracle.mtx_read(str(p), DT[dt])
+        assert a["nnzs"] == o["nnzs"] == 8 and o["declared_nnz"] == 9        # load.h:234-238
+        assert np.array_equal(a["row_ptr"], o["row_ptr"]) and np.array_equal(a["col_idx"], o["col_idx"])
+        assert a["values"].tobytes() == o["values"].tobytes()
+
+
+def test_loader_errors(hs, tmp_path):
+    with pytest.raises(hs.HspmmError) as e:
+        hs.mtx_load(str(tmp_path / "nope.mtx"), 0)
+    assert e.value.code == 4 and "cannot open" in str(e.value)               # load.h:176-180
+    bad = tmp_path / "bad.mtx"
+    bad.write_text("%%MatrixMarket\n% only comments\n")
+    with pytest.raises(hs.HspmmError) as e:
+        hs.mtx_load(str(bad), 0)
+    assert e.value.code == 4                                                 # load.h:190-194
+    oob = tmp_path / "oob.mtx"
+    oob.write_text("2 2 1\n3 1 1.0\n")
+    with pytest.raises(hs.HspmmError):
+        hs.mtx_load(str(oob), 1)
+    with pytest.raises(hs.HspmmError):
+        hs.mtx_load(str(oob), 7)
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_converter_equals_oracle(hs, oracle, dtype):
+    rng = np.random.default_rng(200 + dtype)
+    shapes = [(1, 1, 1.0, 0.0), (8, 16, 0.5, 0.0), (9, 17, 0.5, 0.0), (27, 12, 0.1, 0.7), (64, 500, 0.05, 0.3),
+              (203, 77, 0.3, 0.1), (1000, 1000, 0.004, 0.5), (16, 4000, 0.6, 0.0)]
+    for rows, cols, dens, erp in shapes:
+        A = random_csr(rng, rows, cols, dens, dtype, erp)
+        for tr in (False, True):
+            a = hs.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype, transpose=tr)
+            o = oracle.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], DT[dtype], transpose=tr)
+            _same_btcf(a, o)
+
+
+def test_converter_large_multithreaded_equals_oracle(hs, oracle):
+    # big enough that the library's window loop runs on several threads
+    from hopper_spmm_amd import generators as G
+    A = G.rmat(15, 16, seed=9)
+    a = hs.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], 0)
+    o = oracle.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], "fp16")
+    _same_btcf(a, o)
+    A = G.pruned_weight(1376, 512, 0.1, seed=4)
+    a = hs.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], 1)
+    o = oracle.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], "tf32")
+    _same_btcf(a, o)
+
+
+def test_converter_empty_and_duplicates(hs, oracle):
+    # no stored entry at all: zero effective windows
+    rp = np.zeros(21, np.uint32)
+    b = hs.csr_to_btcf(20, 5, rp, np.zeros(0, np.uint32), np.zeros(0, np.uint16), 0)
+    assert b["eff_row_windows"] == 0 and b["total_tiles"] == 0 and b["rowOffset"].tolist() == [0]
+    # zero rows
+    b = hs.csr_to_btcf(0, 5, np.zeros(1, np.uint32), np.zeros(0, np.uint32), np.zeros(0, np.float32), 1)
+    assert b["eff_row_windows"] == 0 and b["total_row_windows"] == 0
+    # duplicate position: the later stored entry stays (convert.h:215)
+    rp = np.array([0, 3], np.uint32)
+    ci = np.array([4, 4, 9], np.uint32)
+    vv = np.array([1.0, 2.0, 3.0], np.float32)
+    a = hs.csr_to_btcf(1, 10, rp, ci, vv, 1)
+    o = oracle.csr_to_btcf(1, 10, rp, ci, vv, "tf32")
+    _same_btcf(a, o)
+    assert a["data"][0] == 2.0
+    # an explicit zero still claims a tile column
+    a = hs.csr_to_btcf(1, 10, np.array([0, 2], np.uint32), np.array([1, 7], np.uint32), np.array([0.0, 5.0], np.float32), 1)
+    assert a["tcA2B"].tolist()[:2] == [1, 7]

@@ -1,0 +1,85 @@
+"""The host-side work partition (hspmm_partition_preview): every tile belongs to
+exactly one range, partial-sum slots are consistent with the rule the kernel
+applies, and split windows are exactly the windows cut by a range boundary."""
+import numpy as np
+import pytest
+
+NO = 0xFFFFFFFF
+
+
+def simulate(ranges, ro):
+    """Walk each range the way the kernel does; returns {window: [slots in range order]}
+    and the set of windows stored directly."""
+    partial, direct = {}, []
+    for t0, t1, w, head, tail in ranges.tolist():
+        assert ro[w] <= t0 < ro[w + 1]
+        t = t0
+        while t < t1:
+            ws, we = int(ro[w]), int(ro[w + 1])
+            se = min(we, t1)
+            if t == ws and se == we:
+                direct.append(w)
+            else:
+                slot = head if t == t0 else tail
+                assert slot != NO
+                partial.setdefault(w, []).append(slot)
+            t = se
+            if se == we:
+                w += 1
+    return partial, direct
+
+
+def check(hs, ro, target):
+    ro = np.asarray(ro, np.uint32)
+    p = hs.partition_preview(ro, target)
+    r = p["ranges"]
+    W, T = ro.size - 1, int(ro[-1])
+    assert r[0, 0] == 0 and r[-1, 1] == T
+    assert np.array_equal(r[1:, 0], r[:-1, 1]) and np.all(r[:, 1] > r[:, 0])     # exact cover, no empty range
+    assert len(r) <= max(1, target)
+    partial, direct = simulate(r, ro)
+    slots = [s for w in sorted(partial) for s in partial[w]]
+    assert sorted(slots) == list(range(p["n_partial_slots"]))                     # each slot used once
+    assert p["n_split_windows"] == len(partial)
+    assert sorted(direct + list(partial)) == list(range(W))                       # every window finished once
+    assert all(len(v) >= 2 for v in partial.values())
+    used = set(r[:, 3].tolist()) | set(r[:, 4].tolist())
+    used.discard(NO)
+    assert used == set(slots)
+    return p
+
+
+def test_partition_small_cases(hs):
+    check(hs, [0, 1], 1)
+    check(hs, [0, 1], 8)
+    check(hs, [0, 100], 7)                      # one window cut into pieces
+    check(hs, [0, 1, 2, 40, 41], 4)
+    check(hs, np.arange(0, 1001), 16)           # 1000 one-tile windows: cuts snap, nothing split
+    p = check(hs, np.arange(0, 1001), 16)
+    assert p["n_split_windows"] == 0
+
+
+def test_partition_random(hs):
+    rng = np.random.default_rng(0)
+    for _ in range(60):
+        W = int(rng.integers(1, 400))
+        tiles = np.maximum(1, rng.pareto(1.2, W) * rng.integers(1, 8)).astype(np.int64)
+        ro = np.concatenate([[0], np.cumsum(tiles)])
+        check(hs, ro, int(rng.integers(1, 300)))
+
+
+def test_partition_balance_on_power_law(hs):
+    from hopper_spmm_amd import generators as G
+    A = G.rmat(16, 16, seed=5)
+    b = hs.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], 0)
+    p = check(hs, b["rowOffset"], 1024)
+    ln = (p["ranges"][:, 1] - p["ranges"][:, 0]).astype(np.int64)
+    assert ln.max() <= 2.0 * ln.mean()          # no range is more than twice the mean
+    assert p["n_partial_slots"] <= 2 * len(ln)
+
+
+def test_partition_rejects_bad_offsets(hs):
+    with pytest.raises(hs.HspmmError):
+        hs.partition_preview(np.array([0, 5, 5], np.uint32), 4)
+    with pytest.raises(hs.HspmmError):
+        hs.partition_preview(np.array([1, 5], np.uint32), 4)

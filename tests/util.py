@@ -1,0 +1,77 @@
+"""Helpers shared by the tests."""
+import numpy as np
+
+IDX_MAX = 0xFFFFFFFF
+
+
+def dtype_name(dtype):
+    return "fp16" if dtype == 0 else "tf32"
+
+
+def random_csr(rng, rows, cols, density, dtype, empty_row_prob=0.0, heavy_rows=()):
+    """Duplicate-free random CSR; values are fp16 bit patterns or float32."""
+    row_lists = []
+    for r in range(rows):
+        if r in heavy_rows:
+            k = max(1, int(cols * 0.8))
+        elif rng.random() < empty_row_prob:
+            k = 0
+        else:
+            k = rng.binomial(cols, density)
+        c = np.sort(rng.choice(cols, size=min(k, cols), replace=False)).astype(np.uint32)
+        row_lists.append(c)
+    row_ptr = np.zeros(rows + 1, np.uint32)
+    row_ptr[1:] = np.cumsum([len(c) for c in row_lists])
+    col_idx = np.concatenate(row_lists).astype(np.uint32) if rows else np.zeros(0, np.uint32)
+    v = rng.uniform(-1, 1, col_idx.size).astype(np.float32)
+    vals = v.astype(np.float16).view(np.uint16) if dtype == 0 else v
+    return dict(rows=rows, cols=cols, nnzs=int(col_idx.size), dtype=dtype, row_ptr=row_ptr,
+                col_idx=col_idx, values=vals)
+
+
+def csr_to_dense64(A):
+    """Dense float64 copy of a CSR dict (fp16 bits are decoded with numpy)."""
+    vals = A["values"].view(np.float16).astype(np.float64) if A["dtype"] == 0 else A["values"].astype(np.float64)
+    D = np.zeros((A["rows"], A["cols"]), np.float64)
+    rp = A["row_ptr"]
+    for r in range(A["rows"]):
+        D[r, A["col_idx"][rp[r]:rp[r + 1]]] = vals[rp[r]:rp[r + 1]]
+    return D
+
+
+def btcf_to_csr(b):
+    """Expand tiles through tcA2B / rowIdx back to (row, col, value) triples sorted
+    by (row, col): the round trip of the condensed format."""
+    cw = b["cw"]
+    out = []
+    data = b["data"].reshape(-1, 8, cw)
+    a2b = b["tcA2B"].reshape(-1, cw)
+    for w in range(b["eff_row_windows"]):
+        for t in range(b["rowOffset"][w], b["rowOffset"][w + 1]):
+            for k in range(cw):
+                c = a2b[t, k]
+                if c == IDX_MAX:
+                    continue
+                for r in range(8):
+                    v = data[t, r, k]
+                    if v != 0:
+                        out.append((int(b["rowIdx"][w]) + r, int(c), v))
+    out.sort(key=lambda x: (x[0], x[1]))
+    return out
+
+
+def csr_triples(A):
+    rp = A["row_ptr"]
+    out = []
+    for r in range(A["rows"]):
+        for i in range(rp[r], rp[r + 1]):
+            out.append((r, int(A["col_idx"][i]), A["values"][i]))
+    return out
+
+
+def half_ulp_distance(a_bits, b_bits):
+    """Distance in units of the last place between two arrays of half bit patterns."""
+    def key(x):
+        x = x.astype(np.int32)
+        return np.where(x & 0x8000, -(x & 0x7FFF), x & 0x7FFF)
+    return np.abs(key(a_bits) - key(b_bits))
