@@ -1,0 +1,175 @@
+"""Benchmark of the SpMM hot path on one MI355X.
+
+One step = one SpMM C = A*B (hspmm_run through the C ABI) on synthetic inputs that
+are resident in HBM before the timed region starts.  Prints one JSON line:
+effective TFLOP/s (2*nnz*N / t) as `value`, the HBM roofline of the main kernel
+(compulsory bytes / its measured duration against 8 TB/s) and a CPU baseline (the
+oracle's CSR SpMM on this machine's host cores).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--n N]
+                  [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "oracle")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {0: 2500.0, 1: 157.3}   # dense fp16 / fp32 matrix
+
+
+def cpu_baseline(A, B, N, flops_full):
+    """The oracle's CSR SpMM (test infrastructure used as the measured CPU baseline,
+    never as the product path) on a bounded sample of the rows."""
+    import numpy as np
+    import oracle
+    threads = oracle.max_threads()
+    rows = A["rows"]
+    rp = A["row_ptr"].astype(np.int64)
+    # sample: leading rows holding about 1/4 of the stored entries for the single-thread
+    # run, the whole matrix for the all-threads run if it is small enough
+    def sub(frac):
+        r_end = int(np.searchsorted(rp, rp[-1] * frac)) if frac < 1 else rows
+        r_end = max(1, min(rows, r_end))
+        n = int(rp[r_end])
+        return r_end, n
+    def run(r_end, n, nthreads):
+        t = time.perf_counter()
+        if A["dtype"] == 0:
+            oracle.spmm_csr_f16(r_end, N, A["row_ptr"][:r_end + 1], A["col_idx"][:n], A["values"][:n], B, threads=nthreads)
+        else:
+            oracle.spmm_csr_f32(r_end, N, A["row_ptr"][:r_end + 1], A["col_idx"][:n], A["values"][:n], B, threads=nthreads)
+        return time.perf_counter() - t
+    # size the samples from a tiny probe so that each run stays within ~10-15 s
+    r0, n0 = sub(0.01)
+    probe = max(run(r0, n0, 1), 1e-4)
+    per_nnz_1t = probe / max(n0, 1)
+    frac1 = min(1.0, 10.0 / (per_nnz_1t * rp[-1]))
+    r1, n1 = sub(frac1)
+    t1 = run(r1, n1, 1)
+    fracm = min(1.0, 10.0 * threads * 0.7 / (per_nnz_1t * rp[-1]))
+    rm, nm = sub(fracm)
+    tm = run(rm, nm, threads)
+    return {
+        "value": 2.0 * nm * N / tm / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": "oracle CSR SpMM (fp32 accumulate), first %d of %d rows (%d of %d stored entries), %d threads, %.2f s"
+                  % (rm, rows, nm, int(rp[-1]), threads, tm),
+        "single_thread": {"value": 2.0 * n1 * N / t1 / 1e12, "unit": "TFLOP/s", "cores": 1,
+                          "sample": "first %d rows (%d stored entries), %.2f s" % (r1, n1, t1)},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2, help="index into the benchmark configurations (default: 2, the 1M-row power-law graph)")
+    ap.add_argument("--n", type=int, default=0, help="feature dimension (default: the configuration's)")
+    ap.add_argument("--shrink", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--mode", type=int, default=0, help="kernel mode (hspmm_set_kernel_mode)")
+    ap.add_argument("--stages", type=int, default=0)
+    ap.add_argument("--waves-per-group", type=int, default=0)
+    ap.add_argument("--ranges-per-simd", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this operator runs on a single MI355X and nothing here uses a "
+              "second one (--gpus %d refused)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import hopper_spmm_amd as hs
+    from hopper_spmm_amd import generators as G
+
+    if not torch.cuda.is_available():
+        print("bench.py needs the GPU", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    t_gen = time.perf_counter()
+    cfg = G.make_config(args.config, args.shrink)
+    A = cfg["A"]
+    N = args.n or (cfg["N"][0] if args.config != 4 else 64)
+    dt = A["dtype"]
+    b = hs.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], dt)
+    B = G.dense_b(A["cols"], N, cfg["b_seed"], dt)
+    t_gen = time.perf_counter() - t_gen
+
+    hs.set_kernel_mode(args.mode)
+    hs.configure(args.stages, args.waves_per_group, args.ranges_per_simd, 0)
+    plan = hs.Plan(b)
+    if dt == hs.FP16:
+        dB = torch.from_numpy(B.view(np.int16)).cuda()
+        dC = torch.empty((A["rows"], N), dtype=torch.int16, device="cuda")
+    else:
+        dB = torch.from_numpy(B).cuda()
+        dC = torch.empty((A["rows"], N), dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    pB, pC = dB.data_ptr(), dC.data_ptr()
+
+    for _ in range(args.warmup):
+        plan.run(pB, pC, N, stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.run(pB, pC, N, stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    # kernel durations with device events on the launch stream
+    main_ms, fix_ms = plan.profile(pB, pC, N, runs=args.steps, stream=stream)
+    main_ms /= args.steps
+    fix_ms /= args.steps
+    # the reference's own convention: 3 warm-ups, 5 timed launches (src/common.h:48-49)
+    ref_conv_ms = plan.bench(pB, pC, N, warmup=3, runs=5, stream=stream) / 5.0
+
+    nnz = int(A["nnzs"])
+    flops = 2.0 * nnz * N
+    bytes_alg = G.algorithmic_bytes(b, N)
+    bytes_gather = G.gather_bytes(b, N)
+    info = plan.info()
+    traffic = None
+    tfile = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tfile):
+        with open(tfile) as f:
+            traffic = json.load(f).get("config%d_N%d" % (args.config, N))
+
+    out = {
+        "metric": "SpMM effective TFLOP/s (2*nnz*N)",
+        "value": flops / (ms_per_step * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 in, f32 accumulate" if dt == hs.FP16 else "f32 (tf32 variant)",
+        "data": "synthetic",
+        "config": {"workload": "configs[%d]: %s, N=%d" % (args.config, cfg["name"], N),
+                   "rows": A["rows"], "cols": A["cols"], "nnz": nnz, "tiles": int(b["total_tiles"]),
+                   "eff_row_windows": int(b["eff_row_windows"]), "ranges": info["n_ranges"],
+                   "split_windows": info["n_split_windows"]},
+        "effective_gbps": bytes_alg / (ms_per_step * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": bytes_alg / (main_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": bytes_alg / (main_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": traffic,
+                     "kernel": "spmm_mfma_kernel", "kernel_ms": main_ms, "fixup_kernel_ms": fix_ms,
+                     "algorithmic_bytes": bytes_alg, "gather_bytes": bytes_gather,
+                     "mfma_frac_of_peak_useful_flops": flops / (main_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[dt]},
+        "reference_convention_ms": ref_conv_ms,
+        "setup_seconds": t_gen,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(A, B, N, flops)
+    plan.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -59,12 +59,22 @@ def load_library():
         return _lib
     if not os.path.exists(_LIB):
         build_library(force=False)
+    # A process that also uses PyTorch must end up with one HIP runtime.  PyTorch
+    # ships its own libamdhip64 with the same soname as the system one this
+    # library is linked against; whichever is loaded first serves both, and
+    # PyTorch does not find the device through the system copy.  So let PyTorch
+    # load its runtime first when it is installed.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(_LIB)
     u32, vp, i = C.c_uint32, C.c_void_p, C.c_int
     L.hspmm_last_error.restype = C.c_char_p
     L.hspmm_create.argtypes = [C.POINTER(vp), i, u32, u32, u32, u32, vp, vp, vp, vp]
     L.hspmm_run.argtypes = [vp, vp, vp, u32, vp]
     L.hspmm_bench.argtypes = [vp, vp, vp, u32, i, i, vp, C.POINTER(C.c_float)]
+    L.hspmm_profile.argtypes = [vp, vp, vp, u32, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_float)]
     L.hspmm_destroy.argtypes = [vp]
     L.hspmm_destroy.restype = None
     L.hspmm_configure.argtypes = [i, i, i, i]
@@ -198,6 +208,13 @@ class Plan:
         _check(load_library().hspmm_bench(self._h, C.c_void_p(dB_ptr), C.c_void_p(dC_ptr), N, warmup, runs,
                                           C.c_void_p(stream), C.byref(ms)))
         return ms.value
+
+    def profile(self, dB_ptr, dC_ptr, N, runs=5, stream=0):
+        """(main kernel ms, partial-sum kernel ms), totals over `runs` launches."""
+        a, b = C.c_float(), C.c_float()
+        _check(load_library().hspmm_profile(self._h, C.c_void_p(dB_ptr), C.c_void_p(dC_ptr), N, runs,
+                                            C.c_void_p(stream), C.byref(a), C.byref(b)))
+        return a.value, b.value
 
     def info(self):
         inf = PlanInfo()

@@ -210,6 +210,8 @@ int ensure_scratch(hspmm_plan *p, size_t bytes)
 
 }  // namespace
 
+static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream, hipEvent_t mid);
+
 extern "C" {
 
 const char *hspmm_last_error(void) { return g_last_error.c_str(); }
@@ -336,6 +338,15 @@ void hspmm_destroy(hspmm_plan *p)
 
 int hspmm_run(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream)
 {
+    return hspmm_run_marked(p, dB, dC, N, stream, nullptr);
+}
+
+}  // extern "C"
+
+// mid: when not null, an event recorded between the main kernel and the kernel
+// that adds the partial sums of split windows.
+static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream, hipEvent_t mid)
+{
     if (!p) return fail(HSPMM_ERR_INVALID, "null plan");
     if (N == 0) return fail(HSPMM_ERR_INVALID, "feature dimension N = 0");
     if (p->rows == 0) return HSPMM_OK;
@@ -371,8 +382,42 @@ int hspmm_run(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream)
     ka.scratch = p->d_scratch;
     const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage : (p->dtype == HSPMM_FP16 ? 3 : 4);
     const int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
-    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, c.layout, ka, c.V, prefetch, c.narrow, wpg, s));
+    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, c.layout, ka, c.V, prefetch, c.narrow, wpg, s, mid));
     return HSPMM_OK;
+}
+
+extern "C" {
+
+int hspmm_profile(hspmm_plan *p, const void *dB, void *dC, uint32_t N, int runs, void *stream,
+                  float *main_ms, float *fixup_ms)
+{
+    if (!main_ms || !fixup_ms) return fail(HSPMM_ERR_INVALID, "null output");
+    if (runs < 1 || runs > 1000) return fail(HSPMM_ERR_INVALID, "runs %d outside 1..1000", runs);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    std::vector<hipEvent_t> ev(size_t(runs) * 3);
+    for (auto &e : ev) HSPMM_HIP(hipEventCreate(&e));
+    int rc = HSPMM_OK;
+    for (int i = 0; i < runs && !rc; ++i) {
+        HSPMM_HIP(hipEventRecord(ev[3 * i], s));
+        rc = hspmm_run_marked(p, dB, dC, N, stream, ev[3 * i + 1]);
+        HSPMM_HIP(hipEventRecord(ev[3 * i + 2], s));
+    }
+    if (!rc) {
+        HSPMM_HIP(hipStreamSynchronize(s));
+        *main_ms = 0.f; *fixup_ms = 0.f;
+        for (int i = 0; i < runs; ++i) {
+            float a = 0.f, b = 0.f;
+            if (hipEventQuery(ev[3 * i + 1]) == hipSuccess && hipEventElapsedTime(&a, ev[3 * i], ev[3 * i + 1]) == hipSuccess) {
+                HSPMM_HIP(hipEventElapsedTime(&b, ev[3 * i + 1], ev[3 * i + 2]));
+            } else {                          // no split windows (or scalar kernel): one kernel only
+                (void)hipGetLastError();
+                HSPMM_HIP(hipEventElapsedTime(&a, ev[3 * i], ev[3 * i + 2]));
+            }
+            *main_ms += a; *fixup_ms += b;
+        }
+    }
+    for (auto &e : ev) (void)hipEventDestroy(e);
+    return rc;
 }
 
 int hspmm_bench(hspmm_plan *p, const void *dB, void *dC, uint32_t N, int warmup, int runs, void *stream,

@@ -36,8 +36,9 @@ struct KernelArgs {
 // kLayoutDW = word loads, features strided by 32 per lane, N % (32V) == 0.
 constexpr int kLayoutX4 = 0, kLayoutDW = 1;
 // narrow: B < 4 GiB and cols < 2^24 (32-bit gather offsets).
+// mid: optional event recorded between the main kernel and the partial-sum kernel.
 hipError_t launch_spmm_mfma(int dtype, int layout, const KernelArgs &ka, int V, int prefetch, bool narrow,
-                            int waves_per_group, hipStream_t s);
+                            int waves_per_group, hipStream_t s, hipEvent_t mid);
 hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s);
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
 

@@ -342,7 +342,10 @@ struct Fp32Tile {
     }
     template <int p> __device__ static __forceinline__ float word(const BVec &v)
     {
-        if constexpr (V == 1) return __builtin_bit_cast(float, v); else return __builtin_bit_cast(float, v[p]);
+        // (a bit_cast applied directly to a vector element reads element 0: copy first)
+        uint32_t w;
+        if constexpr (V == 1) w = v; else w = v[p];
+        return __builtin_bit_cast(float, w);
     }
     template <int p>
     __device__ static __forceinline__ void mma_one(const float a0, const float a1, const BVec &b0, const BVec &b1,
@@ -370,7 +373,7 @@ struct Fp32Tile {
             const uint32_t row = row0 + 4u * L.g + e;
             uint32_t out[V];
 #pragma unroll
-            for (int p = 0; p < V; ++p) out[p] = __builtin_bit_cast(uint32_t, acc[p][e]);
+            for (int p = 0; p < V; ++p) { const float f = acc[p][e]; out[p] = __builtin_bit_cast(uint32_t, f); }
             if (active && L.g < 2u && row < rows) store_words<V>(c_lane + size_t(row) * row_bytes, out);
         }
     }
@@ -643,7 +646,8 @@ static hipError_t launch_main_n(const KernelArgs &ka, int prefetch, bool narrow,
 }
 
 template <template <int> class TTV>
-static hipError_t launch_mfma(const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, hipStream_t s)
+static hipError_t launch_mfma(const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, hipStream_t s,
+                              hipEvent_t mid)
 {
     const uint32_t items = ka.n_ranges * ka.n_feat_blocks;
     const dim3 block(64u * waves_per_group);
@@ -653,6 +657,7 @@ static hipError_t launch_mfma(const KernelArgs &ka, int V, int prefetch, bool na
     else if (V == 2) e = launch_main_n<TTV<2>, 2>(ka, prefetch, narrow, grid, block, s);
     else e = launch_main_n<TTV<1>, 1>(ka, prefetch, narrow, grid, block, s);
     if (e != hipSuccess || ka.n_split == 0) return e;
+    if (mid && (e = hipEventRecord(mid, s)) != hipSuccess) return e;
     const uint32_t fitems = ka.n_split * ka.n_feat_blocks;
     const dim3 fgrid((fitems + waves_per_group - 1) / waves_per_group);
     if (V == 4) spmm_fixup_kernel<TTV<4>, 4><<<fgrid, block, 0, s>>>(ka);
@@ -662,11 +667,11 @@ static hipError_t launch_mfma(const KernelArgs &ka, int V, int prefetch, bool na
 }
 
 hipError_t launch_spmm_mfma(int dtype, int layout, const KernelArgs &ka, int V, int prefetch, bool narrow,
-                            int waves_per_group, hipStream_t s)
+                            int waves_per_group, hipStream_t s, hipEvent_t mid)
 {
-    if (dtype != 0) return launch_mfma<Fp32Tile>(ka, V, prefetch, narrow, waves_per_group, s);
-    return layout == kLayoutDW ? launch_mfma<Fp16TileDW>(ka, V, prefetch, narrow, waves_per_group, s)
-                               : launch_mfma<Fp16Tile>(ka, V, prefetch, narrow, waves_per_group, s);
+    if (dtype != 0) return launch_mfma<Fp32Tile>(ka, V, prefetch, narrow, waves_per_group, s, mid);
+    return layout == kLayoutDW ? launch_mfma<Fp16TileDW>(ka, V, prefetch, narrow, waves_per_group, s, mid)
+                               : launch_mfma<Fp16Tile>(ka, V, prefetch, narrow, waves_per_group, s, mid);
 }
 
 hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s)

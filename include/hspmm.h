@@ -71,6 +71,13 @@ int hspmm_run(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stre
 int hspmm_bench(hspmm_plan *plan, const void *dB, void *dC, uint32_t N,
                 int warmup, int runs, void *stream, float *total_ms);
 
+/* No reference counterpart (the reference times whole launches only): `runs`
+ * launches with an event between the two kernels of a launch; *main_ms is the
+ * total time of the main kernel, *fixup_ms of the kernel that adds the partial
+ * sums of windows split across waves (0 when no window is split). */
+int hspmm_profile(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, int runs, void *stream,
+                  float *main_ms, float *fixup_ms);
+
 /* Replaces the cudaFree block of fp16_spmm (reference src/fp16.cu:274-279). */
 void hspmm_destroy(hspmm_plan *plan);
 

@@ -1,0 +1,367 @@
+"""Parity of the HIP operator (through the C ABI of libhspmm.so) with the CPU
+oracle on the same seeded inputs.  Needs a real MI355X: run with -m gpu.
+
+Tolerances (from the task's statement of parity):
+  fp16 path : |gpu - ref| <= 1e-2 * |ref| + 1e-5 * sum_k |a_k b_k|
+  tf32 path : |gpu - ref| <= 1e-3 * |ref| + 1e-5 * sum_k |a_k b_k|
+The second term only matters where a sum cancels to (almost) nothing; it is the
+size of fp32 reassociation noise.  Index handling is checked bit-exactly through
+cases whose arithmetic is exact (small integers) and through the format tests.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from util import csr_to_dense64, half_ulp_distance, random_csr
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DT = {0: "fp16", 1: "tf32"}
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return torch
+
+
+def gpu_spmm(torch, hs, btcf, B, N, plan=None, poison=True):
+    """C = A*B on the device through hspmm_run; B, C as numpy (uint16 bits / float32)."""
+    own = plan is None
+    if own:
+        plan = hs.Plan(btcf)
+    dt = btcf["dtype"]
+    rows = btcf["rows"]
+    if dt == 0:
+        dB = torch.from_numpy(np.ascontiguousarray(B, np.uint16).view(np.int16)).cuda()
+        dC = torch.empty((rows, N), dtype=torch.int16, device="cuda")
+        if poison:
+            dC.fill_(0x7E01)                     # a NaN pattern: unwritten elements show up
+    else:
+        dB = torch.from_numpy(np.ascontiguousarray(B, np.float32)).cuda()
+        dC = torch.empty((rows, N), dtype=torch.float32, device="cuda")
+        if poison:
+            dC.fill_(float("nan"))
+    stream = torch.cuda.current_stream().cuda_stream
+    plan.run(dB.data_ptr(), dC.data_ptr(), N, stream)
+    torch.cuda.synchronize()
+    out = dC.cpu().numpy()
+    if own:
+        plan.close()
+    return out.view(np.uint16) if dt == 0 else out
+
+
+def oracle_spmm(oracle, A, B, N):
+    if A["dtype"] == 0:
+        return oracle.spmm_csr_f16(A["rows"], N, A["row_ptr"], A["col_idx"], A["values"], B, want_absdot=True)
+    return oracle.spmm_csr_f32(A["rows"], N, A["row_ptr"], A["col_idx"], A["values"], B, want_absdot=True)
+
+
+def assert_parity(got, ref, absdot, dtype, what=""):
+    if dtype == 0:
+        g = got.view(np.float16).astype(np.float64)
+        r = ref.view(np.float16).astype(np.float64)
+        rel = 1e-2
+    else:
+        g, r, rel = got.astype(np.float64), ref.astype(np.float64), 1e-3
+    assert not np.isnan(g).any(), what + ": unwritten or NaN output"
+    err = np.abs(g - r)
+    bound = rel * np.abs(r) + 1e-5 * absdot.astype(np.float64)
+    bad = err > bound
+    assert not bad.any(), "%s: %d of %d outputs outside tolerance, worst %g at %s" % (
+        what, int(bad.sum()), bad.size, float((err - bound).max()), np.unravel_index(np.argmax(err - bound), err.shape))
+    if dtype == 0 and got.size:
+        # far tighter in practice: fp16 rounding of nearly identical fp32 sums
+        ulp = half_ulp_distance(got, ref)
+        assert (ulp <= 1).mean() > 0.999, what + ": too many outputs differ by more than one half ulp"
+
+
+def make_b(rng, cols, N, dtype):
+    x = rng.normal(size=(cols, N)).astype(np.float32)
+    return x.astype(np.float16).view(np.uint16) if dtype == 0 else x
+
+
+def convert(hs, A):
+    return hs.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], A["dtype"])
+
+
+# ------------------------------------------------------------------ golden files
+def test_golden_files_end_to_end(torch_cuda, hs, oracle):
+    rng = np.random.default_rng(1)
+    for name, dt in (("tiny.mtx", 0), ("gap.mtx", 1)):
+        A = hs.mtx_load(os.path.join(GOLD, name), dt)
+        A["dtype"] = dt
+        b = convert(hs, A)
+        for N in (1, 2, 3, 8, 16, 40, 64, 128):
+            B = make_b(rng, A["cols"], N, dt)
+            got = gpu_spmm(torch_cuda, hs, b, B, N)
+            ref, mag = oracle_spmm(oracle, A, B, N)
+            assert_parity(got, ref, mag, dt, "%s N=%d" % (name, N))
+            # gap.mtx: rows 8..23 lie in no effective window and the last window has
+            # three real rows; all of that must come out as exact zeros
+            dense = csr_to_dense64(A)
+            empty = ~dense.any(axis=1)
+            assert not got[empty].any()
+
+
+# ------------------------------------------------------------------ exact arithmetic: bit-exact
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_exact_integer_inputs_are_bit_exact(torch_cuda, hs, oracle, dtype, mode):
+    rng = np.random.default_rng(40 + dtype)
+    rows, cols = 203, 310
+    D = rng.integers(-3, 4, (rows, cols)) * (rng.random((rows, cols)) < 0.15)
+    D[40:56] = 0                                    # two empty windows in the middle
+    rp = np.zeros(rows + 1, np.uint32)
+    ci, vv = [], []
+    for r in range(rows):
+        nz = np.nonzero(D[r])[0]
+        ci += nz.tolist(); vv += D[r, nz].tolist()
+        rp[r + 1] = len(ci)
+    vals = np.array(vv, np.float32)
+    A = dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=np.array(ci, np.uint32),
+             values=vals.astype(np.float16).view(np.uint16) if dtype == 0 else vals)
+    hs.set_kernel_mode(mode)
+    try:
+        b = convert(hs, A)
+        for N in (4, 32, 64, 128, 160):
+            Bm = rng.integers(-4, 5, (cols, N))
+            B = Bm.astype(np.float16).view(np.uint16) if dtype == 0 else Bm.astype(np.float32)
+            got = gpu_spmm(torch_cuda, hs, b, B, N)
+            want = D @ Bm
+            g = got.view(np.float16).astype(np.int64) if dtype == 0 else got.astype(np.int64)
+            assert np.array_equal(g, want), "mode %d N %d" % (mode, N)
+    finally:
+        hs.set_kernel_mode(0)
+
+
+# ------------------------------------------------------------------ shapes, tails, splits
+SHAPES = [
+    # rows, cols, density, empty-row probability, heavy rows
+    (1, 1, 1.0, 0.0, ()),
+    (7, 33, 0.4, 0.0, ()),
+    (8, 16, 1.0, 0.0, ()),
+    (27, 100, 0.1, 0.5, ()),
+    (130, 257, 0.05, 0.3, ()),
+    (300, 3000, 0.004, 0.2, (5, 100, 101, 299)),    # heavy windows: cut across ranges
+    (1000, 700, 0.01, 0.6, (512,)),
+]
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_random_shapes_and_feature_dims(torch_cuda, hs, oracle, dtype, shape):
+    rows, cols, dens, erp, heavy = shape
+    rng = np.random.default_rng(hash((rows, cols, dtype)) & 0xFFFF)
+    A = random_csr(rng, rows, cols, dens, dtype, erp, heavy)
+    b = convert(hs, A)
+    # many ranges, so that heavy windows are split and partial sums are exercised
+    hs.configure(producer_warp_group_num=16)
+    try:
+        plan = hs.Plan(b)
+    finally:
+        hs.configure()
+    if heavy:
+        assert plan.info()["n_split_windows"] > 0
+    for N in (1, 2, 6, 8, 16, 24, 32, 64, 72, 96, 128, 200, 256, 384):
+        B = make_b(rng, cols, N, dtype)
+        got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        assert_parity(got, ref, mag, dtype, "shape %s N=%d" % (shape[:2], N))
+    plan.close()
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("mode", [1, 2, 3])
+@pytest.mark.parametrize("stages", [1, 2, 4, 6, 8])
+def test_kernel_variants_agree_with_oracle(torch_cuda, hs, oracle, dtype, mode, stages):
+    rng = np.random.default_rng(77)
+    A = random_csr(rng, 260, 2000, 0.01, dtype, 0.2, (17, 130))
+    b = convert(hs, A)
+    hs.set_kernel_mode(mode)
+    hs.configure(buffer_stage=stages, consumer_warp_num=1 + stages % 4, producer_warp_group_num=8)
+    try:
+        plan = hs.Plan(b)
+        for N in (32, 64, 128, 512):
+            B = make_b(rng, 2000, N, dtype)
+            got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+            ref, mag = oracle_spmm(oracle, A, B, N)
+            assert_parity(got, ref, mag, dtype, "mode %d stages %d N=%d" % (mode, stages, N))
+        plan.close()
+    finally:
+        hs.set_kernel_mode(0)
+        hs.configure()
+
+
+def test_unaligned_and_odd_feature_dims_use_the_all_shapes_kernel(torch_cuda, hs, oracle):
+    rng = np.random.default_rng(5)
+    A = random_csr(rng, 90, 120, 0.1, 0, 0.2)
+    b = convert(hs, A)
+    for N in (1, 3, 7, 33, 129):
+        B = make_b(rng, 120, N, 0)
+        got = gpu_spmm(torch_cuda, hs, b, B, N)
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        assert_parity(got, ref, mag, 0, "odd N=%d" % N)
+
+
+def test_matrix_without_entries_gives_zeros(torch_cuda, hs):
+    for dt in (0, 1):
+        vt = np.uint16 if dt == 0 else np.float32
+        b = hs.csr_to_btcf(21, 9, np.zeros(22, np.uint32), np.zeros(0, np.uint32), np.zeros(0, vt), dt)
+        for N in (1, 5, 64):
+            got = gpu_spmm(torch_cuda, hs, b, np.ones((9, N), vt), N)
+            assert got.shape == (21, N) and not got.any()
+
+
+def test_plan_reuse_is_deterministic(torch_cuda, hs, oracle):
+    rng = np.random.default_rng(9)
+    A = random_csr(rng, 400, 4000, 0.003, 0, 0.1, (3, 200))
+    b = convert(hs, A)
+    hs.configure(producer_warp_group_num=16)
+    try:
+        plan = hs.Plan(b)
+    finally:
+        hs.configure()
+    B = make_b(rng, 4000, 128, 0)
+    first = gpu_spmm(torch_cuda, hs, b, B, 128, plan=plan)
+    # a wider N in between makes the plan regrow its scratch memory
+    B2 = make_b(rng, 4000, 512, 0)
+    wide = gpu_spmm(torch_cuda, hs, b, B2, 512, plan=plan)
+    ref2, mag2 = oracle_spmm(oracle, A, B2, 512)
+    assert_parity(wide, ref2, mag2, 0, "N=512 after N=128")
+    for _ in range(3):
+        again = gpu_spmm(torch_cuda, hs, b, B, 128, plan=plan)
+        assert np.array_equal(first, again)           # fixed summation order: bit-identical
+    plan.close()
+
+
+def test_bench_entry_point_and_errors(torch_cuda, hs, oracle):
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    A = random_csr(rng, 64, 64, 0.2, 0)
+    b = convert(hs, A)
+    plan = hs.Plan(b)
+    B = make_b(rng, 64, 64, 0)
+    dB = torch.from_numpy(B.view(np.int16)).cuda()
+    dC = torch.zeros((64, 64), dtype=torch.int16, device="cuda")
+    ms = plan.bench(dB.data_ptr(), dC.data_ptr(), 64, warmup=3, runs=5)      # src/common.h:48-49
+    assert ms > 0
+    ref, mag = oracle_spmm(oracle, A, B, 64)
+    assert_parity(dC.cpu().numpy().view(np.uint16), ref, mag, 0, "after bench")
+    with pytest.raises(hs.HspmmError):
+        plan.run(dB.data_ptr(), dC.data_ptr(), 0)                            # N = 0
+    with pytest.raises(hs.HspmmError):
+        plan.run(0, dC.data_ptr(), 64)                                       # null B
+    with pytest.raises(hs.HspmmError):
+        plan.run(dB.data_ptr(), 0, 64)                                       # null C
+    with pytest.raises(hs.HspmmError):
+        plan.bench(dB.data_ptr(), dC.data_ptr(), 64, warmup=0, runs=0)
+    info = plan.info()
+    assert info["rows"] == 64 and info["compute_units"] > 0 and info["device_bytes"] > 0
+    plan.close()
+
+
+# ------------------------------------------------------------------ the five configurations
+@pytest.mark.parametrize("index,shrink", [(0, 1), (1, 8), (2, 64), (3, 8), (4, 8)])
+def test_benchmark_configurations_reduced(torch_cuda, hs, oracle, index, shrink):
+    from hopper_spmm_amd import generators as G
+    cfg = G.make_config(index, shrink)
+    A = cfg["A"]
+    b = convert(hs, A)
+    plan = hs.Plan(b)
+    for N in cfg["N"]:
+        B = G.dense_b(A["cols"], N, cfg["b_seed"], A["dtype"])
+        got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        assert_parity(got, ref, mag, A["dtype"], "%s N=%d" % (cfg["name"], N))
+    plan.close()
+
+
+def _rows_subproblem(A, rows_sel):
+    rp = A["row_ptr"].astype(np.int64)
+    lens = rp[rows_sel + 1] - rp[rows_sel]
+    sub_rp = np.zeros(rows_sel.size + 1, np.uint32)
+    sub_rp[1:] = np.cumsum(lens)
+    idx = np.concatenate([np.arange(rp[r], rp[r + 1]) for r in rows_sel]) if rows_sel.size else np.zeros(0, np.int64)
+    return dict(rows=int(rows_sel.size), cols=A["cols"], dtype=A["dtype"], row_ptr=sub_rp,
+                col_idx=A["col_idx"][idx], values=A["values"][idx])
+
+
+@pytest.mark.parametrize("index", [1, 2, 3, 4])
+def test_benchmark_configurations_full_size(torch_cuda, hs, oracle, index):
+    """At full size the oracle is run on a sample of rows only (the heaviest rows
+    and a random sample), and size-independent properties cover the rest:
+    B = 1 gives the row sums, rows without entries are zero, and the all-shapes
+    kernel - an independent implementation - agrees on every element."""
+    from hopper_spmm_amd import generators as G
+    cfg = G.make_config(index, 1)
+    A = cfg["A"]
+    dt = A["dtype"]
+    b = convert(hs, A)
+    N = cfg["N"][0] if index != 4 else 64
+    plan = hs.Plan(b)
+    B = G.dense_b(A["cols"], N, cfg["b_seed"], dt)
+    got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+    rng = np.random.default_rng(index)
+    lens = np.diff(A["row_ptr"].astype(np.int64))
+    sel = np.unique(np.concatenate([np.argsort(lens)[-40:], rng.choice(A["rows"], 3000, replace=False)]))
+    sub = _rows_subproblem(A, sel)
+    ref, mag = oracle_spmm(oracle, sub, B, N)
+    assert_parity(got[sel], ref, mag, dt, "%s sampled rows" % cfg["name"])
+    assert not got[lens == 0].any()
+    # independent implementation on all elements
+    hs.set_kernel_mode(1)
+    try:
+        plan_s = hs.Plan(b)
+    finally:
+        hs.set_kernel_mode(0)
+    other = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan_s)
+    plan_s.close()
+    if dt == 0:
+        assert (half_ulp_distance(got, other) <= 1).mean() > 0.999
+        assert np.allclose(got.view(np.float16).astype(np.float32), other.view(np.float16).astype(np.float32),
+                           rtol=1e-2, atol=1e-3)
+    else:
+        assert np.allclose(got, other, rtol=1e-3, atol=1e-4)
+    # B = 1: C[r, :] = sum of row r (R-MAT rows sum to 1 by construction)
+    ones = np.full((A["cols"], N), 0x3C00, np.uint16) if dt == 0 else np.ones((A["cols"], N), np.float32)
+    c1 = gpu_spmm(torch_cuda, hs, b, ones, N, plan=plan)
+    vals = A["values"].view(np.float16).astype(np.float64) if dt == 0 else A["values"].astype(np.float64)
+    rowsum = np.add.reduceat(np.concatenate([vals, [0.0]]), np.minimum(A["row_ptr"][:-1], vals.size).astype(np.int64))
+    rowsum[lens == 0] = 0.0
+    absum = np.add.reduceat(np.concatenate([np.abs(vals), [0.0]]), np.minimum(A["row_ptr"][:-1], vals.size).astype(np.int64))
+    absum[lens == 0] = 0.0
+    c1f = c1.view(np.float16).astype(np.float64) if dt == 0 else c1.astype(np.float64)
+    tol = (2e-3 if dt == 0 else 1e-5) * np.abs(rowsum) + 1e-5 * absum + 1e-7
+    assert np.all(np.abs(c1f - rowsum[:, None]) <= tol[:, None])
+    assert np.all(c1f == c1f[:, :1])                     # every feature column identical
+    plan.close()
+
+
+def test_columns_beyond_the_32_bit_offset_range(torch_cuda, hs, oracle):
+    """B larger than 4 GiB: the gather uses 64-bit addresses."""
+    torch = torch_cuda
+    cols, N = (1 << 24) + 96, 128
+    rng = np.random.default_rng(12)
+    used = np.unique(np.concatenate([rng.choice(cols, 300, replace=False), [0, cols - 1, (1 << 24) - 1, 1 << 24]]))
+    rows = 40
+    rl = [np.sort(rng.choice(used, int(rng.integers(0, 30)), replace=False)).astype(np.uint32) for _ in range(rows)]
+    rp = np.zeros(rows + 1, np.uint32)
+    rp[1:] = np.cumsum([len(x) for x in rl])
+    ci = np.concatenate(rl).astype(np.uint32)
+    vals = rng.uniform(-1, 1, ci.size).astype(np.float32).astype(np.float16).view(np.uint16)
+    b = hs.csr_to_btcf(rows, cols, rp, ci, vals, 0)
+    small = make_b(rng, used.size, N, 0)                 # B rows that are referenced
+    dB = torch.zeros((cols, N), dtype=torch.int16, device="cuda")
+    dB[torch.from_numpy(used.astype(np.int64)).cuda()] = torch.from_numpy(small.view(np.int16)).cuda()
+    dC = torch.empty((rows, N), dtype=torch.int16, device="cuda")
+    plan = hs.Plan(b)
+    plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    got = dC.cpu().numpy().view(np.uint16)
+    plan.close()
+    remap = np.searchsorted(used, ci).astype(np.uint32)
+    ref, mag = oracle.spmm_csr_f16(rows, N, rp, remap, vals, small, want_absdot=True)
+    assert_parity(got, ref, mag, 0, "wide B")
