@@ -78,6 +78,8 @@ def main():
     ap.add_argument("--stages", type=int, default=0)
     ap.add_argument("--waves-per-group", type=int, default=0)
     ap.add_argument("--ranges-per-simd", type=int, default=0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain device copy of 1 GiB (reference point for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this operator runs on a single MI355X and nothing here uses a "
@@ -130,6 +132,14 @@ def main():
     fix_ms /= args.steps
     # the reference's own convention: 3 warm-ups, 5 timed launches (src/common.h:48-49)
     ref_conv_ms = plan.bench(pB, pC, N, warmup=3, runs=5, stream=stream) / 5.0
+
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")       # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     nnz = int(A["nnzs"])
     flops = 2.0 * nnz * N

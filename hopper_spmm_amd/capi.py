@@ -36,7 +36,17 @@ def build_library(force=True):
     if force:
         cmd.insert(1, "-B")
     subprocess.check_call(cmd, stdout=subprocess.DEVNULL)
+    # the command-line drivers (fp16_test / tf32_test) link against the library
+    cli = ["make", "-C", os.path.join(_HERE, "host")]
+    if force:
+        cli.insert(1, "-B")
+    subprocess.check_call(cli + ["fp16_test", "tf32_test"], stdout=subprocess.DEVNULL)
     return _LIB
+
+
+def cli_path(name):
+    """Path of a built command-line driver: 'fp16_test' or 'tf32_test'."""
+    return os.path.join(_HERE, "host", name)
 
 
 class _Csr(C.Structure):

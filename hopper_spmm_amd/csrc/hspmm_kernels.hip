@@ -55,6 +55,34 @@ __device__ __forceinline__ void load_words(const void *p, uint32_t (&dst)[V])
     }
 }
 
+// The tiles, the column ids and C are touched once per launch; the rows of B are
+// touched again and again.  HSPMM_NT_LOAD / HSPMM_NT_STORE mark the former
+// non-temporal so that they do not push B out of the L2.
+#ifndef HSPMM_NT_LOAD
+#define HSPMM_NT_LOAD 0
+#endif
+#ifndef HSPMM_NT_STORE
+#define HSPMM_NT_STORE 1
+#endif
+template <class T>
+__device__ __forceinline__ T stream_load(const T *p)
+{
+#if HSPMM_NT_LOAD
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+template <class T>
+__device__ __forceinline__ void stream_store(T *p, const T v)
+{
+#if HSPMM_NT_STORE
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
+}
+
 template <int V>
 __device__ __forceinline__ void store_words(void *p, const uint32_t (&src)[V])
 {
@@ -64,7 +92,7 @@ __device__ __forceinline__ void store_words(void *p, const uint32_t (&src)[V])
 #pragma unroll
         for (int i = 0; i < V; ++i) v[i] = src[i];
     }
-    *reinterpret_cast<typename Vec<V>::type *>(p) = v;
+    stream_store(reinterpret_cast<typename Vec<V>::type *>(p), v);
 }
 
 template <int V>
@@ -170,7 +198,7 @@ struct Fp16Tile {
 
     __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t tile)
     {
-        return *reinterpret_cast<const u32x4 *>(L.idx_src + size_t(tile) * 16u);
+        return stream_load(reinterpret_cast<const u32x4 *>(L.idx_src + size_t(tile) * 16u));
     }
     // The registers of one tile in flight are separate variables of the caller
     // (b0..b3: the lane's words of four B rows, a: its two words of the sparse tile).
@@ -182,7 +210,7 @@ struct Fp16Tile {
         b1 = *reinterpret_cast<const BVec *>(gat.row(idx[1]));
         b2 = *reinterpret_cast<const BVec *>(gat.row(idx[2]));
         b3 = *reinterpret_cast<const BVec *>(gat.row(idx[3]));
-        a = *reinterpret_cast<const u32x2 *>(L.a_src + size_t(tile) * 64u);
+        a = stream_load(reinterpret_cast<const u32x2 *>(L.a_src + size_t(tile) * 64u));
     }
     template <int p> __device__ static __forceinline__ uint32_t word(const BVec &v)
     {
@@ -248,7 +276,7 @@ struct Fp16TileDW {
 
     __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t tile)
     {
-        return *reinterpret_cast<const u32x4 *>(L.idx_src + size_t(tile) * 16u);
+        return stream_load(reinterpret_cast<const u32x4 *>(L.idx_src + size_t(tile) * 16u));
     }
     template <class G>
     __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t tile, const Idx idx, const G &gat,
@@ -262,7 +290,7 @@ struct Fp16TileDW {
             if constexpr (V > 2) b2[q] = src[32];
             if constexpr (V > 3) b3[q] = src[48];
         }
-        a = *reinterpret_cast<const u32x2 *>(L.a_src + size_t(tile) * 64u);
+        a = stream_load(reinterpret_cast<const u32x2 *>(L.a_src + size_t(tile) * 64u));
     }
     __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
                                                const BVec &b3, const u32x2 &a, f32x4 (&acc)[kAcc])
@@ -283,7 +311,7 @@ struct Fp16TileDW {
             if (active && row < rows) {
                 uint32_t *dst = reinterpret_cast<uint32_t *>(c_lane + size_t(row) * row_bytes);
 #pragma unroll
-                for (int p = 0; p < V; ++p) dst[16 * p] = pack_half2_rn(acc[p][2 * rr], acc[p][2 * rr + 1]);
+                for (int p = 0; p < V; ++p) stream_store(dst + 16 * p, pack_half2_rn(acc[p][2 * rr], acc[p][2 * rr + 1]));
             }
         }
     }
@@ -294,7 +322,7 @@ struct Fp16TileDW {
         for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) {
             uint32_t *dst = reinterpret_cast<uint32_t *>(c_lane + size_t(r) * row_bytes);
 #pragma unroll
-            for (int p = 0; p < V; ++p) dst[16 * p] = 0u;
+            for (int p = 0; p < V; ++p) stream_store(dst + 16 * p, 0u);
         }
     }
 };
@@ -328,7 +356,7 @@ struct Fp32Tile {
     __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t tile)
     {
         const uint32_t *p = L.idx_src + size_t(tile) * 8u;
-        Idx r; r[0] = p[0]; r[1] = p[4];
+        Idx r; r[0] = stream_load(p); r[1] = stream_load(p + 4);
         return r;
     }
     template <class G>
@@ -338,7 +366,7 @@ struct Fp32Tile {
         b0 = *reinterpret_cast<const BVec *>(gat.row(idx[0]));
         b1 = *reinterpret_cast<const BVec *>(gat.row(idx[1]));
         const uint32_t *p = L.a_src + size_t(tile) * 64u;
-        a[0] = p[0]; a[1] = p[4];
+        a[0] = stream_load(p); a[1] = stream_load(p + 4);
     }
     template <int p> __device__ static __forceinline__ float word(const BVec &v)
     {

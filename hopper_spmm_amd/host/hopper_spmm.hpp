@@ -1,0 +1,246 @@
+// C++ host interface with the names and argument meaning of the reference's
+// host code, implemented on the C ABI of libhspmm.so (include/hspmm.h):
+//
+//   compile-time element type   -DUSE_FP16 / -DUSE_TF32      reference src/common.h:14-43
+//   CSR_MTX, DENSE_MTX, BTCF_MTX_NO_BITMAP, PERF_RESULT      reference src/utils/class.h:30-48, 74-85; src/common.h:51-59
+//   load_matrix, free_csr_matrix                             reference src/utils/load.h:152-355
+//   CSR2BTCFNOBITMAP                                         reference src/utils/convert.h:146-225
+//   fp16_spmm / tf32_spmm                                    reference src/fp16.cu:221-281
+//   Scheduler                                                reference src/scheduler.h:5-42
+//   verify_dense_matrix                                      reference src/utils/verify.h:18-42
+//
+// Differences from the reference, all deliberate: errors are reported (message on
+// stderr, exit code 1) from this layer only, the library below never exits; the
+// operator copies C back to the host (the reference stops after the timing loop,
+// src/fp16.cu:269); tf32_spmm exists (the reference has no such entry point).
+#pragma once
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cmath>
+#include <vector>
+
+#include <hip/hip_runtime.h>
+#include "../../include/hspmm.h"
+
+#if !defined(USE_FP16) && !defined(USE_TF32)
+#error "define USE_FP16 or USE_TF32 (as the reference's Makefile does)"
+#endif
+
+#define MAT_PTR_TYPE uint32_t
+#define MAT_IDX_TYPE uint32_t
+#define vint uint32_t
+#define ROW_WINDOW 8
+#define IDX_MAX UINT32_MAX
+#define WARMUP_RUNS 3
+#define RUNS 5
+#ifdef USE_FP16
+#define MAT_VAL_TYPE _Float16
+#define COL_WINDOW 16
+#define HSPMM_BUILD_DTYPE HSPMM_FP16
+#else
+#define MAT_VAL_TYPE float
+#define COL_WINDOW 8
+#define HSPMM_BUILD_DTYPE HSPMM_TF32
+#endif
+
+struct PERF_RESULT {
+    float time;      // total milliseconds of `runs` launches
+    int runs;
+    void print() const
+    {
+        std::printf("SpMM total time: %.3f ms\n", time);
+        std::printf("SpMM timed runs: %d\n", runs);
+        std::printf("SpMM mean time: %.3f ms\n", time / static_cast<float>(runs));
+    }
+};
+
+struct CSR_MTX {
+    vint rows, cols, nnzs;
+    MAT_PTR_TYPE *row_ptr;
+    MAT_IDX_TYPE *col_idx;
+    MAT_VAL_TYPE *values;
+};
+
+struct DENSE_MTX {
+    vint rows, cols;
+    MAT_VAL_TYPE *values;      // row-major
+};
+
+struct BTCF_MTX_NO_BITMAP {
+    vint rows, cols, nnzs;
+    vint total_row_windows, eff_row_windows;
+    std::vector<MAT_PTR_TYPE> rowOffset;
+    std::vector<MAT_IDX_TYPE> tcA2B;
+    std::vector<MAT_VAL_TYPE> data;
+    std::vector<MAT_IDX_TYPE> rowIdx;
+    uint32_t total_tiles;
+};
+
+namespace hspmm_cpp {
+[[noreturn]] inline void die(const char *what)
+{
+    std::fprintf(stderr, "%s: %s\n", what, hspmm_last_error());
+    std::exit(EXIT_FAILURE);
+}
+inline void check_hip(hipError_t e, const char *what)
+{
+    if (e != hipSuccess) {
+        std::fprintf(stderr, "%s: %s\n", what, hipGetErrorString(e));
+        std::exit(EXIT_FAILURE);
+    }
+}
+}  // namespace hspmm_cpp
+
+// An unreadable file gives an empty matrix and a message, as in the reference
+// (src/utils/load.h:176-180, 190-194).  enable_validation re-checks the CSR
+// structure (the checks of src/utils/load.h:44-73).
+inline CSR_MTX load_matrix(const char *filename, int enable_validation = 0)
+{
+    CSR_MTX m{0, 0, 0, nullptr, nullptr, nullptr};
+    hspmm_csr c;
+    if (hspmm_mtx_load(filename, HSPMM_BUILD_DTYPE, &c) != HSPMM_OK) {
+        std::printf("error: %s\n", hspmm_last_error());
+        return m;
+    }
+    m.rows = c.rows; m.cols = c.cols; m.nnzs = c.nnzs;
+    m.row_ptr = c.row_ptr; m.col_idx = c.col_idx; m.values = static_cast<MAT_VAL_TYPE *>(c.values);
+    if (enable_validation) {
+        int bad = (m.row_ptr[0] != 0) + (m.row_ptr[m.rows] != m.nnzs);
+        for (vint i = 0; i < m.rows; ++i) bad += m.row_ptr[i] > m.row_ptr[i + 1];
+        for (vint i = 0; i < m.nnzs; ++i) bad += m.col_idx[i] >= m.cols;
+        std::printf(bad ? "CSR validation failed: %d violations\n" : "CSR validation passed\n", bad);
+    }
+    std::printf("loaded matrix: %u x %u, %u stored entries\n", m.rows, m.cols, m.nnzs);
+    return m;
+}
+
+inline void free_csr_matrix(CSR_MTX *m)
+{
+    if (!m) return;
+    hspmm_csr c{m->rows, m->cols, m->nnzs, m->row_ptr, m->col_idx, m->values};
+    hspmm_csr_free(&c);
+    *m = CSR_MTX{0, 0, 0, nullptr, nullptr, nullptr};
+}
+
+inline void CSR2BTCFNOBITMAP(const CSR_MTX &csr, BTCF_MTX_NO_BITMAP &btcf)
+{
+    btcf.rows = csr.rows; btcf.cols = csr.cols; btcf.nnzs = csr.nnzs;
+    btcf.total_row_windows = (csr.rows + ROW_WINDOW - 1) / ROW_WINDOW;
+    uint32_t W = 0, T = 0;
+    static const MAT_PTR_TYPE zero_ptr[1] = {0};
+    const MAT_PTR_TYPE *rp = csr.row_ptr ? csr.row_ptr : zero_ptr;
+    if (hspmm_btcf_sizes(HSPMM_BUILD_DTYPE, csr.rows, rp, csr.col_idx, &W, &T) != HSPMM_OK)
+        hspmm_cpp::die("CSR2BTCFNOBITMAP");
+    btcf.rowOffset.assign(size_t(W) + 1, 0);
+    btcf.tcA2B.assign(size_t(T) * COL_WINDOW, 0);
+    btcf.data.assign(size_t(T) * ROW_WINDOW * COL_WINDOW, MAT_VAL_TYPE(0));
+    btcf.rowIdx.assign(W, 0);
+#ifdef SPARSE_A_TRANSPOSE
+    const int transpose = 1;
+#else
+    const int transpose = 0;
+#endif
+    if (hspmm_btcf_fill(HSPMM_BUILD_DTYPE, csr.rows, rp, csr.col_idx, csr.values, transpose, btcf.rowOffset.data(),
+                        btcf.tcA2B.data(), btcf.data.data(), btcf.rowIdx.data()) != HSPMM_OK)
+        hspmm_cpp::die("CSR2BTCFNOBITMAP");
+    btcf.eff_row_windows = W;
+    btcf.total_tiles = T;
+    std::printf("CSR -> condensed tiles: %u effective row windows, %u tiles of %d x %d\n", W, T, ROW_WINDOW, COL_WINDOW);
+}
+
+// The reference's singleton of launch knobs; here they reach the library.
+class Scheduler {
+    int BUFFER_STAGE = 0, CONSUMER_WARP_NUM = 0, PRODUCER_WARP_GROUP_NUM = 0, SM_NUM = 0;
+    Scheduler() = default;
+    Scheduler(const Scheduler &) = delete;
+    Scheduler &operator=(const Scheduler &) = delete;
+    void push() const
+    {
+        if (hspmm_configure(BUFFER_STAGE, CONSUMER_WARP_NUM, PRODUCER_WARP_GROUP_NUM, SM_NUM) != HSPMM_OK)
+            hspmm_cpp::die("Scheduler");
+    }
+
+public:
+    static Scheduler &getInstance()
+    {
+        static Scheduler instance;
+        return instance;
+    }
+    void setBufferStage(int v) { BUFFER_STAGE = v; push(); }
+    int getBufferStage() const { return BUFFER_STAGE; }
+    void setConsumerWarpNum(int v) { CONSUMER_WARP_NUM = v; push(); }
+    int getConsumerWarpNum() const { return CONSUMER_WARP_NUM; }
+    void configure(int buffer_stage, int consumer_warp_num, int producer_warp_group_num, int sm_num)
+    {
+        BUFFER_STAGE = buffer_stage; CONSUMER_WARP_NUM = consumer_warp_num;
+        PRODUCER_WARP_GROUP_NUM = producer_warp_group_num; SM_NUM = sm_num;
+        push();
+    }
+    int getSMNum() const { return SM_NUM; }
+};
+
+// C = A * B on the GPU: uploads, WARMUP_RUNS untimed and RUNS timed launches
+// (src/common.h:48-49), downloads C into dense_c.values.
+inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX_NO_BITMAP &a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+{
+    PERF_RESULT perf{0.0f, RUNS};
+    if (dense_b.rows != a.cols || dense_c.rows != a.rows || dense_c.cols != dense_b.cols) {
+        std::fprintf(stderr, "spmm: shapes do not match: A %u x %u, B %u x %u, C %u x %u\n", a.rows, a.cols,
+                     dense_b.rows, dense_b.cols, dense_c.rows, dense_c.cols);
+        std::exit(EXIT_FAILURE);
+    }
+    hspmm_plan *plan = nullptr;
+    if (hspmm_create(&plan, HSPMM_BUILD_DTYPE, a.rows, a.cols, a.eff_row_windows, a.total_tiles, a.rowOffset.data(),
+                     a.tcA2B.data(), a.data.data(), a.rowIdx.data()) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_create");
+    const size_t b_bytes = size_t(dense_b.rows) * dense_b.cols * sizeof(MAT_VAL_TYPE);
+    const size_t c_bytes = size_t(dense_c.rows) * dense_c.cols * sizeof(MAT_VAL_TYPE);
+    void *d_b = nullptr, *d_c = nullptr;
+    hspmm_cpp::check_hip(hipMalloc(&d_b, b_bytes ? b_bytes : 4), "hipMalloc B");
+    hspmm_cpp::check_hip(hipMalloc(&d_c, c_bytes ? c_bytes : 4), "hipMalloc C");
+    hspmm_cpp::check_hip(hipMemcpy(d_b, dense_b.values, b_bytes, hipMemcpyHostToDevice), "copy B");
+    if (dense_c.cols && hspmm_bench(plan, d_b, d_c, dense_c.cols, WARMUP_RUNS, RUNS, nullptr, &perf.time) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_bench");
+    hspmm_cpp::check_hip(hipMemcpy(dense_c.values, d_c, c_bytes, hipMemcpyDeviceToHost), "copy C");
+    hspmm_cpp::check_hip(hipFree(d_b), "hipFree");
+    hspmm_cpp::check_hip(hipFree(d_c), "hipFree");
+    hspmm_destroy(plan);
+    return perf;
+}
+
+#ifdef USE_FP16
+inline PERF_RESULT fp16_spmm(BTCF_MTX_NO_BITMAP &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+{
+    return hspmm_cpp_spmm(btcf_a, dense_b, dense_c);
+}
+#else
+inline PERF_RESULT tf32_spmm(BTCF_MTX_NO_BITMAP &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+{
+    return hspmm_cpp_spmm(btcf_a, dense_b, dense_c);
+}
+#endif
+
+// Element-wise comparison of two dense matrices.  The reference's helper counts
+// |a - b| > 1 (src/utils/verify.h:28); here the bound is the relative / absolute
+// form of its tile checks (src/tf32.cu:46-70): relative `tol` when |b| > 1e-6,
+// absolute 1e-5 * scale otherwise.
+inline bool verify_dense_matrix(const DENSE_MTX *A, const DENSE_MTX *B, double tol = 1e-2)
+{
+    const size_t total = size_t(A->rows) * A->cols;
+    size_t failed = 0;
+    int printed = 0;
+    for (size_t i = 0; i < total; ++i) {
+        const double a = double(A->values[i]), b = double(B->values[i]);
+        const double err = std::fabs(a - b), ref = std::fabs(b);
+        const bool bad = ref > 1e-6 ? !(err / ref <= tol) : !(err <= 1e-5);
+        if (bad) {
+            ++failed;
+            if (printed++ < 20)
+                std::printf("mismatch at [%zu][%zu]: %g vs %g\n", i / A->cols, i % A->cols, a, b);
+        }
+    }
+    if (failed) std::printf("verification: %zu of %zu elements differ (%.2f%%)\n", failed, total, 100.0 * failed / total);
+    return failed == 0;
+}

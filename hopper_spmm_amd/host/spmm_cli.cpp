@@ -1,0 +1,68 @@
+// Command-line driver with the reference's arguments (reference src/fp16.cu:283-319):
+//   fp16_test <matrix_file> <feature_dim> [--seed S] [--verify]
+// built with -DUSE_FP16; the same source with -DUSE_TF32 gives tf32_test.
+// B is filled with rand() / RAND_MAX as in the reference (src/fp16.cu:303-309);
+// --seed calls srand first (the reference never seeds, i.e. seed 1).  --verify
+// repeats the product with the library's scalar all-shapes kernel, a second
+// implementation on the GPU, and compares the two results element by element.
+#include <cstring>
+#include <string>
+
+#include "hopper_spmm.hpp"
+
+int main(int argc, char *argv[])
+{
+    if (argc < 3) {
+        std::printf("Usage: %s <matrix_file> <feature_dim> [--seed S] [--verify]\n", argv[0]);
+        return 1;
+    }
+    const char *matrix_file = argv[1];
+    const int fd = std::atoi(argv[2]);
+    bool verify = false;
+    for (int i = 3; i < argc; ++i) {
+        if (!std::strcmp(argv[i], "--verify")) verify = true;
+        else if (!std::strcmp(argv[i], "--seed") && i + 1 < argc) std::srand(unsigned(std::atol(argv[++i])));
+        else { std::printf("unknown argument %s\n", argv[i]); return 1; }
+    }
+    if (fd <= 0) { std::printf("feature_dim must be positive\n"); return 1; }
+    const vint feature_dim = vint(fd);
+
+    CSR_MTX csr = load_matrix(matrix_file, 0);
+    if (!csr.row_ptr) return 1;                       // the reference carries on with an empty matrix
+    BTCF_MTX_NO_BITMAP btcf;
+    CSR2BTCFNOBITMAP(csr, btcf);
+    std::printf("=== condensed tile matrix ===\n");
+    std::printf("rows: %u\ncols: %u\nstored entries: %u\n", btcf.rows, btcf.cols, btcf.nnzs);
+    std::printf("row windows: %u\nnon-empty row windows: %u\n", btcf.total_row_windows, btcf.eff_row_windows);
+    std::printf("tiles (%d x %d): %zu\n", ROW_WINDOW, COL_WINDOW, btcf.tcA2B.size() / COL_WINDOW);
+
+    DENSE_MTX dense_b{btcf.cols, feature_dim, new MAT_VAL_TYPE[size_t(btcf.cols) * feature_dim]};
+    for (size_t i = 0; i < size_t(dense_b.rows) * dense_b.cols; ++i)
+        dense_b.values[i] = MAT_VAL_TYPE(static_cast<float>(std::rand()) / static_cast<float>(RAND_MAX));
+    DENSE_MTX dense_c{btcf.rows, feature_dim, new MAT_VAL_TYPE[size_t(btcf.rows) * feature_dim]};
+
+#ifdef USE_FP16
+    PERF_RESULT perf = fp16_spmm(btcf, dense_b, dense_c);
+#else
+    PERF_RESULT perf = tf32_spmm(btcf, dense_b, dense_c);
+#endif
+    perf.print();
+    const double t = perf.time / perf.runs * 1e-3;
+    if (t > 0) std::printf("effective rate: %.3f TFLOP/s (2 * nnz * N / t)\n", 2.0 * btcf.nnzs * feature_dim / t / 1e12);
+
+    int rc = 0;
+    if (verify) {
+        DENSE_MTX second{btcf.rows, feature_dim, new MAT_VAL_TYPE[size_t(btcf.rows) * feature_dim]};
+        if (hspmm_set_kernel_mode(1) != HSPMM_OK) hspmm_cpp::die("hspmm_set_kernel_mode");
+        hspmm_cpp_spmm(btcf, dense_b, second);
+        hspmm_set_kernel_mode(0);
+        const bool ok = verify_dense_matrix(&dense_c, &second);
+        std::printf(ok ? "verification passed\n" : "verification FAILED\n");
+        rc = ok ? 0 : 2;
+        delete[] second.values;
+    }
+    delete[] dense_b.values;
+    delete[] dense_c.values;
+    free_csr_matrix(&csr);
+    return rc;
+}
