@@ -106,13 +106,18 @@ def main():
 
     hs.set_kernel_mode(args.mode)
     hs.configure(args.stages, args.waves_per_group, args.ranges_per_simd, 0)
-    plan = hs.Plan(b)
+    torch.zeros(1, device="cuda")                    # runtime initialised before anything is timed
+    torch.cuda.synchronize()
+    t_h2d = time.perf_counter()
+    plan = hs.Plan(b)                                # validation, partition, upload of the four format arrays
     if dt == hs.FP16:
         dB = torch.from_numpy(B.view(np.int16)).cuda()
         dC = torch.empty((A["rows"], N), dtype=torch.int16, device="cuda")
     else:
         dB = torch.from_numpy(B).cuda()
         dC = torch.empty((A["rows"], N), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    t_h2d = time.perf_counter() - t_h2d
     stream = torch.cuda.current_stream().cuda_stream
     pB, pC = dB.data_ptr(), dC.data_ptr()
 
@@ -125,6 +130,10 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
+
+    t_d2h = time.perf_counter()
+    dC.cpu()
+    t_d2h = time.perf_counter() - t_d2h
 
     # kernel durations with device events on the launch stream
     main_ms, fix_ms = plan.profile(pB, pC, N, runs=args.steps, stream=stream)
@@ -173,6 +182,9 @@ def main():
                      "algorithmic_bytes": bytes_alg, "gather_bytes": bytes_gather,
                      "mfma_frac_of_peak_useful_flops": flops / (main_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[dt]},
         "reference_convention_ms": ref_conv_ms,
+        # one call of the host-buffer interface (fp16_spmm): plan + upload, one launch, download of C
+        "host_buffer_call": {"upload_and_plan_ms": t_h2d * 1e3, "download_ms": t_d2h * 1e3,
+                             "tflops_including_transfers": flops / (t_h2d + t_d2h + ms_per_step * 1e-3) / 1e12},
         "setup_seconds": t_gen,
     }
     if not args.no_cpu_baseline:
