@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstdarg>
 #include <cstring>
 #include <string>
@@ -140,7 +141,10 @@ int choose_ranges(const hspmm_plan *p)
 int build_and_upload_partition(hspmm_plan *p, const uint32_t *rowOffset)
 {
     if (p->W == 0) return HSPMM_OK;
-    p->part = hspmm::build_partition(p->W, rowOffset, uint32_t(choose_ranges(p)));
+    double window_cost = 1.5, slack = 0.35;
+    if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);   // tuning overrides
+    if (const char *e = std::getenv("HSPMM_SLACK")) slack = std::atof(e);
+    p->part = hspmm::build_partition(p->W, rowOffset, uint32_t(choose_ranges(p)), window_cost, slack);
     const auto &part = p->part;
     std::vector<uint32_t> rw(part.ranges.size() * hspmm::kRangeWords, 0u);
     for (size_t i = 0; i < part.ranges.size(); ++i) {
@@ -176,6 +180,7 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
     if (mode == 1) { c.scalar = true; return c; }
     if (p->dtype == HSPMM_FP16) {
         if (N % 2 != 0 || (align & 3u)) { c.scalar = true; return c; }
+        // word loads measured equal to or faster than wide loads wherever both apply
         const bool dw_ok = (N % 64 == 0);
         if (mode != 2 && (dw_ok || mode == 3) && N % 32 == 0) {
             c.layout = hspmm::kLayoutDW;

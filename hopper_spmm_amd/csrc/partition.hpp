@@ -43,7 +43,7 @@ struct Partition {
 // slack: a cut closer than slack * (mean tiles per range) to a window boundary
 // moves onto the boundary.
 inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t target_ranges,
-                                 double window_cost = 0.5, double slack = 0.35)
+                                 double window_cost = 1.5, double slack = 0.35)
 {
     Partition P;
     if (W == 0) return P;
