@@ -59,7 +59,8 @@ class PlanInfo(C.Structure):
     _fields_ = [("rows", C.c_uint32), ("cols", C.c_uint32), ("eff_row_windows", C.c_uint32),
                 ("total_tiles", C.c_uint32), ("dtype", C.c_int32), ("n_ranges", C.c_uint32),
                 ("n_split_windows", C.c_uint32), ("n_partial_slots", C.c_uint32),
-                ("compute_units", C.c_uint32), ("device_bytes", C.c_uint64)]
+                ("compute_units", C.c_uint32), ("n_units", C.c_uint32), ("n_paired_units", C.c_uint32),
+                ("device_bytes", C.c_uint64)]
 
 
 def load_library():
@@ -91,6 +92,7 @@ def load_library():
     L.hspmm_get_config.argtypes = [C.POINTER(i)] * 4
     L.hspmm_get_config.restype = None
     L.hspmm_set_kernel_mode.argtypes = [i]
+    L.hspmm_set_window_pairing.argtypes = [i]
     L.hspmm_get_plan_info.argtypes = [vp, C.POINTER(PlanInfo)]
     L.hspmm_get_partition.argtypes = [vp, vp, u32]
     L.hspmm_partition_preview.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
@@ -133,6 +135,11 @@ def get_config():
 
 def set_kernel_mode(mode):
     _check(load_library().hspmm_set_kernel_mode(mode))
+
+
+def set_window_pairing(mode):
+    """0 = automatic, 1 = never, 2 = whenever two adjacent windows share a column list."""
+    _check(load_library().hspmm_set_window_pairing(mode))
 
 
 def mtx_load(path, dtype):

@@ -49,6 +49,7 @@ struct Config {
     int producer_warp_group_num = 0;
     int sm_num = 0;
     int kernel_mode = 0;
+    int pairing = 0;                    // 0 automatic, 1 never, 2 whenever two windows share a column list
 };
 std::mutex g_cfg_mutex;
 Config g_cfg;
@@ -68,11 +69,16 @@ struct hspmm_plan {
     uint32_t cw = 16, elem = 2;
     int compute_units = 0;
     Config cfg;
-    // device copies of the format arrays
+    // device copies of the format arrays as given: scalar kernel
     uint32_t *d_rowOffset = nullptr, *d_rowIdx = nullptr;
-    uint32_t *d_a2b_raw = nullptr;      // as given (padding = IDX_MAX): scalar kernel
-    uint32_t *d_a2b = nullptr;          // padding renamed to the id in front of it: MFMA kernels
+    uint32_t *d_a2b_raw = nullptr;
     void *d_data = nullptr;
+    // the step stream of the MFMA kernels
+    int G = 1;                          // windows per unit: 2 when windows were paired
+    uint32_t n_units = 0, n_paired = 0, n_steps = 0;
+    uint32_t *d_unitOffset = nullptr, *d_unitRow = nullptr;
+    uint32_t *d_ids = nullptr;          // per step, lane order, padding renamed to the id in front of it
+    void *d_tiles = nullptr;            // per step, lane order (== d_data for fp16 without pairs)
     // partition
     hspmm::Partition part;
     uint32_t *d_ranges = nullptr, *d_split = nullptr, *d_fix_slots = nullptr;
@@ -132,19 +138,19 @@ int choose_ranges(const hspmm_plan *p)
 {
     const int waves_per_simd = p->cfg.producer_warp_group_num > 0 ? p->cfg.producer_warp_group_num : 4;
     uint64_t g = uint64_t(p->compute_units) * 4u * uint64_t(waves_per_simd);
-    const uint64_t cap = (uint64_t(p->T) + kMinTilesPerRange - 1) / kMinTilesPerRange;
+    const uint64_t cap = (uint64_t(p->n_steps) + kMinTilesPerRange - 1) / kMinTilesPerRange;
     if (g > cap) g = cap;
     if (g < 1) g = 1;
     return int(g);
 }
 
-int build_and_upload_partition(hspmm_plan *p, const uint32_t *rowOffset)
+int build_and_upload_partition(hspmm_plan *p, const uint32_t *unitOffset)
 {
     if (p->W == 0) return HSPMM_OK;
     double window_cost = 1.5, slack = 0.35;
     if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);   // tuning overrides
     if (const char *e = std::getenv("HSPMM_SLACK")) slack = std::atof(e);
-    p->part = hspmm::build_partition(p->W, rowOffset, uint32_t(choose_ranges(p)), window_cost, slack);
+    p->part = hspmm::build_partition(p->n_units, unitOffset, uint32_t(choose_ranges(p)), window_cost, slack);
     const auto &part = p->part;
     std::vector<uint32_t> rw(part.ranges.size() * hspmm::kRangeWords, 0u);
     for (size_t i = 0; i < part.ranges.size(); ++i) {
@@ -162,6 +168,97 @@ int build_and_upload_partition(hspmm_plan *p, const uint32_t *rowOffset)
     if ((rc = upload(&p->d_split, sw.data(), sw.size(), &p->fixed_bytes))) return rc;
     if ((rc = upload(&p->d_fix_slots, part.fix_slots.data(), part.fix_slots.size(), &p->fixed_bytes))) return rc;
     return HSPMM_OK;
+}
+
+// The step stream: units (single windows, or pairs of vertically adjacent windows
+// with one column list) and, per step, the ids and tiles in the order the lanes
+// of the MFMA kernels read them.
+struct StepStream {
+    int G = 1;
+    std::vector<uint32_t> unitOffset, unitRow, unitWindow;   // unitWindow: first effective window of the unit
+    uint32_t n_paired = 0, n_steps = 0;
+};
+
+StepStream build_units(uint32_t W, uint32_t cw, const uint32_t *rowOffset, const uint32_t *rowIdx,
+                       const std::vector<uint32_t> &ids_clean, int pairing)
+{
+    StepStream st;
+    // which windows could pair with their successor
+    std::vector<uint8_t> can(W, 0);
+    uint64_t paired_tiles = 0;
+    if (pairing != 1) {
+        for (uint32_t w = 0; w + 1 < W; ++w) {
+            const uint32_t n = rowOffset[w + 1] - rowOffset[w];
+            if (rowIdx[w + 1] != rowIdx[w] + HSPMM_ROW_WINDOW || rowOffset[w + 2] - rowOffset[w + 1] != n) continue;
+            const uint32_t *a = ids_clean.data() + size_t(rowOffset[w]) * cw;
+            const uint32_t *b = ids_clean.data() + size_t(rowOffset[w + 1]) * cw;
+            if (std::memcmp(a, b, size_t(n) * cw * 4) == 0) can[w] = 1;
+        }
+        for (uint32_t w = 0; w + 1 < W;) {
+            if (can[w]) { paired_tiles += 2ull * (rowOffset[w + 1] - rowOffset[w]); w += 2; } else ++w;
+        }
+    }
+    // pairs pay off when a fair share of the tiles is in them: an unpaired window in a
+    // paired stream costs a zero tile and an idle MFMA
+    const bool use_pairs = pairing == 2 ? paired_tiles > 0 : (pairing == 0 && paired_tiles * 4ull >= uint64_t(rowOffset[W]));
+    st.G = use_pairs ? 2 : 1;
+    st.unitOffset.push_back(0);
+    for (uint32_t w = 0; w < W;) {
+        const uint32_t n = rowOffset[w + 1] - rowOffset[w];
+        const bool pair = use_pairs && w + 1 < W && can[w];
+        st.unitWindow.push_back(w);
+        st.unitRow.push_back(rowIdx[w] | (pair ? 1u : 0u));
+        st.unitOffset.push_back(st.unitOffset.back() + n);
+        st.n_paired += pair;
+        w += pair ? 2 : 1;
+    }
+    st.n_steps = st.unitOffset.back();
+    return st;
+}
+
+// ids per step in lane order.  fp16: the 16 ids of the step's tile.  fp32: [g][2] = (id g, id g + 4).
+std::vector<uint32_t> lane_order_ids(const StepStream &st, int dtype, const uint32_t *rowOffset,
+                                     const std::vector<uint32_t> &ids_clean)
+{
+    const uint32_t cw = dtype == HSPMM_FP16 ? 16u : 8u;
+    std::vector<uint32_t> out(size_t(st.n_steps) * cw);
+    for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
+        const uint32_t t0 = rowOffset[st.unitWindow[u]];
+        for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
+            const uint32_t *src = ids_clean.data() + size_t(t0 + i) * cw;
+            uint32_t *dst = out.data() + size_t(st.unitOffset[u] + i) * cw;
+            if (dtype == HSPMM_FP16) std::memcpy(dst, src, 64);
+            else for (uint32_t g = 0; g < 4; ++g) { dst[2 * g] = src[g]; dst[2 * g + 1] = src[g + 4]; }
+        }
+    }
+    return out;
+}
+
+// tiles per step in lane order, as 32-bit words.
+//   fp16: [row r][g][window][2 words = halves 4g..4g+3 of row r]
+//   fp32: [row r][g][window][2 words = a[r][g], a[r][g+4]]
+std::vector<uint32_t> lane_order_tiles(const StepStream &st, int dtype, const uint32_t *rowOffset, const void *data)
+{
+    const int G = st.G;
+    const uint32_t *words = static_cast<const uint32_t *>(data);     // a tile is 64 words in both formats
+    std::vector<uint32_t> out(size_t(st.n_steps) * 64u * G, 0u);
+    for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
+        const uint32_t w0 = st.unitWindow[u];
+        const int nwin = (st.unitRow[u] & 1u) ? 2 : 1;
+        for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
+            uint32_t *dst = out.data() + size_t(st.unitOffset[u] + i) * 64u * G;
+            for (int w = 0; w < nwin; ++w) {
+                const uint32_t *src = words + size_t(rowOffset[w0 + w] + i) * 64u;
+                for (uint32_t r = 0; r < 8; ++r)
+                    for (uint32_t g = 0; g < 4; ++g) {
+                        uint32_t *d = dst + ((r * 4 + g) * G + w) * 2;
+                        if (dtype == HSPMM_FP16) { d[0] = src[r * 8 + 2 * g]; d[1] = src[r * 8 + 2 * g + 1]; }
+                        else { d[0] = src[r * 8 + g]; d[1] = src[r * 8 + g + 4]; }
+                    }
+            }
+        }
+    }
+    return out;
 }
 
 struct Choice {
@@ -255,6 +352,14 @@ int hspmm_set_kernel_mode(int mode)
     return HSPMM_OK;
 }
 
+int hspmm_set_window_pairing(int mode)
+{
+    if (mode < 0 || mode > 2) return fail(HSPMM_ERR_INVALID, "pairing mode %d outside 0..2", mode);
+    std::lock_guard<std::mutex> lk(g_cfg_mutex);
+    g_cfg.pairing = mode;
+    return HSPMM_OK;
+}
+
 int hspmm_partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
                             uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges,
                             uint32_t *n_split_windows, uint32_t *n_partial_slots)
@@ -313,20 +418,36 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         if ((rc = upload(&p->d_rowIdx, rowIdx, size_t(p->W), &p->fixed_bytes))) return bail(rc);
         if ((rc = upload(&p->d_a2b_raw, tcA2B, n_ids, &p->fixed_bytes))) return bail(rc);
         {
-            // padding ids -> the real id in front of them (the tile column is all zero)
-            std::vector<uint32_t> clean(tcA2B, tcA2B + n_ids);
-            for (size_t i = 1; i < n_ids; ++i)
-                if (clean[i] == HSPMM_IDX_MAX) clean[i] = clean[i - 1];
-            if ((rc = upload(&p->d_a2b, clean.data(), n_ids, &p->fixed_bytes))) return bail(rc);
-        }
-        {
             uint8_t *dd = nullptr;
             if ((rc = upload(&dd, static_cast<const uint8_t *>(data), size_t(total_tiles) * 8u * cw * elem,
                              &p->fixed_bytes)))
                 return bail(rc);
             p->d_data = dd;
         }
-        if ((rc = build_and_upload_partition(p, rowOffset))) return bail(rc);
+        // padding ids -> the real id in front of them (the tile column is all zero)
+        std::vector<uint32_t> clean(tcA2B, tcA2B + n_ids);
+        for (size_t i = 1; i < n_ids; ++i)
+            if (clean[i] == HSPMM_IDX_MAX) clean[i] = clean[i - 1];
+        const StepStream st = build_units(p->W, cw, rowOffset, rowIdx, clean, p->cfg.pairing);
+        p->G = st.G;
+        p->n_units = uint32_t(st.unitRow.size());
+        p->n_paired = st.n_paired;
+        p->n_steps = st.n_steps;
+        if ((rc = upload(&p->d_unitOffset, st.unitOffset.data(), st.unitOffset.size(), &p->fixed_bytes))) return bail(rc);
+        if ((rc = upload(&p->d_unitRow, st.unitRow.data(), st.unitRow.size(), &p->fixed_bytes))) return bail(rc);
+        {
+            const std::vector<uint32_t> ids = lane_order_ids(st, dtype, rowOffset, clean);
+            if ((rc = upload(&p->d_ids, ids.data(), ids.size(), &p->fixed_bytes))) return bail(rc);
+        }
+        if (dtype == HSPMM_FP16 && st.G == 1) {
+            p->d_tiles = p->d_data;                 // the caller's tile layout already is the lane order
+        } else {
+            const std::vector<uint32_t> tiles = lane_order_tiles(st, dtype, rowOffset, data);
+            uint32_t *dt = nullptr;
+            if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) return bail(rc);
+            p->d_tiles = dt;
+        }
+        if ((rc = build_and_upload_partition(p, st.unitOffset.data()))) return bail(rc);
     }
     *out = p;
     return HSPMM_OK;
@@ -335,8 +456,9 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
 void hspmm_destroy(hspmm_plan *p)
 {
     if (!p) return;
-    (void)hipFree(p->d_rowOffset); (void)hipFree(p->d_rowIdx); (void)hipFree(p->d_a2b_raw); (void)hipFree(p->d_a2b);
-    (void)hipFree(p->d_data); (void)hipFree(p->d_ranges); (void)hipFree(p->d_split); (void)hipFree(p->d_fix_slots);
+    (void)hipFree(p->d_rowOffset); (void)hipFree(p->d_rowIdx); (void)hipFree(p->d_a2b_raw);
+    if (p->d_tiles != p->d_data) (void)hipFree(p->d_tiles);
+    (void)hipFree(p->d_data); (void)hipFree(p->d_unitOffset); (void)hipFree(p->d_unitRow); (void)hipFree(p->d_ids); (void)hipFree(p->d_ranges); (void)hipFree(p->d_split); (void)hipFree(p->d_fix_slots);
     (void)hipFree(p->d_scratch);
     delete p;
 }
@@ -366,28 +488,31 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     }
     const Choice c = choose_kernel(p, dB, dC, N);
     hspmm::KernelArgs ka{};
-    ka.rowOffset = p->d_rowOffset; ka.data = p->d_data; ka.rowIdx = p->d_rowIdx;
+    ka.rowOffset = p->d_rowOffset; ka.data = p->d_data; ka.rowIdx = p->d_rowIdx; ka.tcA2B = p->d_a2b_raw;
     ka.B = dB; ka.C = dC;
     ka.eff_windows = p->W; ka.rows = p->rows; ka.N = N;
     if (c.scalar) {
-        ka.tcA2B = p->d_a2b_raw;
         HSPMM_HIP(hspmm::launch_spmm_scalar(p->dtype, ka, s));
         return HSPMM_OK;
     }
-    ka.tcA2B = p->d_a2b;
+    ka.unitOffset = p->d_unitOffset; ka.unitRow = p->d_unitRow; ka.ids = p->d_ids; ka.tiles = p->d_tiles;
+    ka.n_units = p->n_units;
     ka.ranges = p->d_ranges; ka.split = p->d_split; ka.fix_slots = p->d_fix_slots;
     ka.n_ranges = uint32_t(p->part.ranges.size());
     ka.n_split = uint32_t(p->part.split.size());
     ka.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
     if (uint64_t(ka.n_ranges) * ka.n_feat_blocks > 0x7FFFFFFFull)
         return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many work items", N);
-    const size_t need = size_t(p->part.n_slots) * ka.n_feat_blocks * size_t(c.V) * 64u * 16u;
+    const size_t need = size_t(p->part.n_slots) * ka.n_feat_blocks * size_t(c.V) * size_t(p->G) * 64u * 16u;
     int rc = ensure_scratch(p, need);
     if (rc) return rc;
     ka.scratch = p->d_scratch;
-    const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage : (p->dtype == HSPMM_FP16 ? 3 : 4);
+    // default depth: what fits 128 registers per lane without spilling
+    const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage
+                         : p->dtype != HSPMM_FP16 ? (p->G == 2 && c.V == 4 ? 3 : 4)
+                         : (p->G == 2 && c.V == 4 ? 2 : 3);
     const int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
-    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, c.layout, ka, c.V, prefetch, c.narrow, wpg, s, mid));
+    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, c.layout, p->G, ka, c.V, prefetch, c.narrow, wpg, s, mid));
     return HSPMM_OK;
 }
 
@@ -457,6 +582,8 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_split_windows = uint32_t(p->part.split.size());
     info->n_partial_slots = p->part.n_slots;
     info->compute_units = uint32_t(p->compute_units);
+    info->n_units = p->n_units;
+    info->n_paired_units = p->n_paired;
     info->device_bytes = uint64_t(p->fixed_bytes) + uint64_t(p->scratch_bytes);
     return HSPMM_OK;
 }

@@ -15,19 +15,25 @@ constexpr uint32_t kFixWords = 4u;
 constexpr int kMaxWavesPerGroup = 4;
 
 struct KernelArgs {
-    // the four format arrays (device copies), reference src/fp16.cu:38-41
+    // the four format arrays exactly as given (device copies), reference
+    // src/fp16.cu:38-41: read by the scalar kernel
     const uint32_t *rowOffset;
-    const uint32_t *tcA2B;       // MFMA kernels: padding ids renamed; scalar kernel: as given
+    const uint32_t *tcA2B;
     const void     *data;
     const uint32_t *rowIdx;
+    // the step stream the MFMA kernels walk
+    const uint32_t *unitOffset;  // n_units + 1: first step of every unit
+    const uint32_t *unitRow;     // n_units: first matrix row of the unit | 1 if it is a pair of windows
+    const uint32_t *ids;         // per step, lane order, padding ids renamed
+    const void     *tiles;       // per step, lane order
     // partition
     const uint32_t *ranges;      // n_ranges x kRangeWords
-    const uint32_t *split;       // n_split x kFixWords {window, slot_begin, slot_count, 0}
+    const uint32_t *split;       // n_split x kFixWords {unit, slot_begin, slot_count, 0}
     const uint32_t *fix_slots;
     float          *scratch;     // partial sums: [slot][feature block][acc reg][lane] x 4 floats
     const void     *B;           // cols x N
     void           *C;           // rows x N
-    uint32_t n_ranges, n_split, eff_windows, rows, N, n_feat_blocks;
+    uint32_t n_ranges, n_split, eff_windows, n_units, rows, N, n_feat_blocks;
 };
 
 // dtype: 0 = fp16 tiles 8x16, 1 = fp32 tiles 8x8.  V = 32-bit words a lane loads
@@ -37,7 +43,8 @@ struct KernelArgs {
 constexpr int kLayoutX4 = 0, kLayoutDW = 1;
 // narrow: B < 4 GiB and cols < 2^24 (32-bit gather offsets).
 // mid: optional event recorded between the main kernel and the partial-sum kernel.
-hipError_t launch_spmm_mfma(int dtype, int layout, const KernelArgs &ka, int V, int prefetch, bool narrow,
+// G: windows per unit in the step stream (1, or 2 when the plan paired windows).
+hipError_t launch_spmm_mfma(int dtype, int layout, int G, const KernelArgs &ka, int V, int prefetch, bool narrow,
                             int waves_per_group, hipStream_t s, hipEvent_t mid);
 hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s);
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);

@@ -103,6 +103,12 @@ void hspmm_get_config(int *buffer_stage, int *consumer_warp_num,
  * word loads whenever N is a multiple of 32. */
 int hspmm_set_kernel_mode(int mode);
 
+/* No reference counterpart.  Two vertically adjacent windows with the same
+ * column list (block-clustered weights) can share one gather of B.  Read by the
+ * next hspmm_create: 0 = pair when at least a quarter of the tiles would be in
+ * pairs, 1 = never, 2 = whenever any two windows qualify. */
+int hspmm_set_window_pairing(int mode);
+
 typedef struct {
     uint32_t rows, cols, eff_row_windows, total_tiles;
     int32_t  dtype;
@@ -110,6 +116,8 @@ typedef struct {
     uint32_t n_split_windows;   /* windows whose tiles span more than one range */
     uint32_t n_partial_slots;   /* fp32 partial accumulators the split windows use */
     uint32_t compute_units;
+    uint32_t n_units;           /* units of the step stream: single windows and pairs */
+    uint32_t n_paired_units;    /* units made of two adjacent windows with one column list */
     uint64_t device_bytes;      /* bytes of device memory the plan holds right now */
 } hspmm_plan_info;
 
