@@ -49,6 +49,7 @@ struct Config {
     int producer_warp_group_num = 0;
     int sm_num = 0;
     int kernel_mode = 0;
+    int fused_fixup = 0;                // 1: the last wave of a cut unit adds its partial sums; 0: second kernel
     int pairing = 0;                    // 0 automatic, 1 never, 2 whenever two windows share a column list
 };
 std::mutex g_cfg_mutex;
@@ -80,10 +81,20 @@ struct hspmm_plan {
     uint32_t *d_ids = nullptr;          // per step, lane order, padding renamed to the id in front of it
     void *d_tiles = nullptr;            // per step, lane order (== d_data for fp16 without pairs)
     // partition
-    hspmm::Partition part;
-    uint32_t *d_ranges = nullptr, *d_split = nullptr, *d_fix_slots = nullptr;
+    // partitions of the step stream: [0] for one feature block per wave range (built by
+    // hspmm_create), [1] / [2] with a half / a quarter of the ranges for feature dimensions
+    // that need 2-3 / 4 or more blocks, built on first use (more blocks = more waves per range)
+    struct DevPartition {
+        bool built = false;
+        hspmm::Partition part;
+        uint32_t *d_ranges = nullptr, *d_split = nullptr, *d_fix_slots = nullptr;
+    };
+    DevPartition parts[3];
+    std::vector<uint32_t> h_unitOffset;
     float *d_scratch = nullptr;
     size_t scratch_bytes = 0;
+    uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
+    size_t arrive_words = 0;
     size_t fixed_bytes = 0;
 };
 
@@ -144,19 +155,24 @@ int choose_ranges(const hspmm_plan *p)
     return int(g);
 }
 
-int build_and_upload_partition(hspmm_plan *p, const uint32_t *unitOffset)
+int build_and_upload_partition(hspmm_plan *p, int level)
 {
-    if (p->W == 0) return HSPMM_OK;
+    hspmm_plan::DevPartition &dp = p->parts[level];
+    if (dp.built || p->W == 0) return HSPMM_OK;
     double window_cost = 1.5, slack = 0.35;
     if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);   // tuning overrides
     if (const char *e = std::getenv("HSPMM_SLACK")) slack = std::atof(e);
-    p->part = hspmm::build_partition(p->n_units, unitOffset, uint32_t(choose_ranges(p)), window_cost, slack);
-    const auto &part = p->part;
+    uint32_t target = uint32_t(choose_ranges(p)) >> level;
+    const uint32_t floor_ranges = uint32_t(p->compute_units) * 4u;       // at least one range per SIMD
+    if (target < floor_ranges) target = std::min<uint32_t>(floor_ranges, uint32_t(choose_ranges(p)));
+    dp.part = hspmm::build_partition(p->n_units, p->h_unitOffset.data(), target, window_cost, slack);
+    const auto &part = dp.part;
     std::vector<uint32_t> rw(part.ranges.size() * hspmm::kRangeWords, 0u);
     for (size_t i = 0; i < part.ranges.size(); ++i) {
         uint32_t *d = rw.data() + i * hspmm::kRangeWords;
         d[0] = part.ranges[i].tile_begin; d[1] = part.ranges[i].tile_end; d[2] = part.ranges[i].first_window;
         d[3] = part.ranges[i].head_slot; d[4] = part.ranges[i].tail_slot;
+        d[5] = part.ranges[i].head_split; d[6] = part.ranges[i].tail_split;
     }
     std::vector<uint32_t> sw(part.split.size() * hspmm::kFixWords, 0u);
     for (size_t i = 0; i < part.split.size(); ++i) {
@@ -164,9 +180,10 @@ int build_and_upload_partition(hspmm_plan *p, const uint32_t *unitOffset)
         d[0] = part.split[i].window; d[1] = part.split[i].slot_begin; d[2] = part.split[i].slot_count;
     }
     int rc;
-    if ((rc = upload(&p->d_ranges, rw.data(), rw.size(), &p->fixed_bytes))) return rc;
-    if ((rc = upload(&p->d_split, sw.data(), sw.size(), &p->fixed_bytes))) return rc;
-    if ((rc = upload(&p->d_fix_slots, part.fix_slots.data(), part.fix_slots.size(), &p->fixed_bytes))) return rc;
+    if ((rc = upload(&dp.d_ranges, rw.data(), rw.size(), &p->fixed_bytes))) return rc;
+    if ((rc = upload(&dp.d_split, sw.data(), sw.size(), &p->fixed_bytes))) return rc;
+    if ((rc = upload(&dp.d_fix_slots, part.fix_slots.data(), part.fix_slots.size(), &p->fixed_bytes))) return rc;
+    dp.built = true;
     return HSPMM_OK;
 }
 
@@ -301,6 +318,16 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
     return c;
 }
 
+int ensure_arrive(hspmm_plan *p, size_t words)
+{
+    if (words <= p->arrive_words) return HSPMM_OK;
+    if (p->d_arrive) { HSPMM_HIP(hipFree(p->d_arrive)); p->d_arrive = nullptr; p->arrive_words = 0; }
+    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->d_arrive), words * 4));
+    HSPMM_HIP(hipMemset(p->d_arrive, 0, words * 4));
+    p->arrive_words = words;
+    return HSPMM_OK;
+}
+
 int ensure_scratch(hspmm_plan *p, size_t bytes)
 {
     if (bytes <= p->scratch_bytes) return HSPMM_OK;
@@ -400,6 +427,7 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
     p->dtype = dtype; p->rows = rows; p->cols = cols; p->W = eff_row_windows; p->T = total_tiles;
     p->cw = cw; p->elem = elem;
     { std::lock_guard<std::mutex> lk(g_cfg_mutex); p->cfg = g_cfg; }
+    if (const char *e = std::getenv("HSPMM_FUSED_FIXUP")) p->cfg.fused_fixup = std::atoi(e);     // tuning override
 
     auto bail = [&](int code) { hspmm_destroy(p); return code; };
     hipError_t e = hipGetDevice(&p->device);
@@ -447,7 +475,8 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
             if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) return bail(rc);
             p->d_tiles = dt;
         }
-        if ((rc = build_and_upload_partition(p, st.unitOffset.data()))) return bail(rc);
+        p->h_unitOffset = st.unitOffset;
+        if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
     }
     *out = p;
     return HSPMM_OK;
@@ -458,8 +487,9 @@ void hspmm_destroy(hspmm_plan *p)
     if (!p) return;
     (void)hipFree(p->d_rowOffset); (void)hipFree(p->d_rowIdx); (void)hipFree(p->d_a2b_raw);
     if (p->d_tiles != p->d_data) (void)hipFree(p->d_tiles);
-    (void)hipFree(p->d_data); (void)hipFree(p->d_unitOffset); (void)hipFree(p->d_unitRow); (void)hipFree(p->d_ids); (void)hipFree(p->d_ranges); (void)hipFree(p->d_split); (void)hipFree(p->d_fix_slots);
-    (void)hipFree(p->d_scratch);
+    (void)hipFree(p->d_data); (void)hipFree(p->d_unitOffset); (void)hipFree(p->d_unitRow); (void)hipFree(p->d_ids);
+    for (auto &dp : p->parts) { (void)hipFree(dp.d_ranges); (void)hipFree(dp.d_split); (void)hipFree(dp.d_fix_slots); }
+    (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive);
     delete p;
 }
 
@@ -497,16 +527,31 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     }
     ka.unitOffset = p->d_unitOffset; ka.unitRow = p->d_unitRow; ka.ids = p->d_ids; ka.tiles = p->d_tiles;
     ka.n_units = p->n_units;
-    ka.ranges = p->d_ranges; ka.split = p->d_split; ka.fix_slots = p->d_fix_slots;
-    ka.n_ranges = uint32_t(p->part.ranges.size());
-    ka.n_split = uint32_t(p->part.split.size());
     ka.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
+    // Several feature blocks give several waves per range; fewer, longer ranges then keep
+    // the number of waves, and pay off where units are long enough to be cut into many
+    // pieces (each piece of a cut unit costs a partial sum).
+    int level = 0;
+    {
+        const double steps_per_unit = double(p->n_steps) / double(p->n_units);
+        const double steps_per_range = double(p->n_steps) / double(p->parts[0].part.ranges.size());
+        if (steps_per_unit >= 8.0 * steps_per_range) level = ka.n_feat_blocks >= 4 ? 2 : ka.n_feat_blocks >= 2 ? 1 : 0;
+    }
+    int rc = build_and_upload_partition(p, level);
+    if (rc) return rc;
+    const hspmm_plan::DevPartition &dp = p->parts[level];
+    ka.ranges = dp.d_ranges; ka.split = dp.d_split; ka.fix_slots = dp.d_fix_slots;
+    ka.n_ranges = uint32_t(dp.part.ranges.size());
+    ka.n_split = uint32_t(dp.part.split.size());
     if (uint64_t(ka.n_ranges) * ka.n_feat_blocks > 0x7FFFFFFFull)
         return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many work items", N);
-    const size_t need = size_t(p->part.n_slots) * ka.n_feat_blocks * size_t(c.V) * size_t(p->G) * 64u * 16u;
-    int rc = ensure_scratch(p, need);
-    if (rc) return rc;
+    const size_t need = size_t(dp.part.n_slots) * ka.n_feat_blocks * size_t(c.V) * size_t(p->G) * 64u * 16u;
+    if ((rc = ensure_scratch(p, need))) return rc;
     ka.scratch = p->d_scratch;
+    if (p->cfg.fused_fixup && ka.n_split) {
+        if ((rc = ensure_arrive(p, size_t(ka.n_split) * ka.n_feat_blocks))) return rc;
+        ka.arrive = p->d_arrive;
+    }
     // default depth: what fits 128 registers per lane without spilling
     const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage
                          : p->dtype != HSPMM_FP16 ? (p->G == 2 && c.V == 4 ? 3 : 4)
@@ -578,9 +623,9 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     if (!p || !info) return fail(HSPMM_ERR_INVALID, "null argument");
     info->rows = p->rows; info->cols = p->cols; info->eff_row_windows = p->W; info->total_tiles = p->T;
     info->dtype = p->dtype;
-    info->n_ranges = uint32_t(p->part.ranges.size());
-    info->n_split_windows = uint32_t(p->part.split.size());
-    info->n_partial_slots = p->part.n_slots;
+    info->n_ranges = uint32_t(p->parts[0].part.ranges.size());
+    info->n_split_windows = uint32_t(p->parts[0].part.split.size());
+    info->n_partial_slots = p->parts[0].part.n_slots;
     info->compute_units = uint32_t(p->compute_units);
     info->n_units = p->n_units;
     info->n_paired_units = p->n_paired;
@@ -591,11 +636,11 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
 int hspmm_get_partition(const hspmm_plan *p, uint32_t *ranges, uint32_t capacity_ranges)
 {
     if (!p || !ranges) return fail(HSPMM_ERR_INVALID, "null argument");
-    const size_t n = p->part.ranges.size() < capacity_ranges ? p->part.ranges.size() : capacity_ranges;
+    const size_t n = p->parts[0].part.ranges.size() < capacity_ranges ? p->parts[0].part.ranges.size() : capacity_ranges;
     for (size_t i = 0; i < n; ++i) {
-        ranges[5 * i + 0] = p->part.ranges[i].tile_begin; ranges[5 * i + 1] = p->part.ranges[i].tile_end;
-        ranges[5 * i + 2] = p->part.ranges[i].first_window;
-        ranges[5 * i + 3] = p->part.ranges[i].head_slot; ranges[5 * i + 4] = p->part.ranges[i].tail_slot;
+        ranges[5 * i + 0] = p->parts[0].part.ranges[i].tile_begin; ranges[5 * i + 1] = p->parts[0].part.ranges[i].tile_end;
+        ranges[5 * i + 2] = p->parts[0].part.ranges[i].first_window;
+        ranges[5 * i + 3] = p->parts[0].part.ranges[i].head_slot; ranges[5 * i + 4] = p->parts[0].part.ranges[i].tail_slot;
     }
     return HSPMM_OK;
 }

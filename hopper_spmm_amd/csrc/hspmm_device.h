@@ -31,6 +31,8 @@ struct KernelArgs {
     const uint32_t *split;       // n_split x kFixWords {unit, slot_begin, slot_count, 0}
     const uint32_t *fix_slots;
     float          *scratch;     // partial sums: [slot][feature block][acc reg][lane] x 4 floats
+    uint32_t       *arrive;      // [split unit][feature block] arrival counters (all zero between launches);
+                                 // null: the partial sums are added by a second kernel
     const void     *B;           // cols x N
     void           *C;           // rows x N
     uint32_t n_ranges, n_split, eff_windows, n_units, rows, N, n_feat_blocks;

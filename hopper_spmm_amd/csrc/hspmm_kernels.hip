@@ -81,6 +81,22 @@ __device__ __forceinline__ uint32_t pack_half2_rn(float lo, float hi)
 
 __device__ __forceinline__ uint32_t umin32(uint32_t a, uint32_t b) { return a < b ? a : b; }
 
+// Device-scope ("agent") relaxed accesses, word by word: visible to every XCD.
+__device__ __forceinline__ void store_device_scope(f32x4 *p, const f32x4 v)
+{
+    float *q = reinterpret_cast<float *>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { const float f = v[i]; __hip_atomic_store(q + i, f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+}
+__device__ __forceinline__ f32x4 load_device_scope(const f32x4 *p)
+{
+    const float *q = reinterpret_cast<const float *>(p);
+    f32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __hip_atomic_load(q + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return v;
+}
+
 // Uniform (per-wave) reads of the small index arrays go through the constant
 // address space so that they become scalar loads, which do not share the
 // in-order return queue of the vector loads that stream the tiles.
@@ -449,6 +465,7 @@ void spmm_mfma_kernel(const KernelArgs ka)
     const const_u32_ptr unitRow = as_const(ka.unitRow);
     const uint32_t t0 = rd[0], t1 = rd[1];
     const uint32_t head_slot = rd[3], tail_slot = rd[4];
+    const uint32_t head_split = rd[5], tail_split = rd[6];
     const uint32_t U = ka.n_units, rows = ka.rows;
 
     typename TT::Lane L;
@@ -512,12 +529,49 @@ void spmm_mfma_kernel(const KernelArgs ka)
                     if (paired) TT::template store_window<G - 1>(L, acc, c_lane, row_bytes, row0 + kRowWindow, rows, active);
                 }
             } else {
-                const uint32_t slot = (ww.seg_start == t0) ? head_slot : tail_slot;
+                const bool head = ww.seg_start == t0;
+                const uint32_t slot = head ? head_slot : tail_slot;
                 if (slot != kIdxMax) {
                     f32x4 *dst = reinterpret_cast<f32x4 *>(ka.scratch) +
                                  (size_t(slot) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
+                    if (!ka.arrive) {
 #pragma unroll
-                    for (int p = 0; p < NACC; ++p) dst[p * 64] = acc[p];
+                        for (int p = 0; p < NACC; ++p) dst[p * 64] = acc[p];
+                    } else {
+                        // The wave that brings the last partial sum of a cut unit adds all of
+                        // them, in range order (so the result does not depend on who is last),
+                        // and stores the unit.  The partial sums cross the L2s of different
+                        // XCDs: they are written and read with device-scope accesses (which go
+                        // past the L2 of the XCD), the writes are waited for before the arrival
+                        // is counted, and no whole-cache write-back or invalidate is needed.
+#pragma unroll
+                        for (int p = 0; p < NACC; ++p) store_device_scope(dst + p * 64, acc[p]);
+                        __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): the stores are acknowledged
+                        const uint32_t entry = head ? head_split : tail_split;
+                        const uint32_t *fx = ka.split + size_t(entry) * kFixWords;
+                        uint32_t *ctr = ka.arrive + size_t(entry) * ka.n_feat_blocks + fb;
+                        uint32_t old = 0;
+                        if (lane == 0)
+                            old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        old = __builtin_amdgcn_readfirstlane(old);
+                        const uint32_t sb = fx[1], sc = fx[2];
+                        if (old + 1u == sc) {
+#pragma unroll
+                            for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+                            for (uint32_t i = 0; i < sc; ++i) {
+                                const uint32_t sl = ka.fix_slots[sb + i];
+                                const f32x4 *src = reinterpret_cast<const f32x4 *>(ka.scratch) +
+                                                   (size_t(sl) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
+#pragma unroll
+                                for (int p = 0; p < NACC; ++p) acc[p] += load_device_scope(src + p * 64);
+                            }
+                            TT::template store_window<0>(L, acc, c_lane, row_bytes, row0, rows, active);
+                            if constexpr (G > 1) {
+                                if (paired) TT::template store_window<G - 1>(L, acc, c_lane, row_bytes, row0 + kRowWindow, rows, active);
+                            }
+                            if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                    }
                 }
             }
             if (ww.seg_end == ww.uend) {
@@ -596,6 +650,8 @@ void spmm_fixup_kernel(const KernelArgs ka)
     f32x4 acc[NACC];
 #pragma unroll
     for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // the additions keep the slot order; the loads of four slots are in flight together
+#pragma unroll 4
     for (uint32_t i = 0; i < sc; ++i) {
         const uint32_t slot = ka.fix_slots[sb + i];
         const f32x4 *src = reinterpret_cast<const f32x4 *>(ka.scratch) +
@@ -694,7 +750,7 @@ static hipError_t launch_tt(const KernelArgs &ka, int prefetch, bool narrow, int
     const dim3 grid((items + waves_per_group - 1) / waves_per_group);
     hipError_t e = narrow ? launch_main_p<TT, true>(ka, prefetch, grid, block, s)
                           : launch_main_p<TT, false>(ka, prefetch, grid, block, s);
-    if (e != hipSuccess || ka.n_split == 0) return e;
+    if (e != hipSuccess || ka.n_split == 0 || ka.arrive) return e;
     if (mid && (e = hipEventRecord(mid, s)) != hipSuccess) return e;
     const uint32_t fitems = ka.n_split * ka.n_feat_blocks;
     const dim3 fgrid((fitems + waves_per_group - 1) / waves_per_group);

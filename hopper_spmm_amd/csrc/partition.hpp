@@ -23,6 +23,7 @@ struct Range {
     uint32_t tile_begin, tile_end;    // [begin, end) in the flat tile sequence
     uint32_t first_window;            // effective window holding tile_begin
     uint32_t head_slot, tail_slot;    // partial-sum slots (kNoSlot = none)
+    uint32_t head_split, tail_split;  // index of the cut window's entry in Partition::split
 };
 
 struct SplitWindow {
@@ -85,6 +86,7 @@ inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t
         while (rowOffset[win + 1] <= g.tile_begin) ++win;
         g.first_window = win;
         g.head_slot = g.tail_slot = kNoSlot;
+        g.head_split = g.tail_split = kNoSlot;
     }
     // Partial segments: only the first and the last window segment of a range can
     // be incomplete.  The kernel's rule: an incomplete segment that starts at the
@@ -100,11 +102,13 @@ inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t
             const bool complete = (t == ws) && (se == we);
             if (!complete) {
                 const uint32_t slot = P.n_slots++;
-                if (t == g.tile_begin) g.head_slot = slot; else g.tail_slot = slot;
                 if (cur_split != wv) {
                     P.split.push_back(SplitWindow{wv, uint32_t(P.fix_slots.size()), 0});
                     cur_split = wv;
                 }
+                const uint32_t entry = uint32_t(P.split.size()) - 1u;
+                if (t == g.tile_begin) { g.head_slot = slot; g.head_split = entry; }
+                else { g.tail_slot = slot; g.tail_split = entry; }
                 P.fix_slots.push_back(slot);
                 P.split.back().slot_count++;
             }
