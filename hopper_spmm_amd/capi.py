@@ -12,6 +12,7 @@ import numpy as np
 
 FP16 = 0            # HSPMM_FP16, reference -DUSE_FP16 (src/common.h:14-19)
 TF32 = 1            # HSPMM_TF32, reference -DUSE_TF32 (src/common.h:26-43), fp32 storage
+BF16 = 2            # HSPMM_BF16, reference -DUSE_BF16 (src/common.h:20-25)
 IDX_MAX = 0xFFFFFFFF
 ROW_WINDOW = 8
 
@@ -32,7 +33,7 @@ def library_path():
 
 def build_library(force=True):
     """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU)."""
-    cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j4"]
+    cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j8"]
     if force:
         cmd.insert(1, "-B")
     subprocess.check_call(cmd, stdout=subprocess.DEVNULL)
@@ -40,12 +41,12 @@ def build_library(force=True):
     cli = ["make", "-C", os.path.join(_HERE, "host")]
     if force:
         cli.insert(1, "-B")
-    subprocess.check_call(cli + ["fp16_test", "tf32_test"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(cli + ["fp16_test", "bf16_test", "tf32_test"], stdout=subprocess.DEVNULL)
     return _LIB
 
 
 def cli_path(name):
-    """Path of a built command-line driver: 'fp16_test' or 'tf32_test'."""
+    """Path of a built command-line driver: 'fp16_test', 'bf16_test' or 'tf32_test'."""
     return os.path.join(_HERE, "host", name)
 
 
@@ -115,11 +116,11 @@ def _p(a):
 
 
 def _val_dtype(dtype):
-    if dtype == FP16:
+    if dtype in (FP16, BF16):
         return np.uint16
     if dtype == TF32:
         return np.float32
-    raise ValueError("dtype must be FP16 or TF32")
+    raise ValueError("dtype must be FP16, TF32 or BF16")
 
 
 def configure(buffer_stage=0, consumer_warp_num=0, producer_warp_group_num=0, sm_num=0):
@@ -144,7 +145,7 @@ def set_window_pairing(mode):
 
 def mtx_load(path, dtype):
     """load_matrix of the reference (src/utils/load.h:152): .mtx -> CSR dict.
-    fp16 values are returned as uint16 bit patterns."""
+    fp16 / bf16 values are returned as uint16 bit patterns."""
     L = load_library()
     m = _Csr()
     _check(L.hspmm_mtx_load(os.fsencode(path), dtype, C.byref(m)))
@@ -165,7 +166,7 @@ def csr_to_btcf(rows, cols, row_ptr, col_idx, values, dtype, transpose=False):
     BTCF_MTX_NO_BITMAP fields (src/utils/class.h:74-85) as a dict of numpy arrays."""
     L = load_library()
     vt = _val_dtype(dtype)
-    cw = 16 if dtype == FP16 else 8
+    cw = 8 if dtype == TF32 else 16
     row_ptr = np.ascontiguousarray(row_ptr, np.uint32)
     col_idx = np.ascontiguousarray(col_idx, np.uint32)
     values = np.ascontiguousarray(values, vt)

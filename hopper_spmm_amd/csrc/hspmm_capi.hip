@@ -237,14 +237,14 @@ StepStream build_units(uint32_t W, uint32_t cw, const uint32_t *rowOffset, const
 std::vector<uint32_t> lane_order_ids(const StepStream &st, int dtype, const uint32_t *rowOffset,
                                      const std::vector<uint32_t> &ids_clean)
 {
-    const uint32_t cw = dtype == HSPMM_FP16 ? 16u : 8u;
+    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
     std::vector<uint32_t> out(size_t(st.n_steps) * cw);
     for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
         const uint32_t t0 = rowOffset[st.unitWindow[u]];
         for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
             const uint32_t *src = ids_clean.data() + size_t(t0 + i) * cw;
             uint32_t *dst = out.data() + size_t(st.unitOffset[u] + i) * cw;
-            if (dtype == HSPMM_FP16) std::memcpy(dst, src, 64);
+            if (dtype != HSPMM_TF32) std::memcpy(dst, src, 64);
             else for (uint32_t g = 0; g < 4; ++g) { dst[2 * g] = src[g]; dst[2 * g + 1] = src[g + 4]; }
         }
     }
@@ -269,7 +269,7 @@ std::vector<uint32_t> lane_order_tiles(const StepStream &st, int dtype, const ui
                 for (uint32_t r = 0; r < 8; ++r)
                     for (uint32_t g = 0; g < 4; ++g) {
                         uint32_t *d = dst + ((r * 4 + g) * G + w) * 2;
-                        if (dtype == HSPMM_FP16) { d[0] = src[r * 8 + 2 * g]; d[1] = src[r * 8 + 2 * g + 1]; }
+                        if (dtype != HSPMM_TF32) { d[0] = src[r * 8 + 2 * g]; d[1] = src[r * 8 + 2 * g + 1]; }
                         else { d[0] = src[r * 8 + g]; d[1] = src[r * 8 + g + 4]; }
                     }
             }
@@ -292,7 +292,7 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
     c.narrow = p->cols < (1u << 24) && row_bytes < (1u << 24) && uint64_t(p->cols) * row_bytes <= (1ull << 32);
     const int mode = p->cfg.kernel_mode;
     if (mode == 1) { c.scalar = true; return c; }
-    if (p->dtype == HSPMM_FP16) {
+    if (p->dtype != HSPMM_TF32) {
         if (N % 2 != 0 || (align & 3u)) { c.scalar = true; return c; }
         // word loads measured equal to or faster than wide loads wherever both apply
         const bool dw_ok = (N % 64 == 0);
@@ -416,9 +416,10 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
 {
     if (!out) return fail(HSPMM_ERR_INVALID, "null plan pointer");
     *out = nullptr;
-    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32) return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
-    const uint32_t cw = dtype == HSPMM_FP16 ? 16u : 8u;
-    const uint32_t elem = dtype == HSPMM_FP16 ? 2u : 4u;
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16)
+        return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
+    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
+    const uint32_t elem = dtype == HSPMM_TF32 ? 4u : 2u;
     int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx);
     if (rc) return rc;
 
@@ -467,7 +468,7 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
             const std::vector<uint32_t> ids = lane_order_ids(st, dtype, rowOffset, clean);
             if ((rc = upload(&p->d_ids, ids.data(), ids.size(), &p->fixed_bytes))) return bail(rc);
         }
-        if (dtype == HSPMM_FP16 && st.G == 1) {
+        if (dtype != HSPMM_TF32 && st.G == 1) {
             p->d_tiles = p->d_data;                 // the caller's tile layout already is the lane order
         } else {
             const std::vector<uint32_t> tiles = lane_order_tiles(st, dtype, rowOffset, data);
@@ -554,7 +555,7 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     }
     // default depth: what fits 128 registers per lane without spilling
     const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage
-                         : p->dtype != HSPMM_FP16 ? (p->G == 2 && c.V == 4 ? 3 : 4)
+                         : p->dtype == HSPMM_TF32 ? (p->G == 2 && c.V == 4 ? 3 : 4)
                          : (p->G == 2 && c.V == 4 ? 2 : 3);
     const int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
     HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, c.layout, p->G, ka, c.V, prefetch, c.narrow, wpg, s, mid));

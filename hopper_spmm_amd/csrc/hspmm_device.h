@@ -38,11 +38,13 @@ struct KernelArgs {
     uint32_t n_ranges, n_split, eff_windows, n_units, rows, N, n_feat_blocks;
 };
 
-// dtype: 0 = fp16 tiles 8x16, 1 = fp32 tiles 8x8.  V = 32-bit words a lane loads
+// dtype: 0 = fp16 tiles 8x16, 1 = fp32 tiles 8x8, 2 = bf16 tiles 8x16.  V = 32-bit words a lane loads
 // per B row (1, 2 or 4).
 // layout (fp16 only): kLayoutX4 = wide loads, contiguous features per lane, N % (2V) == 0;
 // kLayoutDW = word loads, features strided by 32 per lane, N % (32V) == 0.
 constexpr int kLayoutX4 = 0, kLayoutDW = 1;
+// element types, numbered as HSPMM_FP16 / HSPMM_TF32 / HSPMM_BF16 of the public header
+constexpr int kDtypeF16 = 0, kDtypeF32 = 1, kDtypeBf16 = 2;
 // narrow: B < 4 GiB and cols < 2^24 (32-bit gather offsets).
 // mid: optional event recorded between the main kernel and the partial-sum kernel.
 // G: windows per unit in the step stream (1, or 2 when the plan paired windows).

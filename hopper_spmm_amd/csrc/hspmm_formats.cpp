@@ -48,6 +48,16 @@ static uint16_t float_to_half_bits(float f)
     return uint16_t(sign | h);
 }
 
+// IEEE binary32 -> bfloat16, round to nearest even (the implicit float ->
+// __nv_bfloat16 conversion of the reference's bf16 build, src/utils/load.h:224).
+static uint16_t float_to_bf16_bits(float f)
+{
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return uint16_t((x >> 16) | 0x0040u);    // NaN stays NaN (quiet)
+    return uint16_t((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+}
+
 static unsigned worker_count(size_t work_items, size_t min_per_worker)
 {
     unsigned hw = std::thread::hardware_concurrency();
@@ -155,7 +165,7 @@ int hspmm_mtx_load(const char *path, int dtype, hspmm_csr *out)
 {
     if (!path || !out) { set_error("null argument"); return HSPMM_ERR_INVALID; }
     std::memset(out, 0, sizeof *out);
-    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
     Triples t;
     std::string err;
     int rc = read_triples(path, t, err);
@@ -168,7 +178,7 @@ int hspmm_mtx_load(const char *path, int dtype, hspmm_csr *out)
             set_error("entry " + std::to_string(i) + " of " + path + " lies outside the declared shape");
             return HSPMM_ERR_IO;
         }
-    const size_t es = dtype == HSPMM_FP16 ? 2 : 4;
+    const size_t es = dtype == HSPMM_TF32 ? 4 : 2;
     uint32_t *row_ptr = static_cast<uint32_t *>(std::calloc(size_t(t.rows) + 1, 4));
     uint32_t *col_idx = static_cast<uint32_t *>(std::malloc((nnz ? nnz : 1) * 4));
     void *values = std::malloc((nnz ? nnz : 1) * es);
@@ -191,7 +201,8 @@ int hspmm_mtx_load(const char *path, int dtype, hspmm_csr *out)
     for (size_t i = 0; i < nnz; ++i) {
         const uint32_t s = order[i];
         col_idx[i] = t.c[s];
-        if (es == 2) static_cast<uint16_t *>(values)[i] = float_to_half_bits(t.v[s]);
+        if (dtype == HSPMM_FP16) static_cast<uint16_t *>(values)[i] = float_to_half_bits(t.v[s]);
+        else if (dtype == HSPMM_BF16) static_cast<uint16_t *>(values)[i] = float_to_bf16_bits(t.v[s]);
         else static_cast<float *>(values)[i] = t.v[s];
     }
     out->rows = t.rows; out->cols = t.cols; out->nnzs = uint32_t(nnz);
@@ -246,12 +257,12 @@ extern "C" {
 int hspmm_btcf_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
                      uint32_t *eff_row_windows, uint32_t *total_tiles)
 {
-    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
     if (!row_ptr || !eff_row_windows || !total_tiles || (!col_idx && row_ptr[rows])) {
         set_error("null argument");
         return HSPMM_ERR_INVALID;
     }
-    const uint32_t cw = dtype == HSPMM_FP16 ? 16u : 8u;
+    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
     std::vector<uint32_t> tiles;
     count_tiles(rows, row_ptr, col_idx, cw, tiles);
     uint64_t W = 0, T = 0;
@@ -266,10 +277,10 @@ int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uin
                     const void *values, int transpose, uint32_t *rowOffset, uint32_t *tcA2B, void *data,
                     uint32_t *rowIdx)
 {
-    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
     if (!row_ptr || !rowOffset) { set_error("null argument"); return HSPMM_ERR_INVALID; }
-    const uint32_t cw = dtype == HSPMM_FP16 ? 16u : 8u;
-    const size_t es = dtype == HSPMM_FP16 ? 2 : 4;
+    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
+    const size_t es = dtype == HSPMM_TF32 ? 4 : 2;
     const size_t tile_elems = size_t(HSPMM_ROW_WINDOW) * cw;
     std::vector<uint32_t> tiles;
     count_tiles(rows, row_ptr, col_idx, cw, tiles);

@@ -1,0 +1,752 @@
+// gfx950 (MI355X) MFMA kernel templates for C = A * B with A in the condensed 8-row-window
+// tile format (reference src/utils/class.h:74-85).  They replace the reference's
+// fp16_spmm_kernel (reference src/fp16.cu:36-175) and supply the fp32-storage
+// ("tf32") variant the reference only sketches (src/common.h:26-43).
+//
+// Design (one wave = one independent pipeline, no LDS, no barriers):
+//   * The plan turns the windows into a flat stream of "steps".  A step is one
+//     tile of one window or - where two vertically adjacent windows have the same
+//     column list, as in block-clustered weights - one tile of each of the two
+//     ("paired unit", G = 2): the gathered rows of B are then loaded once and
+//     multiplied with both tiles.
+//   * A wave owns a contiguous range of steps (a few hundred) and, for feature
+//     dimensions wider than one block, one feature block.  Units are contiguous in
+//     the step stream, so the loads stream through the range without regard to
+//     unit boundaries; only the MFMA stage looks at them (to store a finished
+//     window and clear accumulators).
+//   * Per fp16 step a lane issues one 16-byte load of four column ids, one load
+//     of its part of the sparse tile(s) and the loads of its words of the four B
+//     rows those ids name; the 16 lanes of a quarter-wave cover one B row
+//     contiguously.
+//   * fp16 contraction without any transposition of B: an MFMA operand register
+//     holds two k-slots.  A B register as loaded holds features (2c, 2c+1) of one
+//     gathered row, i.e. "k-slot pair" = (even feature, odd feature).  The sparse
+//     operand is built so that MFMA row 2r holds a[r][k] in the even slot and 0 in
+//     the odd one, MFMA row 2r+1 the reverse.  Output row 2r then is window row r
+//     for the even features, row 2r+1 for the odd ones: all 16 MFMA rows and all
+//     32 k-slots do useful work for an 8-row window, and a lane ends up with
+//     contiguous features of two window rows.
+//   * fp32 ("tf32") contraction uses v_mfma_f32_16x16x4_f32; one B register per
+//     lane per k, no packing issue; MFMA rows 8..15 are zero padding.
+//   * Loads for step t+P are issued before the MFMAs of step t (P = prefetch
+//     depth, registers as the ring buffer); hardware returns vector loads in
+//     order, so the wait before the MFMAs of step t leaves P-1 steps in flight.
+//   * Padding columns (id 0xFFFFFFFF) are renamed, in the plan's device copy of the
+//     ids, to the real column in front of them; their tile column is all zero.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#pragma once
+#include "hspmm_device.h"
+
+namespace hspmm {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float    f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int V> struct Vec;
+template <> struct Vec<1> { typedef uint32_t type; };
+template <> struct Vec<2> { typedef u32x2 type; };
+template <> struct Vec<4> { typedef u32x4 type; };
+
+// C is written once per launch; the rows of B are read again and again.  The
+// stores are marked non-temporal so that C does not push B out of the L2.
+// (Non-temporal loads of the tile / id streams measured slower: not used.)
+template <class T>
+__device__ __forceinline__ void stream_store(T *p, const T v)
+{
+    __builtin_nontemporal_store(v, p);
+}
+
+template <int V>
+__device__ __forceinline__ void store_words(void *p, const uint32_t (&src)[V])
+{
+    typename Vec<V>::type v;
+    if constexpr (V == 1) v = src[0];
+    else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) v[i] = src[i];
+    }
+    stream_store(reinterpret_cast<typename Vec<V>::type *>(p), v);
+}
+
+__device__ __forceinline__ uint32_t pack_half2_rn(float lo, float hi)
+{
+    // float -> half conversion in the default rounding mode (nearest even), as the
+    // reference's store does (src/fp16.cu:167, cvt.rn.f16.f32).
+    _Float16 l = (_Float16)lo, h = (_Float16)hi;
+    uint16_t lb = __builtin_bit_cast(uint16_t, l), hb = __builtin_bit_cast(uint16_t, h);
+    return uint32_t(lb) | (uint32_t(hb) << 16);
+}
+
+__device__ __forceinline__ uint32_t umin32(uint32_t a, uint32_t b) { return a < b ? a : b; }
+
+// The two 16-bit element types share everything but the MFMA instruction and the
+// rounding of the result: BF = false is IEEE half, BF = true bfloat16 (the
+// reference's -DUSE_BF16 build, src/common.h:20-25).  Both round to nearest even.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+template <bool BF> struct HalfOps;
+template <> struct HalfOps<false> {
+    typedef _Float16 elem_t;
+    __device__ static __forceinline__ f32x4 mfma(const u32x4 a, const u32x4 b, const f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ uint32_t pack(float lo, float hi) { return pack_half2_rn(lo, hi); }
+};
+template <> struct HalfOps<true> {
+    typedef __bf16 elem_t;
+    __device__ static __forceinline__ f32x4 mfma(const u32x4 a, const u32x4 b, const f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ uint32_t pack(float lo, float hi)
+    {
+        const __bf16 l = (__bf16)lo, h = (__bf16)hi;
+        return uint32_t(__builtin_bit_cast(uint16_t, l)) | (uint32_t(__builtin_bit_cast(uint16_t, h)) << 16);
+    }
+};
+
+// Device-scope ("agent") relaxed accesses, word by word: visible to every XCD.
+__device__ __forceinline__ void store_device_scope(f32x4 *p, const f32x4 v)
+{
+    float *q = reinterpret_cast<float *>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { const float f = v[i]; __hip_atomic_store(q + i, f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+}
+__device__ __forceinline__ f32x4 load_device_scope(const f32x4 *p)
+{
+    const float *q = reinterpret_cast<const float *>(p);
+    f32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __hip_atomic_load(q + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return v;
+}
+
+// Uniform (per-wave) reads of the small index arrays go through the constant
+// address space so that they become scalar loads, which do not share the
+// in-order return queue of the vector loads that stream the tiles.
+typedef const uint32_t __attribute__((address_space(4))) *const_u32_ptr;
+__device__ __forceinline__ const_u32_ptr as_const(const uint32_t *p)
+{
+    return (const_u32_ptr)(uintptr_t)p;
+}
+
+// Where a lane reads its words of B row c.  NARROW: B is smaller than 4 GiB and
+// has fewer than 2^24 rows, so one 24-bit multiply-add gives a 32-bit offset
+// from a scalar base.
+template <bool NARROW>
+struct Gather {
+    const char *base;        // B (uniform)
+    uint32_t row_bytes;      // N * element size
+    uint32_t lane_off;       // byte offset of the lane's first feature inside a row
+    __device__ __forceinline__ const char *row(uint32_t c) const
+    {
+        if constexpr (NARROW) {
+            const uint32_t off = __umul24(c, row_bytes) + lane_off;
+            return base + size_t(off);
+        } else {
+            return base + (size_t(c) * row_bytes + lane_off);
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Element-type traits: how one step is loaded, multiplied and stored.
+// V = 32-bit words of a B row a lane owns, G = windows per unit (1 or 2).
+// The plan stores the tiles of a step in lane order (hspmm_capi.hip,
+// build_lane_order): what one lane needs of a step is one contiguous load.
+// ---------------------------------------------------------------------------
+
+// Common part of the two fp16 layouts: the sparse operand.
+//   tiles, G = 1: the caller's tile, [row r][k] halves; lane (g, j) reads
+//                 a[j/2][4g..4g+3] = 8 bytes at (r*16 + 4g) halves.
+//   tiles, G = 2: [row r][g][window][4 halves]; the lane reads 16 bytes.
+template <int G>
+struct Fp16Lane {
+    typedef typename Vec<2 * G>::type AVec;
+    uint32_t g, j;                             // quarter-wave, lane in quarter
+    uint32_t sel_lo, sel_hi;                   // byte selectors for the sparse operand
+    const uint32_t *a_src;                     // lane's words inside step 0
+    const uint32_t *idx_src;                   // lane's ids inside step 0
+    __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
+    {
+        g = lane >> 4; j = lane & 15u;
+        const uint32_t r = j >> 1, parity = j & 1u;
+        // v_perm_b32 selectors: bytes 0-3 come from the second source, 0x0c gives 0x00.
+        //   even MFMA row: value in the low half  -> {lo: b0 b1 0 0}, {hi: b2 b3 0 0}
+        //   odd  MFMA row: value in the high half -> {lo: 0 0 b0 b1}, {hi: 0 0 b2 b3}
+        sel_lo = parity ? 0x01000c0cu : 0x0c0c0100u;
+        sel_hi = parity ? 0x03020c0cu : 0x0c0c0302u;
+        a_src = reinterpret_cast<const uint32_t *>(tiles) + (r * 8u + g * 2u) * G;
+        idx_src = ids + g * 4u;
+    }
+    __device__ __forceinline__ u32x4 load_idx(uint32_t step) const
+    {
+        return *reinterpret_cast<const u32x4 *>(idx_src + size_t(step) * 16u);
+    }
+    __device__ __forceinline__ AVec load_a(uint32_t step) const
+    {
+        return *reinterpret_cast<const AVec *>(a_src + size_t(step) * (64u * G));
+    }
+    // MFMA row 2r carries a[r][k] in the even k-slot of each pair, row 2r+1 in the odd one.
+    template <int W0>
+    __device__ __forceinline__ u32x4 sparse_operand(const AVec &a) const
+    {
+        const uint32_t lo = a[2 * W0], hi = a[2 * W0 + 1];
+        u32x4 aw;
+        aw[0] = __builtin_amdgcn_perm(0u, lo, sel_lo);
+        aw[1] = __builtin_amdgcn_perm(0u, lo, sel_hi);
+        aw[2] = __builtin_amdgcn_perm(0u, hi, sel_lo);
+        aw[3] = __builtin_amdgcn_perm(0u, hi, sel_hi);
+        return aw;
+    }
+};
+
+// fp16, layout "X4": a lane reads 4*V contiguous bytes of each of its four B rows
+// (one wide load per row) and owns 2*V contiguous features.  Any N that is a
+// multiple of 2*V.  The B operand of MFMA p is word p of the four loads, which
+// costs register moves.
+template <int V_, int G_, bool BF = false>
+struct Fp16Tile {
+    static constexpr int V = V_, G = G_;
+    static constexpr int kBlockFeat = 32 * V;      // features one wave covers
+    static constexpr int kLaneFeat = 2 * V;        // lane's first feature = j * kLaneFeat
+    static constexpr int kElem = 2;
+    typedef typename Vec<V>::type BVec;
+    typedef u32x4 Idx;                             // four column ids per lane per step
+    typedef Fp16Lane<G> Lane;
+    typedef typename Lane::AVec AVec;
+
+    __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t step) { return L.load_idx(step); }
+    // The registers of one step in flight are separate variables of the caller
+    // (b0..b3: the lane's words of four B rows, a: its words of the sparse tile(s)).
+    template <class GT>
+    __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t step, const Idx idx, const GT &gat,
+                                                     BVec &b0, BVec &b1, BVec &b2, BVec &b3, AVec &a)
+    {
+        b0 = *reinterpret_cast<const BVec *>(gat.row(idx[0]));
+        b1 = *reinterpret_cast<const BVec *>(gat.row(idx[1]));
+        b2 = *reinterpret_cast<const BVec *>(gat.row(idx[2]));
+        b3 = *reinterpret_cast<const BVec *>(gat.row(idx[3]));
+        a = L.load_a(step);
+    }
+    template <int p> __device__ static __forceinline__ uint32_t word(const BVec &v)
+    {
+        if constexpr (V == 1) return v; else return v[p];
+    }
+    template <int W0, int p>
+    __device__ static __forceinline__ void mma_one(const u32x4 av, const BVec &b0, const BVec &b1, const BVec &b2,
+                                                   const BVec &b3, f32x4 (&acc)[G * V])
+    {
+        if constexpr (p < V) {
+            u32x4 bw;
+            bw[0] = word<p>(b0); bw[1] = word<p>(b1); bw[2] = word<p>(b2); bw[3] = word<p>(b3);
+            acc[W0 * V + p] = HalfOps<BF>::mfma(av, bw, acc[W0 * V + p]);
+        }
+    }
+    template <int W0>
+    __device__ static __forceinline__ void mma_window(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
+                                                      const BVec &b3, const AVec &a, f32x4 (&acc)[G * V])
+    {
+        if constexpr (W0 < G) {
+            const u32x4 av = L.template sparse_operand<W0>(a);
+            mma_one<W0, 0>(av, b0, b1, b2, b3, acc); mma_one<W0, 1>(av, b0, b1, b2, b3, acc);
+            mma_one<W0, 2>(av, b0, b1, b2, b3, acc); mma_one<W0, 3>(av, b0, b1, b2, b3, acc);
+        }
+    }
+    __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
+                                               const BVec &b3, const AVec &a, f32x4 (&acc)[G * V])
+    {
+        mma_window<0>(L, b0, b1, b2, b3, a, acc);
+        mma_window<1>(L, b0, b1, b2, b3, a, acc);
+    }
+    // acc[W0*V + p][e]: MFMA row 4g+e = window row 2g + e/2, feature lane_feat + 2p + (e & 1).
+    template <int W0>
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[G * V], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+            const uint32_t row = row0 + 2u * L.g + rr;
+            uint32_t out[V];
+#pragma unroll
+            for (int p = 0; p < V; ++p) out[p] = HalfOps<BF>::pack(acc[W0 * V + p][2 * rr], acc[W0 * V + p][2 * rr + 1]);
+            if (active && row < rows) store_words<V>(c_lane + size_t(row) * row_bytes, out);
+        }
+    }
+    // Zero rows [r_begin, r_end) of this lane's features.
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        uint32_t z[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) z[i] = 0u;
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) store_words<V>(c_lane + size_t(r) * row_bytes, z);
+    }
+};
+
+// fp16, layout "DW": a lane reads single words, word p of a row at feature
+// 32p + 2j, so that the 16 lanes of a quarter-wave still read 64 contiguous
+// bytes, and the four words that form the B operand of MFMA p (one per B row)
+// are loaded straight into four consecutive registers: no moves.  Needs N to be
+// a multiple of 32*V.
+template <int V_, int G_, bool BF = false>
+struct Fp16TileDW {
+    static constexpr int V = V_, G = G_;
+    static constexpr int kBlockFeat = 32 * V;
+    static constexpr int kLaneFeat = 2;            // lane's first feature = 2j, then +32 per word
+    static constexpr int kElem = 2;
+    typedef u32x4 BVec;                            // b_p = word p of the four B rows
+    typedef u32x4 Idx;
+    typedef Fp16Lane<G> Lane;
+    typedef typename Lane::AVec AVec;
+
+    __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t step) { return L.load_idx(step); }
+    template <class GT>
+    __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t step, const Idx idx, const GT &gat,
+                                                     BVec &b0, BVec &b1, BVec &b2, BVec &b3, AVec &a)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(gat.row(idx[q]));
+            b0[q] = src[0];
+            if constexpr (V > 1) b1[q] = src[16];
+            if constexpr (V > 2) b2[q] = src[32];
+            if constexpr (V > 3) b3[q] = src[48];
+        }
+        a = L.load_a(step);
+    }
+    template <int W0>
+    __device__ static __forceinline__ void mma_window(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
+                                                      const BVec &b3, const AVec &a, f32x4 (&acc)[G * V])
+    {
+        if constexpr (W0 < G) {
+            const u32x4 av = L.template sparse_operand<W0>(a);
+            acc[W0 * V] = HalfOps<BF>::mfma(av, b0, acc[W0 * V]);
+            if constexpr (V > 1) acc[W0 * V + 1] = HalfOps<BF>::mfma(av, b1, acc[W0 * V + 1]);
+            if constexpr (V > 2) acc[W0 * V + 2] = HalfOps<BF>::mfma(av, b2, acc[W0 * V + 2]);
+            if constexpr (V > 3) acc[W0 * V + 3] = HalfOps<BF>::mfma(av, b3, acc[W0 * V + 3]);
+        }
+    }
+    __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
+                                               const BVec &b3, const AVec &a, f32x4 (&acc)[G * V])
+    {
+        mma_window<0>(L, b0, b1, b2, b3, a, acc);
+        mma_window<1>(L, b0, b1, b2, b3, a, acc);
+    }
+    // acc[W0*V + p][e]: MFMA row 4g+e = window row 2g + e/2, feature 32p + 2j + (e & 1).
+    template <int W0>
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[G * V], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+            const uint32_t row = row0 + 2u * L.g + rr;
+            if (active && row < rows) {
+                uint32_t *dst = reinterpret_cast<uint32_t *>(c_lane + size_t(row) * row_bytes);
+#pragma unroll
+                for (int p = 0; p < V; ++p)
+                    stream_store(dst + 16 * p, HalfOps<BF>::pack(acc[W0 * V + p][2 * rr], acc[W0 * V + p][2 * rr + 1]));
+            }
+        }
+    }
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) {
+            uint32_t *dst = reinterpret_cast<uint32_t *>(c_lane + size_t(r) * row_bytes);
+#pragma unroll
+            for (int p = 0; p < V; ++p) stream_store(dst + 16 * p, 0u);
+        }
+    }
+};
+
+// fp32 storage ("tf32" build of the reference): 8x8 tiles, v_mfma_f32_16x16x4_f32.
+// MFMA rows 0..7 are the window rows, rows 8..15 zero; lane (g, j) supplies k = g
+// and k = g + 4 of a tile and V contiguous features.
+//   ids per step, lane order: [g][2] = (id g, id g+4): 8 bytes per lane.
+//   tiles per step, lane order: [row r][g][window][2] = (a[r][g], a[r][g+4]) per window.
+template <int V_, int G_>
+struct Fp32Tile {
+    static constexpr int V = V_, G = G_;
+    static constexpr int kBlockFeat = 16 * V;
+    static constexpr int kLaneFeat = V;
+    static constexpr int kElem = 4;
+    typedef typename Vec<V>::type BVec;
+    typedef u32x2 Idx;                             // two column ids per lane per step
+    typedef typename Vec<2 * G>::type AVec;
+
+    struct Lane {
+        uint32_t g, j;
+        uint32_t a_mask;                           // all ones for MFMA rows 0..7, else 0
+        const uint32_t *a_src;
+        const uint32_t *idx_src;
+        __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
+        {
+            g = lane >> 4; j = lane & 15u;
+            a_mask = j < 8u ? 0xFFFFFFFFu : 0u;
+            a_src = reinterpret_cast<const uint32_t *>(tiles) + ((j & 7u) * 8u + g * 2u) * G;
+            idx_src = ids + g * 2u;
+        }
+    };
+    __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t step)
+    {
+        return *reinterpret_cast<const u32x2 *>(L.idx_src + size_t(step) * 8u);
+    }
+    template <class GT>
+    __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t step, const Idx idx, const GT &gat,
+                                                     BVec &b0, BVec &b1, BVec &, BVec &, AVec &a)
+    {
+        b0 = *reinterpret_cast<const BVec *>(gat.row(idx[0]));
+        b1 = *reinterpret_cast<const BVec *>(gat.row(idx[1]));
+        a = *reinterpret_cast<const AVec *>(L.a_src + size_t(step) * (64u * G));
+    }
+    template <int p> __device__ static __forceinline__ float word(const BVec &v)
+    {
+        // (a bit_cast applied directly to a vector element reads element 0: copy first)
+        uint32_t w;
+        if constexpr (V == 1) w = v; else w = v[p];
+        return __builtin_bit_cast(float, w);
+    }
+    template <int W0, int p>
+    __device__ static __forceinline__ void mma_one(const float a0, const float a1, const BVec &b0, const BVec &b1,
+                                                   f32x4 (&acc)[G * V])
+    {
+        if constexpr (p < V) {
+            acc[W0 * V + p] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, word<p>(b0), acc[W0 * V + p], 0, 0, 0);
+            acc[W0 * V + p] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, word<p>(b1), acc[W0 * V + p], 0, 0, 0);
+        }
+    }
+    template <int W0>
+    __device__ static __forceinline__ void mma_window(const Lane &L, const BVec &b0, const BVec &b1, const AVec &a,
+                                                      f32x4 (&acc)[G * V])
+    {
+        if constexpr (W0 < G) {
+            const uint32_t w0 = a[2 * W0] & L.a_mask, w1 = a[2 * W0 + 1] & L.a_mask;
+            const float a0 = __builtin_bit_cast(float, w0), a1 = __builtin_bit_cast(float, w1);
+            mma_one<W0, 0>(a0, a1, b0, b1, acc); mma_one<W0, 1>(a0, a1, b0, b1, acc);
+            mma_one<W0, 2>(a0, a1, b0, b1, acc); mma_one<W0, 3>(a0, a1, b0, b1, acc);
+        }
+    }
+    __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &,
+                                               const BVec &, const AVec &a, f32x4 (&acc)[G * V])
+    {
+        mma_window<0>(L, b0, b1, a, acc);
+        mma_window<1>(L, b0, b1, a, acc);
+    }
+    // acc[W0*V + p][e]: MFMA row 4g+e (a window row when g < 2), feature lane_feat + p.
+    template <int W0>
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[G * V], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t row = row0 + 4u * L.g + e;
+            uint32_t out[V];
+#pragma unroll
+            for (int p = 0; p < V; ++p) { const float f = acc[W0 * V + p][e]; out[p] = __builtin_bit_cast(uint32_t, f); }
+            if (active && L.g < 2u && row < rows) store_words<V>(c_lane + size_t(row) * row_bytes, out);
+        }
+    }
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        uint32_t z[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) z[i] = 0u;
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) store_words<V>(c_lane + size_t(r) * row_bytes, z);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Main kernel: one wave per (step range, feature block).
+// ---------------------------------------------------------------------------
+// State of the unit walk (all wave-uniform, kept in scalar registers).  A unit is
+// one window, or two adjacent windows with one column list (bit 0 of unitRow).
+struct UnitWalk {
+    uint32_t u;            // current unit
+    uint32_t ustart, uend; // its step span
+    uint32_t row;          // its first matrix row | paired bit
+    uint32_t next_row;     // first row of the next unit (or rows)
+    uint32_t seg_start, seg_end;   // part of the span inside this wave's range
+};
+
+template <class TT, int P, bool NARROW>
+__global__ __launch_bounds__(kMaxWavesPerGroup * 64, (P <= 4 ? 4 : 2))
+void spmm_mfma_kernel(const KernelArgs ka)
+{
+    constexpr int G = TT::G, V = TT::V, NACC = G * V;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t item = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    if (item >= ka.n_ranges * ka.n_feat_blocks) return;
+    const uint32_t range = item / ka.n_feat_blocks;
+    const uint32_t fb = item - range * ka.n_feat_blocks;
+    const const_u32_ptr rd = as_const(ka.ranges) + size_t(range) * kRangeWords;
+    const const_u32_ptr unitOffset = as_const(ka.unitOffset);
+    const const_u32_ptr unitRow = as_const(ka.unitRow);
+    const uint32_t t0 = rd[0], t1 = rd[1];
+    const uint32_t head_slot = rd[3], tail_slot = rd[4];
+    const uint32_t head_split = rd[5], tail_split = rd[6];
+    const uint32_t U = ka.n_units, rows = ka.rows;
+
+    typename TT::Lane L;
+    L.init(lane, ka.tiles, ka.ids);
+    const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
+    const bool active = feat < ka.N;
+    const size_t row_bytes = size_t(ka.N) * TT::kElem;
+    char *c_lane = reinterpret_cast<char *>(ka.C) + size_t(feat) * TT::kElem;
+    Gather<NARROW> gat;
+    gat.base = reinterpret_cast<const char *>(ka.B);
+    gat.row_bytes = uint32_t(row_bytes);
+    gat.lane_off = active ? feat * TT::kElem : 0u;     // lanes past N read (and drop) the row start
+
+    UnitWalk ww;
+    ww.u = rd[2];
+    ww.ustart = unitOffset[ww.u];
+    ww.uend = unitOffset[ww.u + 1u];
+    ww.row = unitRow[ww.u];
+    ww.next_row = (ww.u + 1u < U) ? (unitRow[ww.u + 1u] & ~7u) : rows;
+    ww.seg_start = t0;
+    ww.seg_end = umin32(ww.uend, t1);
+
+    // Rows before the first effective window belong to the wave that starts at step 0.
+    if (t0 == 0u) TT::zero_rows(L, c_lane, row_bytes, 0u, unitRow[0] & ~7u, active);
+
+    f32x4 acc[NACC];
+#pragma unroll
+    for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t tlast = t1 - 1u;
+    typedef typename TT::BVec BVec;
+    typedef typename TT::AVec AVec;
+#define HSPMM_FOR_STAGES(X) \
+    X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7)
+#define HSPMM_DECL(k) BVec b0_##k, b1_##k, b2_##k, b3_##k; AVec a_##k; typename TT::Idx I##k;
+#define HSPMM_REGS(k) b0_##k, b1_##k, b2_##k, b3_##k, a_##k
+    HSPMM_FOR_STAGES(HSPMM_DECL)
+#define HSPMM_PRO_IDX(k) if constexpr (P > k) I##k = TT::load_idx(L, umin32(t0 + k, tlast));
+#define HSPMM_PRO_TILE(k) if constexpr (P > k) { \
+        TT::load_tile(L, umin32(t0 + k, tlast), I##k, gat, HSPMM_REGS(k)); \
+        I##k = TT::load_idx(L, umin32(t0 + P + k, tlast)); \
+        __builtin_amdgcn_sched_barrier(0); }
+    // The order of the loads below must be the order of the steady state (the
+    // compiler derives the steady state's wait counts from both ways into the
+    // loop), hence the scheduling barriers.
+    HSPMM_FOR_STAGES(HSPMM_PRO_IDX)
+    __builtin_amdgcn_sched_barrier(0);
+    HSPMM_FOR_STAGES(HSPMM_PRO_TILE)
+
+    // MFMAs of `step` from its registers, then the unit bookkeeping.
+    auto compute = [&](const BVec &b0, const BVec &b1, const BVec &b2, const BVec &b3, const AVec &a,
+                       const uint32_t step) __attribute__((always_inline)) {
+        TT::mma(L, b0, b1, b2, b3, a, acc);
+        if (step + 1u == ww.seg_end) {
+            const uint32_t row0 = ww.row & ~7u;
+            const bool paired = (G > 1) && (ww.row & 1u);
+            const bool complete = (ww.seg_start == ww.ustart) && (ww.seg_end == ww.uend);
+            if (complete) {
+                TT::template store_window<0>(L, acc, c_lane, row_bytes, row0, rows, active);
+                if constexpr (G > 1) {
+                    if (paired) TT::template store_window<G - 1>(L, acc, c_lane, row_bytes, row0 + kRowWindow, rows, active);
+                }
+            } else {
+                const bool head = ww.seg_start == t0;
+                const uint32_t slot = head ? head_slot : tail_slot;
+                if (slot != kIdxMax) {
+                    f32x4 *dst = reinterpret_cast<f32x4 *>(ka.scratch) +
+                                 (size_t(slot) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
+                    if (!ka.arrive) {
+#pragma unroll
+                        for (int p = 0; p < NACC; ++p) dst[p * 64] = acc[p];
+                    } else {
+                        // The wave that brings the last partial sum of a cut unit adds all of
+                        // them, in range order (so the result does not depend on who is last),
+                        // and stores the unit.  The partial sums cross the L2s of different
+                        // XCDs: they are written and read with device-scope accesses (which go
+                        // past the L2 of the XCD), the writes are waited for before the arrival
+                        // is counted, and no whole-cache write-back or invalidate is needed.
+#pragma unroll
+                        for (int p = 0; p < NACC; ++p) store_device_scope(dst + p * 64, acc[p]);
+                        __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): the stores are acknowledged
+                        const uint32_t entry = head ? head_split : tail_split;
+                        const uint32_t *fx = ka.split + size_t(entry) * kFixWords;
+                        uint32_t *ctr = ka.arrive + size_t(entry) * ka.n_feat_blocks + fb;
+                        uint32_t old = 0;
+                        if (lane == 0)
+                            old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        old = __builtin_amdgcn_readfirstlane(old);
+                        const uint32_t sb = fx[1], sc = fx[2];
+                        if (old + 1u == sc) {
+#pragma unroll
+                            for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+                            for (uint32_t i = 0; i < sc; ++i) {
+                                const uint32_t sl = ka.fix_slots[sb + i];
+                                const f32x4 *src = reinterpret_cast<const f32x4 *>(ka.scratch) +
+                                                   (size_t(sl) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
+#pragma unroll
+                                for (int p = 0; p < NACC; ++p) acc[p] += load_device_scope(src + p * 64);
+                            }
+                            TT::template store_window<0>(L, acc, c_lane, row_bytes, row0, rows, active);
+                            if constexpr (G > 1) {
+                                if (paired) TT::template store_window<G - 1>(L, acc, c_lane, row_bytes, row0 + kRowWindow, rows, active);
+                            }
+                            if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                    }
+                }
+            }
+            if (ww.seg_end == ww.uend) {
+                // this wave holds the unit's last step: it also clears the empty
+                // windows that follow (rows up to the next effective window)
+                const uint32_t gap_begin = row0 + (paired ? 2u * kRowWindow : kRowWindow);
+                if (gap_begin < ww.next_row) TT::zero_rows(L, c_lane, row_bytes, gap_begin, ww.next_row, active);
+            }
+#pragma unroll
+            for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+            // next unit (the reads are clamped; values past the end are not used)
+            ++ww.u;
+            ww.ustart = ww.uend;
+            ww.uend = unitOffset[umin32(ww.u + 1u, U)];
+            ww.row = unitRow[umin32(ww.u, U - 1u)];
+            ww.next_row = (ww.u + 1u < U) ? (unitRow[ww.u + 1u] & ~7u) : rows;
+            ww.seg_start = ww.seg_end;
+            ww.seg_end = umin32(ww.uend, t1);
+        }
+    };
+
+    // Steady state: every stage computes its step and reloads its registers with
+    // the step P further on, without conditions, so that the wait in front of a
+    // stage's MFMAs leaves the loads of the P-1 younger stages in flight.
+    uint32_t t = t0;
+    for (; t + 2u * P <= t1; t += P) {
+#define HSPMM_STEADY(k) if constexpr (P > k) { \
+        compute(HSPMM_REGS(k), t + k); \
+        TT::load_tile(L, t + k + P, I##k, gat, HSPMM_REGS(k)); \
+        I##k = TT::load_idx(L, umin32(t + k + 2u * P, tlast)); \
+        __builtin_amdgcn_sched_barrier(0); }
+        HSPMM_FOR_STAGES(HSPMM_STEADY)
+    }
+    // Drain: fewer than 2P steps are left; loads stop at the end of the range.
+    for (; t < t1; t += P) {
+#define HSPMM_DRAIN(k) if constexpr (P > k) { \
+        if (t + k < t1) compute(HSPMM_REGS(k), t + k); \
+        if (t + k + P < t1) { \
+            TT::load_tile(L, t + k + P, I##k, gat, HSPMM_REGS(k)); \
+            I##k = TT::load_idx(L, umin32(t + k + 2u * P, tlast)); } }
+        HSPMM_FOR_STAGES(HSPMM_DRAIN)
+    }
+#undef HSPMM_DRAIN
+#undef HSPMM_STEADY
+#undef HSPMM_PRO_TILE
+#undef HSPMM_PRO_IDX
+#undef HSPMM_REGS
+#undef HSPMM_DECL
+#undef HSPMM_FOR_STAGES
+}
+
+// ---------------------------------------------------------------------------
+// Second kernel: adds, in range order, the fp32 partial sums of every unit
+// whose steps were cut across ranges, and stores its window(s).
+// ---------------------------------------------------------------------------
+template <class TT>
+__global__ __launch_bounds__(kMaxWavesPerGroup * 64)
+void spmm_fixup_kernel(const KernelArgs ka)
+{
+    constexpr int G = TT::G, V = TT::V, NACC = G * V;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t item = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    if (item >= ka.n_split * ka.n_feat_blocks) return;
+    const uint32_t entry = item / ka.n_feat_blocks;
+    const uint32_t fb = item - entry * ka.n_feat_blocks;
+    const uint32_t *fx = ka.split + size_t(entry) * kFixWords;
+    const uint32_t u = fx[0], sb = fx[1], sc = fx[2];
+
+    typename TT::Lane L;
+    L.init(lane, ka.tiles, ka.ids);
+    const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
+    const bool active = feat < ka.N;
+    const size_t row_bytes = size_t(ka.N) * TT::kElem;
+    char *c_lane = reinterpret_cast<char *>(ka.C) + size_t(feat) * TT::kElem;
+
+    f32x4 acc[NACC];
+#pragma unroll
+    for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // the additions keep the slot order; the loads of four slots are in flight together
+#pragma unroll 4
+    for (uint32_t i = 0; i < sc; ++i) {
+        const uint32_t slot = ka.fix_slots[sb + i];
+        const f32x4 *src = reinterpret_cast<const f32x4 *>(ka.scratch) +
+                           (size_t(slot) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
+#pragma unroll
+        for (int p = 0; p < NACC; ++p) acc[p] += src[p * 64];
+    }
+    const uint32_t row = ka.unitRow[u];
+    TT::template store_window<0>(L, acc, c_lane, row_bytes, row & ~7u, ka.rows, active);
+    if constexpr (G > 1) {
+        if (row & 1u) TT::template store_window<G - 1>(L, acc, c_lane, row_bytes, (row & ~7u) + kRowWindow, ka.rows, active);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Launch helpers (host).  The instantiations are spread over several source
+// files (one per element type and unit width) so that they compile in parallel.
+// ---------------------------------------------------------------------------
+template <class TT, bool NARROW>
+static hipError_t launch_main_p(const KernelArgs &ka, int prefetch, dim3 grid, dim3 block, hipStream_t s)
+{
+    switch (prefetch) {
+    case 1: spmm_mfma_kernel<TT, 1, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 2: spmm_mfma_kernel<TT, 2, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 4: spmm_mfma_kernel<TT, 4, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 6: spmm_mfma_kernel<TT, 6, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 8: spmm_mfma_kernel<TT, 8, NARROW><<<grid, block, 0, s>>>(ka); break;
+    default: spmm_mfma_kernel<TT, 3, NARROW><<<grid, block, 0, s>>>(ka); break;
+    }
+    return hipGetLastError();
+}
+
+template <class TT>
+static hipError_t launch_tt(const KernelArgs &ka, int prefetch, bool narrow, int waves_per_group, hipStream_t s,
+                            hipEvent_t mid)
+{
+    const uint32_t items = ka.n_ranges * ka.n_feat_blocks;
+    const dim3 block(64u * waves_per_group);
+    const dim3 grid((items + waves_per_group - 1) / waves_per_group);
+    hipError_t e = narrow ? launch_main_p<TT, true>(ka, prefetch, grid, block, s)
+                          : launch_main_p<TT, false>(ka, prefetch, grid, block, s);
+    if (e != hipSuccess || ka.n_split == 0 || ka.arrive) return e;
+    if (mid && (e = hipEventRecord(mid, s)) != hipSuccess) return e;
+    const uint32_t fitems = ka.n_split * ka.n_feat_blocks;
+    const dim3 fgrid((fitems + waves_per_group - 1) / waves_per_group);
+    spmm_fixup_kernel<TT><<<fgrid, block, 0, s>>>(ka);
+    return hipGetLastError();
+}
+
+template <template <int, int> class TTV, int G>
+static hipError_t launch_v(const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, hipStream_t s,
+                           hipEvent_t mid)
+{
+    if (V == 4) return launch_tt<TTV<4, G>>(ka, prefetch, narrow, waves_per_group, s, mid);
+    if (V == 2) return launch_tt<TTV<2, G>>(ka, prefetch, narrow, waves_per_group, s, mid);
+    return launch_tt<TTV<1, G>>(ka, prefetch, narrow, waves_per_group, s, mid);
+}
+
+template <template <int, int> class TTV>
+static hipError_t launch_g(const KernelArgs &ka, int G, int V, int prefetch, bool narrow, int waves_per_group,
+                           hipStream_t s, hipEvent_t mid)
+{
+    return G == 2 ? launch_v<TTV, 2>(ka, V, prefetch, narrow, waves_per_group, s, mid)
+                  : launch_v<TTV, 1>(ka, V, prefetch, narrow, waves_per_group, s, mid);
+}
+
+template <int V, int G> using Fp16X4 = Fp16Tile<V, G, false>;
+template <int V, int G> using Fp16DW = Fp16TileDW<V, G, false>;
+template <int V, int G> using Bf16X4 = Fp16Tile<V, G, true>;
+template <int V, int G> using Bf16DW = Fp16TileDW<V, G, true>;
+
+}  // namespace hspmm

@@ -13,7 +13,7 @@ a row.  fp16 values are returned as uint16 bit patterns (round to nearest even).
 """
 import numpy as np
 
-FP16, TF32 = 0, 1
+FP16, TF32, BF16 = 0, 1, 2
 
 
 def _rng(seed):
@@ -25,6 +25,25 @@ def half_bits(x):
     return np.asarray(x, np.float32).astype(np.float16).view(np.uint16)
 
 
+def bf16_bits(x):
+    """float array -> bfloat16 bit patterns (uint16), round to nearest even."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = np.isnan(np.asarray(x, np.float32))
+    if nan.any():
+        r = np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), r)
+    return r
+
+
+def encode(x, dtype):
+    """float values -> the storage of `dtype` (uint16 bits for fp16 / bf16, float32 otherwise)."""
+    if dtype == FP16:
+        return half_bits(x)
+    if dtype == BF16:
+        return bf16_bits(x)
+    return np.asarray(x, np.float32)
+
+
 def csr_from_keys(rows, cols, keys, values_fn, dtype):
     """keys: sorted unique int64 array of row * cols + col."""
     r = (keys // cols).astype(np.int64)
@@ -33,7 +52,7 @@ def csr_from_keys(rows, cols, keys, values_fn, dtype):
     row_ptr = np.zeros(rows + 1, np.uint32)
     np.cumsum(counts, out=row_ptr[1:])
     vals = values_fn(r, c, counts)
-    vals = half_bits(vals) if dtype == FP16 else np.asarray(vals, np.float32)
+    vals = encode(vals, dtype)
     return dict(rows=int(rows), cols=int(cols), nnzs=int(keys.size), dtype=dtype,
                 row_ptr=row_ptr, col_idx=c, values=vals)
 
@@ -119,7 +138,7 @@ def dense_b(cols, N, seed, dtype=FP16):
     """B = N(0, 1), row-major cols x N; uint16 half bits for fp16, float32 otherwise."""
     g = _rng(seed)
     x = g.standard_normal((cols, N), dtype=np.float32)
-    return half_bits(x) if dtype == FP16 else x
+    return encode(x, dtype)
 
 
 # The five configurations the benchmark names; `shrink` divides the sizes for
@@ -156,7 +175,7 @@ def algorithmic_bytes(btcf, N):
     """Compulsory bytes of one SpMM: every array touched once - the tiles, the
     column ids, rowOffset, rowIdx, each B row that is referenced at least once,
     and all of C."""
-    s = 2 if btcf["dtype"] == FP16 else 4
+    s = 4 if btcf["dtype"] == TF32 else 2
     cw = btcf["cw"]
     T, W, M = int(btcf["total_tiles"]), int(btcf["eff_row_windows"]), int(btcf["rows"])
     ids = btcf["tcA2B"]
@@ -166,7 +185,7 @@ def algorithmic_bytes(btcf, N):
 
 def gather_bytes(btcf, N):
     """Same with every gathered B row counted every time it is read."""
-    s = 2 if btcf["dtype"] == FP16 else 4
+    s = 4 if btcf["dtype"] == TF32 else 2
     cw = btcf["cw"]
     T, W, M = int(btcf["total_tiles"]), int(btcf["eff_row_windows"]), int(btcf["rows"])
     ids = btcf["tcA2B"]

@@ -1,7 +1,7 @@
 // C++ host interface with the names and argument meaning of the reference's
 // host code, implemented on the C ABI of libhspmm.so (include/hspmm.h):
 //
-//   compile-time element type   -DUSE_FP16 / -DUSE_TF32      reference src/common.h:14-43
+//   compile-time element type   -DUSE_FP16 / -DUSE_BF16 / -DUSE_TF32   reference src/common.h:14-43
 //   CSR_MTX, DENSE_MTX, BTCF_MTX_NO_BITMAP, PERF_RESULT      reference src/utils/class.h:30-48, 74-85; src/common.h:51-59
 //   load_matrix, free_csr_matrix                             reference src/utils/load.h:152-355
 //   CSR2BTCFNOBITMAP                                         reference src/utils/convert.h:146-225
@@ -12,7 +12,7 @@
 // Differences from the reference, all deliberate: errors are reported (message on
 // stderr, exit code 1) from this layer only, the library below never exits; the
 // operator copies C back to the host (the reference stops after the timing loop,
-// src/fp16.cu:269); tf32_spmm exists (the reference has no such entry point).
+// src/fp16.cu:269); tf32_spmm and bf16_spmm exist (the reference has no such entry points).
 #pragma once
 
 #include <cstdint>
@@ -24,8 +24,8 @@
 #include <hip/hip_runtime.h>
 #include "../../include/hspmm.h"
 
-#if !defined(USE_FP16) && !defined(USE_TF32)
-#error "define USE_FP16 or USE_TF32 (as the reference's Makefile does)"
+#if !defined(USE_FP16) && !defined(USE_TF32) && !defined(USE_BF16)
+#error "define USE_FP16, USE_BF16 or USE_TF32 (as the reference's Makefile does)"
 #endif
 
 #define MAT_PTR_TYPE uint32_t
@@ -35,10 +35,14 @@
 #define IDX_MAX UINT32_MAX
 #define WARMUP_RUNS 3
 #define RUNS 5
-#ifdef USE_FP16
+#if defined(USE_FP16)
 #define MAT_VAL_TYPE _Float16
 #define COL_WINDOW 16
 #define HSPMM_BUILD_DTYPE HSPMM_FP16
+#elif defined(USE_BF16)
+#define MAT_VAL_TYPE __bf16
+#define COL_WINDOW 16
+#define HSPMM_BUILD_DTYPE HSPMM_BF16
 #else
 #define MAT_VAL_TYPE float
 #define COL_WINDOW 8
@@ -135,7 +139,7 @@ inline void CSR2BTCFNOBITMAP(const CSR_MTX &csr, BTCF_MTX_NO_BITMAP &btcf)
         hspmm_cpp::die("CSR2BTCFNOBITMAP");
     btcf.rowOffset.assign(size_t(W) + 1, 0);
     btcf.tcA2B.assign(size_t(T) * COL_WINDOW, 0);
-    btcf.data.assign(size_t(T) * ROW_WINDOW * COL_WINDOW, MAT_VAL_TYPE(0));
+    btcf.data.assign(size_t(T) * ROW_WINDOW * COL_WINDOW, MAT_VAL_TYPE(0.0f));
     btcf.rowIdx.assign(W, 0);
 #ifdef SPARSE_A_TRANSPOSE
     const int transpose = 1;
@@ -210,8 +214,13 @@ inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX_NO_BITMAP &a, DENSE_MTX &dense_b, DEN
     return perf;
 }
 
-#ifdef USE_FP16
+#if defined(USE_FP16)
 inline PERF_RESULT fp16_spmm(BTCF_MTX_NO_BITMAP &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+{
+    return hspmm_cpp_spmm(btcf_a, dense_b, dense_c);
+}
+#elif defined(USE_BF16)
+inline PERF_RESULT bf16_spmm(BTCF_MTX_NO_BITMAP &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
 {
     return hspmm_cpp_spmm(btcf_a, dense_b, dense_c);
 }

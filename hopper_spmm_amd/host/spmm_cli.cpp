@@ -1,6 +1,7 @@
 // Command-line driver with the reference's arguments (reference src/fp16.cu:283-319):
 //   fp16_test <matrix_file> <feature_dim> [--seed S] [--verify]
-// built with -DUSE_FP16; the same source with -DUSE_TF32 gives tf32_test.
+// built with -DUSE_FP16; the same source with -DUSE_TF32 / -DUSE_BF16 gives
+// tf32_test / bf16_test.
 // B is filled with rand() / RAND_MAX as in the reference (src/fp16.cu:303-309);
 // --seed calls srand first (the reference never seeds, i.e. seed 1).  --verify
 // repeats the product with the library's scalar all-shapes kernel, a second
@@ -41,8 +42,10 @@ int main(int argc, char *argv[])
         dense_b.values[i] = MAT_VAL_TYPE(static_cast<float>(std::rand()) / static_cast<float>(RAND_MAX));
     DENSE_MTX dense_c{btcf.rows, feature_dim, new MAT_VAL_TYPE[size_t(btcf.rows) * feature_dim]};
 
-#ifdef USE_FP16
+#if defined(USE_FP16)
     PERF_RESULT perf = fp16_spmm(btcf, dense_b, dense_c);
+#elif defined(USE_BF16)
+    PERF_RESULT perf = bf16_spmm(btcf, dense_b, dense_c);
 #else
     PERF_RESULT perf = tf32_spmm(btcf, dense_b, dense_c);
 #endif

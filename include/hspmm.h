@@ -8,11 +8,12 @@
  *   tcA2B[T*CW]     column id of every tile column, IDX_MAX (0xFFFFFFFF) = padding
  *   data[T*8*CW]    dense 8 x CW tiles, row-major inside a tile
  *   rowIdx[W]       first matrix row of each effective window (multiple of 8)
- * with CW = 16 and 2-byte IEEE half values for HSPMM_FP16, CW = 8 and 4-byte
- * float values for HSPMM_TF32 (reference src/common.h:14-43).
+ * with CW = 16 and 2-byte values for HSPMM_FP16 (IEEE half) and HSPMM_BF16
+ * (bfloat16), CW = 8 and 4-byte float values for HSPMM_TF32 (reference
+ * src/common.h:14-43).
  * B is dense cols x N, C is dense rows x N, both row-major, same element type
  * as `data` (reference src/fp16.cu:36-46, 163-170).  Accumulation is fp32; the
- * fp16 path rounds once to nearest-even on store.
+ * 16-bit paths round once to nearest-even on store.
  *
  * All functions return 0 (HSPMM_OK) or a positive error code; the text of the
  * last error on the calling thread is available from hspmm_last_error().
@@ -30,6 +31,7 @@ extern "C" {
 
 #define HSPMM_FP16 0            /* reference -DUSE_FP16 build, src/common.h:14-19 */
 #define HSPMM_TF32 1            /* reference -DUSE_TF32 build, src/common.h:26-43 (fp32 storage) */
+#define HSPMM_BF16 2            /* reference -DUSE_BF16 build, src/common.h:20-25 (the reference has no bf16 program) */
 #define HSPMM_IDX_MAX 0xFFFFFFFFu   /* reference src/common.h:47 */
 #define HSPMM_ROW_WINDOW 8u         /* reference src/common.h:17 */
 
@@ -50,7 +52,7 @@ typedef struct hspmm_plan hspmm_plan;
  * src/fp16.cu:228-249) and create_tma_desc_A (src/fp16.cu:177-219): validates
  * the four format arrays (host pointers), copies them to the current HIP
  * device and builds the work partition the kernels walk.  `dtype` is
- * HSPMM_FP16 or HSPMM_TF32. */
+ * HSPMM_FP16, HSPMM_TF32 or HSPMM_BF16. */
 int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
                  uint32_t eff_row_windows, uint32_t total_tiles,
                  const uint32_t *rowOffset, const uint32_t *tcA2B,

@@ -12,6 +12,7 @@
  *
  * Parity status of each function (what pins it):
  *   orc_f32_to_f16 / orc_f16_to_f32  exhaustive comparison with numpy float16
+ *   orc_f32_to_bf16 / orc_bf16_to_f32 comparison with torch.bfloat16 (CPU), all 65536 patterns back
  *   orc_mtx_read                     reference-produced golden vectors (tiny.mtx,
  *                                    gap.mtx), scipy COO->CSR cross-check
  *   orc_btcf_count / orc_btcf_fill   the same golden vectors, round-trip to CSR,
@@ -88,6 +89,25 @@ float orc_f16_to_f32(uint16_t h)
     return f;
 }
 
+/* float <-> bfloat16 (round to nearest even), the implicit conversions of the
+ * reference's bf16 build (MAT_VAL_TYPE __nv_bfloat16, src/common.h:20-25; value
+ * assignment at src/utils/load.h:224). */
+uint16_t orc_f32_to_bf16(float f)
+{
+    uint32_t x; memcpy(&x, &f, 4);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    uint32_t lsb = (x >> 16) & 1u;
+    return (uint16_t)((x + 0x7FFFu + lsb) >> 16);
+}
+float orc_bf16_to_f32(uint16_t h)
+{
+    uint32_t x = (uint32_t)h << 16; float f; memcpy(&f, &x, 4); return f;
+}
+void orc_f32_to_bf16_array(const float *src, uint16_t *dst, size_t n)
+{ for (size_t i = 0; i < n; ++i) dst[i] = orc_f32_to_bf16(src[i]); }
+void orc_bf16_to_f32_array(const uint16_t *src, float *dst, size_t n)
+{ for (size_t i = 0; i < n; ++i) dst[i] = orc_bf16_to_f32(src[i]); }
+
 void orc_f32_to_f16_array(const float *src, uint16_t *dst, size_t n)
 { for (size_t i = 0; i < n; ++i) dst[i] = orc_f32_to_f16(src[i]); }
 
@@ -119,10 +139,12 @@ static int orc_key_cmp(const void *a, const void *b)
     return x->seq < y->seq ? -1 : (x->seq > y->seq);
 }
 
-/* elem_size: 2 = fp16 build (USE_FP16, value rounded with RN, load.h:226),
- *            4 = fp32 storage (USE_TF32, value kept as parsed, load.h:224). */
-orc_csr *orc_mtx_read(const char *path, int elem_size)
+/* kind: 2 = fp16 build (USE_FP16, value rounded with RN, load.h:226),
+ *       4 = fp32 storage (USE_TF32, value kept as parsed, load.h:224),
+ *       3 = bf16 build (USE_BF16, value rounded with RN by the assignment, load.h:224). */
+orc_csr *orc_mtx_read(const char *path, int kind)
 {
+    const int elem_size = kind == 4 ? 4 : 2;
     orc_csr *m = (orc_csr *)calloc(1, sizeof(orc_csr));
     if (!m) return NULL;
     FILE *f = fopen(path, "r");
@@ -167,7 +189,8 @@ orc_csr *orc_mtx_read(const char *path, int elem_size)
     for (uint32_t i = 0; i < nnz; ++i) {                               /* load.h:284-300 */
         uint32_t s = keys[i].seq;
         m->col_idx[i] = ci[s];
-        if (elem_size == 2) ((uint16_t *)m->values)[i] = orc_f32_to_f16(vf[s]);
+        if (kind == 2) ((uint16_t *)m->values)[i] = orc_f32_to_f16(vf[s]);
+        else if (kind == 3) ((uint16_t *)m->values)[i] = orc_f32_to_bf16(vf[s]);
         else                ((float *)m->values)[i] = vf[s];
         m->row_ptr[ri[s] + 1]++;
     }
@@ -288,8 +311,20 @@ int orc_max_threads(void) { return orc_threads(0); }
 
 /* C[rows x N] (fp16) = A_csr (fp16) * B[cols x N] (fp16).  absdot, when not NULL,
  * receives sum_k |a||b| per output (fp32) for error bounds in tests. */
+static void orc_spmm_csr_16(int bf, uint32_t rows, uint32_t N, const uint32_t *row_ptr, const uint32_t *col_idx,
+                            const uint16_t *vals, const uint16_t *B, uint16_t *C, float *absdot, int nthreads);
+
 void orc_spmm_csr_f16(uint32_t rows, uint32_t N, const uint32_t *row_ptr, const uint32_t *col_idx,
                       const uint16_t *vals, const uint16_t *B, uint16_t *C, float *absdot, int nthreads)
+{ orc_spmm_csr_16(0, rows, N, row_ptr, col_idx, vals, B, C, absdot, nthreads); }
+
+/* Same arithmetic with bfloat16 storage (the reference's -DUSE_BF16 types). */
+void orc_spmm_csr_bf16(uint32_t rows, uint32_t N, const uint32_t *row_ptr, const uint32_t *col_idx,
+                       const uint16_t *vals, const uint16_t *B, uint16_t *C, float *absdot, int nthreads)
+{ orc_spmm_csr_16(1, rows, N, row_ptr, col_idx, vals, B, C, absdot, nthreads); }
+
+static void orc_spmm_csr_16(int bf, uint32_t rows, uint32_t N, const uint32_t *row_ptr, const uint32_t *col_idx,
+                            const uint16_t *vals, const uint16_t *B, uint16_t *C, float *absdot, int nthreads)
 {
     int nt = orc_threads(nthreads); (void)nt;
     #pragma omp parallel num_threads(nt)
@@ -300,14 +335,15 @@ void orc_spmm_csr_f16(uint32_t rows, uint32_t N, const uint32_t *row_ptr, const 
         for (int64_t r = 0; r < (int64_t)rows; ++r) {
             for (uint32_t j = 0; j < N; ++j) { acc[j] = 0.0f; mag[j] = 0.0f; }
             for (uint32_t id = row_ptr[r]; id < row_ptr[r + 1]; ++id) {
-                float a = orc_f16_to_f32(vals[id]);
+                float a = bf ? orc_bf16_to_f32(vals[id]) : orc_f16_to_f32(vals[id]);
                 const uint16_t *b = B + (size_t)col_idx[id] * N;
                 if (absdot) for (uint32_t j = 0; j < N; ++j) {
-                    float p = a * orc_f16_to_f32(b[j]); acc[j] += p; mag[j] += fabsf(p);
-                } else for (uint32_t j = 0; j < N; ++j) acc[j] += a * orc_f16_to_f32(b[j]);
+                    float p = a * (bf ? orc_bf16_to_f32(b[j]) : orc_f16_to_f32(b[j])); acc[j] += p; mag[j] += fabsf(p);
+                } else if (bf) for (uint32_t j = 0; j < N; ++j) acc[j] += a * orc_bf16_to_f32(b[j]);
+                else for (uint32_t j = 0; j < N; ++j) acc[j] += a * orc_f16_to_f32(b[j]);
             }
             uint16_t *c = C + (size_t)r * N;
-            for (uint32_t j = 0; j < N; ++j) c[j] = orc_f32_to_f16(acc[j]);
+            for (uint32_t j = 0; j < N; ++j) c[j] = bf ? orc_f32_to_bf16(acc[j]) : orc_f32_to_f16(acc[j]);
             if (absdot) memcpy(absdot + (size_t)r * N, mag, (size_t)N * 4);
         }
         free(acc);
@@ -349,9 +385,21 @@ void orc_spmm_csr_f32(uint32_t rows, uint32_t N, const uint32_t *row_ptr, const 
  * data[t][r][k] * B[tcA2B[t][k]][:] in fp32; C[rowIdx[w]+r][:] = RN16(acc).
  * Rows outside every effective window, and nothing beyond `rows`, are written
  * as zero (the reference leaves them uninitialised; zero is the SpMM value). */
+static void orc_spmm_btcf_16(int bf, uint32_t rows, uint32_t N, uint32_t eff_windows,
+                             const uint32_t *rowOffset, const uint32_t *tcA2B, const uint16_t *data,
+                             const uint32_t *rowIdx, const uint16_t *B, uint16_t *C);
 void orc_spmm_btcf_f16(uint32_t rows, uint32_t N, uint32_t eff_windows,
                        const uint32_t *rowOffset, const uint32_t *tcA2B, const uint16_t *data,
                        const uint32_t *rowIdx, const uint16_t *B, uint16_t *C)
+{ orc_spmm_btcf_16(0, rows, N, eff_windows, rowOffset, tcA2B, data, rowIdx, B, C); }
+void orc_spmm_btcf_bf16(uint32_t rows, uint32_t N, uint32_t eff_windows,
+                        const uint32_t *rowOffset, const uint32_t *tcA2B, const uint16_t *data,
+                        const uint32_t *rowIdx, const uint16_t *B, uint16_t *C)
+{ orc_spmm_btcf_16(1, rows, N, eff_windows, rowOffset, tcA2B, data, rowIdx, B, C); }
+
+static void orc_spmm_btcf_16(int bf, uint32_t rows, uint32_t N, uint32_t eff_windows,
+                             const uint32_t *rowOffset, const uint32_t *tcA2B, const uint16_t *data,
+                             const uint32_t *rowIdx, const uint16_t *B, uint16_t *C)
 {
     const uint32_t cw = 16;
     memset(C, 0, (size_t)rows * N * 2);
@@ -364,14 +412,17 @@ void orc_spmm_btcf_f16(uint32_t rows, uint32_t N, uint32_t eff_windows,
                 if (col == ORC_IDX_MAX) continue;
                 const uint16_t *b = B + (size_t)col * N;
                 for (uint32_t r = 0; r < ORC_ROW_WINDOW; ++r) {
-                    float a = orc_f16_to_f32(data[((size_t)t * ORC_ROW_WINDOW + r) * cw + k]);
+                    uint16_t ab = data[((size_t)t * ORC_ROW_WINDOW + r) * cw + k];
+                    float a = bf ? orc_bf16_to_f32(ab) : orc_f16_to_f32(ab);
                     float *ar = acc + (size_t)r * N;
-                    for (uint32_t j = 0; j < N; ++j) ar[j] += a * orc_f16_to_f32(b[j]);
+                    if (bf) for (uint32_t j = 0; j < N; ++j) ar[j] += a * orc_bf16_to_f32(b[j]);
+                    else for (uint32_t j = 0; j < N; ++j) ar[j] += a * orc_f16_to_f32(b[j]);
                 }
             }
         for (uint32_t r = 0; r < ORC_ROW_WINDOW && rowIdx[w] + r < rows; ++r)
             for (uint32_t j = 0; j < N; ++j)
-                C[(size_t)(rowIdx[w] + r) * N + j] = orc_f32_to_f16(acc[(size_t)r * N + j]);
+                C[(size_t)(rowIdx[w] + r) * N + j] = bf ? orc_f32_to_bf16(acc[(size_t)r * N + j])
+                                                        : orc_f32_to_f16(acc[(size_t)r * N + j]);
     }
     free(acc);
 }

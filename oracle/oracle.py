@@ -75,12 +75,26 @@ def f16_bits_to_f32(h):
     return out
 
 
+def f32_to_bf16_bits(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().orc_f32_to_bf16_array(_p(x), _p(out), C.c_size_t(x.size))
+    return out
+
+
+def bf16_bits_to_f32(h):
+    h = _c(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().orc_bf16_to_f32_array(_p(h), _p(out), C.c_size_t(h.size))
+    return out
+
+
 def mtx_read(path, dtype):
-    """dtype 'fp16' -> values as uint16 bit patterns; 'tf32' -> float32.
+    """dtype 'fp16' / 'bf16' -> values as uint16 bit patterns; 'tf32' -> float32.
     Returns dict(rows, cols, nnzs, declared_nnz, row_ptr, col_idx, values) or
     raises OSError / ValueError following the oracle's status code."""
-    es = 2 if dtype == "fp16" else 4
-    m = lib().orc_mtx_read(os.fsencode(path), es)
+    es = 4 if dtype == "tf32" else 2
+    m = lib().orc_mtx_read(os.fsencode(path), {"fp16": 2, "bf16": 3, "tf32": 4}[dtype])
     try:
         s = m.contents
         if s.status == 1:
@@ -112,9 +126,9 @@ def csr_validate(rows, cols, row_ptr, col_idx):
 
 def csr_to_btcf(rows, cols, row_ptr, col_idx, values, dtype, transpose=False, cw=None):
     """CSR -> condensed tiles (no bitmap).  values: uint16 bits (fp16) or float32 (tf32)."""
-    es = 2 if dtype == "fp16" else 4
+    es = 4 if dtype == "tf32" else 2
     if cw is None:
-        cw = 16 if dtype == "fp16" else 8
+        cw = 8 if dtype == "tf32" else 16
     vt = np.uint16 if es == 2 else np.float32
     row_ptr = _c(row_ptr, np.uint32)
     col_idx = _c(col_idx, np.uint32)
@@ -149,6 +163,18 @@ def spmm_csr_f16(rows, N, row_ptr, col_idx, vals_bits, B_bits, want_absdot=False
     return (Cm, mag) if want_absdot else Cm
 
 
+def spmm_csr_bf16(rows, N, row_ptr, col_idx, vals_bits, B_bits, want_absdot=False, threads=0):
+    row_ptr = _c(row_ptr, np.uint32)
+    col_idx = _c(col_idx, np.uint32)
+    vals_bits = _c(vals_bits, np.uint16)
+    B_bits = _c(B_bits, np.uint16)
+    Cm = np.empty((rows, N), np.uint16)
+    mag = np.empty((rows, N), np.float32) if want_absdot else None
+    lib().orc_spmm_csr_bf16(C.c_uint32(rows), C.c_uint32(N), _p(row_ptr), _p(col_idx), _p(vals_bits),
+                            _p(B_bits), _p(Cm), _p(mag) if want_absdot else None, C.c_int(threads))
+    return (Cm, mag) if want_absdot else Cm
+
+
 def spmm_csr_f32(rows, N, row_ptr, col_idx, vals, B, want_absdot=False, trunc_tf32=False, threads=0):
     row_ptr = _c(row_ptr, np.uint32)
     col_idx = _c(col_idx, np.uint32)
@@ -165,11 +191,12 @@ def spmm_csr_f32(rows, N, row_ptr, col_idx, vals, B, want_absdot=False, trunc_tf
 def spmm_btcf(btcf, B, N):
     """Tile-order SpMM on a dict as returned by csr_to_btcf (row-major tiles only)."""
     rows, W = btcf["rows"], btcf["eff_row_windows"]
-    if btcf["dtype"] == "fp16":
+    if btcf["dtype"] in ("fp16", "bf16"):
         assert btcf["cw"] == 16
         B = _c(B, np.uint16)
         Cm = np.empty((rows, N), np.uint16)
-        lib().orc_spmm_btcf_f16(C.c_uint32(rows), C.c_uint32(N), C.c_uint32(W), _p(btcf["rowOffset"]),
+        fn = lib().orc_spmm_btcf_f16 if btcf["dtype"] == "fp16" else lib().orc_spmm_btcf_bf16
+        fn(C.c_uint32(rows), C.c_uint32(N), C.c_uint32(W), _p(btcf["rowOffset"]),
                                 _p(btcf["tcA2B"]), _p(btcf["data"]), _p(btcf["rowIdx"]), _p(B), _p(Cm))
     else:
         B = _c(B, np.float32)

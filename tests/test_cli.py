@@ -44,7 +44,7 @@ def test_cli_end_to_end_with_verification(hs, tmp_path):
         f.write("%%MatrixMarket matrix coordinate real general\n%d %d %d\n" % (rows, cols, nnz))
         for k in flat:
             f.write("%d %d %.6g\n" % (k // cols + 1, k % cols + 1, rng.normal()))
-    for name, n in (("fp16_test", "128"), ("fp16_test", "7"), ("tf32_test", "64")):
+    for name, n in (("fp16_test", "128"), ("fp16_test", "7"), ("tf32_test", "64"), ("bf16_test", "128"), ("bf16_test", "5")):
         r = run(hs, name, str(p), n, "--seed", "42", "--verify")
         assert r.returncode == 0, r.stdout + r.stderr
         assert "verification passed" in r.stdout

@@ -10,7 +10,7 @@ import pytest
 from util import random_csr
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-DT = {0: "fp16", 1: "tf32"}
+DT = {0: "fp16", 1: "tf32", 2: "bf16"}
 
 
 def _same_btcf(a, b):
@@ -43,7 +43,7 @@ def test_golden_vectors_through_the_library(hs):
             assert np.array_equal(b["data"].view(np.float16).astype(np.float32).reshape(want.shape), want)
 
 
-@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("dtype", [0, 1, 2])
 def test_loader_equals_oracle(hs, oracle, tmp_path, dtype):
     rng = np.random.default_rng(100 + dtype)
     for case in range(6):
@@ -98,7 +98,7 @@ def test_loader_errors(hs, tmp_path):
         hs.mtx_load(str(oob), 7)
 
 
-@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("dtype", [0, 1, 2])
 def test_converter_equals_oracle(hs, oracle, dtype):
     rng = np.random.default_rng(200 + dtype)
     shapes = [(1, 1, 1.0, 0.0), (8, 16, 0.5, 0.0), (9, 17, 0.5, 0.0), (27, 12, 0.1, 0.7), (64, 500, 0.05, 0.3),

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import scipy.sparse as sp
 
-from util import IDX_MAX, btcf_to_csr, csr_to_dense64, csr_triples, random_csr
+from util import IDX_MAX, btcf_to_csr, csr_to_dense64, csr_triples, decode, dtype_name, encode, random_csr
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
@@ -47,6 +47,27 @@ def test_float_to_half_against_numpy(oracle):
         want = x.astype(np.float16).view(np.uint16)
     assert np.array_equal(got, want)
     assert np.isnan(oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(np.array([np.nan], np.float32))))[0]
+
+
+def test_bfloat16_conversions_against_torch(oracle):
+    import torch
+    bits = np.arange(65536, dtype=np.uint16)
+    got = oracle.bf16_bits_to_f32(bits)
+    want = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16).to(torch.float32).numpy()
+    assert got.tobytes() == want.tobytes()                      # NaN payloads included
+    rng = np.random.default_rng(8)
+    f = bits.astype(np.uint32) << 16
+    # every bf16 value, the exact midpoints to the next one (ties), their neighbours, random patterns
+    cases = [f, f | 0x8000, f | 0x7FFF, f | 0x8001, rng.integers(0, 2 ** 32, 300000, dtype=np.uint64).astype(np.uint32)]
+    x = np.concatenate(cases).astype(np.uint32).view(np.float32)
+    x = x[~np.isnan(x)]
+    got = oracle.f32_to_bf16_bits(x)
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+    assert np.isnan(oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(np.array([np.nan], np.float32))))[0]
+    # the benchmark generator's own conversion agrees as well
+    from hopper_spmm_amd import generators as G
+    assert np.array_equal(G.bf16_bits(x), want)
 
 
 # ---------------------------------------------------------------- loader
@@ -259,17 +280,14 @@ def test_spmm_exact_integer_case(oracle):
         assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("dtype", [0, 1, 2])
 def test_spmm_against_dense_float64(oracle, dtype):
     rng = np.random.default_rng(31 + dtype)
     rows, cols, N = 50, 70, 24
     A = random_csr(rng, rows, cols, 0.2, dtype, 0.2)
     Bf = rng.normal(size=(cols, N)).astype(np.float32)
-    if dtype == 0:
-        B = Bf.astype(np.float16).view(np.uint16)
-        B64 = B.view(np.float16).astype(np.float64)
-    else:
-        B, B64 = Bf, Bf.astype(np.float64)
+    B = encode(Bf, dtype)
+    B64 = decode(B, dtype)
     exact = csr_to_dense64(A) @ B64
     mag = np.abs(csr_to_dense64(A)) @ np.abs(B64)
     if dtype == 0:
@@ -277,14 +295,19 @@ def test_spmm_against_dense_float64(oracle, dtype):
         got = C.view(np.float16).astype(np.float64)
         # one fp16 rounding of an fp32 sum: half an ulp of the result plus fp32 noise
         assert np.all(np.abs(got - exact) <= np.abs(exact) * 2.0 ** -11 + mag * 1e-6 + 1e-7)
+    elif dtype == 2:
+        C, absdot = oracle.spmm_csr_bf16(rows, N, A["row_ptr"], A["col_idx"], A["values"], B, want_absdot=True)
+        got = decode(C, 2)
+        # one bf16 rounding (8 significant bits: half an ulp is at most 2^-8 relative) of an fp32 sum
+        assert np.all(np.abs(got - exact) <= np.abs(exact) * 2.0 ** -8 + mag * 1e-6 + 1e-30)
     else:
         C, absdot = oracle.spmm_csr_f32(rows, N, A["row_ptr"], A["col_idx"], A["values"], B, want_absdot=True)
         assert np.all(np.abs(C - exact) <= mag * 1e-6)
     assert np.allclose(absdot, mag, rtol=1e-5, atol=1e-7)
     # tile order and CSR order agree to reassociation error (identical here: both go k ascending)
-    b = oracle.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], "fp16" if dtype == 0 else "tf32")
+    b = oracle.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype_name(dtype))
     Ct = oracle.spmm_btcf(b, B, N)
-    if dtype == 0:
+    if dtype != 1:
         assert np.array_equal(Ct, C)
     else:
         assert np.allclose(Ct, C, rtol=1e-6, atol=1e-6)

@@ -4,6 +4,7 @@ oracle on the same seeded inputs.  Needs a real MI355X: run with -m gpu.
 Tolerances (from the task's statement of parity):
   fp16 path : |gpu - ref| <= 1e-2 * |ref| + 1e-5 * sum_k |a_k b_k|
   tf32 path : |gpu - ref| <= 1e-3 * |ref| + 1e-5 * sum_k |a_k b_k|
+  bf16 path : the fp16 bound (one bf16 rounding is 2^-9 relative)
 The second term only matters where a sum cancels to (almost) nothing; it is the
 size of fp32 reassociation noise.  Index handling is checked bit-exactly through
 cases whose arithmetic is exact (small integers) and through the format tests.
@@ -13,11 +14,11 @@ import os
 import numpy as np
 import pytest
 
-from util import csr_to_dense64, half_ulp_distance, random_csr
+from util import csr_to_dense64, decode, encode, half_ulp_distance, random_csr
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-DT = {0: "fp16", 1: "tf32"}
+DT = {0: "fp16", 1: "tf32", 2: "bf16"}
 
 
 @pytest.fixture(scope="module")
@@ -34,7 +35,7 @@ def gpu_spmm(torch, hs, btcf, B, N, plan=None, poison=True):
         plan = hs.Plan(btcf)
     dt = btcf["dtype"]
     rows = btcf["rows"]
-    if dt == 0:
+    if dt != 1:
         dB = torch.from_numpy(np.ascontiguousarray(B, np.uint16).view(np.int16)).cuda()
         dC = torch.empty((rows, N), dtype=torch.int16, device="cuda")
         if poison:
@@ -50,20 +51,20 @@ def gpu_spmm(torch, hs, btcf, B, N, plan=None, poison=True):
     out = dC.cpu().numpy()
     if own:
         plan.close()
-    return out.view(np.uint16) if dt == 0 else out
+    return out.view(np.uint16) if dt != 1 else out
 
 
 def oracle_spmm(oracle, A, B, N):
+    if A["dtype"] == 2:
+        return oracle.spmm_csr_bf16(A["rows"], N, A["row_ptr"], A["col_idx"], A["values"], B, want_absdot=True)
     if A["dtype"] == 0:
         return oracle.spmm_csr_f16(A["rows"], N, A["row_ptr"], A["col_idx"], A["values"], B, want_absdot=True)
     return oracle.spmm_csr_f32(A["rows"], N, A["row_ptr"], A["col_idx"], A["values"], B, want_absdot=True)
 
 
 def assert_parity(got, ref, absdot, dtype, what=""):
-    if dtype == 0:
-        g = got.view(np.float16).astype(np.float64)
-        r = ref.view(np.float16).astype(np.float64)
-        rel = 1e-2
+    if dtype != 1:
+        g, r, rel = decode(got, dtype), decode(ref, dtype), 1e-2
     else:
         g, r, rel = got.astype(np.float64), ref.astype(np.float64), 1e-3
     assert not np.isnan(g).any(), what + ": unwritten or NaN output"
@@ -72,15 +73,15 @@ def assert_parity(got, ref, absdot, dtype, what=""):
     bad = err > bound
     assert not bad.any(), "%s: %d of %d outputs outside tolerance, worst %g at %s" % (
         what, int(bad.sum()), bad.size, float((err - bound).max()), np.unravel_index(np.argmax(err - bound), err.shape))
-    if dtype == 0 and got.size:
-        # far tighter in practice: fp16 rounding of nearly identical fp32 sums
+    if dtype != 1 and got.size:
+        # far tighter in practice: one rounding of nearly identical fp32 sums
         ulp = half_ulp_distance(got, ref)
         assert (ulp <= 1).mean() > 0.999, what + ": too many outputs differ by more than one half ulp"
 
 
 def make_b(rng, cols, N, dtype):
     x = rng.normal(size=(cols, N)).astype(np.float32)
-    return x.astype(np.float16).view(np.uint16) if dtype == 0 else x
+    return encode(x, dtype)
 
 
 def convert(hs, A):
@@ -107,7 +108,7 @@ def test_golden_files_end_to_end(torch_cuda, hs, oracle):
 
 
 # ------------------------------------------------------------------ exact arithmetic: bit-exact
-@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("dtype", [0, 1, 2])
 @pytest.mark.parametrize("mode", [0, 1, 2, 3])
 def test_exact_integer_inputs_are_bit_exact(torch_cuda, hs, oracle, dtype, mode):
     rng = np.random.default_rng(40 + dtype)
@@ -122,17 +123,20 @@ def test_exact_integer_inputs_are_bit_exact(torch_cuda, hs, oracle, dtype, mode)
         rp[r + 1] = len(ci)
     vals = np.array(vv, np.float32)
     A = dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=np.array(ci, np.uint32),
-             values=vals.astype(np.float16).view(np.uint16) if dtype == 0 else vals)
+             values=encode(vals, dtype))
     hs.set_kernel_mode(mode)
     try:
         b = convert(hs, A)
         for N in (4, 32, 64, 128, 160):
             Bm = rng.integers(-4, 5, (cols, N))
-            B = Bm.astype(np.float16).view(np.uint16) if dtype == 0 else Bm.astype(np.float32)
+            B = encode(Bm, dtype)
             got = gpu_spmm(torch_cuda, hs, b, B, N)
-            want = D @ Bm
-            g = got.view(np.float16).astype(np.int64) if dtype == 0 else got.astype(np.int64)
-            assert np.array_equal(g, want), "mode %d N %d" % (mode, N)
+            # the sums are exact in fp32, so the output is the one rounding of the
+            # exact integer result to the storage type
+            want = encode(D @ Bm, dtype)
+            assert np.array_equal(got, want), "mode %d N %d" % (mode, N)
+            if dtype != 2:
+                assert np.array_equal(decode(got, dtype).astype(np.int64), D @ Bm)
     finally:
         hs.set_kernel_mode(0)
 
@@ -150,7 +154,7 @@ SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("dtype", [0, 1, 2])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_random_shapes_and_feature_dims(torch_cuda, hs, oracle, dtype, shape):
     rows, cols, dens, erp, heavy = shape
@@ -173,7 +177,7 @@ def test_random_shapes_and_feature_dims(torch_cuda, hs, oracle, dtype, shape):
     plan.close()
 
 
-@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("dtype", [0, 1, 2])
 @pytest.mark.parametrize("mode", [1, 2, 3])
 @pytest.mark.parametrize("stages", [1, 2, 4, 6, 8])
 def test_kernel_variants_agree_with_oracle(torch_cuda, hs, oracle, dtype, mode, stages):
@@ -216,10 +220,10 @@ def _block_matrix(rng, rows, cols, brows, bcols, keep, dtype, break_some=False):
         rp[r + 1] = len(ci)
     vals = np.array(vv, np.float32)
     return dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=np.array(ci, np.uint32),
-                values=vals.astype(np.float16).view(np.uint16) if dtype == 0 else vals)
+                values=encode(vals, dtype))
 
 
-@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("dtype", [0, 1, 2])
 @pytest.mark.parametrize("case", ["blocks16", "blocks32", "mixed", "ragged"])
 def test_windows_with_one_column_list_share_their_gather(torch_cuda, hs, oracle, dtype, case):
     rng = np.random.default_rng(60 + dtype)
@@ -256,18 +260,19 @@ def test_windows_with_one_column_list_share_their_gather(torch_cuda, hs, oracle,
 
 def test_unaligned_and_odd_feature_dims_use_the_all_shapes_kernel(torch_cuda, hs, oracle):
     rng = np.random.default_rng(5)
-    A = random_csr(rng, 90, 120, 0.1, 0, 0.2)
-    b = convert(hs, A)
-    for N in (1, 3, 7, 33, 129):
-        B = make_b(rng, 120, N, 0)
-        got = gpu_spmm(torch_cuda, hs, b, B, N)
-        ref, mag = oracle_spmm(oracle, A, B, N)
-        assert_parity(got, ref, mag, 0, "odd N=%d" % N)
+    for dt in (0, 2):
+        A = random_csr(rng, 90, 120, 0.1, dt, 0.2)
+        b = convert(hs, A)
+        for N in (1, 3, 7, 33, 129):
+            B = make_b(rng, 120, N, dt)
+            got = gpu_spmm(torch_cuda, hs, b, B, N)
+            ref, mag = oracle_spmm(oracle, A, B, N)
+            assert_parity(got, ref, mag, dt, "%s odd N=%d" % (DT[dt], N))
 
 
 def test_matrix_without_entries_gives_zeros(torch_cuda, hs):
-    for dt in (0, 1):
-        vt = np.uint16 if dt == 0 else np.float32
+    for dt in (0, 1, 2):
+        vt = np.float32 if dt == 1 else np.uint16
         b = hs.csr_to_btcf(21, 9, np.zeros(22, np.uint32), np.zeros(0, np.uint32), np.zeros(0, vt), dt)
         for N in (1, 5, 64):
             got = gpu_spmm(torch_cuda, hs, b, np.ones((9, N), vt), N)

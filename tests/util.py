@@ -5,11 +5,33 @@ IDX_MAX = 0xFFFFFFFF
 
 
 def dtype_name(dtype):
-    return "fp16" if dtype == 0 else "tf32"
+    return {0: "fp16", 1: "tf32", 2: "bf16"}[dtype]
+
+
+def encode(x, dtype):
+    """float values -> storage of dtype: uint16 bits (fp16 = 0, bf16 = 2) or float32 (1).
+    bf16 goes through torch's CPU conversion, which is independent of both the
+    library's and the oracle's."""
+    x = np.ascontiguousarray(x, np.float32)
+    if dtype == 0:
+        return x.astype(np.float16).view(np.uint16)
+    if dtype == 2:
+        import torch
+        return torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    return x
+
+
+def decode(v, dtype):
+    """storage of dtype -> float64."""
+    if dtype == 0:
+        return np.ascontiguousarray(v).view(np.float16).astype(np.float64)
+    if dtype == 2:
+        return (np.ascontiguousarray(v).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    return np.asarray(v).astype(np.float64)
 
 
 def random_csr(rng, rows, cols, density, dtype, empty_row_prob=0.0, heavy_rows=()):
-    """Duplicate-free random CSR; values are fp16 bit patterns or float32."""
+    """Duplicate-free random CSR; values are fp16 / bf16 bit patterns or float32."""
     row_lists = []
     for r in range(rows):
         if r in heavy_rows:
@@ -24,14 +46,14 @@ def random_csr(rng, rows, cols, density, dtype, empty_row_prob=0.0, heavy_rows=(
     row_ptr[1:] = np.cumsum([len(c) for c in row_lists])
     col_idx = np.concatenate(row_lists).astype(np.uint32) if rows else np.zeros(0, np.uint32)
     v = rng.uniform(-1, 1, col_idx.size).astype(np.float32)
-    vals = v.astype(np.float16).view(np.uint16) if dtype == 0 else v
+    vals = encode(v, dtype)
     return dict(rows=rows, cols=cols, nnzs=int(col_idx.size), dtype=dtype, row_ptr=row_ptr,
                 col_idx=col_idx, values=vals)
 
 
 def csr_to_dense64(A):
-    """Dense float64 copy of a CSR dict (fp16 bits are decoded with numpy)."""
-    vals = A["values"].view(np.float16).astype(np.float64) if A["dtype"] == 0 else A["values"].astype(np.float64)
+    """Dense float64 copy of a CSR dict."""
+    vals = decode(A["values"], A["dtype"])
     D = np.zeros((A["rows"], A["cols"]), np.float64)
     rp = A["row_ptr"]
     for r in range(A["rows"]):
@@ -70,7 +92,8 @@ def csr_triples(A):
 
 
 def half_ulp_distance(a_bits, b_bits):
-    """Distance in units of the last place between two arrays of half bit patterns."""
+    """Distance in units of the last place between two arrays of 16-bit float bit
+    patterns (fp16 or bf16: sign-magnitude ordering holds for both)."""
     def key(x):
         x = x.astype(np.int32)
         return np.where(x & 0x8000, -(x & 0x7FFF), x & 0x7FFF)
