@@ -102,6 +102,13 @@ def load_library():
     L.hspmm_csr_free.restype = None
     L.hspmm_btcf_sizes.argtypes = [i, u32, vp, vp, C.POINTER(u32), C.POINTER(u32)]
     L.hspmm_btcf_fill.argtypes = [i, u32, vp, vp, vp, i, vp, vp, vp, vp]
+    L.hspmm_bitmap_sizes.argtypes = [i, u32, vp, vp, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
+    L.hspmm_bitmap_fill.argtypes = [i, u32, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp]
+    L.hspmm_bitmap_expand.argtypes = [i, u32, vp, vp, vp, vp]
+    L.hspmm_create_bitmap.argtypes = [C.POINTER(vp), i, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp]
+    L.hspmm_group_sizes.argtypes = [u32, vp, u32, C.POINTER(u32), C.POINTER(u32)]
+    L.hspmm_group_fill.argtypes = [u32, vp, vp, u32, vp, vp, vp]
+    L.hspmm_create_grouped.argtypes = [C.POINTER(vp), i, u32, u32, u32, vp, vp, vp, vp, vp, vp, vp]
     _lib = L
     return L
 
@@ -186,6 +193,81 @@ def csr_to_btcf(rows, cols, row_ptr, col_idx, values, dtype, transpose=False):
                 total_tiles=T, rowOffset=rowOffset, tcA2B=tcA2B, data=data, rowIdx=rowIdx)
 
 
+BITS_PER_TILE = 0       # HSPMM_BITS_PER_TILE: every tile owns its bitmap words
+BITS_AS_REFERENCE = 1   # HSPMM_BITS_AS_REFERENCE: word index as written in src/utils/convert.h:96-101
+
+
+def csr_to_bitmap(rows, cols, row_ptr, col_idx, values, dtype, transpose=False, bit_layout=BITS_PER_TILE):
+    """CSR2BTCF of the reference (src/utils/convert.h:22): returns the BTCF_MTX
+    fields (src/utils/class.h:55-67) as a dict of numpy arrays."""
+    L = load_library()
+    vt = _val_dtype(dtype)
+    cw = 8 if dtype == TF32 else 16
+    words = 1 if dtype == TF32 else 2
+    row_ptr = np.ascontiguousarray(row_ptr, np.uint32)
+    col_idx = np.ascontiguousarray(col_idx, np.uint32)
+    values = np.ascontiguousarray(values, vt)
+    if row_ptr.size != rows + 1:
+        raise ValueError("row_ptr must have rows + 1 entries")
+    W, T, S = C.c_uint32(), C.c_uint32(), C.c_uint32()
+    _check(L.hspmm_bitmap_sizes(dtype, rows, _p(row_ptr), _p(col_idx), C.byref(W), C.byref(T), C.byref(S)))
+    W, T, S = W.value, T.value, S.value
+    rowOffset = np.zeros(W + 1, np.uint32)
+    nnzOffset = np.zeros(T + 1, np.uint32)
+    tcA2B = np.empty(T * cw, np.uint32)
+    tcBit = np.empty(T * words, np.uint64)
+    data = np.empty(S, vt)
+    rowIdx = np.empty(W, np.uint32)
+    _check(L.hspmm_bitmap_fill(dtype, rows, _p(row_ptr), _p(col_idx), _p(values), int(transpose), int(bit_layout),
+                               rowOffset.ctypes.data_as(C.c_void_p), nnzOffset.ctypes.data_as(C.c_void_p),
+                               _p(tcA2B), _p(tcBit), _p(data), _p(rowIdx)))
+    return dict(rows=rows, cols=cols, nnzs=int(col_idx.size), dtype=dtype, cw=cw,
+                total_row_windows=(rows + ROW_WINDOW - 1) // ROW_WINDOW, eff_row_windows=W,
+                total_tiles=T, rowOffset=rowOffset, nnzOffset=nnzOffset, tcA2B=tcA2B, tcBit=tcBit,
+                data=data, rowIdx=rowIdx)
+
+
+def bitmap_expand(bitmap):
+    """Bitmap tiles -> the dense tiles of the uncompressed format (a BTCF_MTX_NO_BITMAP dict)."""
+    L = load_library()
+    dtype = bitmap["dtype"]
+    vt = _val_dtype(dtype)
+    cw = 8 if dtype == TF32 else 16
+    T = int(bitmap["total_tiles"])
+    nnzOffset = np.ascontiguousarray(bitmap["nnzOffset"], np.uint32)
+    tcBit = np.ascontiguousarray(bitmap["tcBit"], np.uint64)
+    packed = np.ascontiguousarray(bitmap["data"], vt)
+    dense = np.empty(T * ROW_WINDOW * cw, vt)
+    _check(L.hspmm_bitmap_expand(dtype, T, _p(nnzOffset), _p(tcBit), _p(packed), _p(dense)))
+    out = {k: bitmap[k] for k in ("rows", "cols", "nnzs", "dtype", "total_row_windows", "eff_row_windows",
+                                  "total_tiles", "rowOffset", "tcA2B", "rowIdx")}
+    out["cw"] = cw
+    out["data"] = dense
+    return out
+
+
+def bitmap_to_grouped(bitmap, min_len=32):
+    """BTCF2GBTCF of the reference (src/utils/convert.h:232): returns the GBTCF_MTX
+    fields (src/utils/class.h:93-108); the tile arrays are shared with `bitmap`."""
+    L = load_library()
+    rowOffset = np.ascontiguousarray(bitmap["rowOffset"], np.uint32)
+    rowIdx = np.ascontiguousarray(bitmap["rowIdx"], np.uint32)
+    W = int(bitmap["eff_row_windows"])
+    tgl, n = C.c_uint32(), C.c_uint32()
+    _check(L.hspmm_group_sizes(W, _p(rowOffset), min_len, C.byref(tgl), C.byref(n)))
+    n = n.value
+    groupOffset = np.zeros(n + 1, np.uint32)
+    groupRowIdx = np.zeros(n, np.uint32)
+    atomic = np.zeros(n, np.uint8)
+    _check(L.hspmm_group_fill(W, _p(rowOffset), _p(rowIdx), tgl.value,
+                              groupOffset.ctypes.data_as(C.c_void_p), _p(groupRowIdx), _p(atomic)))
+    out = {k: bitmap[k] for k in ("rows", "cols", "nnzs", "dtype", "cw", "nnzOffset", "tcA2B", "tcBit", "data")}
+    # the reference sets both window counts to groupOffset.size() (convert.h:267-268)
+    out.update(total_groups=n, tgl=tgl.value, groupOffset=groupOffset, rowIdx=groupRowIdx, atomic=atomic,
+               total_row_windows=n + 1, eff_row_windows=n + 1)
+    return out
+
+
 def partition_preview(rowOffset, target_ranges):
     """The work partition hspmm_create would build (host only)."""
     L = load_library()
@@ -203,15 +285,33 @@ class Plan:
     """Device-resident A plus its work partition (hspmm_create / hspmm_destroy)."""
 
     def __init__(self, btcf):
+        """btcf: a dict as returned by csr_to_btcf (uncompressed tiles), csr_to_bitmap
+        (it has "tcBit") or bitmap_to_grouped (it has "groupOffset")."""
         L = load_library()
         self._h = C.c_void_p()
         self.dtype = btcf["dtype"]
         self.rows, self.cols = int(btcf["rows"]), int(btcf["cols"])
         vt = _val_dtype(self.dtype)
-        ro = np.ascontiguousarray(btcf["rowOffset"], np.uint32)
         a2b = np.ascontiguousarray(btcf["tcA2B"], np.uint32)
         data = np.ascontiguousarray(btcf["data"], vt)
         ri = np.ascontiguousarray(btcf["rowIdx"], np.uint32)
+        if "groupOffset" in btcf:
+            go = np.ascontiguousarray(btcf["groupOffset"], np.uint32)
+            no = np.ascontiguousarray(btcf["nnzOffset"], np.uint32)
+            bits = np.ascontiguousarray(btcf["tcBit"], np.uint64)
+            at = np.ascontiguousarray(btcf["atomic"], np.uint8)
+            _check(L.hspmm_create_grouped(C.byref(self._h), self.dtype, self.rows, self.cols,
+                                          int(btcf["total_groups"]), go.ctypes.data_as(C.c_void_p), _p(no), _p(a2b),
+                                          _p(bits), _p(data), _p(ri), _p(at)))
+            return
+        ro = np.ascontiguousarray(btcf["rowOffset"], np.uint32)
+        if "tcBit" in btcf:
+            no = np.ascontiguousarray(btcf["nnzOffset"], np.uint32)
+            bits = np.ascontiguousarray(btcf["tcBit"], np.uint64)
+            _check(L.hspmm_create_bitmap(C.byref(self._h), self.dtype, self.rows, self.cols,
+                                         int(btcf["eff_row_windows"]), int(btcf["total_tiles"]),
+                                         _p(ro), _p(no), _p(a2b), _p(bits), _p(data), _p(ri)))
+            return
         _check(L.hspmm_create(C.byref(self._h), self.dtype, self.rows, self.cols,
                               int(btcf["eff_row_windows"]), int(btcf["total_tiles"]),
                               _p(ro), _p(a2b), _p(data), _p(ri)))

@@ -483,6 +483,55 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
     return HSPMM_OK;
 }
 
+int hspmm_create_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
+                        uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *nnzOffset,
+                        const uint32_t *tcA2B, const uint64_t *tcBit, const void *data, const uint32_t *rowIdx)
+{
+    if (!out) return fail(HSPMM_ERR_INVALID, "null plan pointer");
+    *out = nullptr;
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16)
+        return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
+    if (total_tiles && (!nnzOffset || !tcBit)) return fail(HSPMM_ERR_INVALID, "null nnzOffset or tcBit");
+    const size_t tile_bytes = size_t(HSPMM_ROW_WINDOW) * (dtype == HSPMM_TF32 ? 8u * 4u : 16u * 2u);
+    std::vector<uint8_t> dense;
+    try { dense.resize(size_t(total_tiles) * tile_bytes); }
+    catch (const std::bad_alloc &) { return fail(HSPMM_ERR_ALLOC, "out of host memory"); }
+    // hspmm_bitmap_expand leaves its own message behind on failure
+    const int rc = hspmm_bitmap_expand(dtype, total_tiles, nnzOffset, tcBit, data, dense.data());
+    if (rc) return rc;
+    return hspmm_create(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, tcA2B, dense.data(), rowIdx);
+}
+
+int hspmm_create_grouped(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t total_groups,
+                         const uint32_t *groupOffset, const uint32_t *nnzOffset, const uint32_t *tcA2B,
+                         const uint64_t *tcBit, const void *data, const uint32_t *groupRowIdx,
+                         const uint8_t *atomic)
+{
+    if (!out) return fail(HSPMM_ERR_INVALID, "null plan pointer");
+    *out = nullptr;
+    if (total_groups && (!groupOffset || !groupRowIdx || !atomic))
+        return fail(HSPMM_ERR_INVALID, "null groupOffset, rowIdx or atomic");
+    // consecutive groups with one row index are one window again
+    std::vector<uint32_t> rowOffset(1, total_groups ? groupOffset[0] : 0u), rowIdx;
+    for (uint32_t g = 0; g < total_groups; ++g) {
+        if (groupOffset[g + 1] <= groupOffset[g])
+            return fail(HSPMM_ERR_INVALID, "groupOffset does not increase at group %u", g);
+        const bool first = g == 0 || groupRowIdx[g] != groupRowIdx[g - 1];
+        const bool last = g + 1 == total_groups || groupRowIdx[g + 1] != groupRowIdx[g];
+        const bool shared = !(first && last);
+        if ((atomic[g] != 0) != shared)
+            return fail(HSPMM_ERR_INVALID, "atomic[%u] = %u but the group %s its rows with a neighbour", g,
+                        unsigned(atomic[g]), shared ? "shares" : "does not share");
+        if (first) rowIdx.push_back(groupRowIdx[g]);
+        if (last) rowOffset.push_back(groupOffset[g + 1]);
+    }
+    // groups of one window that are not adjacent show up as a row index that does
+    // not increase, which the checks of hspmm_create reject
+    const uint32_t W = uint32_t(rowIdx.size());
+    return hspmm_create_bitmap(out, dtype, rows, cols, W, rowOffset.back(), rowOffset.data(), nnzOffset, tcA2B, tcBit,
+                               data, rowIdx.data());
+}
+
 void hspmm_destroy(hspmm_plan *p)
 {
     if (!p) return;

@@ -1,9 +1,10 @@
 // Host-side format functions of the C ABI (include/hspmm.h): MatrixMarket
-// loading and the CSR -> condensed-tile conversion.  They produce the same arrays
-// as the reference's load_matrix (reference src/utils/load.h:152-322) and
-// CSR2BTCFNOBITMAP (reference src/utils/convert.h:146-225), built differently:
-// whole-file parsing with strtoul/strtof, a counting sort by row, and a
-// two-pass, multi-threaded window conversion without hash maps.
+// loading and the CSR -> condensed-tile conversions.  They produce the same arrays
+// as the reference's load_matrix (reference src/utils/load.h:152-322),
+// CSR2BTCFNOBITMAP (src/utils/convert.h:146-225), CSR2BTCF (convert.h:22-139) and
+// BTCF2GBTCF (convert.h:232-276), built differently: whole-file parsing with
+// strtoul/strtof, a counting sort by row, and two-pass, multi-threaded window
+// conversions without hash maps or growing vectors.
 #include <algorithm>
 #include <cerrno>
 #include <cstdint>
@@ -321,6 +322,205 @@ int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uin
                 }
         }
     });
+    return HSPMM_OK;
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------
+// Bitmap-compressed tiles (reference CSR2BTCF, src/utils/convert.h:22-139)
+// ---------------------------------------------------------------------------
+extern "C" {
+
+int hspmm_bitmap_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                       uint32_t *eff_row_windows, uint32_t *total_tiles, uint32_t *stored)
+{
+    const int rc = hspmm_btcf_sizes(dtype, rows, row_ptr, col_idx, eff_row_windows, total_tiles);
+    if (rc) return rc;
+    if (stored) *stored = row_ptr[rows];      // every CSR entry is stored (convert.h:114-119)
+    return HSPMM_OK;
+}
+
+int hspmm_bitmap_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                      const void *values, int transpose, int bit_layout,
+                      uint32_t *rowOffset, uint32_t *nnzOffset, uint32_t *tcA2B, uint64_t *tcBit,
+                      void *data, uint32_t *rowIdx)
+{
+    using namespace hspmm_host;
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    if (bit_layout != HSPMM_BITS_PER_TILE && bit_layout != HSPMM_BITS_AS_REFERENCE) {
+        set_error("unknown bit layout");
+        return HSPMM_ERR_INVALID;
+    }
+    if (!row_ptr || !rowOffset || !nnzOffset) { set_error("null argument"); return HSPMM_ERR_INVALID; }
+    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
+    const uint32_t wpt = HSPMM_BITMAP_WORDS(dtype);
+    const size_t es = dtype == HSPMM_TF32 ? 4 : 2;
+    std::vector<uint32_t> tiles;
+    count_tiles(rows, row_ptr, col_idx, cw, tiles);
+    const size_t nwin = tiles.size();
+    std::vector<uint32_t> eff_index(nwin + 1, 0u), first_tile(nwin + 1, 0u);
+    for (size_t w = 0; w < nwin; ++w) {
+        eff_index[w + 1] = eff_index[w] + (tiles[w] != 0);
+        first_tile[w + 1] = first_tile[w] + tiles[w];
+    }
+    const uint32_t T = first_tile[nwin];
+    rowOffset[0] = 0;                                                        // convert.h:29
+    nnzOffset[0] = 0;                                                        // convert.h:136
+    if (T && (!tcA2B || !tcBit || !data || !rowIdx || !col_idx || !values)) {
+        set_error("null argument");
+        return HSPMM_ERR_INVALID;
+    }
+    if (T) std::memset(tcBit, 0, size_t(T) * wpt * 8);                       // convert.h:67
+    // The reference's word index for 8 x 16 tiles lets neighbouring tiles, and so
+    // neighbouring windows, share a word: that layout is filled by one thread.
+    const bool shared_words = bit_layout == HSPMM_BITS_AS_REFERENCE && wpt == 2;
+    auto convert_windows = [&](size_t wb, size_t we) {
+        std::vector<uint32_t> uniq, start, cursor;
+        for (size_t w = wb; w < we; ++w) {
+            if (!tiles[w]) continue;
+            const uint32_t r0 = uint32_t(w * HSPMM_ROW_WINDOW);
+            const uint32_t r1 = std::min<uint64_t>(uint64_t(r0) + HSPMM_ROW_WINDOW, rows);
+            const uint32_t u = window_columns(row_ptr, col_idx, r0, r1, uniq);
+            const uint32_t ew = eff_index[w], ft = first_tile[w], nt = tiles[w];
+            rowOffset[ew + 1] = ft + nt;                                     // convert.h:58
+            rowIdx[ew] = r0;                                                 // convert.h:68
+            uint32_t *ids = tcA2B + size_t(ft) * cw;
+            for (uint32_t i = 0; i < nt * cw; ++i) ids[i] = i < u ? uniq[i] : HSPMM_IDX_MAX;   // convert.h:50-56
+            // Stored entries are grouped by tile, and inside a tile by (row, position in
+            // the row) - or by (tile column, row) with `transpose` (convert.h:114-133).  Count
+            // per sub-bucket, scan, place.  All entries of earlier windows come first, so
+            // the window's part of `data` starts at row_ptr[r0].
+            const uint32_t sub = transpose ? cw : 1u;
+            start.assign(size_t(nt) * sub + 1, 0u);
+            for (uint32_t id = row_ptr[r0]; id < row_ptr[r1]; ++id) {
+                const uint32_t rank = uint32_t(std::lower_bound(uniq.begin(), uniq.end(), col_idx[id]) - uniq.begin());
+                ++start[size_t(rank / cw) * sub + (transpose ? rank % cw : 0u) + 1];
+            }
+            for (size_t i = 0; i < size_t(nt) * sub; ++i) start[i + 1] += start[i];
+            for (uint32_t t = 0; t < nt; ++t)
+                nnzOffset[ft + t + 1] = row_ptr[r0] + start[size_t(t + 1) * sub];             // convert.h:84,135-137
+            cursor.assign(start.begin(), start.end() - 1);
+            for (uint32_t r = r0; r < r1; ++r)
+                for (uint32_t id = row_ptr[r]; id < row_ptr[r + 1]; ++id) {
+                    const uint32_t rank = uint32_t(std::lower_bound(uniq.begin(), uniq.end(), col_idx[id]) - uniq.begin());
+                    const uint32_t tc = rank / cw, lc = rank % cw, lr = r % HSPMM_ROW_WINDOW;
+                    const uint32_t bit = transpose ? lc * HSPMM_ROW_WINDOW + lr              // convert.h:90
+                                                   : lr * cw + lc;                           // convert.h:93
+                    const size_t word = shared_words ? size_t(ft + tc) + bit / 64u           // convert.h:97-101
+                                                     : size_t(ft + tc) * wpt + bit / 64u;
+                    tcBit[word] |= uint64_t(1) << (bit % 64u);
+                    const uint32_t pos = row_ptr[r0] + cursor[size_t(tc) * sub + (transpose ? lc : 0u)]++;
+                    std::memcpy(static_cast<unsigned char *>(data) + size_t(pos) * es,
+                                static_cast<const unsigned char *>(values) + size_t(id) * es, es);
+                }
+        }
+    };
+    if (shared_words) convert_windows(0, nwin);
+    else parallel_blocks(nwin, 2048, convert_windows);
+    return HSPMM_OK;
+}
+
+int hspmm_bitmap_expand(int dtype, uint32_t total_tiles, const uint32_t *nnzOffset, const uint64_t *tcBit,
+                        const void *data, void *dense_tiles)
+{
+    using namespace hspmm_host;
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    if (total_tiles && (!nnzOffset || !tcBit || !dense_tiles)) { set_error("null argument"); return HSPMM_ERR_INVALID; }
+    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
+    const uint32_t wpt = HSPMM_BITMAP_WORDS(dtype);
+    const size_t es = dtype == HSPMM_TF32 ? 4 : 2;
+    const size_t tile_bytes = size_t(HSPMM_ROW_WINDOW) * cw * es;
+    if (total_tiles && nnzOffset[0] != 0) { set_error("nnzOffset must start at 0"); return HSPMM_ERR_INVALID; }
+    if (total_tiles && nnzOffset[total_tiles] && !data) { set_error("null argument"); return HSPMM_ERR_INVALID; }
+    // every worker records the first inconsistent tile of its block
+    const unsigned nw = worker_count(total_tiles, 1u << 14);
+    std::vector<uint32_t> bad_per_block(nw, HSPMM_IDX_MAX);
+    uint32_t first_bad = HSPMM_IDX_MAX;
+    auto work = [&](unsigned wi) {
+        const size_t b = size_t(total_tiles) * wi / nw, e = size_t(total_tiles) * (wi + 1) / nw;
+        for (size_t t = b; t < e; ++t) {
+            unsigned char *tile = static_cast<unsigned char *>(dense_tiles) + t * tile_bytes;
+            std::memset(tile, 0, tile_bytes);
+            if (nnzOffset[t + 1] < nnzOffset[t]) { if (bad_per_block[wi] == HSPMM_IDX_MAX) bad_per_block[wi] = uint32_t(t); continue; }
+            uint32_t count = 0;
+            for (uint32_t k = 0; k < wpt; ++k) count += uint32_t(__builtin_popcountll(tcBit[t * wpt + k]));
+            if (count != nnzOffset[t + 1] - nnzOffset[t]) { if (bad_per_block[wi] == HSPMM_IDX_MAX) bad_per_block[wi] = uint32_t(t); continue; }
+            size_t src = nnzOffset[t];
+            for (uint32_t k = 0; k < wpt; ++k) {
+                uint64_t bits = tcBit[t * wpt + k];
+                while (bits) {
+                    const uint32_t bit = uint32_t(__builtin_ctzll(bits)) + 64u * k;
+                    bits &= bits - 1;
+                    std::memcpy(tile + size_t(bit) * es, static_cast<const unsigned char *>(data) + src * es, es);
+                    ++src;
+                }
+            }
+        }
+    };
+    if (nw <= 1) work(0);
+    else {
+        std::vector<std::thread> th;
+        for (unsigned i = 0; i < nw; ++i) th.emplace_back(work, i);
+        for (auto &t : th) t.join();
+    }
+    for (uint32_t b : bad_per_block) if (b < first_bad) first_bad = b;
+    if (first_bad != HSPMM_IDX_MAX) {
+        set_error("tile " + std::to_string(first_bad) + ": the number of set bits differs from its nnzOffset span");
+        return HSPMM_ERR_INVALID;
+    }
+    return HSPMM_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Grouped format (reference BTCF2GBTCF, src/utils/convert.h:232-276)
+// ---------------------------------------------------------------------------
+int hspmm_group_sizes(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t min_len,
+                      uint32_t *tgl, uint32_t *total_groups)
+{
+    using namespace hspmm_host;
+    if (eff_row_windows && !rowOffset) { set_error("null argument"); return HSPMM_ERR_INVALID; }
+    if (min_len == 0) { set_error("min_len must be positive"); return HSPMM_ERR_INVALID; }
+    for (uint32_t w = 0; w < eff_row_windows; ++w)
+        if (rowOffset[w + 1] <= rowOffset[w]) { set_error("rowOffset must increase strictly"); return HSPMM_ERR_INVALID; }
+    // mean tiles per window: the reference adds the counts up as doubles and truncates
+    // the quotient (convert.h:239,243); the sum is exact in a double (< 2^53).
+    uint32_t mean = 0;
+    if (eff_row_windows)
+        mean = uint32_t(double(rowOffset[eff_row_windows] - rowOffset[0]) / double(eff_row_windows));
+    const uint32_t len = std::max(mean, min_len);                            // convert.h:243
+    uint64_t groups = 0;
+    for (uint32_t w = 0; w < eff_row_windows; ++w) {
+        const uint32_t n = rowOffset[w + 1] - rowOffset[w];
+        groups += (uint64_t(n) + len - 1) / len;                             // convert.h:249
+    }
+    if (groups > 0xFFFFFFFEull) { set_error("group count exceeds 32 bits"); return HSPMM_ERR_UNSUPPORTED; }
+    if (tgl) *tgl = len;
+    if (total_groups) *total_groups = uint32_t(groups);
+    return HSPMM_OK;
+}
+
+int hspmm_group_fill(uint32_t eff_row_windows, const uint32_t *rowOffset, const uint32_t *rowIdx,
+                     uint32_t tgl, uint32_t *groupOffset, uint32_t *groupRowIdx, uint8_t *atomic)
+{
+    using namespace hspmm_host;
+    if (!groupOffset || (eff_row_windows && (!rowOffset || !rowIdx || !groupRowIdx || !atomic))) {
+        set_error("null argument");
+        return HSPMM_ERR_INVALID;
+    }
+    if (tgl == 0) { set_error("tgl must be positive"); return HSPMM_ERR_INVALID; }
+    size_t g = 0;
+    for (uint32_t w = 0; w < eff_row_windows; ++w) {
+        const uint32_t n = rowOffset[w + 1] - rowOffset[w];
+        const uint32_t group_num = uint32_t((uint64_t(n) + tgl - 1) / tgl);                   // convert.h:249
+        const uint32_t stride = group_num ? uint32_t((uint64_t(n) + group_num - 1) / group_num) : 0u;
+        for (uint32_t j = 0; j < group_num; ++j, ++g) {
+            groupOffset[g] = rowOffset[w] + stride * j;                      // convert.h:251-252
+            groupRowIdx[g] = rowIdx[w];                                      // convert.h:253
+            atomic[g] = group_num == 1 ? 0 : 1;                              // convert.h:254-257
+        }
+    }
+    groupOffset[g] = eff_row_windows ? rowOffset[eff_row_windows] : 0u;      // convert.h:261
     return HSPMM_OK;
 }
 

@@ -19,6 +19,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cmath>
+#include <cstring>
 #include <vector>
 
 #include <hip/hip_runtime.h>
@@ -80,6 +81,34 @@ struct BTCF_MTX_NO_BITMAP {
     std::vector<MAT_VAL_TYPE> data;
     std::vector<MAT_IDX_TYPE> rowIdx;
     uint32_t total_tiles;
+};
+
+// Bitmap-compressed tiles (reference src/utils/class.h:55-67).  For 8 x 16 tiles
+// tcBit holds two words per tile, tile t in words 2t and 2t + 1.
+#define MAT_MAP_TYPE uint64_t
+#define ATOMIC_TYPE uint8_t
+struct BTCF_MTX {
+    vint rows, cols, nnzs;
+    vint total_row_windows, eff_row_windows;
+    std::vector<MAT_PTR_TYPE> rowOffset;
+    std::vector<MAT_PTR_TYPE> nnzOffset;
+    std::vector<MAT_IDX_TYPE> tcA2B;
+    std::vector<MAT_MAP_TYPE> tcBit;
+    std::vector<MAT_VAL_TYPE> data;       // stored entries only, indexed through nnzOffset
+    std::vector<MAT_IDX_TYPE> rowIdx;
+};
+
+// Grouped tiles (reference src/utils/class.h:93-108).
+struct GBTCF_MTX {
+    vint rows, cols, nnzs;
+    vint total_row_windows, total_groups, eff_row_windows;
+    std::vector<MAT_PTR_TYPE> groupOffset;
+    std::vector<MAT_PTR_TYPE> nnzOffset;
+    std::vector<MAT_IDX_TYPE> tcA2B;
+    std::vector<MAT_MAP_TYPE> tcBit;
+    std::vector<MAT_VAL_TYPE> data;
+    std::vector<MAT_IDX_TYPE> rowIdx;     // one per group
+    std::vector<ATOMIC_TYPE> atomic;      // 1 where a window was cut into several groups
 };
 
 namespace hspmm_cpp {
@@ -154,6 +183,86 @@ inline void CSR2BTCFNOBITMAP(const CSR_MTX &csr, BTCF_MTX_NO_BITMAP &btcf)
     std::printf("CSR -> condensed tiles: %u effective row windows, %u tiles of %d x %d\n", W, T, ROW_WINDOW, COL_WINDOW);
 }
 
+// CSR2BTCF of the reference (src/utils/convert.h:22-139).
+inline void CSR2BTCF(const CSR_MTX &csr, BTCF_MTX &btcf)
+{
+    btcf.rows = csr.rows; btcf.cols = csr.cols; btcf.nnzs = csr.nnzs;
+    btcf.total_row_windows = (csr.rows + ROW_WINDOW - 1) / ROW_WINDOW;
+    uint32_t W = 0, T = 0, S = 0;
+    static const MAT_PTR_TYPE zero_ptr[1] = {0};
+    const MAT_PTR_TYPE *rp = csr.row_ptr ? csr.row_ptr : zero_ptr;
+    if (hspmm_bitmap_sizes(HSPMM_BUILD_DTYPE, csr.rows, rp, csr.col_idx, &W, &T, &S) != HSPMM_OK)
+        hspmm_cpp::die("CSR2BTCF");
+    btcf.rowOffset.assign(size_t(W) + 1, 0);
+    btcf.nnzOffset.assign(size_t(T) + 1, 0);
+    btcf.tcA2B.assign(size_t(T) * COL_WINDOW, 0);
+    btcf.tcBit.assign(size_t(T) * HSPMM_BITMAP_WORDS(HSPMM_BUILD_DTYPE), 0);
+    btcf.data.assign(S, MAT_VAL_TYPE(0.0f));
+    btcf.rowIdx.assign(W, 0);
+#ifdef SPARSE_A_TRANSPOSE
+    const int transpose = 1;
+#else
+    const int transpose = 0;
+#endif
+    if (hspmm_bitmap_fill(HSPMM_BUILD_DTYPE, csr.rows, rp, csr.col_idx, csr.values, transpose, HSPMM_BITS_PER_TILE,
+                          btcf.rowOffset.data(), btcf.nnzOffset.data(), btcf.tcA2B.data(), btcf.tcBit.data(),
+                          btcf.data.data(), btcf.rowIdx.data()) != HSPMM_OK)
+        hspmm_cpp::die("CSR2BTCF");
+    btcf.eff_row_windows = W;
+    std::printf("CSR -> bitmap tiles: %u effective row windows, %u tiles, %u stored entries\n", W, T, S);
+}
+
+// BTCF2GBTCF of the reference (src/utils/convert.h:232-276).
+inline void BTCF2GBTCF(BTCF_MTX &btcf, GBTCF_MTX &gbtcf)
+{
+    uint32_t tgl = 0, groups = 0;
+    if (hspmm_group_sizes(btcf.eff_row_windows, btcf.rowOffset.data(), 32, &tgl, &groups) != HSPMM_OK)
+        hspmm_cpp::die("BTCF2GBTCF");
+    std::printf("tgl : %u\n", tgl);
+    gbtcf.groupOffset.assign(size_t(groups) + 1, 0);
+    gbtcf.rowIdx.assign(groups, 0);
+    gbtcf.atomic.assign(groups, 0);
+    if (hspmm_group_fill(btcf.eff_row_windows, btcf.rowOffset.data(), btcf.rowIdx.data(), tgl, gbtcf.groupOffset.data(),
+                         gbtcf.rowIdx.data(), gbtcf.atomic.data()) != HSPMM_OK)
+        hspmm_cpp::die("BTCF2GBTCF");
+    std::printf("total groups : %u\n", groups);
+    gbtcf.total_groups = groups;
+    gbtcf.rows = btcf.rows; gbtcf.cols = btcf.cols; gbtcf.nnzs = btcf.nnzs;
+    gbtcf.total_row_windows = groups + 1;          // groupOffset.size(), as the reference sets both (convert.h:267-268)
+    gbtcf.eff_row_windows = groups + 1;
+    gbtcf.nnzOffset = btcf.nnzOffset; gbtcf.tcA2B = btcf.tcA2B; gbtcf.tcBit = btcf.tcBit; gbtcf.data = btcf.data;
+}
+
+// The checks of the reference's validateBTCF2GBTCFConversion (src/utils/convert.h:283-402)
+// with the group count of every window derived from the converter's own group
+// length; the reference's check still assumes a fixed length of 4 tiles
+// (convert.h:317-318) and rejects every real conversion.
+inline bool validateBTCF2GBTCFConversion(const BTCF_MTX &btcf, const GBTCF_MTX &gbtcf)
+{
+    if (btcf.rows != gbtcf.rows || btcf.cols != gbtcf.cols || btcf.nnzs != gbtcf.nnzs) return false;
+    if (gbtcf.groupOffset.size() != size_t(gbtcf.total_groups) + 1) return false;
+    if (gbtcf.atomic.size() != gbtcf.total_groups || gbtcf.rowIdx.size() != gbtcf.total_groups) return false;
+    for (size_t i = 0; i + 1 < gbtcf.groupOffset.size(); ++i)
+        if (gbtcf.groupOffset[i] >= gbtcf.groupOffset[i + 1]) return false;
+    uint32_t tgl = 0, groups = 0;
+    if (hspmm_group_sizes(btcf.eff_row_windows, btcf.rowOffset.data(), 32, &tgl, &groups) != HSPMM_OK) return false;
+    if (groups != gbtcf.total_groups) return false;
+    size_t g = 0;
+    for (vint w = 0; w < btcf.eff_row_windows; ++w) {
+        const vint n = btcf.rowOffset[w + 1] - btcf.rowOffset[w];
+        const vint expected = (n + tgl - 1) / tgl;
+        if (gbtcf.groupOffset[g] != btcf.rowOffset[w]) return false;
+        for (vint j = 0; j < expected; ++j, ++g) {
+            if (gbtcf.rowIdx[g] != btcf.rowIdx[w] || gbtcf.atomic[g] != (expected > 1)) return false;
+            if (gbtcf.groupOffset[g + 1] > btcf.rowOffset[w + 1]) return false;
+        }
+        if (gbtcf.groupOffset[g] != btcf.rowOffset[w + 1]) return false;
+    }
+    return gbtcf.nnzOffset == btcf.nnzOffset && gbtcf.tcA2B == btcf.tcA2B && gbtcf.tcBit == btcf.tcBit &&
+           gbtcf.data.size() == btcf.data.size() &&
+           std::memcmp(gbtcf.data.data(), btcf.data.data(), btcf.data.size() * sizeof(MAT_VAL_TYPE)) == 0;
+}
+
 // The reference's singleton of launch knobs; here they reach the library.
 class Scheduler {
     int BUFFER_STAGE = 0, CONSUMER_WARP_NUM = 0, PRODUCER_WARP_GROUP_NUM = 0, SM_NUM = 0;
@@ -187,18 +296,56 @@ public:
 
 // C = A * B on the GPU: uploads, WARMUP_RUNS untimed and RUNS timed launches
 // (src/common.h:48-49), downloads C into dense_c.values.
-inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX_NO_BITMAP &a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+namespace hspmm_cpp {
+inline void check_shapes(vint a_rows, vint a_cols, const DENSE_MTX &dense_b, const DENSE_MTX &dense_c)
 {
-    PERF_RESULT perf{0.0f, RUNS};
-    if (dense_b.rows != a.cols || dense_c.rows != a.rows || dense_c.cols != dense_b.cols) {
-        std::fprintf(stderr, "spmm: shapes do not match: A %u x %u, B %u x %u, C %u x %u\n", a.rows, a.cols,
+    if (dense_b.rows != a_cols || dense_c.rows != a_rows || dense_c.cols != dense_b.cols) {
+        std::fprintf(stderr, "spmm: shapes do not match: A %u x %u, B %u x %u, C %u x %u\n", a_rows, a_cols,
                      dense_b.rows, dense_b.cols, dense_c.rows, dense_c.cols);
         std::exit(EXIT_FAILURE);
     }
+}
+inline PERF_RESULT run_plan(hspmm_plan *plan, DENSE_MTX &dense_b, DENSE_MTX &dense_c);
+}  // namespace hspmm_cpp
+
+inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX_NO_BITMAP &a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+{
+    hspmm_cpp::check_shapes(a.rows, a.cols, dense_b, dense_c);
     hspmm_plan *plan = nullptr;
     if (hspmm_create(&plan, HSPMM_BUILD_DTYPE, a.rows, a.cols, a.eff_row_windows, a.total_tiles, a.rowOffset.data(),
                      a.tcA2B.data(), a.data.data(), a.rowIdx.data()) != HSPMM_OK)
         hspmm_cpp::die("hspmm_create");
+    return hspmm_cpp::run_plan(plan, dense_b, dense_c);
+}
+
+// The same operator for a matrix held as bitmap tiles or as groups; the
+// reference has no kernel for either format.
+inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX &a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+{
+    hspmm_cpp::check_shapes(a.rows, a.cols, dense_b, dense_c);
+    hspmm_plan *plan = nullptr;
+    const uint32_t tiles = a.rowOffset.empty() ? 0u : a.rowOffset.back();
+    if (hspmm_create_bitmap(&plan, HSPMM_BUILD_DTYPE, a.rows, a.cols, a.eff_row_windows, tiles, a.rowOffset.data(),
+                            a.nnzOffset.data(), a.tcA2B.data(), a.tcBit.data(), a.data.data(),
+                            a.rowIdx.data()) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_create_bitmap");
+    return hspmm_cpp::run_plan(plan, dense_b, dense_c);
+}
+
+inline PERF_RESULT hspmm_cpp_spmm(GBTCF_MTX &a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+{
+    hspmm_cpp::check_shapes(a.rows, a.cols, dense_b, dense_c);
+    hspmm_plan *plan = nullptr;
+    if (hspmm_create_grouped(&plan, HSPMM_BUILD_DTYPE, a.rows, a.cols, a.total_groups, a.groupOffset.data(),
+                             a.nnzOffset.data(), a.tcA2B.data(), a.tcBit.data(), a.data.data(), a.rowIdx.data(),
+                             a.atomic.data()) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_create_grouped");
+    return hspmm_cpp::run_plan(plan, dense_b, dense_c);
+}
+
+inline PERF_RESULT hspmm_cpp::run_plan(hspmm_plan *plan, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+{
+    PERF_RESULT perf{0.0f, RUNS};
     const size_t b_bytes = size_t(dense_b.rows) * dense_b.cols * sizeof(MAT_VAL_TYPE);
     const size_t c_bytes = size_t(dense_c.rows) * dense_c.cols * sizeof(MAT_VAL_TYPE);
     void *d_b = nullptr, *d_c = nullptr;
@@ -214,18 +361,23 @@ inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX_NO_BITMAP &a, DENSE_MTX &dense_b, DEN
     return perf;
 }
 
+// With BTCF_MTX_NO_BITMAP this is the reference's signature; BTCF_MTX and
+// GBTCF_MTX are accepted as well.
 #if defined(USE_FP16)
-inline PERF_RESULT fp16_spmm(BTCF_MTX_NO_BITMAP &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+template <class SPARSE_MTX>
+inline PERF_RESULT fp16_spmm(SPARSE_MTX &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
 {
     return hspmm_cpp_spmm(btcf_a, dense_b, dense_c);
 }
 #elif defined(USE_BF16)
-inline PERF_RESULT bf16_spmm(BTCF_MTX_NO_BITMAP &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+template <class SPARSE_MTX>
+inline PERF_RESULT bf16_spmm(SPARSE_MTX &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
 {
     return hspmm_cpp_spmm(btcf_a, dense_b, dense_c);
 }
 #else
-inline PERF_RESULT tf32_spmm(BTCF_MTX_NO_BITMAP &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
+template <class SPARSE_MTX>
+inline PERF_RESULT tf32_spmm(SPARSE_MTX &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
 {
     return hspmm_cpp_spmm(btcf_a, dense_b, dense_c);
 }

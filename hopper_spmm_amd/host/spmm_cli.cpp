@@ -1,11 +1,13 @@
 // Command-line driver with the reference's arguments (reference src/fp16.cu:283-319):
-//   fp16_test <matrix_file> <feature_dim> [--seed S] [--verify]
+//   fp16_test <matrix_file> <feature_dim> [--seed S] [--verify] [--format tiles|bitmap|grouped]
 // built with -DUSE_FP16; the same source with -DUSE_TF32 / -DUSE_BF16 gives
 // tf32_test / bf16_test.
 // B is filled with rand() / RAND_MAX as in the reference (src/fp16.cu:303-309);
 // --seed calls srand first (the reference never seeds, i.e. seed 1).  --verify
 // repeats the product with the library's scalar all-shapes kernel, a second
 // implementation on the GPU, and compares the two results element by element.
+// --format hands the matrix to the operator as uncompressed tiles (the reference's
+// only path, the default), as bitmap tiles (CSR2BTCF) or as groups (BTCF2GBTCF).
 #include <cstring>
 #include <string>
 
@@ -14,18 +16,25 @@
 int main(int argc, char *argv[])
 {
     if (argc < 3) {
-        std::printf("Usage: %s <matrix_file> <feature_dim> [--seed S] [--verify]\n", argv[0]);
+        std::printf("Usage: %s <matrix_file> <feature_dim> [--seed S] [--verify] [--format tiles|bitmap|grouped]\n",
+                    argv[0]);
         return 1;
     }
     const char *matrix_file = argv[1];
     const int fd = std::atoi(argv[2]);
     bool verify = false;
+    std::string format = "tiles";
     for (int i = 3; i < argc; ++i) {
         if (!std::strcmp(argv[i], "--verify")) verify = true;
+        else if (!std::strcmp(argv[i], "--format") && i + 1 < argc) format = argv[++i];
         else if (!std::strcmp(argv[i], "--seed") && i + 1 < argc) std::srand(unsigned(std::atol(argv[++i])));
         else { std::printf("unknown argument %s\n", argv[i]); return 1; }
     }
     if (fd <= 0) { std::printf("feature_dim must be positive\n"); return 1; }
+    if (format != "tiles" && format != "bitmap" && format != "grouped") {
+        std::printf("unknown format %s\n", format.c_str());
+        return 1;
+    }
     const vint feature_dim = vint(fd);
 
     CSR_MTX csr = load_matrix(matrix_file, 0);
@@ -43,12 +52,25 @@ int main(int argc, char *argv[])
     DENSE_MTX dense_c{btcf.rows, feature_dim, new MAT_VAL_TYPE[size_t(btcf.rows) * feature_dim]};
 
 #if defined(USE_FP16)
-    PERF_RESULT perf = fp16_spmm(btcf, dense_b, dense_c);
+#define SPMM fp16_spmm
 #elif defined(USE_BF16)
-    PERF_RESULT perf = bf16_spmm(btcf, dense_b, dense_c);
+#define SPMM bf16_spmm
 #else
-    PERF_RESULT perf = tf32_spmm(btcf, dense_b, dense_c);
+#define SPMM tf32_spmm
 #endif
+    PERF_RESULT perf{0.0f, RUNS};
+    if (format == "tiles") perf = SPMM(btcf, dense_b, dense_c);
+    else {
+        BTCF_MTX bitmap;
+        CSR2BTCF(csr, bitmap);
+        if (format == "bitmap") perf = SPMM(bitmap, dense_b, dense_c);
+        else {
+            GBTCF_MTX grouped;
+            BTCF2GBTCF(bitmap, grouped);
+            if (!validateBTCF2GBTCFConversion(bitmap, grouped)) { std::printf("grouping failed its checks\n"); return 2; }
+            perf = SPMM(grouped, dense_b, dense_c);
+        }
+    }
     perf.print();
     const double t = perf.time / perf.runs * 1e-3;
     if (t > 0) std::printf("effective rate: %.3f TFLOP/s (2 * nnz * N / t)\n", 2.0 * btcf.nnzs * feature_dim / t / 1e12);

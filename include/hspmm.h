@@ -167,6 +167,78 @@ int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uin
                     const void *values, int transpose,
                     uint32_t *rowOffset, uint32_t *tcA2B, void *data, uint32_t *rowIdx);
 
+/* ---- bitmap-compressed and grouped formats ------------------------------ */
+
+/* Words of tcBit per tile: one 64-bit word for 8 x 8 tiles (HSPMM_TF32), two
+ * for 8 x 16 tiles (reference src/utils/convert.h:61-66). */
+#define HSPMM_BITMAP_WORDS(dtype) ((dtype) == HSPMM_TF32 ? 1u : 2u)
+
+/* Where the bit of element (r, k) of tile t goes for 8 x 16 tiles.
+ * HSPMM_BITS_PER_TILE: word 2t + bit/64, so every tile owns its two words; this
+ * is the layout the plan functions below read.
+ * HSPMM_BITS_AS_REFERENCE: word t + bit/64 in an array of 2 x tiles words, as
+ * the reference indexes it (src/utils/convert.h:83,96-101): the high word of
+ * tile t is also the low word of tile t + 1, which cannot be decoded; kept so
+ * that the converter's output can be compared bit for bit.  Both layouts are
+ * the same thing for 8 x 8 tiles. */
+#define HSPMM_BITS_PER_TILE 0
+#define HSPMM_BITS_AS_REFERENCE 1
+
+/* Replaces CSR2BTCF (reference src/utils/convert.h:22-139; struct BTCF_MTX,
+ * src/utils/class.h:55-67) in two calls.  Besides rowOffset, tcA2B and rowIdx
+ * of the uncompressed format it gives nnzOffset (total_tiles + 1 prefix sums of
+ * the stored entries per tile), tcBit (HSPMM_BITMAP_WORDS x total_tiles words,
+ * bit r * COL_WINDOW + k set for a stored element, or k * 8 + r with
+ * `transpose`) and `data` with the stored entries only, tile after tile in
+ * ascending bit order.  *stored = entries of `data` = row_ptr[rows]. */
+int hspmm_bitmap_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                       uint32_t *eff_row_windows, uint32_t *total_tiles, uint32_t *stored);
+int hspmm_bitmap_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                      const void *values, int transpose, int bit_layout,
+                      uint32_t *rowOffset, uint32_t *nnzOffset, uint32_t *tcA2B, uint64_t *tcBit,
+                      void *data, uint32_t *rowIdx);
+
+/* No reference counterpart (the reference never decodes its bitmaps): expands
+ * bitmap tiles (HSPMM_BITS_PER_TILE layout) to the dense 8 x COL_WINDOW tiles
+ * of the uncompressed format; the k-th stored entry of a tile goes to the
+ * offset of its k-th set bit.  Fails when a tile's bit count differs from its
+ * nnzOffset span. */
+int hspmm_bitmap_expand(int dtype, uint32_t total_tiles, const uint32_t *nnzOffset, const uint64_t *tcBit,
+                        const void *data, void *dense_tiles);
+
+/* Same as hspmm_create for a matrix held as bitmap tiles (row-major bit order,
+ * HSPMM_BITS_PER_TILE).  The tiles are expanded once, here, into the plan's own
+ * device layout; the kernels and their results are those of hspmm_create on
+ * the expanded arrays. */
+int hspmm_create_bitmap(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
+                        uint32_t eff_row_windows, uint32_t total_tiles,
+                        const uint32_t *rowOffset, const uint32_t *nnzOffset, const uint32_t *tcA2B,
+                        const uint64_t *tcBit, const void *data, const uint32_t *rowIdx);
+
+/* Replaces BTCF2GBTCF (reference src/utils/convert.h:232-276; struct GBTCF_MTX,
+ * src/utils/class.h:93-108) in two calls: windows are cut into groups of at
+ * most tgl tiles, tgl = max(floor(mean tiles per window), min_len) with the
+ * reference's min_len = 32 (convert.h:242-243); a window of n tiles gets
+ * g = ceil(n / tgl) groups starting ceil(n / g) tiles apart (convert.h:249-252).
+ * groupOffset has total_groups + 1 entries, groupRowIdx and atomic one per
+ * group (atomic = 1 where a window has more than one group, convert.h:254-257).
+ * The tile arrays (nnzOffset, tcA2B, tcBit, data) are shared with the bitmap
+ * format unchanged (convert.h:271-274). */
+int hspmm_group_sizes(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t min_len,
+                      uint32_t *tgl, uint32_t *total_groups);
+int hspmm_group_fill(uint32_t eff_row_windows, const uint32_t *rowOffset, const uint32_t *rowIdx,
+                     uint32_t tgl, uint32_t *groupOffset, uint32_t *groupRowIdx, uint8_t *atomic);
+
+/* Same as hspmm_create_bitmap for the grouped format: consecutive groups with
+ * one row index are one window again (their partial results are summed in a
+ * fixed order by the plan's own partition, not with atomics).  Fails when
+ * groupOffset does not increase strictly, when groups of one window are not
+ * adjacent, or when an atomic flag contradicts the grouping. */
+int hspmm_create_grouped(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
+                         uint32_t total_groups, const uint32_t *groupOffset, const uint32_t *nnzOffset,
+                         const uint32_t *tcA2B, const uint64_t *tcBit, const void *data,
+                         const uint32_t *groupRowIdx, const uint8_t *atomic);
+
 #ifdef __cplusplus
 }
 #endif

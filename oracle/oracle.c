@@ -17,6 +17,11 @@
  *                                    gap.mtx), scipy COO->CSR cross-check
  *   orc_btcf_count / orc_btcf_fill   the same golden vectors, round-trip to CSR,
  *                                    brute force on small dense matrices
+ *   orc_bitmap_fill                  golden nnzOffset / packed data / as-written tcBit
+ *                                    words of tiny.mtx, popcounts, expansion through
+ *                                    the set bits equals the uncompressed tiles
+ *   orc_group                        hand-computed cases, closed-form group sizes,
+ *                                    coverage of every window by its groups
  *   orc_spmm_csr_* / orc_spmm_btcf_* dense numpy float64 product on the same
  *                                    rounded inputs, closed forms, CSR-order vs
  *                                    tile-order agreement
@@ -290,6 +295,125 @@ void orc_btcf_fill(uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_i
         W++; T += tiles;
     }
     free(uniq);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Bitmap-compressed tiles.  Follows CSR2BTCF, src/utils/convert.h:22-139.   */
+/* ------------------------------------------------------------------------- */
+/* Sizes are those of orc_btcf_count (same windows and tiles, convert.h:40-58);
+ * `data` holds one entry per stored CSR entry (convert.h:118,130).
+ *   rowOffset[W+1], nnzOffset[T+1], tcA2B[T*cw], tcBit[T*words] (zeroed here),
+ *   data[nnz*elem_size], rowIdx[W];  words = 2 for cw = 16, 1 for cw = 8
+ *   (convert.h:61-66).
+ * as_reference != 0: the word of bit b of tile t is t + b/64, exactly as written
+ * (convert.h:83,96-101), so neighbouring 8 x 16 tiles share a word;
+ * as_reference == 0: word words*t + b/64 (every tile owns its words).
+ * The reference collects the entries of every tile in growing vectors
+ * (convert.h:71-79,114-119) and appends them tile after tile (convert.h:122-133);
+ * here the vectors are linked lists threaded through `next`. */
+void orc_bitmap_fill(uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                     const void *values, uint32_t elem_size, uint32_t cw, int transpose, int as_reference,
+                     uint32_t *rowOffset, uint32_t *nnzOffset, uint32_t *tcA2B, uint64_t *tcBit,
+                     void *data, uint32_t *rowIdx)
+{
+    const uint32_t words = cw == 16 ? 2u : 1u;
+    uint32_t W = 0, T = 0, cap = 0, lcap = 0;
+    uint32_t *uniq = NULL, *next = NULL, *head = NULL, *tail = NULL;
+    size_t out = 0;                                /* entries appended to data so far */
+    uint32_t eff = 0, tot = 0;
+    orc_btcf_count(rows, row_ptr, col_idx, cw, &eff, &tot);
+    memset(tcBit, 0, (size_t)tot * words * 8);
+    rowOffset[0] = 0;                                                             /* convert.h:29 */
+    nnzOffset[0] = 0;                                                             /* convert.h:136 */
+    for (uint32_t r0 = 0; r0 < rows; r0 += ORC_ROW_WINDOW) {
+        uint32_t r1 = r0 + ORC_ROW_WINDOW < rows ? r0 + ORC_ROW_WINDOW : rows;    /* convert.h:34 */
+        uint32_t b = row_ptr[r0], e = row_ptr[r1], n = e - b;
+        if (n == 0) continue;                                                     /* convert.h:38 */
+        if (n > cap) {
+            cap = n;
+            uniq = (uint32_t *)realloc(uniq, (size_t)cap * 4);
+            next = (uint32_t *)realloc(next, (size_t)cap * 4);
+        }
+        memcpy(uniq, col_idx + b, (size_t)n * 4);
+        qsort(uniq, n, 4, orc_u32_cmp);                                           /* convert.h:42 */
+        uint32_t u = 1;
+        for (uint32_t i = 1; i < n; ++i) if (uniq[i] != uniq[i - 1]) uniq[u++] = uniq[i];   /* convert.h:44 */
+        uint32_t tiles = (u + cw - 1) / cw;                                       /* convert.h:51-57 */
+        uint32_t *a2b = tcA2B + (size_t)T * cw;
+        for (uint32_t i = 0; i < tiles * cw; ++i) a2b[i] = i < u ? uniq[i] : ORC_IDX_MAX;   /* convert.h:51-56 */
+        rowOffset[W + 1] = rowOffset[W] + tiles;                                  /* convert.h:58 */
+        rowIdx[W] = r0;                                                           /* convert.h:68 */
+        /* one list per tile, or per tile column in the transposed order */
+        uint32_t lists = transpose ? tiles * cw : tiles;
+        if (lists > lcap) {
+            lcap = lists;
+            head = (uint32_t *)realloc(head, (size_t)lcap * 4);
+            tail = (uint32_t *)realloc(tail, (size_t)lcap * 4);
+        }
+        for (uint32_t i = 0; i < lists; ++i) head[i] = tail[i] = ORC_IDX_MAX;
+        for (uint32_t r = r0; r < r1; ++r) {                                      /* convert.h:81 */
+            for (uint32_t id = row_ptr[r]; id < row_ptr[r + 1]; ++id) {           /* convert.h:82 */
+                uint32_t c = col_idx[id], lo = 0, hi = u;
+                while (hi - lo > 1) { uint32_t mid = (lo + hi) / 2; if (uniq[mid] <= c) lo = mid; else hi = mid; }
+                uint32_t tc = lo / cw, lc = lo % cw, lr = r % ORC_ROW_WINDOW;     /* convert.h:83 */
+                uint32_t bit = transpose ? lc * ORC_ROW_WINDOW + lr               /* convert.h:90 */
+                                         : lr * cw + lc;                          /* convert.h:93 */
+                size_t tile = (size_t)T + tc;                                     /* offset_index, convert.h:83 */
+                if (words == 2) {
+                    size_t base = as_reference ? tile : tile * 2;
+                    if (bit < 64) tcBit[base] |= 1ull << bit;                     /* convert.h:97-98 */
+                    else tcBit[base + 1] |= 1ull << (bit - 64);                   /* convert.h:99-100 */
+                } else if (bit < 64) tcBit[tile] |= 1ull << bit;                  /* convert.h:104-106 */
+                uint32_t list = transpose ? tc * cw + lc : tc;                    /* convert.h:112,116 */
+                uint32_t k = id - b;
+                next[k] = ORC_IDX_MAX;
+                if (head[list] == ORC_IDX_MAX) head[list] = k; else next[tail[list]] = k;
+                tail[list] = k;
+            }
+        }
+        uint32_t per = transpose ? cw : 1u;
+        for (uint32_t t = 0; t < tiles; ++t) {                                    /* convert.h:122-133 */
+            for (uint32_t l = t * per; l < (t + 1) * per; ++l)
+                for (uint32_t k = head[l]; k != ORC_IDX_MAX; k = next[k]) {
+                    memcpy((unsigned char *)data + out * elem_size,
+                           (const unsigned char *)values + ((size_t)b + k) * elem_size, elem_size);
+                    out++;
+                }
+            nnzOffset[T + t + 1] = (uint32_t)out;                                 /* convert.h:84,135-137 */
+        }
+        W++; T += tiles;
+    }
+    free(uniq); free(next); free(head); free(tail);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Grouped format.  Follows BTCF2GBTCF, src/utils/convert.h:232-276.         */
+/* ------------------------------------------------------------------------- */
+/* Returns the number of groups; *tgl_out = max((u32)mean tiles per window,
+ * min_len) (convert.h:239-243; the reference fixes min_len = 32).  Pass NULL
+ * arrays to get the sizes only.  groupOffset[groups+1], groupRowIdx[groups],
+ * atomic[groups]. */
+uint32_t orc_group(uint32_t eff_windows, const uint32_t *rowOffset, const uint32_t *rowIdx, uint32_t min_len,
+                   uint32_t *tgl_out, uint32_t *groupOffset, uint32_t *groupRowIdx, uint8_t *atomic)
+{
+    double sum = 0.0;
+    for (uint32_t i = 0; i < eff_windows; ++i) sum += (double)(rowOffset[i + 1] - rowOffset[i]);   /* convert.h:235-239 */
+    uint32_t mean = eff_windows ? (uint32_t)(sum / (double)eff_windows) : 0u;
+    uint32_t tgl = mean > min_len ? mean : min_len;                               /* convert.h:243 */
+    if (tgl_out) *tgl_out = tgl;
+    uint32_t g = 0;
+    for (uint32_t i = 0; i < eff_windows; ++i) {
+        uint32_t n = rowOffset[i + 1] - rowOffset[i];
+        uint32_t group_num = (n + tgl - 1) / tgl;                                 /* convert.h:249 */
+        for (uint32_t j = 0; j < group_num; ++j, ++g) {
+            if (!groupOffset) continue;
+            groupOffset[g] = rowOffset[i] + (n + group_num - 1) / group_num * j;  /* convert.h:251 */
+            groupRowIdx[g] = rowIdx[i];                                           /* convert.h:253 */
+            atomic[g] = group_num == 1 ? 0 : 1;                                   /* convert.h:254-257 */
+        }
+    }
+    if (groupOffset) groupOffset[g] = eff_windows ? rowOffset[eff_windows] : 0u;  /* convert.h:261 */
+    return g;
 }
 
 /* ------------------------------------------------------------------------- */

@@ -151,6 +151,52 @@ def csr_to_btcf(rows, cols, row_ptr, col_idx, values, dtype, transpose=False, cw
                 rowOffset=rowOffset, tcA2B=tcA2B, data=data, rowIdx=rowIdx)
 
 
+def csr_to_bitmap(rows, cols, row_ptr, col_idx, values, dtype, transpose=False, as_reference=False):
+    """CSR -> bitmap-compressed tiles.  as_reference=True indexes tcBit exactly as
+    the reference does (neighbouring 8 x 16 tiles share a word)."""
+    es = 4 if dtype == "tf32" else 2
+    cw = 8 if dtype == "tf32" else 16
+    words = 1 if cw == 8 else 2
+    vt = np.uint16 if es == 2 else np.float32
+    row_ptr = _c(row_ptr, np.uint32)
+    col_idx = _c(col_idx, np.uint32)
+    values = _c(values, vt)
+    W = C.c_uint32()
+    T = C.c_uint32()
+    lib().orc_btcf_count(C.c_uint32(rows), _p(row_ptr), _p(col_idx), C.c_uint32(cw), C.byref(W), C.byref(T))
+    W, T = W.value, T.value
+    nnz = int(row_ptr[rows])
+    rowOffset = np.zeros(W + 1, np.uint32)
+    nnzOffset = np.zeros(T + 1, np.uint32)
+    tcA2B = np.empty(T * cw, np.uint32)
+    tcBit = np.zeros(T * words, np.uint64)
+    data = np.zeros(nnz, vt)
+    rowIdx = np.empty(W, np.uint32)
+    lib().orc_bitmap_fill(C.c_uint32(rows), _p(row_ptr), _p(col_idx), _p(values), C.c_uint32(es), C.c_uint32(cw),
+                          C.c_int(int(transpose)), C.c_int(int(as_reference)),
+                          _p(rowOffset), _p(nnzOffset), _p(tcA2B), _p(tcBit), _p(data), _p(rowIdx))
+    return dict(rows=rows, cols=cols, nnzs=nnz, dtype=dtype, cw=cw,
+                total_row_windows=(rows + ROW_WINDOW - 1) // ROW_WINDOW, eff_row_windows=W, total_tiles=T,
+                rowOffset=rowOffset, nnzOffset=nnzOffset, tcA2B=tcA2B, tcBit=tcBit, data=data, rowIdx=rowIdx)
+
+
+def group(rowOffset, rowIdx, min_len=32):
+    """Window list -> groups of at most tgl tiles: (tgl, groupOffset, groupRowIdx, atomic)."""
+    rowOffset = _c(rowOffset, np.uint32)
+    rowIdx = _c(rowIdx, np.uint32)
+    W = rowIdx.size
+    tgl = C.c_uint32()
+    L = lib()
+    L.orc_group.restype = C.c_uint32
+    n = L.orc_group(C.c_uint32(W), _p(rowOffset), _p(rowIdx), C.c_uint32(min_len), C.byref(tgl), None, None, None)
+    groupOffset = np.zeros(n + 1, np.uint32)
+    groupRowIdx = np.zeros(n, np.uint32)
+    atomic = np.zeros(n, np.uint8)
+    L.orc_group(C.c_uint32(W), _p(rowOffset), _p(rowIdx), C.c_uint32(min_len), C.byref(tgl),
+                _p(groupOffset), _p(groupRowIdx), _p(atomic))
+    return tgl.value, groupOffset, groupRowIdx, atomic
+
+
 def spmm_csr_f16(rows, N, row_ptr, col_idx, vals_bits, B_bits, want_absdot=False, threads=0):
     row_ptr = _c(row_ptr, np.uint32)
     col_idx = _c(col_idx, np.uint32)

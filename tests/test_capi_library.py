@@ -74,6 +74,36 @@ def test_create_rejects_malformed_formats_before_touching_the_device(hs):
     assert b"dtype" in L.hspmm_last_error() and not h.value
 
 
+def test_bitmap_and_grouped_plans_reject_malformed_arrays_before_touching_the_device(hs):
+    from util import random_csr
+    rng = np.random.default_rng(21)
+    A = random_csr(rng, 64, 900, 0.2, 0, 0.0, heavy_rows=(3,))
+    b = hs.csr_to_bitmap(64, 900, A["row_ptr"], A["col_idx"], A["values"], 0)
+    g = hs.bitmap_to_grouped(b, min_len=4)
+    assert g["atomic"].any() and not g["atomic"].all()
+
+    def broken(src, **kw):
+        d = dict(src)
+        for k, f in kw.items():
+            a = src[k].copy()
+            f(a)
+            d[k] = a
+        return d
+
+    def flip(a): a[5] ^= np.uint64(2)
+    def shift(a): a[2] += 1
+    def flag_one(a): a[int(np.argmax(g["atomic"] == 0))] = 1
+    def flag_zero(a): a[int(np.argmax(g["atomic"] == 1))] = 0
+    def stall(a): a[3] = a[2]
+    def scatter(a): a[-1] = a[0]
+    cases = [broken(b, tcBit=flip), broken(b, nnzOffset=shift), broken(g, tcBit=flip), broken(g, atomic=flag_one),
+             broken(g, atomic=flag_zero), broken(g, groupOffset=stall), broken(g, rowIdx=scatter)]
+    for c in cases:
+        with pytest.raises(hs.HspmmError) as e:
+            hs.Plan(c)
+        assert e.value.code == 1, str(e.value)           # HSPMM_ERR_INVALID from host-side checks
+
+
 def test_operator_fails_loudly_without_a_gfx950_device(hs):
     import torch
     if torch.cuda.is_available():

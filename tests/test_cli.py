@@ -32,6 +32,12 @@ def test_cli_fails_loudly_without_a_device(hs):
     r = run(hs, "fp16_test", os.path.join(GOLD, "tiny.mtx"), "64")
     assert r.returncode == 1 and "hspmm_create" in r.stderr
     assert "tiles (8 x 16): 2" in r.stdout                           # the format statistics of src/fp16.cu:295-301
+    for fmt, entry in (("bitmap", "hspmm_create_bitmap"), ("grouped", "hspmm_create_grouped")):
+        r = run(hs, "fp16_test", os.path.join(GOLD, "tiny.mtx"), "64", "--format", fmt)
+        assert r.returncode == 1 and entry in r.stderr
+        assert "2 tiles, 9 stored entries" in r.stdout
+    r = run(hs, "fp16_test", os.path.join(GOLD, "tiny.mtx"), "64", "--format", "csr")
+    assert r.returncode == 1 and "unknown format" in r.stdout
 
 
 @pytest.mark.gpu
@@ -44,8 +50,10 @@ def test_cli_end_to_end_with_verification(hs, tmp_path):
         f.write("%%MatrixMarket matrix coordinate real general\n%d %d %d\n" % (rows, cols, nnz))
         for k in flat:
             f.write("%d %d %.6g\n" % (k // cols + 1, k % cols + 1, rng.normal()))
-    for name, n in (("fp16_test", "128"), ("fp16_test", "7"), ("tf32_test", "64"), ("bf16_test", "128"), ("bf16_test", "5")):
-        r = run(hs, name, str(p), n, "--seed", "42", "--verify")
+    for name, n, fmt in (("fp16_test", "128", "tiles"), ("fp16_test", "7", "tiles"), ("tf32_test", "64", "tiles"),
+                         ("bf16_test", "128", "tiles"), ("bf16_test", "5", "tiles"), ("fp16_test", "64", "bitmap"),
+                         ("tf32_test", "32", "grouped"), ("bf16_test", "64", "grouped")):
+        r = run(hs, name, str(p), n, "--seed", "42", "--verify", "--format", fmt)
         assert r.returncode == 0, r.stdout + r.stderr
         assert "verification passed" in r.stdout
         assert "SpMM timed runs: 5" in r.stdout                      # RUNS, src/common.h:49

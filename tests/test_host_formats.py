@@ -143,3 +143,82 @@ def test_converter_empty_and_duplicates(hs, oracle):
     # an explicit zero still claims a tile column
     a = hs.csr_to_btcf(1, 10, np.array([0, 2], np.uint32), np.array([1, 7], np.uint32), np.array([0.0, 5.0], np.float32), 1)
     assert a["tcA2B"].tolist()[:2] == [1, 7]
+
+
+# ------------------------------------------------------------------ bitmap tiles and groups
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_bitmap_converter_equals_oracle(hs, oracle, dtype):
+    rng = np.random.default_rng(400 + dtype)
+    shapes = [(1, 1, 1.0, 0.0), (8, 16, 0.5, 0.0), (9, 17, 0.5, 0.0), (27, 12, 0.1, 0.7), (64, 500, 0.05, 0.3),
+              (203, 77, 0.3, 0.1), (1000, 1000, 0.004, 0.5), (16, 4000, 0.6, 0.0)]
+    for rows, cols, dens, erp in shapes:
+        A = random_csr(rng, rows, cols, dens, dtype, erp)
+        for tr in (False, True):
+            for layout in (hs.BITS_PER_TILE, hs.BITS_AS_REFERENCE):
+                a = hs.csr_to_bitmap(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype, tr, layout)
+                o = oracle.csr_to_bitmap(rows, cols, A["row_ptr"], A["col_idx"], A["values"], DT[dtype], tr,
+                                         layout == hs.BITS_AS_REFERENCE)
+                for k in ("rowOffset", "nnzOffset", "tcA2B", "tcBit", "rowIdx"):
+                    assert np.array_equal(a[k], o[k]), k
+                assert a["data"].tobytes() == o["data"].tobytes()
+                assert (a["eff_row_windows"], a["total_tiles"]) == (o["eff_row_windows"], o["total_tiles"])
+            # expansion gives back the uncompressed converter's tiles, in both tile orders
+            e = hs.bitmap_expand(hs.csr_to_bitmap(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype, tr))
+            d = hs.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype, transpose=tr)
+            _same_btcf(e, d)
+
+
+def test_bitmap_golden_vector_through_the_library(hs):
+    import json
+    with open(os.path.join(GOLD, "expected.json")) as f:
+        g = json.load(f)["tiny"]
+    A = hs.mtx_load(os.path.join(GOLD, "tiny.mtx"), 0)
+    b = hs.csr_to_bitmap(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], 0,
+                         bit_layout=hs.BITS_AS_REFERENCE)
+    assert b["nnzOffset"].tolist() == g["bitmap"]["nnzOffset"]
+    assert b["data"].view(np.float16).astype(np.float32).tolist() == g["bitmap"]["data"]
+    assert [int(x) for x in b["tcBit"]] == [int(x, 16) for x in g["bitmap"]["tcBit_as_reference"]]
+
+
+def test_bitmap_large_multithreaded_equals_oracle(hs, oracle):
+    from hopper_spmm_amd import generators as G
+    A = G.rmat(15, 16, seed=9)
+    a = hs.csr_to_bitmap(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], 0)
+    o = oracle.csr_to_bitmap(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], "fp16")
+    for k in ("rowOffset", "nnzOffset", "tcA2B", "tcBit", "rowIdx"):
+        assert np.array_equal(a[k], o[k]), k
+    assert a["data"].tobytes() == o["data"].tobytes()
+    _same_btcf(hs.bitmap_expand(a), hs.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], 0))
+
+
+def test_bitmap_expand_rejects_inconsistent_tiles(hs):
+    rng = np.random.default_rng(3)
+    A = random_csr(rng, 40, 60, 0.2, 0)
+    b = hs.csr_to_bitmap(40, 60, A["row_ptr"], A["col_idx"], A["values"], 0)
+    bad = dict(b)
+    bad["tcBit"] = b["tcBit"].copy()
+    bad["tcBit"][3] ^= np.uint64(1) << np.uint64(63)             # one bit more or less than nnzOffset says
+    with pytest.raises(hs.HspmmError) as e:
+        hs.bitmap_expand(bad)
+    assert "tile 1" in str(e.value)
+    bad = dict(b)
+    bad["nnzOffset"] = b["nnzOffset"].copy()
+    bad["nnzOffset"][0] = 1
+    with pytest.raises(hs.HspmmError):
+        hs.bitmap_expand(bad)
+
+
+def test_grouping_equals_oracle(hs, oracle):
+    rng = np.random.default_rng(12)
+    A = random_csr(rng, 400, 3000, 0.02, 0, 0.2, heavy_rows=(5, 100, 399))
+    b = hs.csr_to_bitmap(400, 3000, A["row_ptr"], A["col_idx"], A["values"], 0)
+    for min_len in (1, 3, 32, 1000):
+        g = hs.bitmap_to_grouped(b, min_len)
+        tgl, go, ri, at = oracle.group(b["rowOffset"], b["rowIdx"], min_len)
+        assert g["tgl"] == tgl and g["total_groups"] == at.size
+        assert np.array_equal(g["groupOffset"], go) and np.array_equal(g["rowIdx"], ri)
+        assert np.array_equal(g["atomic"], at)
+        assert g["eff_row_windows"] == go.size                      # as the reference sets it (convert.h:267-268)
+    empty = hs.csr_to_bitmap(9, 9, np.zeros(10, np.uint32), np.zeros(0, np.uint32), np.zeros(0, np.uint16), 0)
+    g = hs.bitmap_to_grouped(empty)
+    assert g["total_groups"] == 0 and g["groupOffset"].tolist() == [0] and g["tgl"] == 32

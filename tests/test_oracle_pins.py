@@ -229,6 +229,106 @@ def test_converter_brute_force_dense(oracle):
         assert np.array_equal(b["data"].reshape(-1, 8, 8), np.array(exp_tiles))
 
 
+# ---------------------------------------------------------------- bitmap tiles and groups
+def _expand_bitmap(b):
+    """Definition of the bitmap format, in numpy: the k-th stored entry of a tile
+    sits where its k-th set bit is."""
+    cw, T = b["cw"], b["total_tiles"]
+    words = b["tcBit"].size // max(T, 1) if T else 1
+    dense = np.zeros((T, 8 * cw), b["data"].dtype)
+    for t in range(T):
+        bits = 0
+        for k in range(words):
+            bits |= int(b["tcBit"][t * words + k]) << (64 * k)
+        pos = [i for i in range(8 * cw) if bits >> i & 1]
+        seg = b["data"][b["nnzOffset"][t]:b["nnzOffset"][t + 1]]
+        assert len(pos) == seg.size
+        dense[t, pos] = seg
+    return dense.ravel()
+
+
+def test_bitmap_golden_vector(oracle):
+    g = gold()["tiny"]
+    m = oracle.mtx_read(os.path.join(GOLD, g["file"]), "fp16")
+    b = oracle.csr_to_bitmap(m["rows"], m["cols"], m["row_ptr"], m["col_idx"], m["values"], "fp16", as_reference=True)
+    assert b["nnzOffset"].tolist() == g["bitmap"]["nnzOffset"]
+    assert b["data"].view(np.float16).astype(np.float32).tolist() == g["bitmap"]["data"]
+    assert [int(x) for x in b["tcBit"]] == [int(x, 16) for x in g["bitmap"]["tcBit_as_reference"]]
+    assert b["rowOffset"].tolist() == g["rowOffset"] and b["tcA2B"].tolist() == g["tcA2B"]
+    assert b["rowIdx"].tolist() == g["rowIdx"]
+    # the per-tile layout holds the same bits, two words to a tile
+    c = oracle.csr_to_bitmap(m["rows"], m["cols"], m["row_ptr"], m["col_idx"], m["values"], "fp16")
+    want = np.zeros((2, 128), bool)
+    for t, r, k, _ in g["tile_nonzeros"]:
+        want[t, r * 16 + k] = True
+    got = np.array([[int(c["tcBit"][2 * t + i // 64]) >> (i % 64) & 1 for i in range(128)] for t in range(2)], bool)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_bitmap_expands_to_the_uncompressed_tiles(oracle, dtype):
+    rng = np.random.default_rng(300 + dtype)
+    name = dtype_name(dtype)
+    for rows, cols, dens, erp in [(1, 1, 1.0, 0), (7, 5, 0.5, 0), (8, 40, 0.9, 0.0), (27, 100, 0.1, 0.5),
+                                  (64, 33, 0.4, 0.0), (100, 300, 0.02, 0.6)]:
+        A = random_csr(rng, rows, cols, dens, dtype, erp)
+        A["values"][A["values"] == 0] = encode(np.float32(0.5), dtype)    # stored zeros would hide a misplaced entry
+        for tr in (False, True):
+            b = oracle.csr_to_bitmap(rows, cols, A["row_ptr"], A["col_idx"], A["values"], name, transpose=tr)
+            d = oracle.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], name, transpose=tr)
+            for k in ("rowOffset", "tcA2B", "rowIdx"):
+                assert np.array_equal(b[k], d[k])
+            assert b["nnzOffset"][0] == 0 and b["nnzOffset"][-1] == A["nnzs"] and b["data"].size == A["nnzs"]
+            assert np.array_equal(_expand_bitmap(b).view(np.uint8), d["data"].view(np.uint8))
+            # as-reference indexing: 8 x 8 tiles are unaffected; for 8 x 16 tiles word w is the
+            # low word of tile w or-ed with the high word of tile w - 1
+            r = oracle.csr_to_bitmap(rows, cols, A["row_ptr"], A["col_idx"], A["values"], name, transpose=tr,
+                                     as_reference=True)
+            if dtype == 1:
+                assert np.array_equal(r["tcBit"], b["tcBit"])
+            else:
+                T = b["total_tiles"]
+                lo, hi = b["tcBit"][0::2], b["tcBit"][1::2]
+                want = np.zeros(2 * T, np.uint64)
+                want[:T] |= lo
+                want[1:T + 1] |= hi
+                assert np.array_equal(r["tcBit"], want)
+
+
+def test_grouping_hand_computed_and_closed_form(oracle):
+    # tiles per window 5, 65, 1, 129: mean 50 -> tgl 50; 65 -> 2 groups 33 apart; 129 -> 3 groups 43 apart
+    tgl, go, ri, at = oracle.group(np.array([0, 5, 70, 71, 200]), np.array([0, 8, 24, 32]))
+    assert tgl == 50
+    assert go.tolist() == [0, 5, 38, 70, 71, 114, 157, 200]
+    assert ri.tolist() == [0, 8, 8, 24, 32, 32, 32]
+    assert at.tolist() == [0, 1, 1, 0, 1, 1, 1]
+    # mean below the floor of 32 tiles: tgl = 32
+    tgl, go, ri, at = oracle.group(np.array([0, 3, 36]), np.array([8, 16]))
+    assert tgl == 32 and go.tolist() == [0, 3, 20, 36] and at.tolist() == [0, 1, 1] and ri.tolist() == [8, 16, 16]
+    # no window at all
+    tgl, go, ri, at = oracle.group(np.array([0]), np.zeros(0, np.uint32))
+    assert tgl == 32 and go.tolist() == [0] and ri.size == 0
+    rng = np.random.default_rng(5)
+    for min_len in (1, 4, 32):
+        n = rng.integers(1, 400, 60)
+        ro = np.concatenate([[0], np.cumsum(n)])
+        ri_in = np.arange(60) * 8
+        tgl, go, ri, at = oracle.group(ro, ri_in, min_len)
+        assert tgl == max(int(n.sum() / 60), min_len)
+        g = 0
+        for w in range(60):
+            k = -(-int(n[w]) // tgl)
+            step = -(-int(n[w]) // k)
+            assert go[g:g + k].tolist() == [int(ro[w]) + step * j for j in range(k)]
+            assert np.all(ri[g:g + k] == ri_in[w]) and np.all(at[g:g + k] == (k > 1))
+            # every group holds at least one and at most tgl tiles, together exactly the window
+            ends = go[g + 1:g + k + 1].astype(np.int64)
+            sizes = ends - go[g:g + k]
+            assert ends[-1] == ro[w + 1] and np.all(sizes >= 1) and np.all(sizes <= tgl)
+            g += k
+        assert g == at.size and go[-1] == ro[-1]
+
+
 def test_converter_duplicate_entries_last_one_wins(oracle):
     # convert.h:215 assigns, it does not add: of two stored entries at one position
     # the later one (in CSR order) stays

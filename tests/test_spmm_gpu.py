@@ -258,6 +258,38 @@ def test_windows_with_one_column_list_share_their_gather(torch_cuda, hs, oracle,
         plan.close()
 
 
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_plans_from_bitmap_and_grouped_formats(torch_cuda, hs, oracle, dtype):
+    """The compressed and the grouped format describe the same matrix: their plans
+    give bit for bit what the plan of the uncompressed tiles gives, and that agrees
+    with the oracle."""
+    rng = np.random.default_rng(90 + dtype)
+    for rows, cols, dens, erp, heavy in [(27, 100, 0.1, 0.5, ()), (300, 3000, 0.004, 0.2, (5, 100, 101, 299)),
+                                         (1000, 700, 0.01, 0.6, (512,))]:
+        A = random_csr(rng, rows, cols, dens, dtype, erp, heavy)
+        plain = convert(hs, A)
+        bitmap = hs.csr_to_bitmap(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype)
+        assert bitmap["data"].size == A["nnzs"] < plain["data"].size
+        grouped = hs.bitmap_to_grouped(bitmap, min_len=4)
+        if heavy:
+            assert grouped["atomic"].any()
+        for N in (8, 64, 136):
+            B = make_b(rng, cols, N, dtype)
+            want = gpu_spmm(torch_cuda, hs, plain, B, N)
+            ref, mag = oracle_spmm(oracle, A, B, N)
+            assert_parity(want, ref, mag, dtype, "plain %dx%d N=%d" % (rows, cols, N))
+            for name, fmt in (("bitmap", bitmap), ("grouped", grouped), ("grouped-32", hs.bitmap_to_grouped(bitmap))):
+                got = gpu_spmm(torch_cuda, hs, fmt, B, N)
+                assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "%s %dx%d N=%d" % (name, rows, cols, N)
+    # golden file through the compressed format
+    A = hs.mtx_load(os.path.join(GOLD, "tiny.mtx"), dtype)
+    A["dtype"] = dtype
+    bitmap = hs.csr_to_bitmap(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], dtype)
+    B = make_b(rng, A["cols"], 32, dtype)
+    ref, mag = oracle_spmm(oracle, A, B, 32)
+    assert_parity(gpu_spmm(torch_cuda, hs, bitmap, B, 32), ref, mag, dtype, "tiny.mtx bitmap")
+
+
 def test_unaligned_and_odd_feature_dims_use_the_all_shapes_kernel(torch_cuda, hs, oracle):
     rng = np.random.default_rng(5)
     for dt in (0, 2):
