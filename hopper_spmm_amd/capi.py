@@ -122,6 +122,15 @@ def _p(a):
     return a.ctypes.data_as(C.c_void_p) if a is not None and a.size else None
 
 
+def _copy_out(ptr, count, dt):
+    """numpy copy of `count` elements of type dt at the C pointer `ptr`."""
+    if count == 0:
+        return np.zeros(0, dt)
+    addr = C.cast(ptr, C.c_void_p).value
+    nbytes = count * np.dtype(dt).itemsize
+    return np.frombuffer((C.c_char * nbytes).from_address(addr), dtype=dt).copy()
+
+
 def _val_dtype(dtype):
     if dtype in (FP16, BF16):
         return np.uint16
@@ -159,10 +168,9 @@ def mtx_load(path, dtype):
     try:
         n = m.nnzs
         vt = _val_dtype(dtype)
-        row_ptr = np.ctypeslib.as_array(m.row_ptr, (m.rows + 1,)).copy()
-        col_idx = np.ctypeslib.as_array(m.col_idx, (max(n, 1),))[:n].copy()
-        vals = np.ctypeslib.as_array(C.cast(m.values, C.POINTER(np.ctypeslib.as_ctypes_type(vt))),
-                                     (max(n, 1),))[:n].copy()
+        row_ptr = _copy_out(m.row_ptr, m.rows + 1, np.uint32)
+        col_idx = _copy_out(m.col_idx, n, np.uint32)
+        vals = _copy_out(m.values, n, vt)
         return dict(rows=m.rows, cols=m.cols, nnzs=n, row_ptr=row_ptr, col_idx=col_idx, values=vals)
     finally:
         L.hspmm_csr_free(C.byref(m))

@@ -5,6 +5,11 @@
 // BTCF2GBTCF (convert.h:232-276), built differently: whole-file parsing with
 // strtoul/strtof, a counting sort by row, and two-pass, multi-threaded window
 // conversions without hash maps or growing vectors.
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
 #include <algorithm>
 #include <cerrno>
 #include <cstdint>
@@ -83,27 +88,105 @@ static void parallel_blocks(size_t n, size_t min_per_worker, F &&fn)
     for (auto &t : th) t.join();
 }
 
-// One parsed text line in the manner of sscanf(line, "%u %u %f") == 3
-// (reference src/utils/load.h:219).
-static bool parse_triple(const char *p, uint32_t &r, uint32_t &c, float &v)
+// ---------------------------------------------------------------------------
+// Text parsing.  A data line counts when sscanf(line, "%u %u %f") == 3
+// (reference src/utils/load.h:219); the functions below give the same values
+// for the text between `p` and `end` without copying the line.
+// ---------------------------------------------------------------------------
+static inline bool is_space(char ch)
 {
-    char *end;
-    auto parse_u = [&](uint32_t &out) -> bool {
-        while (*p == ' ' || *p == '\t' || *p == '\n' || *p == '\v' || *p == '\f' || *p == '\r') ++p;
-        const char *q = p;
-        if (*q == '+' || *q == '-') ++q;
-        if (*q < '0' || *q > '9') return false;
-        errno = 0;
-        const unsigned long val = std::strtoul(p, &end, 10);
-        out = uint32_t(val);
-        p = end;
-        return true;
-    };
-    if (!parse_u(r) || !parse_u(c)) return false;
-    errno = 0;
-    const float f = std::strtof(p, &end);
-    if (end == p) return false;
-    v = f;
+    return ch == ' ' || ch == '\t' || ch == '\n' || ch == '\v' || ch == '\f' || ch == '\r';
+}
+
+// %u: white space, an optional sign, decimal digits.  Values beyond 64 bits
+// saturate as strtoul does; the result is then cut to 32 bits.
+static inline bool parse_u32(const char *&p, const char *end, uint32_t &out)
+{
+    while (p < end && is_space(*p)) ++p;
+    bool neg = false;
+    if (p < end && (*p == '+' || *p == '-')) { neg = *p == '-'; ++p; }
+    if (p >= end || *p < '0' || *p > '9') return false;
+    uint64_t v = 0;
+    bool over = false;
+    while (p < end && *p >= '0' && *p <= '9') {
+        const uint64_t d = uint64_t(*p - '0');
+        if (v > (UINT64_MAX - d) / 10u) over = true; else v = v * 10u + d;
+        ++p;
+    }
+    if (over) v = UINT64_MAX;
+    else if (neg) v = 0u - v;
+    out = uint32_t(v);
+    return true;
+}
+
+// strtof on a copy: every form that the quick path below leaves alone (inf, nan,
+// hexadecimal, more than 19 digits, exponents beyond +-22, results near the ends
+// of the float range).
+static bool parse_float_slow(const char *start, const char *end, float &out)
+{
+    char buf[1024];
+    size_t n = size_t(end - start);
+    if (n > sizeof buf - 1) n = sizeof buf - 1;
+    std::memcpy(buf, start, n);
+    buf[n] = 0;
+    char *stop;
+    const float f = std::strtof(buf, &stop);
+    if (stop == buf) return false;
+    out = f;
+    return true;
+}
+
+// %f.  Quick path: a decimal significand m < 2^53 and a power of ten up to
+// 10^22 are both exact doubles, so m * 10^e (or m / 10^-e) is the correctly
+// rounded double of the decimal value.  Rounding that double to float gives the
+// correctly rounded float unless the double sits exactly half way between two
+// floats (then the digits that were rounded away decide, and strtof is asked).
+static bool parse_float(const char *p, const char *end, float &out)
+{
+    static const double p10[23] = {1e0, 1e1, 1e2, 1e3, 1e4, 1e5, 1e6, 1e7, 1e8, 1e9, 1e10, 1e11,
+                                   1e12, 1e13, 1e14, 1e15, 1e16, 1e17, 1e18, 1e19, 1e20, 1e21, 1e22};
+    while (p < end && is_space(*p)) ++p;
+    const char *start = p;
+    bool neg = false;
+    if (p < end && (*p == '+' || *p == '-')) { neg = *p == '-'; ++p; }
+    if (p + 1 < end && p[0] == '0' && (p[1] == 'x' || p[1] == 'X')) return parse_float_slow(start, end, out);
+    uint64_t m = 0;
+    int e10 = 0, ndig = 0;
+    bool any = false;
+    while (p < end && *p >= '0' && *p <= '9') {
+        any = true;
+        if (m || *p != '0') { if (++ndig > 19) return parse_float_slow(start, end, out); m = m * 10u + uint64_t(*p - '0'); }
+        ++p;
+    }
+    if (p < end && *p == '.') {
+        ++p;
+        while (p < end && *p >= '0' && *p <= '9') {
+            any = true;
+            if (m || *p != '0') { if (++ndig > 19) return parse_float_slow(start, end, out); m = m * 10u + uint64_t(*p - '0'); }
+            --e10;
+            ++p;
+        }
+    }
+    if (!any) return parse_float_slow(start, end, out);          // inf, nan, or nothing
+    if (p < end && (*p == 'e' || *p == 'E')) {
+        const char *q = p + 1;
+        bool eneg = false;
+        if (q < end && (*q == '+' || *q == '-')) { eneg = *q == '-'; ++q; }
+        if (q < end && *q >= '0' && *q <= '9') {
+            int ev = 0;
+            while (q < end && *q >= '0' && *q <= '9') { if (ev < 100000) ev = ev * 10 + (*q - '0'); ++q; }
+            e10 += eneg ? -ev : ev;
+        }
+    }
+    if (m == 0) { out = neg ? -0.0f : 0.0f; return true; }
+    if (m >= (uint64_t(1) << 53) || e10 < -22 || e10 > 22) return parse_float_slow(start, end, out);
+    double d = double(m);
+    d = e10 < 0 ? d / p10[-e10] : d * p10[e10];
+    if (!(d > 1e-30 && d < 1e30)) return parse_float_slow(start, end, out);
+    uint64_t bits;
+    std::memcpy(&bits, &d, 8);
+    if ((bits & 0x1FFFFFFFull) == 0x10000000ull) return parse_float_slow(start, end, out);
+    out = float(neg ? -d : d);
     return true;
 }
 
@@ -113,45 +196,118 @@ struct Triples {
     std::vector<float> v;
 };
 
-// Reads the file the way the reference's fgets loop sees it: pieces of at most
-// 1023 characters ending at a newline (reference src/utils/load.h:155, 183, 215).
+// The whole file, read-only, through mmap (or read() where mapping fails).
+struct FileText {
+    const char *data = nullptr;
+    size_t size = 0;
+    bool mapped = false;
+    std::string owned;
+    ~FileText() { if (mapped) munmap(const_cast<char *>(data), size); }
+    bool open(const char *path)
+    {
+        const int fd = ::open(path, O_RDONLY);
+        if (fd < 0) return false;
+        struct stat st;
+        if (fstat(fd, &st) == 0 && S_ISREG(st.st_mode) && st.st_size > 0) {
+            void *m = mmap(nullptr, size_t(st.st_size), PROT_READ, MAP_PRIVATE, fd, 0);
+            if (m != MAP_FAILED) { data = static_cast<const char *>(m); size = size_t(st.st_size); mapped = true; }
+        }
+        if (!mapped) {
+            char buf[1 << 16];
+            ssize_t n;
+            while ((n = ::read(fd, buf, sizeof buf)) > 0) owned.append(buf, size_t(n));
+            data = owned.data(); size = owned.size();
+        }
+        ::close(fd);
+        return true;
+    }
+};
+
+// The reference reads with fgets into a 1024-byte buffer (src/utils/load.h:155,
+// 183, 215): a "line" is a piece of at most 1023 characters that ends after a
+// newline, and sscanf stops at a NUL byte.  [pos, return value) is the next piece.
+static inline size_t piece_end(const char *txt, size_t pos, size_t size)
+{
+    const size_t limit = std::min(size, pos + 1023);
+    const void *nl = std::memchr(txt + pos, '\n', limit - pos);
+    return nl ? size_t(static_cast<const char *>(nl) - txt) + 1 : limit;
+}
+
+static inline bool parse_piece(const char *b, const char *e, uint32_t &r, uint32_t &c, float &v)
+{
+    if (const void *nul = std::memchr(b, 0, size_t(e - b))) e = static_cast<const char *>(nul);
+    const char *p = b;
+    return parse_u32(p, e, r) && parse_u32(p, e, c) && parse_float(p, e, v);
+}
+
+// Header and size line on one thread, then the data lines in blocks that start
+// after a newline (every such position starts a piece), one block per worker.
 static int read_triples(const char *path, Triples &t, std::string &err)
 {
-    FILE *f = std::fopen(path, "rb");
-    if (!f) { err = std::string("cannot open file ") + path; return HSPMM_ERR_IO; }
-    std::string text;
-    {
-        char buf[1 << 16];
-        size_t n;
-        while ((n = std::fread(buf, 1, sizeof buf, f)) > 0) text.append(buf, n);
-    }
-    std::fclose(f);
-    size_t pos = 0;
-    std::string line;
-    auto next_line = [&]() -> bool {
-        if (pos >= text.size()) return false;
-        size_t e = pos;
-        const size_t limit = std::min(text.size(), pos + 1023);
-        while (e < limit && text[e] != '\n') ++e;
-        if (e < limit) ++e;                         // keep the newline, like fgets
-        line.assign(text, pos, e - pos);
-        pos = e;
-        return true;
-    };
+    FileText f;
+    if (!f.open(path)) { err = std::string("cannot open file ") + path; return HSPMM_ERR_IO; }
+    const char *txt = f.data;
+    const size_t size = f.size;
+    size_t pos = 0, line_b = 0, line_e = 0;
     bool have = false;
-    while (next_line()) { have = true; if (line[0] != '%') break; }     // load.h:183-187
-    unsigned rows, cols, nnz;
-    if (!have || std::sscanf(line.c_str(), "%u %u %u", &rows, &cols, &nnz) != 3) {   // load.h:190
-        err = std::string("cannot parse the size line of ") + path;
-        return HSPMM_ERR_IO;
+    while (pos < size) {                                                // load.h:183-187
+        line_b = pos; line_e = piece_end(txt, pos, size); pos = line_e;
+        have = true;
+        if (txt[line_b] != '%') break;
+    }
+    unsigned rows = 0, cols = 0, nnz = 0;
+    {
+        std::string line(have ? txt + line_b : "", have ? line_e - line_b : 0);
+        if (!have || std::sscanf(line.c_str(), "%u %u %u", &rows, &cols, &nnz) != 3) {   // load.h:190
+            err = std::string("cannot parse the size line of ") + path;
+            return HSPMM_ERR_IO;
+        }
     }
     t.rows = rows; t.cols = cols; t.declared = nnz;
-    t.r.reserve(nnz); t.c.reserve(nnz); t.v.reserve(nnz);
-    while (t.r.size() < nnz && next_line()) {                           // load.h:215
-        uint32_t r, c; float v;
-        if (parse_triple(line.c_str(), r, c, v)) {
-            t.r.push_back(r - 1u); t.c.push_back(c - 1u); t.v.push_back(v);   // load.h:221-222
+    const size_t body = pos;
+    const unsigned nw = worker_count(size - body, size_t(1) << 20);
+    std::vector<size_t> cut(nw + 1, size);
+    cut[0] = body;
+    for (unsigned i = 1; i < nw; ++i) {
+        size_t want = body + (size - body) / nw * i;
+        if (want < cut[i - 1]) want = cut[i - 1];
+        const void *nl = want < size ? std::memchr(txt + want, '\n', size - want) : nullptr;
+        cut[i] = nl ? size_t(static_cast<const char *>(nl) - txt) + 1 : size;
+    }
+    std::vector<Triples> part(nw);
+    auto work = [&](unsigned wi) {
+        Triples &o = part[wi];
+        const size_t b = cut[wi], e = cut[wi + 1];
+        const size_t guess = (e - b) / 12 + 16;
+        o.r.reserve(guess); o.c.reserve(guess); o.v.reserve(guess);
+        for (size_t p = b; p < e;) {
+            const size_t pe = piece_end(txt, p, e);
+            uint32_t r, c; float v;
+            if (parse_piece(txt + p, txt + pe, r, c, v)) {
+                o.r.push_back(r - 1u); o.c.push_back(c - 1u); o.v.push_back(v);   // load.h:221-222
+            }
+            p = pe;
         }
+    };
+    if (nw <= 1) work(0);
+    else {
+        std::vector<std::thread> th;
+        for (unsigned i = 0; i < nw; ++i) th.emplace_back(work, i);
+        for (auto &x : th) x.join();
+    }
+    // the reference stops reading once the declared number of entries is there (load.h:215)
+    size_t total = 0;
+    for (const Triples &o : part) total += o.r.size();
+    if (total > nnz) total = nnz;
+    t.r.resize(total); t.c.resize(total); t.v.resize(total);
+    size_t at = 0;
+    for (const Triples &o : part) {
+        const size_t n = std::min(o.r.size(), total - at);
+        std::memcpy(t.r.data() + at, o.r.data(), n * 4);
+        std::memcpy(t.c.data() + at, o.c.data(), n * 4);
+        std::memcpy(t.v.data() + at, o.v.data(), n * 4);
+        at += n;
+        if (at == total) break;
     }
     return HSPMM_OK;
 }
@@ -199,13 +355,15 @@ int hspmm_mtx_load(const char *path, int dtype, hspmm_csr *out)
             std::stable_sort(order.begin() + row_ptr[r], order.begin() + row_ptr[r + 1],
                              [&](uint32_t a, uint32_t b) { return t.c[a] < t.c[b]; });
     });
-    for (size_t i = 0; i < nnz; ++i) {
-        const uint32_t s = order[i];
-        col_idx[i] = t.c[s];
-        if (dtype == HSPMM_FP16) static_cast<uint16_t *>(values)[i] = float_to_half_bits(t.v[s]);
-        else if (dtype == HSPMM_BF16) static_cast<uint16_t *>(values)[i] = float_to_bf16_bits(t.v[s]);
-        else static_cast<float *>(values)[i] = t.v[s];
-    }
+    parallel_blocks(nnz, size_t(1) << 16, [&](size_t ib, size_t ie) {
+        for (size_t i = ib; i < ie; ++i) {
+            const uint32_t s = order[i];
+            col_idx[i] = t.c[s];
+            if (dtype == HSPMM_FP16) static_cast<uint16_t *>(values)[i] = float_to_half_bits(t.v[s]);
+            else if (dtype == HSPMM_BF16) static_cast<uint16_t *>(values)[i] = float_to_bf16_bits(t.v[s]);
+            else static_cast<float *>(values)[i] = t.v[s];
+        }
+    });
     out->rows = t.rows; out->cols = t.cols; out->nnzs = uint32_t(nnz);
     out->row_ptr = row_ptr; out->col_idx = col_idx; out->values = values;
     return HSPMM_OK;

@@ -81,6 +81,71 @@ def test_loader_special_values_and_short_files(hs, oracle, tmp_path):
         assert a["values"].tobytes() == o["values"].tobytes()
 
 
+def test_loader_number_forms_equal_the_c_library(hs, oracle, tmp_path):
+    """The loader's own number parsing against sscanf (the oracle reads with it):
+    digit counts on both sides of what fits a double exactly, exponents on both sides
+    of 10^22, ties between two floats, subnormal and overflowing values, signs,
+    hexadecimal, inf and nan, indices with signs and beyond 32 bits."""
+    rng = np.random.default_rng(77)
+    vals = ["0", "-0", "+0.0", ".5", "5.", "-.25e1", "+1.5E+3", "1e", "1e+", "2.5e-3x", "inf", "-inf", "nan", "INFINITY",
+            "0x1p3", "0x1.8p-2", "1e-42", "1e-46", "3.4028235e38", "3.4028236e38", "1e40", "-1e40",
+            "16777217", "16777217.0000000001", "9007199254740993", "0.1", "123456789012345678901234567890",
+            "0.000000000000000000000000000001", "1e22", "1e23", "8.5e-23", "1.17549435e-38", "1.17549421e-38"]
+    for _ in range(3000):
+        nd = int(rng.integers(1, 26))
+        digits = "".join(rng.choice(list("0123456789"), nd))
+        point = int(rng.integers(0, nd + 1))
+        txt = digits[:point] + "." + digits[point:] if rng.random() < 0.7 else digits
+        if rng.random() < 0.6:
+            txt += "e%d" % int(rng.integers(-45, 40))
+        vals.append(("-" if rng.random() < 0.3 else "") + txt)
+    # exact ties: the midpoint of two neighbouring floats, written out in full
+    f = np.abs(rng.normal(size=400).astype(np.float32)) * np.float32(10.0) ** rng.integers(-8, 9, 400).astype(np.float32)
+    mid = (f.astype(np.float64) + np.nextafter(f, np.float32(np.inf)).astype(np.float64)) / 2
+    from decimal import Decimal
+    for m in mid:
+        d = Decimal(float(m))
+        vals += [format(d, "f"), format(d + d * Decimal(10) ** -25, "f"), format(d - d * Decimal(10) ** -25, "f")]
+    rows = len(vals)
+    p = tmp_path / "forms.mtx"
+    with open(p, "w") as fh:
+        fh.write("%d %d %d\n" % (rows, 7, rows + 6))
+        for i, v in enumerate(vals):
+            fh.write("%d %d %s\n" % (i + 1, 1 + i % 7, v))
+        fh.write("+3 +2 1.5\n1 -4294967294 2.5\n4294967297 4294967298 3.5\n")   # signs and wrap-around: (3,2) (1,2) (1,2)
+        fh.write("2 x 1\n2 3\n 5\t6\t7.5 trailing words\n")
+    for dt in (1, 0):
+        a = hs.mtx_load(str(p), dt)
+        o = oracle.mtx_read(str(p), DT[dt])
+        assert a["nnzs"] == o["nnzs"] and a["nnzs"] >= rows
+        assert np.array_equal(a["row_ptr"], o["row_ptr"]) and np.array_equal(a["col_idx"], o["col_idx"])
+        assert a["values"].tobytes() == o["values"].tobytes()
+
+
+def test_loader_blocks_of_a_large_file_equal_the_oracle(hs, oracle, tmp_path):
+    # several megabytes, so that the data lines are parsed in more than one block; a few
+    # over-long lines (cut into 1023-character pieces like fgets does) and blank lines
+    rng = np.random.default_rng(78)
+    rows, cols, nnz = 3000, 2500, 400000
+    flat = rng.choice(rows * cols, size=nnz, replace=False)
+    v = rng.normal(size=nnz)
+    p = tmp_path / "big.mtx"
+    with open(p, "w") as fh:
+        fh.write("%%MatrixMarket matrix coordinate real general\n%d %d %d\n" % (rows, cols, nnz))
+        for i in range(nnz):
+            if i % 50021 == 7:
+                fh.write(" " * 2500 + "\n")
+            if i % 70001 == 11:
+                fh.write("\n")
+            fh.write("%d %d %.8g\n" % (flat[i] // cols + 1, flat[i] % cols + 1, v[i]))
+    assert os.path.getsize(p) > 6 << 20
+    a = hs.mtx_load(str(p), 0)
+    o = oracle.mtx_read(str(p), "fp16")
+    assert a["nnzs"] == o["nnzs"] == nnz
+    assert np.array_equal(a["row_ptr"], o["row_ptr"]) and np.array_equal(a["col_idx"], o["col_idx"])
+    assert a["values"].tobytes() == o["values"].tobytes()
+
+
 def test_loader_errors(hs, tmp_path):
     with pytest.raises(hs.HspmmError) as e:
         hs.mtx_load(str(tmp_path / "nope.mtx"), 0)
