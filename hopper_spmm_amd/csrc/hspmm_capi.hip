@@ -159,13 +159,14 @@ int build_and_upload_partition(hspmm_plan *p, int level)
 {
     hspmm_plan::DevPartition &dp = p->parts[level];
     if (dp.built || p->W == 0) return HSPMM_OK;
-    double window_cost = 1.5, slack = 0.35;
+    double window_cost = 1.5, slack = 0.35, margin = 32.0;
     if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);   // tuning overrides
     if (const char *e = std::getenv("HSPMM_SLACK")) slack = std::atof(e);
+    if (const char *e = std::getenv("HSPMM_WHOLE_WINDOW_MARGIN")) margin = std::atof(e);
     uint32_t target = uint32_t(choose_ranges(p)) >> level;
     const uint32_t floor_ranges = uint32_t(p->compute_units) * 4u;       // at least one range per SIMD
     if (target < floor_ranges) target = std::min<uint32_t>(floor_ranges, uint32_t(choose_ranges(p)));
-    dp.part = hspmm::build_partition(p->n_units, p->h_unitOffset.data(), target, window_cost, slack);
+    dp.part = hspmm::build_partition(p->n_units, p->h_unitOffset.data(), target, window_cost, slack, margin);
     const auto &part = dp.part;
     std::vector<uint32_t> rw(part.ranges.size() * hspmm::kRangeWords, 0u);
     for (size_t i = 0; i < part.ranges.size(); ++i) {

@@ -333,6 +333,52 @@ def test_plan_reuse_is_deterministic(torch_cuda, hs, oracle):
     plan.close()
 
 
+def test_run_captured_in_a_hip_graph_replays_correctly(torch_cuda, hs, oracle):
+    """After one eager call (which sizes the plan's scratch memory) hspmm_run only
+    launches kernels, so a stream capture records it; every replay, with eager work
+    and new contents of B in between, must give what the eager call gives."""
+    torch = torch_cuda
+    rng = np.random.default_rng(15)
+    for dtype in (0, 1):
+        A = random_csr(rng, 400, 4000, 0.003, dtype, 0.1, (3, 200))
+        b = convert(hs, A)
+        hs.configure(producer_warp_group_num=16)
+        try:
+            plan = hs.Plan(b)
+        finally:
+            hs.configure()
+        assert plan.info()["n_split_windows"] > 0              # two kernels per call
+        N = 64
+        tt = torch.int16 if dtype == 0 else torch.float32
+        Bs = [make_b(rng, 4000, N, dtype) for _ in range(3)]
+        as_t = (lambda x: torch.from_numpy(x.view(np.int16))) if dtype == 0 else torch.from_numpy
+        dB = as_t(Bs[0]).cuda()
+        dC = torch.empty((400, N), dtype=tt, device="cuda")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            plan.run(dB.data_ptr(), dC.data_ptr(), N, side.cuda_stream)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)
+        for rep in range(6):
+            Bh = Bs[rep % 3]
+            dB.copy_(as_t(Bh).cuda())
+            dC.fill_(0x7E01 if dtype == 0 else float("nan"))
+            (dB.float().sum() + 1).item()                       # eager work and a synchronisation between replays
+            graph.replay()
+            torch.cuda.synchronize()
+            got = dC.cpu().numpy()
+            got = got.view(np.uint16) if dtype == 0 else got
+            want = gpu_spmm(torch, hs, b, Bh, N, plan=plan)
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "replay %d" % rep
+            ref, mag = oracle_spmm(oracle, A, Bh, N)
+            assert_parity(got, ref, mag, dtype, "graph replay %d" % rep)
+        del graph
+        plan.close()
+
+
 def test_bench_entry_point_and_errors(torch_cuda, hs, oracle):
     torch = torch_cuda
     rng = np.random.default_rng(3)
