@@ -91,6 +91,17 @@ struct hspmm_plan {
     };
     DevPartition parts[3];
     std::vector<uint32_t> h_unitOffset;
+    // LDS-panel kernels (matrices whose windows touch a large share of the columns):
+    // the unit stream re-tiled panel by panel, built by hspmm_create when it pays
+    struct Panel {
+        bool built = false;
+        uint32_t n_panels = 0, n_steps = 0;
+        uint32_t *d_poff = nullptr, *d_ids = nullptr, *d_step_panel = nullptr;
+        void *d_tiles = nullptr;
+        uint32_t *d_split = nullptr, *d_fix_slots = nullptr;    // one split entry per unit, for the chunk sums
+        uint32_t split_chunks = 0;                               // chunk count d_split was built for
+        size_t fix_slot_count = 0;
+    } panel;
     float *d_scratch = nullptr;
     size_t scratch_bytes = 0;
     uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
@@ -279,6 +290,151 @@ std::vector<uint32_t> lane_order_tiles(const StepStream &st, int dtype, const ui
     return out;
 }
 
+
+// Re-tiles the matrix panel by panel for the LDS-panel kernels (spmm_panel_kernel.hpp):
+// inside every window the columns of one panel of kPanelRows columns get tiles of
+// their own.  Every step carries the number of panels it lies behind the step in
+// front of it (4 bits; a longer run of panels without a step gets an all-zero step
+// every 15 panels).  Returns false when the kernels would not pay (criteria inside).
+bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *rowOffset, const uint32_t *tcA2B,
+                        const void *data, bool forced, int *rc_out)
+{
+    *rc_out = HSPMM_OK;
+    const uint32_t cw = p->cw, W = p->W;
+    const uint32_t KP = hspmm::kPanelRows;
+    const uint32_t NP = (p->cols + KP - 1) / KP;
+    const uint32_t U = uint32_t(st.unitRow.size());
+    constexpr uint32_t kMaxJump = 15;
+    if (U == 0 || NP == 0) return false;
+    // worth it when a unit has a few steps in every panel it meets: the panel image is
+    // then read from LDS several times per load from the L2
+    if (!forced && double(st.n_steps) < 2.0 * double(U) * double(NP)) return false;
+    if (uint64_t(U) * (NP + 1) > (1ull << 28)) return false;
+    const size_t es = p->elem, tile_bytes = size_t(8) * cw * es;
+    std::vector<uint32_t> rt_rowOffset(size_t(W) + 1, 0u), rt_ids, rt_panel;
+    std::vector<uint8_t> rt_data;
+    rt_ids.reserve(size_t(p->T) * cw * 5 / 4);
+    rt_panel.reserve(size_t(p->T) * 5 / 4);
+    rt_data.reserve(size_t(p->T) * tile_bytes * 5 / 4);
+    const uint8_t *src_data = static_cast<const uint8_t *>(data);
+    for (uint32_t w = 0; w < W; ++w) {
+        const uint32_t t0 = rowOffset[w], t1 = rowOffset[w + 1];
+        const uint32_t *col = tcA2B + size_t(t0) * cw;
+        uint32_t nreal = (t1 - t0) * cw;
+        while (nreal && col[nreal - 1] == HSPMM_IDX_MAX) --nreal;
+        uint32_t i = 0, tiles = 0, last_pn = 0;
+        while (i < nreal) {
+            const uint32_t pn = col[i] / KP, a = i;
+            while (i < nreal && col[i] / KP == pn) ++i;
+            while (tiles && pn - last_pn > kMaxJump) {           // all-zero step that only carries the jump
+                last_pn += kMaxJump;
+                rt_ids.resize(rt_ids.size() + cw, 0u);
+                rt_data.resize(rt_data.size() + tile_bytes, 0);
+                rt_panel.push_back(last_pn);
+                ++tiles;
+            }
+            const uint32_t nt = (i - a + cw - 1) / cw;
+            const size_t id_at = rt_ids.size(), data_at = rt_data.size();
+            rt_ids.resize(id_at + size_t(nt) * cw);
+            rt_data.resize(data_at + size_t(nt) * tile_bytes, 0);
+            rt_panel.resize(rt_panel.size() + nt, pn);
+            for (uint32_t k = 0; k < nt * cw; ++k) {
+                const uint32_t srci = a + k;
+                if (srci < i) {
+                    rt_ids[id_at + k] = col[srci] - pn * KP;     // row inside the panel
+                    const uint8_t *st_tile = src_data + size_t(t0 + srci / cw) * tile_bytes;
+                    uint8_t *dt_tile = rt_data.data() + data_at + size_t(k / cw) * tile_bytes;
+                    for (uint32_t r = 0; r < 8; ++r)
+                        std::memcpy(dt_tile + (size_t(r) * cw + k % cw) * es, st_tile + (size_t(r) * cw + srci % cw) * es, es);
+                } else {
+                    rt_ids[id_at + k] = rt_ids[id_at + k - 1];   // padding: the row in front, its tile column is zero
+                }
+            }
+            tiles += nt;
+            last_pn = pn;
+        }
+        rt_rowOffset[w + 1] = rt_rowOffset[w] + tiles;
+    }
+    // the same units as the gather kernels walk, with the re-tiled step counts
+    StepStream ps;
+    ps.G = st.G; ps.unitRow = st.unitRow; ps.unitWindow = st.unitWindow; ps.n_paired = st.n_paired;
+    ps.unitOffset.assign(1, 0u);
+    for (uint32_t u = 0; u < U; ++u) {
+        const uint32_t w = st.unitWindow[u];
+        ps.unitOffset.push_back(ps.unitOffset.back() + (rt_rowOffset[w + 1] - rt_rowOffset[w]));
+    }
+    ps.n_steps = ps.unitOffset.back();
+    // padding inside every panel must not eat the gain
+    if (!forced && double(ps.n_steps) > 1.35 * double(st.n_steps)) return false;
+    // poff[u][pn]: first step of unit u at or behind panel pn; step_panel[s]: panel of step s
+    std::vector<uint32_t> poff(size_t(U) * (NP + 1)), step_panel(ps.n_steps ? ps.n_steps : 1, 0u);
+    // per step four words; word g packs the panel rows quarter-wave g reads, 7 bits each (16-bit types:
+    // ids 4g..4g+3, fp32: ids g and g + 4), and in bits 28..31 the panels the step lies behind its predecessor
+    std::vector<uint32_t> ids(size_t(ps.n_steps) * 4u);
+    for (uint32_t u = 0; u < U; ++u) {
+        const uint32_t t0 = rt_rowOffset[st.unitWindow[u]], n = ps.unitOffset[u + 1] - ps.unitOffset[u];
+        uint32_t *po = poff.data() + size_t(u) * (NP + 1);
+        uint32_t at = 0;
+        for (uint32_t pn = 0; pn <= NP; ++pn) {
+            while (at < n && rt_panel[t0 + at] < pn) ++at;
+            po[pn] = ps.unitOffset[u] + at;
+        }
+        for (uint32_t i = 0; i < n; ++i) {
+            const uint32_t *src = rt_ids.data() + size_t(t0 + i) * cw;
+            uint32_t *dst = ids.data() + size_t(ps.unitOffset[u] + i) * 4u;
+            const uint32_t jump = i ? rt_panel[t0 + i] - rt_panel[t0 + i - 1] : 0u;     // <= kMaxJump by construction
+            step_panel[ps.unitOffset[u] + i] = rt_panel[t0 + i];
+            for (uint32_t g = 0; g < 4; ++g)
+                dst[g] = (cw == 16 ? (src[4 * g] | src[4 * g + 1] << 7 | src[4 * g + 2] << 14 | src[4 * g + 3] << 21)
+                                   : (src[g] | src[g + 4] << 7)) | jump << 28;
+        }
+    }
+    hspmm_plan::Panel &pl = p->panel;
+    int rc;
+    if ((rc = upload(&pl.d_poff, poff.data(), poff.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
+    if ((rc = upload(&pl.d_step_panel, step_panel.data(), step_panel.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
+    if ((rc = upload(&pl.d_ids, ids.data(), ids.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
+    {
+        const std::vector<uint32_t> tiles = lane_order_tiles(ps, p->dtype, rt_rowOffset.data(), rt_data.data());
+        uint32_t *dt = nullptr;
+        if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
+        pl.d_tiles = dt;
+    }
+    pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.built = true;
+    return true;
+}
+
+// Split table for the chunk sums of the panel kernels: unit u owns slots
+// u * chunks .. u * chunks + chunks - 1, added in that order.
+int ensure_panel_split(hspmm_plan *p, uint32_t chunks)
+{
+    hspmm_plan::Panel &pl = p->panel;
+    const size_t slots = size_t(p->n_units) * chunks;
+    if (slots > pl.fix_slot_count) {
+        if (pl.d_fix_slots) { HSPMM_HIP(hipFree(pl.d_fix_slots)); pl.d_fix_slots = nullptr; pl.fix_slot_count = 0; }
+        std::vector<uint32_t> ident(slots);
+        for (size_t i = 0; i < slots; ++i) ident[i] = uint32_t(i);
+        size_t dummy = 0;
+        int rc = upload(&pl.d_fix_slots, ident.data(), ident.size(), &dummy);
+        if (rc) return rc;
+        pl.fix_slot_count = slots;
+    }
+    if (pl.split_chunks != chunks) {
+        if (pl.d_split) { HSPMM_HIP(hipFree(pl.d_split)); pl.d_split = nullptr; pl.split_chunks = 0; }
+        std::vector<uint32_t> sp(size_t(p->n_units) * hspmm::kFixWords, 0u);
+        for (uint32_t u = 0; u < p->n_units; ++u) {
+            sp[size_t(u) * hspmm::kFixWords + 0] = u;
+            sp[size_t(u) * hspmm::kFixWords + 1] = u * chunks;
+            sp[size_t(u) * hspmm::kFixWords + 2] = chunks;
+        }
+        size_t dummy = 0;
+        int rc = upload(&pl.d_split, sp.data(), sp.size(), &dummy);
+        if (rc) return rc;
+        pl.split_chunks = chunks;
+    }
+    return HSPMM_OK;
+}
+
 struct Choice {
     bool scalar;
     int layout, V, block_feat;
@@ -374,7 +530,7 @@ void hspmm_get_config(int *buffer_stage, int *consumer_warp_num, int *producer_w
 
 int hspmm_set_kernel_mode(int mode)
 {
-    if (mode < 0 || mode > 3) return fail(HSPMM_ERR_INVALID, "kernel mode %d outside 0..3", mode);
+    if (mode < 0 || mode > 4) return fail(HSPMM_ERR_INVALID, "kernel mode %d outside 0..4", mode);
     std::lock_guard<std::mutex> lk(g_cfg_mutex);
     g_cfg.kernel_mode = mode;
     return HSPMM_OK;
@@ -479,6 +635,11 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         }
         p->h_unitOffset = st.unitOffset;
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
+        if (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 4) {
+            int prc = HSPMM_OK;
+            (void)build_panel_stream(p, st, rowOffset, tcA2B, data, p->cfg.kernel_mode == 4, &prc);
+            if (prc) return bail(prc);
+        }
     }
     *out = p;
     return HSPMM_OK;
@@ -540,6 +701,9 @@ void hspmm_destroy(hspmm_plan *p)
     if (p->d_tiles != p->d_data) (void)hipFree(p->d_tiles);
     (void)hipFree(p->d_data); (void)hipFree(p->d_unitOffset); (void)hipFree(p->d_unitRow); (void)hipFree(p->d_ids);
     for (auto &dp : p->parts) { (void)hipFree(dp.d_ranges); (void)hipFree(dp.d_split); (void)hipFree(dp.d_fix_slots); }
+    (void)hipFree(p->panel.d_poff); (void)hipFree(p->panel.d_ids); (void)hipFree(p->panel.d_tiles);
+    (void)hipFree(p->panel.d_step_panel);
+    (void)hipFree(p->panel.d_split); (void)hipFree(p->panel.d_fix_slots);
     (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive);
     delete p;
 }
@@ -550,6 +714,54 @@ int hspmm_run(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream)
 }
 
 }  // extern "C"
+
+// Launch through the LDS-panel kernels.  Grid = row blocks x feature blocks x chunks of
+// panels; the chunk count is what it takes to have about two workgroups per compute unit.
+static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStream_t s, hipEvent_t mid)
+{
+    const hspmm_plan::Panel &pl = p->panel;
+    hspmm::PanelArgs pa{};
+    pa.unitRow = p->d_unitRow; pa.poff = pl.d_poff; pa.step_panel = pl.d_step_panel; pa.ids = pl.d_ids;
+    pa.tiles = pl.d_tiles; pa.n_steps = pl.n_steps;
+    pa.B = dB; pa.C = dC;
+    pa.n_units = p->n_units; pa.rows = p->rows; pa.cols = p->cols; pa.N = N;
+    pa.n_feat_blocks = N / (hspmm::kPanelRowBytes / p->elem);
+    pa.n_panels = pl.n_panels;
+    // 16 waves per workgroup fill a compute unit (two workgroups with 64 KB of LDS each
+    // do not become resident together): 14 units where the LDS reads bind (paired
+    // units), 12 otherwise, which spreads the consumer waves evenly over the SIMDs.
+    int units = p->G == 2 ? 14 : 12;
+    if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) {                                      // tuning overrides
+        const int v = std::atoi(e);
+        units = (v == 14 || v == 12 || v == 8) ? v : 6;
+    }
+    // chunks of panels: as many as keep the workgroups within one round over the compute units
+    const uint64_t row_blocks = (uint64_t(p->n_units) + units - 1) / units;
+    const uint64_t base = row_blocks * pa.n_feat_blocks;
+    uint64_t chunks = uint64_t(p->compute_units) / base;
+    if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) chunks = uint64_t(std::atoi(e));
+    if (chunks < 1) chunks = 1;
+    if (chunks > pl.n_panels) chunks = pl.n_panels;
+    pa.panels_per_chunk = uint32_t((pl.n_panels + chunks - 1) / chunks);
+    pa.n_chunks = (pl.n_panels + pa.panels_per_chunk - 1) / pa.panels_per_chunk;
+    if (base * pa.n_chunks > 0x7FFFFFFFull)
+        return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many workgroups", N);
+    hspmm::KernelArgs ka{};
+    if (pa.n_chunks > 1) {
+        int rc = ensure_panel_split(p, pa.n_chunks);
+        if (rc) return rc;
+        const size_t need = size_t(p->n_units) * pa.n_chunks * pa.n_feat_blocks * 4u * size_t(p->G) * 64u * 16u;
+        if ((rc = ensure_scratch(p, need))) return rc;
+        pa.scratch = p->d_scratch;
+        ka.unitRow = p->d_unitRow; ka.ids = pl.d_ids; ka.tiles = pl.d_tiles;
+        ka.split = pl.d_split; ka.fix_slots = pl.d_fix_slots; ka.scratch = p->d_scratch;
+        ka.C = dC; ka.B = dB;
+        ka.n_split = p->n_units; ka.n_units = p->n_units; ka.rows = p->rows; ka.N = N;
+        ka.n_feat_blocks = pa.n_feat_blocks;
+    }
+    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, p->G, pa, ka, units, s, mid));
+    return HSPMM_OK;
+}
 
 // mid: when not null, an event recorded between the main kernel and the kernel
 // that adds the partial sums of split windows.
@@ -562,10 +774,23 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     if (!dB && p->W) return fail(HSPMM_ERR_INVALID, "null B");
     if (reinterpret_cast<uintptr_t>(dC) % p->elem || reinterpret_cast<uintptr_t>(dB) % p->elem)
         return fail(HSPMM_ERR_INVALID, "B and C must be aligned to the element size");
+    {
+        // the plan's arrays live on the device that was current in hspmm_create
+        int dev = -1;
+        HSPMM_HIP(hipGetDevice(&dev));
+        if (dev != p->device)
+            return fail(HSPMM_ERR_INVALID, "the plan was created on device %d, the current device is %d", p->device, dev);
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (p->W == 0) {
         HSPMM_HIP(hspmm::launch_fill_zero(dC, size_t(p->rows) * N * p->elem, s));
         return HSPMM_OK;
+    }
+    if (p->panel.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 4)) {
+        // LDS-panel kernels: a workgroup covers 256 bytes of every B row with 16-byte accesses
+        const uint32_t block_feat = hspmm::kPanelRowBytes / p->elem;
+        const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
+        if (N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid);
     }
     const Choice c = choose_kernel(p, dB, dC, N);
     hspmm::KernelArgs ka{};
@@ -681,6 +906,8 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_units = p->n_units;
     info->n_paired_units = p->n_paired;
     info->device_bytes = uint64_t(p->fixed_bytes) + uint64_t(p->scratch_bytes);
+    info->n_panels = p->panel.built ? p->panel.n_panels : 0u;
+    info->n_panel_steps = p->panel.built ? p->panel.n_steps : 0u;
     return HSPMM_OK;
 }
 

@@ -51,6 +51,29 @@ constexpr int kDtypeF16 = 0, kDtypeF32 = 1, kDtypeBf16 = 2;
 hipError_t launch_spmm_mfma(int dtype, int layout, int G, const KernelArgs &ka, int V, int prefetch, bool narrow,
                             int waves_per_group, hipStream_t s, hipEvent_t mid);
 hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s);
+
+// LDS-panel kernels (spmm_panel_kernel.hpp).
+constexpr uint32_t kPanelRows = 128;           // B rows per panel
+constexpr uint32_t kPanelRowBytes = 256;       // bytes of a B row one workgroup covers (128 halves / 64 floats)
+constexpr uint32_t kPanelBytes = kPanelRows * kPanelRowBytes;
+
+struct PanelArgs {
+    const uint32_t *unitRow;     // n_units: first matrix row of the unit | 1 if it is a pair of windows
+    const uint32_t *poff;        // n_units x (n_panels + 1): first step of the unit at or behind every panel
+    const uint32_t *step_panel;  // per step: its panel
+    const uint32_t *ids;         // per step four words: the rows (inside the panel) each quarter-wave reads, 7 bits
+                                 // each; bits 28..31: panels between the step and the one in front of it
+    const void     *tiles;       // per step, lane order
+    float          *scratch;     // partial sums [unit * n_chunks + chunk][feature block][acc reg][lane]
+    const void     *B;
+    void           *C;
+    uint32_t n_units, n_steps, rows, cols, N, n_feat_blocks, n_panels, n_chunks, panels_per_chunk;
+};
+
+// units: 6, 8, 12 or 14 units (consumer waves) per workgroup; 2 more waves copy B to LDS.  ka: arguments of the kernel that adds
+// the chunk sums (split table with one entry per unit), used when pa.n_chunks > 1.
+hipError_t launch_spmm_panel(int dtype, int G, const PanelArgs &pa, const KernelArgs &ka, int units, hipStream_t s,
+                             hipEvent_t mid);
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
 
 }  // namespace hspmm

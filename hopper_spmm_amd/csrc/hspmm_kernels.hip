@@ -1,7 +1,8 @@
 // gfx950 (MI355X) kernels for C = A * B with A in the condensed 8-row-window
 // tile format (reference src/utils/class.h:74-85): the all-shapes scalar kernel,
 // the clear kernel, and the dispatch to the MFMA kernels (spmm_mfma_kernel.hpp,
-// instantiated in spmm_mfma_<type>_g<n>.hip).
+// instantiated in spmm_mfma_<type>_g<n>.hip; spmm_panel_kernel.hpp, instantiated in
+// spmm_panel_<type>.hip).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "hspmm_device.h"
@@ -87,6 +88,18 @@ hipError_t launch_spmm_mfma(int dtype, int layout, int G, const KernelArgs &ka, 
                       : launch_mfma_bf16_g1(layout, ka, V, prefetch, narrow, waves_per_group, s, mid);
     return G == 2 ? launch_mfma_f16_g2(layout, ka, V, prefetch, narrow, waves_per_group, s, mid)
                   : launch_mfma_f16_g1(layout, ka, V, prefetch, narrow, waves_per_group, s, mid);
+}
+
+hipError_t launch_panel_f16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid);
+hipError_t launch_panel_bf16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid);
+hipError_t launch_panel_f32(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid);
+
+hipError_t launch_spmm_panel(int dtype, int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s,
+                             hipEvent_t mid)
+{
+    if (dtype == kDtypeF32) return launch_panel_f32(G, pa, ka, waves, s, mid);
+    if (dtype == kDtypeBf16) return launch_panel_bf16(G, pa, ka, waves, s, mid);
+    return launch_panel_f16(G, pa, ka, waves, s, mid);
 }
 
 hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s)

@@ -1,0 +1,15 @@
+// Instantiations of the LDS-panel kernel: element type f16.
+#include <hip/hip_runtime.h>
+#include "spmm_panel_kernel.hpp"
+
+namespace hspmm {
+
+template <int G> using PanelTile = Fp16X4<4, G>;
+
+hipError_t launch_panel_f16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid)
+{
+    return G == 2 ? launch_panel_nw<PanelTile<2>>(pa, ka, waves, s, mid)
+                  : launch_panel_nw<PanelTile<1>>(pa, ka, waves, s, mid);
+}
+
+}  // namespace hspmm

@@ -1,0 +1,244 @@
+// gfx950 (MI355X) kernel family for matrices whose row windows touch a large share
+// of all columns (pruned dense weights, block-clustered weights): the rows of B are
+// staged through LDS once per workgroup and shared by all its waves, instead of
+// every wave gathering its own copy from the L2 (spmm_mfma_kernel.hpp).  It serves
+// the same entry point, the reference's fp16_spmm (reference src/fp16.cu:221-281),
+// and what the reference sketches with its producer / consumer shared-memory ring
+// (src/fp16.cu:56-175).
+//
+//   * Columns are cut into panels of kPanelRows.  The plan re-tiles every unit (a
+//     window, or a pair of windows with one column list) panel by panel: the
+//     unit's columns inside a panel are condensed into tiles of their own, so no
+//     tile straddles a panel; ids are row numbers inside the panel (one byte each,
+//     the four - fp32: two - ids of a lane in one word).  poff[u][p] is the first
+//     step of unit u in panel p.
+//   * A workgroup owns NC consecutive units (one per consumer wave), one block of
+//     256 bytes of every B row (128 halves / 64 floats of the feature dimension)
+//     and a contiguous chunk of panels.  Per panel its producer waves copy the
+//     panel's slice of B (kPanelRows x 256 bytes, coalesced 16-byte loads) to LDS;
+//     every consumer wave then runs the steps its unit has in the panel, reading
+//     its four (two for fp32) B rows per step from LDS with 16-byte reads: the 16
+//     lanes of a quarter-wave read one whole 256-byte row, so the reads of a
+//     quarter never share a bank.
+//   * Two LDS buffers and one barrier per panel: the producers fill the buffer of
+//     panel p+1 while the consumers multiply panel p.
+//   * The unit's tiles and ids stream from global memory through a small register
+//     ring, as in the gather kernels.
+//   * With more than one chunk of panels per unit, every chunk leaves fp32 partial
+//     sums in scratch slots that spmm_fixup_kernel adds in chunk order.
+#pragma once
+#include "spmm_mfma_kernel.hpp"
+
+namespace hspmm {
+
+// B rows a lane reads per step: four for the 16-bit types, two for fp32.
+template <class TT> struct PanelRows { static constexpr int value = 4; };
+template <int V, int G> struct PanelRows<Fp32Tile<V, G>> { static constexpr int value = 2; };
+
+// One barrier of the workgroup with the LDS writes in front of it visible behind it.
+__device__ __forceinline__ void panel_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// NC consumer waves (one unit each) and NPW producer waves that do nothing but copy
+// panel images to LDS: the consumers' register ring of tile / id loads then never
+// has to wait for a panel load (vector loads return in order, and a wave that had
+// both kinds in flight would drain its ring at every panel).
+template <class TT, int NC, int NPW>
+__global__ __launch_bounds__((NC + NPW) * 64)
+void spmm_panel_kernel(const PanelArgs pa)
+{
+    constexpr int G = TT::G, V = TT::V, NACC = G * V;
+    constexpr int kPieces = int(kPanelBytes / 16u) / (NPW * 64);   // 16-byte pieces of a panel per producer thread
+    static_assert(V == 4, "a lane owns 16 bytes of a B row");
+    static_assert(kPieces * NPW * 64 * 16 == int(kPanelBytes), "panel must divide among the producers");
+    __shared__ __attribute__((aligned(16))) char smem[2 * kPanelBytes];
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // blockIdx.x = (row block * feature blocks + feature block) * chunks + chunk
+    const uint32_t per_rb = pa.n_feat_blocks * pa.n_chunks;
+    const uint32_t rb = blockIdx.x / per_rb;
+    const uint32_t rest = blockIdx.x - rb * per_rb;
+    const uint32_t fb = rest / pa.n_chunks;
+    const uint32_t chunk = rest - fb * pa.n_chunks;
+    const uint32_t p_begin = chunk * pa.panels_per_chunk;
+    const uint32_t p_end = umin32(p_begin + pa.panels_per_chunk, pa.n_panels);
+    const size_t row_bytes = size_t(pa.N) * TT::kElem;
+
+    if (wave >= uint32_t(NC)) {
+        // ---- producer: panel q goes to buffer q & 1, then the barrier that releases it.
+        // Buffer q & 1 was last read for panel q - 2, which every consumer left before
+        // the barrier of panel q - 1.
+        const uint32_t pt = threadIdx.x - uint32_t(NC) * 64u;       // 0 .. NPW*64-1
+        // piece c = pt + i * NPW*64 is bytes [16c, 16c + 16) of the image: row c / 16, 16-byte column c % 16
+        const char *b_col = reinterpret_cast<const char *>(pa.B) + size_t(fb) * kPanelRowBytes + (pt & 15u) * 16u;
+        const uint32_t piece_row0 = pt >> 4;
+        // The loads of panel q + 1 are in flight (in registers) while the consumers multiply
+        // panel q - 1 .. q: a panel has a whole barrier period to arrive.
+        u32x4 X[kPieces];
+        auto issue = [&](uint32_t q) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < kPieces; ++i) {
+                uint32_t row = q * kPanelRows + piece_row0 + uint32_t(i) * (NPW * 4);
+                row = umin32(row, pa.cols - 1u);                   // rows past the matrix are never referenced
+                X[i] = *reinterpret_cast<const u32x4 *>(b_col + size_t(row) * row_bytes);
+            }
+        };
+        issue(p_begin);
+        for (uint32_t q = p_begin; q < p_end; ++q) {
+            char *img = smem + (q & 1u) * kPanelBytes + pt * 16u;
+#pragma unroll
+            for (int i = 0; i < kPieces; ++i)
+                *reinterpret_cast<u32x4 *>(img + uint32_t(i) * (NPW * 64 * 16)) = X[i];
+            if (q + 1u < p_end) issue(q + 1u);
+            panel_barrier();
+        }
+        return;
+    }
+
+    // ---- consumer
+    const uint32_t u = rb * NC + wave;
+    const bool has_unit = u < pa.n_units;
+    const const_u32_ptr poff = as_const(pa.poff) + size_t(has_unit ? u : 0u) * (pa.n_panels + 1u);
+
+    typename TT::Lane L;
+    L.init(lane, pa.tiles, pa.ids);
+    const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
+    char *c_lane = reinterpret_cast<char *>(pa.C) + size_t(feat) * TT::kElem;
+
+    // steps [t0, t1) of the unit lie in this chunk of panels; a wave without a unit has none
+    const uint32_t t0 = has_unit ? poff[p_begin] : 0u;
+    const uint32_t t1 = has_unit ? poff[p_end] : 0u;
+    // loads past the last step are clamped to it (their values are not used)
+    const uint32_t tlast = t1 > t0 ? t1 - 1u : umin32(t0, pa.n_steps - 1u);
+    // barriers this wave owes: one per panel of the chunk, with or without steps in it
+    uint32_t owed = p_end - p_begin;
+    // panels in front of the chunk's first step (the count stored with that step refers
+    // to its predecessor, which may lie in another chunk)
+    uint32_t first_jump = t1 > t0 ? as_const(pa.step_panel)[t0] - p_begin : 0u;
+
+    f32x4 acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    typedef typename TT::AVec AVec;
+    const uint32_t *id_src = pa.ids + L.g;
+    auto ring_idx = [&](uint32_t step) __attribute__((always_inline)) -> uint32_t {
+        return id_src[size_t(umin32(step, tlast)) * 4u];
+    };
+    auto ring_a = [&](uint32_t step) __attribute__((always_inline)) -> AVec {
+        return *reinterpret_cast<const AVec *>(L.a_src + size_t(umin32(step, tlast)) * (64u * G));
+    };
+    // register ring of kRing steps (separate variables: an array would go to scratch)
+#define HSPMM_RING(X) X(0) X(1) X(2) X(3) X(4) X(5)
+    constexpr uint32_t kRing = 6;
+#define HSPMM_RING_DECL(k) uint32_t I##k = ring_idx(t0 + k##u); AVec A##k = ring_a(t0 + k##u);
+    HSPMM_RING(HSPMM_RING_DECL)
+#undef HSPMM_RING_DECL
+    panel_barrier();                                                // panel p_begin is in its buffer
+    --owed;
+    // the lane's 16 bytes of a row, in the buffer of the current panel
+    uint32_t img = (p_begin & 1u) * kPanelBytes + L.j * 16u;
+
+    // One step: first the barriers that lie between it and the step in front of it.
+    auto step = [&](const uint32_t I, const AVec &A, const uint32_t jump) __attribute__((always_inline)) {
+        for (uint32_t n = jump; n && owed; --n) {                   // never more barriers than the producers pass
+            panel_barrier();
+            img ^= kPanelBytes;
+            --owed;
+        }
+        typename TT::BVec b0, b1, b2 = {}, b3 = {};
+        b0 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 0, 7) << 8));
+        b1 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 7, 7) << 8));
+        if constexpr (PanelRows<TT>::value == 4) {
+            b2 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 14, 7) << 8));
+            b3 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 21, 7) << 8));
+        }
+        TT::mma(L, b0, b1, b2, b3, A, acc);
+    };
+    auto jump_of = [&](const uint32_t I, const uint32_t t) __attribute__((always_inline)) -> uint32_t {
+        const uint32_t stored = __builtin_amdgcn_readfirstlane(I) >> 28;
+        return t == t0 ? first_jump : stored;
+    };
+
+    uint32_t t = t0;
+    // Steady state: every slot runs its step and reloads its registers with the step kRing
+    // further on, without conditions on the loads.
+    for (; t + 2u * kRing <= t1; t += kRing) {
+#define HSPMM_PANEL_STEADY(k) \
+        step(I##k, A##k, jump_of(I##k, t + k##u)); \
+        I##k = ring_idx(t + k##u + kRing); A##k = ring_a(t + k##u + kRing);
+        HSPMM_RING(HSPMM_PANEL_STEADY)
+#undef HSPMM_PANEL_STEADY
+    }
+    for (; t < t1; t += kRing) {
+#define HSPMM_PANEL_DRAIN(k) \
+        if (t + k##u < t1) step(I##k, A##k, jump_of(I##k, t + k##u)); \
+        if (t + k##u + kRing < t1) { I##k = ring_idx(t + k##u + kRing); A##k = ring_a(t + k##u + kRing); }
+        HSPMM_RING(HSPMM_PANEL_DRAIN)
+#undef HSPMM_PANEL_DRAIN
+    }
+#undef HSPMM_RING
+    // the panels behind the unit's last step
+    for (; owed; --owed) panel_barrier();
+
+    if (!has_unit) return;
+    const uint32_t row = pa.unitRow[u];
+    const uint32_t row0 = row & ~7u;
+    const bool paired = (G > 1) && (row & 1u);
+    if (pa.n_chunks == 1u) {
+        TT::template store_window<0>(L, acc, c_lane, row_bytes, row0, pa.rows, true);
+        if constexpr (G > 1) {
+            if (paired) TT::template store_window<G - 1>(L, acc, c_lane, row_bytes, row0 + kRowWindow, pa.rows, true);
+        }
+    } else {
+        f32x4 *dst = reinterpret_cast<f32x4 *>(pa.scratch) +
+                     ((size_t(u) * pa.n_chunks + chunk) * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) dst[i * 64] = acc[i];
+    }
+    if (chunk == 0u) {
+        // rows of the windows without entries behind this unit, and in front of the first one
+        const uint32_t next_row = (u + 1u < pa.n_units) ? (pa.unitRow[u + 1u] & ~7u) : pa.rows;
+        const uint32_t gap_begin = row0 + (paired ? 2u * kRowWindow : kRowWindow);
+        if (gap_begin < next_row) TT::zero_rows(L, c_lane, row_bytes, gap_begin, next_row, true);
+        if (u == 0u) TT::zero_rows(L, c_lane, row_bytes, 0u, row0, true);
+    }
+}
+
+// Units (consumer waves) per workgroup; two more waves are producers.  Waves go to
+// the four SIMDs of a compute unit round-robin: 8 and 12 consumers spread evenly.
+constexpr int kPanelUnitChoices[] = {6, 8, 12, 14};
+
+// ka: the arguments of spmm_fixup_kernel for the chunk sums (split table with one
+// entry per unit); used only when pa.n_chunks > 1.
+template <class TT, int NC, int NPW>
+static hipError_t launch_panel_tt(const PanelArgs &pa, const KernelArgs &ka, hipStream_t s, hipEvent_t mid)
+{
+    const uint32_t row_blocks = (pa.n_units + NC - 1) / NC;
+    const dim3 grid(row_blocks * pa.n_feat_blocks * pa.n_chunks), block((NC + NPW) * 64);
+    spmm_panel_kernel<TT, NC, NPW><<<grid, block, 0, s>>>(pa);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || pa.n_chunks == 1u) return e;
+    if (mid && (e = hipEventRecord(mid, s)) != hipSuccess) return e;
+    const uint32_t fitems = ka.n_split * ka.n_feat_blocks;
+    spmm_fixup_kernel<TT><<<dim3((fitems + 3u) / 4u), dim3(256), 0, s>>>(ka);
+    return hipGetLastError();
+}
+
+template <class TT>
+static hipError_t launch_panel_nw(const PanelArgs &pa, const KernelArgs &ka, int units, hipStream_t s, hipEvent_t mid)
+{
+    switch (units) {
+    case 14: return launch_panel_tt<TT, 14, 2>(pa, ka, s, mid);
+    case 12: return launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
+    case 8: return launch_panel_tt<TT, 8, 2>(pa, ka, s, mid);
+    default: return launch_panel_tt<TT, 6, 2>(pa, ka, s, mid);
+    }
+}
+
+}  // namespace hspmm

@@ -100,9 +100,12 @@ void hspmm_get_config(int *buffer_stage, int *consumer_warp_num,
                       int *producer_warp_group_num, int *sm_num);
 
 /* Kernel selection, read by the next hspmm_create: 0 = automatic (MFMA kernels
- * whenever the feature dimension allows), 1 = always the scalar all-shapes
- * kernel, 2 = fp16 MFMA kernel with wide loads only, 3 = fp16 MFMA kernel with
- * word loads whenever N is a multiple of 32. */
+ * whenever the feature dimension allows; the kernels that stage B through LDS
+ * for matrices whose windows touch a large share of the columns), 1 = always the
+ * scalar all-shapes kernel, 2 = 16-bit MFMA kernel with wide loads only, 3 =
+ * 16-bit MFMA kernel with word loads whenever N is a multiple of 32, 4 = the
+ * LDS-staging kernels for every matrix (whenever N is a multiple of 128 for the
+ * 16-bit types, of 64 for fp32, and B and C are 16-byte aligned). */
 int hspmm_set_kernel_mode(int mode);
 
 /* No reference counterpart.  Two vertically adjacent windows with the same
@@ -121,6 +124,8 @@ typedef struct {
     uint32_t n_units;           /* units of the step stream: single windows and pairs */
     uint32_t n_paired_units;    /* units made of two adjacent windows with one column list */
     uint64_t device_bytes;      /* bytes of device memory the plan holds right now */
+    uint32_t n_panels;          /* column panels of the LDS-staging kernels; 0: the plan does not use them */
+    uint32_t n_panel_steps;     /* steps of the unit stream re-tiled panel by panel */
 } hspmm_plan_info;
 
 /* No reference counterpart (the reference prints its statistics from main,

@@ -290,6 +290,101 @@ def test_plans_from_bitmap_and_grouped_formats(torch_cuda, hs, oracle, dtype):
     assert_parity(gpu_spmm(torch_cuda, hs, bitmap, B, 32), ref, mag, dtype, "tiny.mtx bitmap")
 
 
+PANEL_SHAPES = [
+    # rows, cols, density, empty-row probability, heavy rows
+    (8, 16, 1.0, 0.0, ()),                      # one window, one panel
+    (27, 100, 0.3, 0.3, ()),                    # ragged last window, one panel
+    (130, 257, 0.2, 0.3, ()),                   # three panels, the last one a single column
+    (300, 1000, 0.1, 0.2, (5, 100, 299)),
+    (1000, 700, 0.01, 0.6, (512,)),             # most units have no step in most panels
+]
+
+
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+@pytest.mark.parametrize("shape", PANEL_SHAPES)
+def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
+    rows, cols, dens, erp, heavy = shape
+    rng = np.random.default_rng(hash((rows, cols, dtype, 4)) & 0xFFFF)
+    A = random_csr(rng, rows, cols, dens, dtype, erp, heavy)
+    b = convert(hs, A)
+    block = 64 if dtype == 1 else 128
+    for units, chunks in (("6", ""), ("14", ""), ("6", "1"), ("14", "3"), ("6", "1000")):
+        os.environ["HSPMM_PANEL_UNITS"] = units
+        if chunks:
+            os.environ["HSPMM_PANEL_CHUNKS"] = chunks
+        hs.set_kernel_mode(4)
+        try:
+            plan = hs.Plan(b)
+            info = plan.info()
+            assert info["n_panels"] == (cols + 127) // 128 and info["n_panel_steps"] >= info["total_tiles"] // 2
+            for N in (block, 2 * block, 5 * block):
+                B = make_b(rng, cols, N, dtype)
+                got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+                ref, mag = oracle_spmm(oracle, A, B, N)
+                assert_parity(got, ref, mag, dtype, "panel units %s chunks %s shape %s N=%d" % (units, chunks, shape[:2], N))
+            # a feature dimension the panel kernels do not take falls back to the gather kernels
+            B = make_b(rng, cols, 24, dtype)
+            got = gpu_spmm(torch_cuda, hs, b, B, 24, plan=plan)
+            ref, mag = oracle_spmm(oracle, A, B, 24)
+            assert_parity(got, ref, mag, dtype, "panel plan, N=24")
+            plan.close()
+        finally:
+            hs.set_kernel_mode(0)
+            os.environ.pop("HSPMM_PANEL_UNITS", None)
+            os.environ.pop("HSPMM_PANEL_CHUNKS", None)
+
+
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_lds_panel_kernels_exact_and_paired(torch_cuda, hs, oracle, dtype):
+    """Block-clustered matrices (paired windows) and exact integer arithmetic: the panel
+    kernels must give the one rounding of the exact result, like the gather kernels."""
+    rng = np.random.default_rng(70 + dtype)
+    block = 64 if dtype == 1 else 128
+    A = _block_matrix(rng, 203, 900, 16, 16, 0.5, dtype)
+    b = convert(hs, A)
+    D = rng.integers(-3, 4, (120, 700)) * (rng.random((120, 700)) < 0.3)
+    rp = np.zeros(121, np.uint32)
+    ci, vv = [], []
+    for r in range(120):
+        nz = np.nonzero(D[r])[0]
+        ci += nz.tolist(); vv += D[r, nz].tolist()
+        rp[r + 1] = len(ci)
+    E = dict(rows=120, cols=700, dtype=dtype, row_ptr=rp, col_idx=np.array(ci, np.uint32),
+             values=encode(np.array(vv, np.float32), dtype))
+    e = convert(hs, E)
+    hs.set_kernel_mode(4)
+    try:
+        for pairing in (0, 1, 2):
+            hs.set_window_pairing(pairing)
+            plan = hs.Plan(b)
+            assert plan.info()["n_panels"] == 8
+            if pairing != 1:
+                assert plan.info()["n_paired_units"] > 0
+            for N in (block, 3 * block):
+                B = make_b(rng, 900, N, dtype)
+                got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+                ref, mag = oracle_spmm(oracle, A, B, N)
+                assert_parity(got, ref, mag, dtype, "paired panel pairing %d N=%d" % (pairing, N))
+            plan.close()
+        hs.set_window_pairing(0)
+        plan = hs.Plan(e)
+        Bm = rng.integers(-4, 5, (700, 2 * block))
+        got = gpu_spmm(torch_cuda, hs, e, encode(Bm, dtype), 2 * block, plan=plan)
+        assert np.array_equal(got, encode(D @ Bm, dtype))
+        plan.close()
+    finally:
+        hs.set_kernel_mode(0)
+        hs.set_window_pairing(0)
+
+
+def test_lds_panel_kernels_are_chosen_for_dense_windows_only(torch_cuda, hs):
+    from hopper_spmm_amd import generators as G
+    dense = G.make_config(4, 8)["A"]            # block-clustered: every window meets half of all columns
+    sparse = G.make_config(1, 8)["A"]           # ~16 entries per row
+    assert hs.Plan(convert(hs, dense)).info()["n_panels"] > 0
+    assert hs.Plan(convert(hs, sparse)).info()["n_panels"] == 0
+
+
 def test_unaligned_and_odd_feature_dims_use_the_all_shapes_kernel(torch_cuda, hs, oracle):
     rng = np.random.default_rng(5)
     for dt in (0, 2):
