@@ -732,8 +732,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     // units), 12 otherwise, which spreads the consumer waves evenly over the SIMDs.
     int units = p->G == 2 ? 14 : 12;
     if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) {                                      // tuning overrides
-        const int v = std::atoi(e);
-        units = (v == 14 || v == 12 || v == 8) ? v : 6;
+        units = std::atoi(e) == 14 ? 14 : 12;
     }
     // chunks of panels: as many as keep the workgroups within one round over the compute units
     const uint64_t row_blocks = (uint64_t(p->n_units) + units - 1) / units;

@@ -210,9 +210,8 @@ void spmm_panel_kernel(const PanelArgs pa)
     }
 }
 
-// Units (consumer waves) per workgroup; two more waves are producers.  Waves go to
-// the four SIMDs of a compute unit round-robin: 8 and 12 consumers spread evenly.
-constexpr int kPanelUnitChoices[] = {6, 8, 12, 14};
+// Units (consumer waves) per workgroup: 12 or 14; two more waves are producers.  Waves go
+// to the four SIMDs of a compute unit round-robin, so 12 consumers spread evenly.
 
 // ka: the arguments of spmm_fixup_kernel for the chunk sums (split table with one
 // entry per unit); used only when pa.n_chunks > 1.
@@ -233,12 +232,7 @@ static hipError_t launch_panel_tt(const PanelArgs &pa, const KernelArgs &ka, hip
 template <class TT>
 static hipError_t launch_panel_nw(const PanelArgs &pa, const KernelArgs &ka, int units, hipStream_t s, hipEvent_t mid)
 {
-    switch (units) {
-    case 14: return launch_panel_tt<TT, 14, 2>(pa, ka, s, mid);
-    case 12: return launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
-    case 8: return launch_panel_tt<TT, 8, 2>(pa, ka, s, mid);
-    default: return launch_panel_tt<TT, 6, 2>(pa, ka, s, mid);
-    }
+    return units == 14 ? launch_panel_tt<TT, 14, 2>(pa, ka, s, mid) : launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
 }
 
 }  // namespace hspmm
