@@ -99,6 +99,7 @@ struct hspmm_plan {
         uint32_t *d_poff = nullptr, *d_ids = nullptr, *d_step_panel = nullptr;
         void *d_tiles = nullptr;
         uint32_t *d_split = nullptr, *d_fix_slots = nullptr;    // one split entry per unit, for the chunk sums
+        bool quad = false;                                       // ids in the format of the 4x4x1 fp32 tile
         uint32_t split_chunks = 0;                               // chunk count d_split was built for
         size_t fix_slot_count = 0;
     } panel;
@@ -371,6 +372,9 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     // per step four words; word g packs the panel rows quarter-wave g reads, 7 bits each (16-bit types:
     // ids 4g..4g+3, fp32: ids g and g + 4), and in bits 28..31 the panels the step lies behind its predecessor
     std::vector<uint32_t> ids(size_t(ps.n_steps) * 4u);
+    // fp32 single windows run through the 4x4x1 instruction, which wants row offsets (see Fp32Quad)
+    bool quad = p->dtype == HSPMM_TF32 && st.G == 1;
+    if (const char *e = std::getenv("HSPMM_PANEL_QUAD")) quad = quad && std::atoi(e) != 0;       // tuning override
     for (uint32_t u = 0; u < U; ++u) {
         const uint32_t t0 = rt_rowOffset[st.unitWindow[u]], n = ps.unitOffset[u + 1] - ps.unitOffset[u];
         uint32_t *po = poff.data() + size_t(u) * (NP + 1);
@@ -384,9 +388,13 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
             uint32_t *dst = ids.data() + size_t(ps.unitOffset[u] + i) * 4u;
             const uint32_t jump = i ? rt_panel[t0 + i] - rt_panel[t0 + i - 1] : 0u;     // <= kMaxJump by construction
             step_panel[ps.unitOffset[u] + i] = rt_panel[t0 + i];
-            for (uint32_t g = 0; g < 4; ++g)
-                dst[g] = (cw == 16 ? (src[4 * g] | src[4 * g + 1] << 7 | src[4 * g + 2] << 14 | src[4 * g + 3] << 21)
-                                   : (src[g] | src[g + 4] << 7)) | jump << 28;
+            for (uint32_t g = 0; g < 4; ++g) {
+                if (quad)   // byte offsets of rows g and g + 4 inside the panel image; the jump in bits 0..3 of word 0
+                    dst[g] = (src[g] << 8 | (g == 0 ? jump : 0u)) | (src[g + 4] << 8) << 16;
+                else
+                    dst[g] = (cw == 16 ? (src[4 * g] | src[4 * g + 1] << 7 | src[4 * g + 2] << 14 | src[4 * g + 3] << 21)
+                                       : (src[g] | src[g + 4] << 7)) | jump << 28;
+            }
         }
     }
     hspmm_plan::Panel &pl = p->panel;
@@ -400,7 +408,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
         if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
         pl.d_tiles = dt;
     }
-    pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.built = true;
+    pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.built = true;
     return true;
 }
 
@@ -749,7 +757,8 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     if (pa.n_chunks > 1) {
         int rc = ensure_panel_split(p, pa.n_chunks);
         if (rc) return rc;
-        const size_t need = size_t(p->n_units) * pa.n_chunks * pa.n_feat_blocks * 4u * size_t(p->G) * 64u * 16u;
+        const size_t nacc = pl.quad ? 2u : 4u * size_t(p->G);
+        const size_t need = size_t(p->n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
         if ((rc = ensure_scratch(p, need))) return rc;
         pa.scratch = p->d_scratch;
         ka.unitRow = p->d_unitRow; ka.ids = pl.d_ids; ka.tiles = pl.d_tiles;
@@ -758,7 +767,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         ka.n_split = p->n_units; ka.n_units = p->n_units; ka.rows = p->rows; ka.N = N;
         ka.n_feat_blocks = pa.n_feat_blocks;
     }
-    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, p->G, pa, ka, units, s, mid));
+    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : p->G, pa, ka, units, s, mid));
     return HSPMM_OK;
 }
 

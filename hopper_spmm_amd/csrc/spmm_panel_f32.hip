@@ -6,8 +6,10 @@ namespace hspmm {
 
 template <int G> using PanelTile = Fp32Tile<4, G>;
 
+// G = 0: single windows through the 4x4x1 instruction (the plan's ids are in that tile's format)
 hipError_t launch_panel_f32(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid)
 {
+    if (G == 0) return launch_panel_nw<Fp32Quad>(pa, ka, waves, s, mid);
     return G == 2 ? launch_panel_nw<PanelTile<2>>(pa, ka, waves, s, mid)
                   : launch_panel_nw<PanelTile<1>>(pa, ka, waves, s, mid);
 }

@@ -31,9 +31,134 @@
 
 namespace hspmm {
 
-// B rows a lane reads per step: four for the 16-bit types, two for fp32.
-template <class TT> struct PanelRows { static constexpr int value = 4; };
-template <int V, int G> struct PanelRows<Fp32Tile<V, G>> { static constexpr int value = 2; };
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+
+// fp32 without the 8 -> 16 row padding of v_mfma_f32_16x16x4_f32 (single windows only):
+// v_mfma_f32_4x4x1_16B_f32 multiplies 16 independent 4 x 1 by 1 x 4 blocks.  Block
+// b = lane / 4 is rows 4 * (b / 8) .. + 3 of the window times features 4 * (b % 8) .. + 3
+// of a group of 32 features; one instruction is one k (one B row) for 8 rows x 32
+// features, all of it useful, at the rate of the big instruction.  The B row of a k
+// is the same for all lanes, so its panel offset is a scalar.
+//   tiles per step: the lane order of Fp32Tile, [row r][8 words: k = 0,4,1,5,2,6,3,7]:
+//     a lane reads the 32 bytes of its row.
+//   ids per step: four words, word g = offset of row g | offset of row g + 4 << 16
+//     (offset = row inside the panel x 256); bits 0..3 of word 0: the panel jump.
+struct Fp32Quad {
+    static constexpr int V = 2, G = 1;             // two accumulators: features 0..31 and 32..63 of the block
+    static constexpr int kBlockFeat = 64;
+    static constexpr int kLaneFeat = 1;            // lane's feature = j (+ 32 for the second accumulator)
+    static constexpr int kElem = 4;
+    static constexpr bool kQuad = true;
+    typedef u32x8 AVec;
+    struct Lane {
+        uint32_t g, j;                             // row quad (0, 1), feature inside the group of 32
+        const uint32_t *a_src;
+        const uint32_t *idx_src;
+        __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
+        {
+            g = lane >> 5; j = lane & 31u;
+            a_src = reinterpret_cast<const uint32_t *>(tiles) + (4u * g + (lane & 3u)) * 8u;
+            idx_src = ids;
+        }
+    };
+    // acc[h][e]: window row 4g + e, feature 32h + j
+    template <int W0>
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[2], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t row = row0 + 4u * L.g + e;
+            if (active && row < rows) {
+                float *dst = reinterpret_cast<float *>(c_lane + size_t(row) * row_bytes);
+                const float lo = acc[0][e], hi = acc[1][e];
+                stream_store(dst, lo);
+                stream_store(dst + 32, hi);
+            }
+        }
+    }
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 2u) {
+            float *dst = reinterpret_cast<float *>(c_lane + size_t(r) * row_bytes);
+            stream_store(dst, 0.f);
+            stream_store(dst + 32, 0.f);
+        }
+    }
+};
+
+// How a consumer wave of the panel kernel reads the ids and tiles of a step and runs it.
+template <class TT>
+struct PanelOps {
+    static constexpr int kRows = TT::kElem == 4 ? 2 : 4;         // B rows a lane reads per step
+    typedef uint32_t Idx;                                         // the lane's word of the step's four id words
+    typedef typename TT::AVec AVec;
+    __device__ static __forceinline__ Idx load_idx(const typename TT::Lane &L, const uint32_t *ids, uint32_t step)
+    {
+        return ids[size_t(step) * 4u + L.g];
+    }
+    __device__ static __forceinline__ AVec load_a(const typename TT::Lane &L, uint32_t step)
+    {
+        return *reinterpret_cast<const AVec *>(L.a_src + size_t(step) * (64u * TT::G));
+    }
+    __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) >> 28; }
+    // img: LDS byte offset of the lane's 16 bytes of row 0 of the current panel image
+    __device__ static __forceinline__ void step(const typename TT::Lane &L, const char *smem, uint32_t img, const Idx I,
+                                                const AVec &A, f32x4 (&acc)[TT::G * TT::V])
+    {
+        typename TT::BVec b0, b1, b2 = {}, b3 = {};
+        b0 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 0, 7) << 8));
+        b1 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 7, 7) << 8));
+        if constexpr (kRows == 4) {
+            b2 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 14, 7) << 8));
+            b3 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 21, 7) << 8));
+        }
+        TT::mma(L, b0, b1, b2, b3, A, acc);
+    }
+    __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return L.j * 16u; }
+};
+
+template <>
+struct PanelOps<Fp32Quad> {
+    typedef u32x4 Idx;                                            // all four id words (the same in every lane)
+    typedef u32x8 AVec;
+    // The address is the same in every lane: the compiler makes this a scalar load.
+    __device__ static __forceinline__ Idx load_idx(const Fp32Quad::Lane &, const uint32_t *ids, uint32_t step)
+    {
+        return *reinterpret_cast<const u32x4 *>(ids + size_t(step) * 4u);
+    }
+    __device__ static __forceinline__ AVec load_a(const Fp32Quad::Lane &L, uint32_t step)
+    {
+        return *reinterpret_cast<const u32x8 *>(L.a_src + size_t(step) * 64u);
+    }
+    __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I[0]) & 15u; }
+    __device__ static __forceinline__ void step(const Fp32Quad::Lane &, const char *smem, uint32_t img, const Idx I,
+                                                const AVec &A, f32x4 (&acc)[2])
+    {
+        // word w holds the offsets of the rows whose tile values are A[2w] and A[2w + 1]
+        float lo[8], hi[8];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t word = I[w];
+            const uint32_t sw = __builtin_amdgcn_readfirstlane(word);
+            const uint32_t off0 = sw & 0xFF00u, off1 = sw >> 16;
+            const float *r0 = reinterpret_cast<const float *>(smem + (img + off0));
+            const float *r1 = reinterpret_cast<const float *>(smem + (img + off1));
+            lo[2 * w] = r0[0]; hi[2 * w] = r0[32];
+            lo[2 * w + 1] = r1[0]; hi[2 * w + 1] = r1[32];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t aw = A[i];
+            const float a = __builtin_bit_cast(float, aw);
+            acc[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, lo[i], acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, hi[i], acc[1], 0, 0, 0);
+        }
+    }
+    __device__ static __forceinline__ uint32_t lane_bytes(const Fp32Quad::Lane &L) { return L.j * 4u; }
+};
 
 // One barrier of the workgroup with the LDS writes in front of it visible behind it.
 __device__ __forceinline__ void panel_barrier()
@@ -53,7 +178,6 @@ void spmm_panel_kernel(const PanelArgs pa)
 {
     constexpr int G = TT::G, V = TT::V, NACC = G * V;
     constexpr int kPieces = int(kPanelBytes / 16u) / (NPW * 64);   // 16-byte pieces of a panel per producer thread
-    static_assert(V == 4, "a lane owns 16 bytes of a B row");
     static_assert(kPieces * NPW * 64 * 16 == int(kPanelBytes), "panel must divide among the producers");
     __shared__ __attribute__((aligned(16))) char smem[2 * kPanelBytes];
 
@@ -125,43 +249,37 @@ void spmm_panel_kernel(const PanelArgs pa)
 #pragma unroll
     for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    typedef typename TT::AVec AVec;
-    const uint32_t *id_src = pa.ids + L.g;
-    auto ring_idx = [&](uint32_t step) __attribute__((always_inline)) -> uint32_t {
-        return id_src[size_t(umin32(step, tlast)) * 4u];
+    typedef PanelOps<TT> Ops;
+    typedef typename Ops::AVec AVec;
+    typedef typename Ops::Idx Idx;
+    auto ring_idx = [&](uint32_t step) __attribute__((always_inline)) -> Idx {
+        return Ops::load_idx(L, pa.ids, umin32(step, tlast));
     };
     auto ring_a = [&](uint32_t step) __attribute__((always_inline)) -> AVec {
-        return *reinterpret_cast<const AVec *>(L.a_src + size_t(umin32(step, tlast)) * (64u * G));
+        return Ops::load_a(L, umin32(step, tlast));
     };
     // register ring of kRing steps (separate variables: an array would go to scratch)
 #define HSPMM_RING(X) X(0) X(1) X(2) X(3) X(4) X(5)
     constexpr uint32_t kRing = 6;
-#define HSPMM_RING_DECL(k) uint32_t I##k = ring_idx(t0 + k##u); AVec A##k = ring_a(t0 + k##u);
+#define HSPMM_RING_DECL(k) Idx I##k = ring_idx(t0 + k##u); AVec A##k = ring_a(t0 + k##u);
     HSPMM_RING(HSPMM_RING_DECL)
 #undef HSPMM_RING_DECL
     panel_barrier();                                                // panel p_begin is in its buffer
     --owed;
-    // the lane's 16 bytes of a row, in the buffer of the current panel
-    uint32_t img = (p_begin & 1u) * kPanelBytes + L.j * 16u;
+    // the lane's bytes of a row, in the buffer of the current panel
+    uint32_t img = (p_begin & 1u) * kPanelBytes + Ops::lane_bytes(L);
 
     // One step: first the barriers that lie between it and the step in front of it.
-    auto step = [&](const uint32_t I, const AVec &A, const uint32_t jump) __attribute__((always_inline)) {
+    auto step = [&](const Idx &I, const AVec &A, const uint32_t jump) __attribute__((always_inline)) {
         for (uint32_t n = jump; n && owed; --n) {                   // never more barriers than the producers pass
             panel_barrier();
             img ^= kPanelBytes;
             --owed;
         }
-        typename TT::BVec b0, b1, b2 = {}, b3 = {};
-        b0 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 0, 7) << 8));
-        b1 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 7, 7) << 8));
-        if constexpr (PanelRows<TT>::value == 4) {
-            b2 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 14, 7) << 8));
-            b3 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 21, 7) << 8));
-        }
-        TT::mma(L, b0, b1, b2, b3, A, acc);
+        Ops::step(L, smem, img, I, A, acc);
     };
-    auto jump_of = [&](const uint32_t I, const uint32_t t) __attribute__((always_inline)) -> uint32_t {
-        const uint32_t stored = __builtin_amdgcn_readfirstlane(I) >> 28;
+    auto jump_of = [&](const Idx &I, const uint32_t t) __attribute__((always_inline)) -> uint32_t {
+        const uint32_t stored = Ops::jump(I);
         return t == t0 ? first_jump : stored;
     };
 
