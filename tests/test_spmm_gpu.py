@@ -434,16 +434,24 @@ def test_run_captured_in_a_hip_graph_replays_correctly(torch_cuda, hs, oracle):
     and new contents of B in between, must give what the eager call gives."""
     torch = torch_cuda
     rng = np.random.default_rng(15)
-    for dtype in (0, 1):
-        A = random_csr(rng, 400, 4000, 0.003, dtype, 0.1, (3, 200))
-        b = convert(hs, A)
-        hs.configure(producer_warp_group_num=16)
-        try:
+    for dtype, panels in ((0, False), (1, False), (0, True), (1, True)):
+        if panels:
+            # dense windows: the LDS-panel kernel and the kernel that adds its chunk sums
+            A = random_csr(rng, 400, 4000, 0.1, dtype, 0.1)
+            b = convert(hs, A)
             plan = hs.Plan(b)
-        finally:
-            hs.configure()
-        assert plan.info()["n_split_windows"] > 0              # two kernels per call
-        N = 64
+            assert plan.info()["n_panels"] > 0
+            N = 128
+        else:
+            A = random_csr(rng, 400, 4000, 0.003, dtype, 0.1, (3, 200))
+            b = convert(hs, A)
+            hs.configure(producer_warp_group_num=16)
+            try:
+                plan = hs.Plan(b)
+            finally:
+                hs.configure()
+            assert plan.info()["n_split_windows"] > 0          # two kernels per call
+            N = 64
         tt = torch.int16 if dtype == 0 else torch.float32
         Bs = [make_b(rng, 4000, N, dtype) for _ in range(3)]
         as_t = (lambda x: torch.from_numpy(x.view(np.int16))) if dtype == 0 else torch.from_numpy
