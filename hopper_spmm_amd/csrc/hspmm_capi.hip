@@ -738,12 +738,15 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     // 16 waves per workgroup fill a compute unit (two workgroups with 64 KB of LDS each
     // do not become resident together): 14 units where the LDS reads bind (paired
     // units), 12 otherwise, which spreads the consumer waves evenly over the SIMDs.
-    int units = p->G == 2 ? 14 : 12;
+    // (code 13 = 12 units and four producer waves: few enough registers for two workgroups per
+    // compute unit, which the 4x4x1 fp32 kernel needs to keep its short MFMAs fed)
+    int units = pl.quad ? 13 : p->G == 2 ? 14 : 12;
     if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) {                                      // tuning overrides
-        units = std::atoi(e) == 14 ? 14 : 12;
+        units = std::atoi(e) == 14 ? 14 : std::atoi(e) == 13 ? 13 : 12;
     }
     // chunks of panels: as many as keep the workgroups within one round over the compute units
-    const uint64_t row_blocks = (uint64_t(p->n_units) + units - 1) / units;
+    const int units_per_group = units == 13 ? 12 : units;
+    const uint64_t row_blocks = (uint64_t(p->n_units) + units_per_group - 1) / units_per_group;
     const uint64_t base = row_blocks * pa.n_feat_blocks;
     uint64_t chunks = uint64_t(p->compute_units) / base;
     if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) chunks = uint64_t(std::atoi(e));

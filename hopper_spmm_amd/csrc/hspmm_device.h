@@ -70,7 +70,7 @@ struct PanelArgs {
     uint32_t n_units, n_steps, rows, cols, N, n_feat_blocks, n_panels, n_chunks, panels_per_chunk;
 };
 
-// units: 12 or 14 units (consumer waves) per workgroup; 2 more waves copy B to LDS.
+// units: 12 or 14 units (consumer waves) per workgroup, 2 more waves copy B to LDS; 13 = 12 units and 4 such waves.
 // G: windows per unit; 0 = fp32 single windows with ids in the format of the 4x4x1 tile.  ka: arguments of the kernel that adds
 // the chunk sums (split table with one entry per unit), used when pa.n_chunks > 1.
 hipError_t launch_spmm_panel(int dtype, int G, const PanelArgs &pa, const KernelArgs &ka, int units, hipStream_t s,

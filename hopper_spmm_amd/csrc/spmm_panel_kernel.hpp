@@ -93,6 +93,9 @@ struct Fp32Quad {
 template <class TT>
 struct PanelOps {
     static constexpr int kRows = TT::kElem == 4 ? 2 : 4;         // B rows a lane reads per step
+    static constexpr uint32_t kRing = 6;                          // steps of tiles and ids in flight
+    static constexpr int kLive = TT::G * TT::V;                   // accumulator registers the step loop keeps
+    __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
     typedef uint32_t Idx;                                         // the lane's word of the step's four id words
     typedef typename TT::AVec AVec;
     __device__ static __forceinline__ Idx load_idx(const typename TT::Lane &L, const uint32_t *ids, uint32_t step)
@@ -106,7 +109,7 @@ struct PanelOps {
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) >> 28; }
     // img: LDS byte offset of the lane's 16 bytes of row 0 of the current panel image
     __device__ static __forceinline__ void step(const typename TT::Lane &L, const char *smem, uint32_t img, const Idx I,
-                                                const AVec &A, f32x4 (&acc)[TT::G * TT::V])
+                                                const AVec &A, f32x4 (&acc)[kLive])
     {
         typename TT::BVec b0, b1, b2 = {}, b3 = {};
         b0 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 0, 7) << 8));
@@ -122,6 +125,11 @@ struct PanelOps {
 
 template <>
 struct PanelOps<Fp32Quad> {
+    static constexpr uint32_t kRing = 3;                          // few registers: two workgroups per compute unit
+    // Two accumulators per 32-feature half, used in turn: an MFMA then never reads the result of
+    // the one two instructions in front of it.  fold() adds the pairs once, at the end of the unit.
+    static constexpr int kLive = 4;
+    __device__ static __forceinline__ void fold(f32x4 (&acc)[4]) { acc[0] += acc[2]; acc[1] += acc[3]; }
     typedef u32x4 Idx;                                            // all four id words (the same in every lane)
     typedef u32x8 AVec;
     // The address is the same in every lane: the compiler makes this a scalar load.
@@ -135,7 +143,7 @@ struct PanelOps<Fp32Quad> {
     }
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I[0]) & 15u; }
     __device__ static __forceinline__ void step(const Fp32Quad::Lane &, const char *smem, uint32_t img, const Idx I,
-                                                const AVec &A, f32x4 (&acc)[2])
+                                                const AVec &A, f32x4 (&acc)[4])
     {
         // word w holds the offsets of the rows whose tile values are A[2w] and A[2w + 1]
         float lo[8], hi[8];
@@ -153,8 +161,8 @@ struct PanelOps<Fp32Quad> {
         for (int i = 0; i < 8; ++i) {
             const uint32_t aw = A[i];
             const float a = __builtin_bit_cast(float, aw);
-            acc[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, lo[i], acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, hi[i], acc[1], 0, 0, 0);
+            acc[2 * (i & 1)] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, lo[i], acc[2 * (i & 1)], 0, 0, 0);
+            acc[2 * (i & 1) + 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, hi[i], acc[2 * (i & 1) + 1], 0, 0, 0);
         }
     }
     __device__ static __forceinline__ uint32_t lane_bytes(const Fp32Quad::Lane &L) { return L.j * 4u; }
@@ -245,11 +253,11 @@ void spmm_panel_kernel(const PanelArgs pa)
     // to its predecessor, which may lie in another chunk)
     uint32_t first_jump = t1 > t0 ? as_const(pa.step_panel)[t0] - p_begin : 0u;
 
-    f32x4 acc[NACC];
-#pragma unroll
-    for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-
     typedef PanelOps<TT> Ops;
+    f32x4 live[Ops::kLive];
+#pragma unroll
+    for (int i = 0; i < Ops::kLive; ++i) live[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
     typedef typename Ops::AVec AVec;
     typedef typename Ops::Idx Idx;
     auto ring_idx = [&](uint32_t step) __attribute__((always_inline)) -> Idx {
@@ -260,8 +268,10 @@ void spmm_panel_kernel(const PanelArgs pa)
     };
     // register ring of kRing steps (separate variables: an array would go to scratch)
 #define HSPMM_RING(X) X(0) X(1) X(2) X(3) X(4) X(5)
-    constexpr uint32_t kRing = 6;
-#define HSPMM_RING_DECL(k) Idx I##k = ring_idx(t0 + k##u); AVec A##k = ring_a(t0 + k##u);
+    constexpr uint32_t kRing = Ops::kRing;
+    static_assert(kRing >= 1 && kRing <= 6, "ring slots are named variables");
+#define HSPMM_RING_DECL(k) Idx I##k = {}; AVec A##k = {}; \
+    if constexpr (kRing > k) { I##k = ring_idx(t0 + k##u); A##k = ring_a(t0 + k##u); }
     HSPMM_RING(HSPMM_RING_DECL)
 #undef HSPMM_RING_DECL
     panel_barrier();                                                // panel p_begin is in its buffer
@@ -276,7 +286,7 @@ void spmm_panel_kernel(const PanelArgs pa)
             img ^= kPanelBytes;
             --owed;
         }
-        Ops::step(L, smem, img, I, A, acc);
+        Ops::step(L, smem, img, I, A, live);
     };
     auto jump_of = [&](const Idx &I, const uint32_t t) __attribute__((always_inline)) -> uint32_t {
         const uint32_t stored = Ops::jump(I);
@@ -287,16 +297,16 @@ void spmm_panel_kernel(const PanelArgs pa)
     // Steady state: every slot runs its step and reloads its registers with the step kRing
     // further on, without conditions on the loads.
     for (; t + 2u * kRing <= t1; t += kRing) {
-#define HSPMM_PANEL_STEADY(k) \
+#define HSPMM_PANEL_STEADY(k) if constexpr (kRing > k) { \
         step(I##k, A##k, jump_of(I##k, t + k##u)); \
-        I##k = ring_idx(t + k##u + kRing); A##k = ring_a(t + k##u + kRing);
+        I##k = ring_idx(t + k##u + kRing); A##k = ring_a(t + k##u + kRing); }
         HSPMM_RING(HSPMM_PANEL_STEADY)
 #undef HSPMM_PANEL_STEADY
     }
     for (; t < t1; t += kRing) {
-#define HSPMM_PANEL_DRAIN(k) \
+#define HSPMM_PANEL_DRAIN(k) if constexpr (kRing > k) { \
         if (t + k##u < t1) step(I##k, A##k, jump_of(I##k, t + k##u)); \
-        if (t + k##u + kRing < t1) { I##k = ring_idx(t + k##u + kRing); A##k = ring_a(t + k##u + kRing); }
+        if (t + k##u + kRing < t1) { I##k = ring_idx(t + k##u + kRing); A##k = ring_a(t + k##u + kRing); } }
         HSPMM_RING(HSPMM_PANEL_DRAIN)
 #undef HSPMM_PANEL_DRAIN
     }
@@ -305,6 +315,10 @@ void spmm_panel_kernel(const PanelArgs pa)
     for (; owed; --owed) panel_barrier();
 
     if (!has_unit) return;
+    Ops::fold(live);
+    f32x4 acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) acc[i] = live[i];
     const uint32_t row = pa.unitRow[u];
     const uint32_t row0 = row & ~7u;
     const bool paired = (G > 1) && (row & 1u);
@@ -328,8 +342,9 @@ void spmm_panel_kernel(const PanelArgs pa)
     }
 }
 
-// Units (consumer waves) per workgroup: 12 or 14; two more waves are producers.  Waves go
-// to the four SIMDs of a compute unit round-robin, so 12 consumers spread evenly.
+// Units (consumer waves) per workgroup: 12 or 14; two more waves are producers (four in
+// the shape the 4x4x1 fp32 kernel uses).  Waves go to the four SIMDs of a compute unit
+// round-robin, so 12 consumers spread evenly.
 
 // ka: the arguments of spmm_fixup_kernel for the chunk sums (split table with one
 // entry per unit); used only when pa.n_chunks > 1.
@@ -350,7 +365,9 @@ static hipError_t launch_panel_tt(const PanelArgs &pa, const KernelArgs &ka, hip
 template <class TT>
 static hipError_t launch_panel_nw(const PanelArgs &pa, const KernelArgs &ka, int units, hipStream_t s, hipEvent_t mid)
 {
-    return units == 14 ? launch_panel_tt<TT, 14, 2>(pa, ka, s, mid) : launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
+    if (units == 14) return launch_panel_tt<TT, 14, 2>(pa, ka, s, mid);
+    if (units == 13) return launch_panel_tt<TT, 12, 4>(pa, ka, s, mid);      // 12 units, four producer waves
+    return launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
 }
 
 }  // namespace hspmm

@@ -308,8 +308,9 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
     A = random_csr(rng, rows, cols, dens, dtype, erp, heavy)
     b = convert(hs, A)
     block = 64 if dtype == 1 else 128
-    for units, chunks in (("12", ""), ("14", ""), ("12", "1"), ("14", "3"), ("12", "1000")):
-        os.environ["HSPMM_PANEL_UNITS"] = units
+    for units, chunks in (("", ""), ("12", ""), ("14", ""), ("13", "2"), ("12", "1"), ("14", "3"), ("12", "1000")):
+        if units:
+            os.environ["HSPMM_PANEL_UNITS"] = units
         if chunks:
             os.environ["HSPMM_PANEL_CHUNKS"] = chunks
         hs.set_kernel_mode(4)
