@@ -413,13 +413,9 @@ struct Fp32Tile {
         return __builtin_bit_cast(float, w);
     }
     template <int W0, int p>
-    __device__ static __forceinline__ void mma_one(const float a0, const float a1, const BVec &b0, const BVec &b1,
-                                                   f32x4 (&acc)[G * V])
+    __device__ static __forceinline__ void mma_one(const float a, const BVec &b, f32x4 (&acc)[G * V])
     {
-        if constexpr (p < V) {
-            acc[W0 * V + p] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, word<p>(b0), acc[W0 * V + p], 0, 0, 0);
-            acc[W0 * V + p] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, word<p>(b1), acc[W0 * V + p], 0, 0, 0);
-        }
+        if constexpr (p < V) acc[W0 * V + p] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, word<p>(b), acc[W0 * V + p], 0, 0, 0);
     }
     template <int W0>
     __device__ static __forceinline__ void mma_window(const Lane &L, const BVec &b0, const BVec &b1, const AVec &a,
@@ -428,8 +424,10 @@ struct Fp32Tile {
         if constexpr (W0 < G) {
             const uint32_t w0 = a[2 * W0] & L.a_mask, w1 = a[2 * W0 + 1] & L.a_mask;
             const float a0 = __builtin_bit_cast(float, w0), a1 = __builtin_bit_cast(float, w1);
-            mma_one<W0, 0>(a0, a1, b0, b1, acc); mma_one<W0, 1>(a0, a1, b0, b1, acc);
-            mma_one<W0, 2>(a0, a1, b0, b1, acc); mma_one<W0, 3>(a0, a1, b0, b1, acc);
+            // first half of k for every accumulator, then the second: an MFMA does not read the
+            // result of the one right in front of it
+            mma_one<W0, 0>(a0, b0, acc); mma_one<W0, 1>(a0, b0, acc); mma_one<W0, 2>(a0, b0, acc); mma_one<W0, 3>(a0, b0, acc);
+            mma_one<W0, 0>(a1, b1, acc); mma_one<W0, 1>(a1, b1, acc); mma_one<W0, 2>(a1, b1, acc); mma_one<W0, 3>(a1, b1, acc);
         }
     }
     __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &,
