@@ -292,6 +292,29 @@ std::vector<uint32_t> lane_order_tiles(const StepStream &st, int dtype, const ui
 }
 
 
+// 16-bit steps of 32 columns for the LDS-panel kernels (Fp16Tr in spmm_panel_kernel.hpp): a re-tiled
+// step of a window is [row r][32 halves]; lane l = (g, m) of the step's 1 KB gets the 16 bytes
+// a[m][8g .. 8g + 7], m = row of the unit's 16 rows (rows 8..15: the second window of a pair, else zero).
+std::vector<uint32_t> lane_order_wide_steps(const StepStream &st, const uint32_t *rowOffset, const void *data)
+{
+    const uint16_t *halves = static_cast<const uint16_t *>(data);   // a step of a window is 8 x 32 halves
+    std::vector<uint32_t> out(size_t(st.n_steps) * 256u, 0u);
+    for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
+        const uint32_t w0 = st.unitWindow[u];
+        const int nwin = (st.unitRow[u] & 1u) ? 2 : 1;
+        for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
+            uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * 256u);
+            for (int w = 0; w < nwin; ++w) {
+                const uint16_t *src = halves + size_t(rowOffset[w0 + w] + i) * 256u;
+                for (uint32_t r = 0; r < 8; ++r)
+                    for (uint32_t g = 0; g < 4; ++g)
+                        std::memcpy(dst + ((g * 16u + 8u * w + r) * 8u), src + r * 32u + 8u * g, 16);
+            }
+        }
+    }
+    return out;
+}
+
 // Re-tiles the matrix panel by panel for the LDS-panel kernels (spmm_panel_kernel.hpp):
 // inside every window the columns of one panel of kPanelRows columns get tiles of
 // their own.  Every step carries the number of panels it lies behind the step in
@@ -311,12 +334,14 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     // then read from LDS several times per load from the L2
     if (!forced && double(st.n_steps) < 2.0 * double(U) * double(NP)) return false;
     if (uint64_t(U) * (NP + 1) > (1ull << 28)) return false;
-    const size_t es = p->elem, tile_bytes = size_t(8) * cw * es;
+    // columns per re-tiled step: the 16-bit kernels contract 32 columns per step, fp32 a tile's 8
+    const uint32_t rw = cw == 16 ? 32u : cw;
+    const size_t es = p->elem, src_tile_bytes = size_t(8) * cw * es, tile_bytes = size_t(8) * rw * es;
     std::vector<uint32_t> rt_rowOffset(size_t(W) + 1, 0u), rt_ids, rt_panel;
     std::vector<uint8_t> rt_data;
     rt_ids.reserve(size_t(p->T) * cw * 5 / 4);
     rt_panel.reserve(size_t(p->T) * 5 / 4);
-    rt_data.reserve(size_t(p->T) * tile_bytes * 5 / 4);
+    rt_data.reserve(size_t(p->T) * src_tile_bytes * 5 / 4);
     const uint8_t *src_data = static_cast<const uint8_t *>(data);
     for (uint32_t w = 0; w < W; ++w) {
         const uint32_t t0 = rowOffset[w], t1 = rowOffset[w + 1];
@@ -329,26 +354,50 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
             while (i < nreal && col[i] / KP == pn) ++i;
             while (tiles && pn - last_pn > kMaxJump) {           // all-zero step that only carries the jump
                 last_pn += kMaxJump;
-                rt_ids.resize(rt_ids.size() + cw, 0u);
+                rt_ids.resize(rt_ids.size() + rw, 0u);
                 rt_data.resize(rt_data.size() + tile_bytes, 0);
                 rt_panel.push_back(last_pn);
                 ++tiles;
             }
-            const uint32_t nt = (i - a + cw - 1) / cw;
+            const uint32_t nt = (i - a + rw - 1) / rw;
             const size_t id_at = rt_ids.size(), data_at = rt_data.size();
-            rt_ids.resize(id_at + size_t(nt) * cw);
+            rt_ids.resize(id_at + size_t(nt) * rw);
             rt_data.resize(data_at + size_t(nt) * tile_bytes, 0);
             rt_panel.resize(rt_panel.size() + nt, pn);
-            for (uint32_t k = 0; k < nt * cw; ++k) {
-                const uint32_t srci = a + k;
-                if (srci < i) {
-                    rt_ids[id_at + k] = col[srci] - pn * KP;     // row inside the panel
-                    const uint8_t *st_tile = src_data + size_t(t0 + srci / cw) * tile_bytes;
-                    uint8_t *dt_tile = rt_data.data() + data_at + size_t(k / cw) * tile_bytes;
-                    for (uint32_t r = 0; r < 8; ++r)
-                        std::memcpy(dt_tile + (size_t(r) * cw + k % cw) * es, st_tile + (size_t(r) * cw + srci % cw) * es, es);
+            for (uint32_t tl = 0; tl < nt; ++tl) {
+                // The columns of the step.  16-bit types: one LDS instruction reads, in each block of 16
+                // lanes, the rows of four consecutive columns of the step (block g, instruction h: columns
+                // 8g + 4h .. + 3), the LDS serves two blocks (g = 0, 1 or g = 2, 3) at a time, and rows
+                // whose numbers differ mod 8 lie in different banks: columns ordered by row number mod 8
+                // (stable) and dealt out over the four sets of eight that are read together put
+                // different remainders into a set wherever the step has them.
+                const uint32_t first = a + tl * rw, n = std::min(rw, i - first);
+                uint32_t order[32];
+                if (rw == 32) {
+                    uint32_t sorted[32], m = 0;
+                    for (uint32_t res = 0; res < 8; ++res)
+                        for (uint32_t k = 0; k < rw; ++k) {
+                            // padding takes the row of the last real column (its tile column stays zero)
+                            const uint32_t c = col[first + std::min(k, n - 1)] - pn * KP;
+                            if ((c & 7u) == res) sorted[m++] = k;
+                        }
+                    for (uint32_t k = 0; k < rw; ++k) {
+                        const uint32_t set = k % 4, e = k / 4;          // set = 2 * (g / 2) + h
+                        const uint32_t g = 2 * (set / 2) + e / 4, h = set % 2;
+                        order[8 * g + 4 * h + e % 4] = sorted[k];
+                    }
                 } else {
-                    rt_ids[id_at + k] = rt_ids[id_at + k - 1];   // padding: the row in front, its tile column is zero
+                    for (uint32_t k = 0; k < rw; ++k) order[k] = k;
+                }
+                uint8_t *dt_tile = rt_data.data() + data_at + size_t(tl) * tile_bytes;
+                for (uint32_t k = 0; k < rw; ++k) {
+                    const uint32_t from = order[k];
+                    const uint32_t srci = first + std::min(from, n - 1);
+                    rt_ids[id_at + size_t(tl) * rw + k] = col[srci] - pn * KP;      // row inside the panel
+                    if (from >= n) continue;
+                    const uint8_t *st_tile = src_data + size_t(t0 + srci / cw) * src_tile_bytes;
+                    for (uint32_t r = 0; r < 8; ++r)
+                        std::memcpy(dt_tile + (size_t(r) * rw + k) * es, st_tile + (size_t(r) * cw + srci % cw) * es, es);
                 }
             }
             tiles += nt;
@@ -366,12 +415,15 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     }
     ps.n_steps = ps.unitOffset.back();
     // padding inside every panel must not eat the gain
-    if (!forced && double(ps.n_steps) > 1.35 * double(st.n_steps)) return false;
+    if (!forced && double(ps.n_steps) * double(rw / cw) > 1.35 * double(st.n_steps)) return false;
     // poff[u][pn]: first step of unit u at or behind panel pn; step_panel[s]: panel of step s
     std::vector<uint32_t> poff(size_t(U) * (NP + 1)), step_panel(ps.n_steps ? ps.n_steps : 1, 0u);
-    // per step four words; word g packs the panel rows quarter-wave g reads, 7 bits each (16-bit types:
-    // ids 4g..4g+3, fp32: ids g and g + 4), and in bits 28..31 the panels the step lies behind its predecessor
-    std::vector<uint32_t> ids(size_t(ps.n_steps) * 4u);
+    // fp32, per step four words: word g packs the panel rows quarter-wave g reads (ids g and g + 4, 7 bits
+    // each) and in bits 28..31 the panels the step lies behind its predecessor.
+    // 16-bit types, per step one word per lane (g = l / 16, i = l % 16): 9 x the panel rows of columns
+    // 8g + i / 4 (bits 4..14) and 8g + 4 + i / 4 (bits 16..26); bits 0..3: the panel count.
+    const uint32_t id_words = cw == 16 ? 64u : 4u;
+    std::vector<uint32_t> ids(size_t(ps.n_steps) * id_words);
     // fp32 single windows run through the 4x4x1 instruction, which wants row offsets (see Fp32Quad)
     bool quad = p->dtype == HSPMM_TF32 && st.G == 1;
     if (const char *e = std::getenv("HSPMM_PANEL_QUAD")) quad = quad && std::atoi(e) != 0;       // tuning override
@@ -384,16 +436,22 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
             po[pn] = ps.unitOffset[u] + at;
         }
         for (uint32_t i = 0; i < n; ++i) {
-            const uint32_t *src = rt_ids.data() + size_t(t0 + i) * cw;
-            uint32_t *dst = ids.data() + size_t(ps.unitOffset[u] + i) * 4u;
+            const uint32_t *src = rt_ids.data() + size_t(t0 + i) * rw;
+            uint32_t *dst = ids.data() + size_t(ps.unitOffset[u] + i) * id_words;
             const uint32_t jump = i ? rt_panel[t0 + i] - rt_panel[t0 + i - 1] : 0u;     // <= kMaxJump by construction
             step_panel[ps.unitOffset[u] + i] = rt_panel[t0 + i];
+            if (cw == 16) {
+                for (uint32_t l = 0; l < 64; ++l) {
+                    const uint32_t c0 = 8u * (l >> 4) + ((l & 15u) >> 2);
+                    dst[l] = jump | (src[c0] * 9u) << 4 | (src[c0 + 4] * 9u) << 16;
+                }
+                continue;
+            }
             for (uint32_t g = 0; g < 4; ++g) {
                 if (quad)   // byte offsets of rows g and g + 4 inside the panel image; the jump in bits 0..3 of word 0
                     dst[g] = (src[g] << 8 | (g == 0 ? jump : 0u)) | (src[g + 4] << 8) << 16;
                 else
-                    dst[g] = (cw == 16 ? (src[4 * g] | src[4 * g + 1] << 7 | src[4 * g + 2] << 14 | src[4 * g + 3] << 21)
-                                       : (src[g] | src[g + 4] << 7)) | jump << 28;
+                    dst[g] = (src[g] | src[g + 4] << 7) | jump << 28;
             }
         }
     }
@@ -403,7 +461,8 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     if ((rc = upload(&pl.d_step_panel, step_panel.data(), step_panel.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     if ((rc = upload(&pl.d_ids, ids.data(), ids.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     {
-        const std::vector<uint32_t> tiles = lane_order_tiles(ps, p->dtype, rt_rowOffset.data(), rt_data.data());
+        const std::vector<uint32_t> tiles = cw == 16 ? lane_order_wide_steps(ps, rt_rowOffset.data(), rt_data.data())
+                                                     : lane_order_tiles(ps, p->dtype, rt_rowOffset.data(), rt_data.data());
         uint32_t *dt = nullptr;
         if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
         pl.d_tiles = dt;
@@ -740,7 +799,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     // units), 12 otherwise, which spreads the consumer waves evenly over the SIMDs.
     // (code 13 = 12 units and four producer waves: few enough registers for two workgroups per
     // compute unit, which the 4x4x1 fp32 kernel needs to keep its short MFMAs fed)
-    int units = pl.quad ? 13 : p->G == 2 ? 14 : 12;
+    int units = pl.quad ? 13 : (p->G == 2 || p->dtype != HSPMM_TF32) ? 14 : 12;
     if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) {                                      // tuning overrides
         units = std::atoi(e) == 14 ? 14 : std::atoi(e) == 13 ? 13 : 12;
     }
@@ -760,7 +819,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     if (pa.n_chunks > 1) {
         int rc = ensure_panel_split(p, pa.n_chunks);
         if (rc) return rc;
-        const size_t nacc = pl.quad ? 2u : 4u * size_t(p->G);
+        const size_t nacc = pl.quad ? 2u : p->dtype != HSPMM_TF32 ? 8u : 4u * size_t(p->G);
         const size_t need = size_t(p->n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
         if ((rc = ensure_scratch(p, need))) return rc;
         pa.scratch = p->d_scratch;

@@ -61,8 +61,9 @@ struct PanelArgs {
     const uint32_t *unitRow;     // n_units: first matrix row of the unit | 1 if it is a pair of windows
     const uint32_t *poff;        // n_units x (n_panels + 1): first step of the unit at or behind every panel
     const uint32_t *step_panel;  // per step: its panel
-    const uint32_t *ids;         // per step four words: the rows (inside the panel) each quarter-wave reads, 7 bits
-                                 // each; bits 28..31: panels between the step and the one in front of it
+    const uint32_t *ids;         // per step: the rows (inside the panel) each quarter-wave reads and the panels
+                                 // between the step and the one in front of it; the format depends on the element
+                                 // type (PanelOps in spmm_panel_kernel.hpp)
     const void     *tiles;       // per step, lane order
     float          *scratch;     // partial sums [unit * n_chunks + chunk][feature block][acc reg][lane]
     const void     *B;

@@ -4,7 +4,7 @@
 
 namespace hspmm {
 
-template <int G> using PanelTile = Bf16X4<4, G>;
+template <int G> using PanelTile = Fp16Tr<G, true>;
 
 hipError_t launch_panel_bf16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid)
 {

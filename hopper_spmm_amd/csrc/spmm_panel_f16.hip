@@ -4,7 +4,7 @@
 
 namespace hspmm {
 
-template <int G> using PanelTile = Fp16X4<4, G>;
+template <int G> using PanelTile = Fp16Tr<G, false>;
 
 hipError_t launch_panel_f16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid)
 {

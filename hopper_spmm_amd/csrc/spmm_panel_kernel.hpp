@@ -92,7 +92,8 @@ struct Fp32Quad {
 // How a consumer wave of the panel kernel reads the ids and tiles of a step and runs it.
 template <class TT>
 struct PanelOps {
-    static constexpr int kRows = TT::kElem == 4 ? 2 : 4;         // B rows a lane reads per step
+    static_assert(TT::kElem == 4, "the 16-bit types have ops of their own");
+    static constexpr uint32_t kPitch = kPanelRowBytes;            // bytes from one row of the LDS image to the next
     static constexpr uint32_t kRing = 6;                          // steps of tiles and ids in flight
     static constexpr int kLive = TT::G * TT::V;                   // accumulator registers the step loop keeps
     __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
@@ -114,17 +115,125 @@ struct PanelOps {
         typename TT::BVec b0, b1, b2 = {}, b3 = {};
         b0 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 0, 7) << 8));
         b1 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 7, 7) << 8));
-        if constexpr (kRows == 4) {
-            b2 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 14, 7) << 8));
-            b3 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 21, 7) << 8));
-        }
         TT::mma(L, b0, b1, b2, b3, A, acc);
     }
     __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return L.j * 16u; }
 };
 
+// 16-bit element types: B rows stay row-major in LDS and the transposing LDS read of
+// gfx950 (ds_read_b64_tr_b16) turns them into MFMA operands.  In every block of 16 lanes
+// that instruction treats the 16 x 4 halves the lanes address as a 4 x 16 matrix (lane i
+// supplies columns 4 (i % 4) .. + 3 of row i / 4) and returns column j to lane j: with
+// lane i addressing 8 bytes of gathered row i / 4 at features 16 p + 4 (i % 4), lane j
+// receives B[row 0..3][16 p + j] - four consecutive k of feature j, which is what
+// v_mfma_f32_16x16x32 wants of its second operand.  Two reads give a lane its eight k.
+// The rows are gathered by the address alone, so the contraction needs neither the
+// even / odd trick of the gather kernels (half of every MFMA multiplies zeros there) nor
+// any register moves:
+//   * a step is 32 columns of a unit; quarter-wave g covers columns 8g .. 8g + 7;
+//   * first operand: the lane's 16 bytes of the plan's tile copy, A[row l % 16 of the
+//     unit's 16 rows][columns 8g .. 8g + 7] (rows 8 .. 15 are the second window of a
+//     pair, zero for a single window);
+//   * accumulator p (of 8): features 16 p .. 16 p + 15 of the block; register e of lane
+//     (g, j): unit row 4g + e, feature 16 p + j.
+// The rows of the LDS image are 288 bytes apart: the four rows one block of lanes reads
+// lie in different banks when their numbers differ mod 4, and the plan orders the
+// columns of a step accordingly (hspmm_capi.hip, build_panel_stream).
+//   ids per step: 64 words, one per lane: bits 4..14 = 9 x (panel row of column
+//     8g + i / 4), bits 16..26 = 9 x (panel row of column 8g + 4 + i / 4) (i = l % 16;
+//     x 32 = byte offset in the image); bits 0..3: the panel jump.
+typedef short tr16x4 __attribute__((ext_vector_type(4)));
+typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
+
+template <int G_, bool BF>
+struct Fp16Tr {
+    static constexpr int G = G_, V = 8 / G_;       // G * V = 8 accumulators
+    static constexpr int kBlockFeat = 128;
+    static constexpr int kLaneFeat = 1;            // lane's feature = j (+ 16 per accumulator)
+    static constexpr int kElem = 2;
+    typedef u32x4 AVec;
+    typedef typename HalfOps<BF>::elem_t elem_t;
+    struct Lane {
+        uint32_t g, j;
+        const uint32_t *a_src;
+        const uint32_t *idx_src;
+        __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
+        {
+            g = lane >> 4; j = lane & 15u;
+            a_src = reinterpret_cast<const uint32_t *>(tiles) + lane * 4u;
+            idx_src = ids + lane;
+        }
+    };
+    // Window W0 of the unit is held by quarter-waves 2 W0 and 2 W0 + 1.
+    template <int W0>
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[8], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+        if ((L.g >> 1) != uint32_t(W0)) return;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t row = row0 + 4u * (L.g & 1u) + e;
+            if (active && row < rows) {
+                elem_t *dst = reinterpret_cast<elem_t *>(c_lane + size_t(row) * row_bytes);
+#pragma unroll
+                for (int p = 0; p < 8; ++p) stream_store(dst + 16 * p, (elem_t)acc[p][e]);
+            }
+        }
+    }
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) {
+            elem_t *dst = reinterpret_cast<elem_t *>(c_lane + size_t(r) * row_bytes);
+#pragma unroll
+            for (int p = 0; p < 8; ++p) stream_store(dst + 16 * p, (elem_t)0.f);
+        }
+    }
+};
+
+template <int G_, bool BF>
+struct PanelOps<Fp16Tr<G_, BF>> {
+    typedef Fp16Tr<G_, BF> TT;
+    static constexpr uint32_t kPitch = kPanelRowBytes + 32u;
+    static constexpr uint32_t kRing = 6;
+    static constexpr int kLive = 8;
+    __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
+    typedef uint32_t Idx;
+    typedef u32x4 AVec;
+    __device__ static __forceinline__ Idx load_idx(const typename TT::Lane &L, const uint32_t *, uint32_t step)
+    {
+        return L.idx_src[size_t(step) * 64u];
+    }
+    __device__ static __forceinline__ AVec load_a(const typename TT::Lane &L, uint32_t step)
+    {
+        return *reinterpret_cast<const u32x4 *>(L.a_src + size_t(step) * 256u);
+    }
+    __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) & 15u; }
+    typedef tr16x4 __attribute__((address_space(3))) *lds_tr_ptr;
+    __device__ static __forceinline__ void step(const typename TT::Lane &, const char *smem, uint32_t img, const Idx I,
+                                                const AVec &A, f32x4 (&acc)[kLive])
+    {
+        typedef __attribute__((address_space(3))) char *lds_char_ptr;
+        const lds_char_ptr base = (lds_char_ptr)smem + img;
+        const lds_char_ptr a0 = base + (__builtin_amdgcn_ubfe(I, 4, 11) << 5);
+        const lds_char_ptr a1 = base + (__builtin_amdgcn_ubfe(I, 16, 11) << 5);
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const tr16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a0 + 32 * p));
+            const tr16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a1 + 32 * p));
+            u32x4 b;
+            const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+            b[0] = l2[0]; b[1] = l2[1]; b[2] = h2[0]; b[3] = h2[1];
+            acc[p] = HalfOps<BF>::mfma(A, b, acc[p]);
+        }
+    }
+    __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return (L.j & 3u) * 8u; }
+};
+
 template <>
 struct PanelOps<Fp32Quad> {
+    static constexpr uint32_t kPitch = kPanelRowBytes;
     static constexpr uint32_t kRing = 3;                          // few registers: two workgroups per compute unit
     // Two accumulators per 32-feature half, used in turn: an MFMA then never reads the result of
     // the one two instructions in front of it.  fold() adds the pairs once, at the end of the unit.
@@ -185,9 +294,11 @@ __global__ __launch_bounds__((NC + NPW) * 64)
 void spmm_panel_kernel(const PanelArgs pa)
 {
     constexpr int G = TT::G, V = TT::V, NACC = G * V;
+    typedef PanelOps<TT> Ops;
     constexpr int kPieces = int(kPanelBytes / 16u) / (NPW * 64);   // 16-byte pieces of a panel per producer thread
     static_assert(kPieces * NPW * 64 * 16 == int(kPanelBytes), "panel must divide among the producers");
-    __shared__ __attribute__((aligned(16))) char smem[2 * kPanelBytes];
+    constexpr uint32_t kPitch = Ops::kPitch, kImage = kPanelRows * kPitch;   // one panel image in LDS
+    __shared__ __attribute__((aligned(16))) char smem[2 * kImage];
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -210,7 +321,8 @@ void spmm_panel_kernel(const PanelArgs pa)
         const char *b_col = reinterpret_cast<const char *>(pa.B) + size_t(fb) * kPanelRowBytes + (pt & 15u) * 16u;
         const uint32_t piece_row0 = pt >> 4;
         // The loads of panel q + 1 are in flight (in registers) while the consumers multiply
-        // panel q - 1 .. q: a panel has a whole barrier period to arrive.
+        // panel q: a panel has a whole barrier period to arrive.  (Three panels in flight, with
+        // four producer waves, measured no faster.)
         u32x4 X[kPieces];
         auto issue = [&](uint32_t q) __attribute__((always_inline)) {
 #pragma unroll
@@ -222,10 +334,10 @@ void spmm_panel_kernel(const PanelArgs pa)
         };
         issue(p_begin);
         for (uint32_t q = p_begin; q < p_end; ++q) {
-            char *img = smem + (q & 1u) * kPanelBytes + pt * 16u;
+            char *img = smem + (q & 1u) * kImage + piece_row0 * kPitch + (pt & 15u) * 16u;
 #pragma unroll
             for (int i = 0; i < kPieces; ++i)
-                *reinterpret_cast<u32x4 *>(img + uint32_t(i) * (NPW * 64 * 16)) = X[i];
+                *reinterpret_cast<u32x4 *>(img + uint32_t(i) * (NPW * 4) * kPitch) = X[i];
             if (q + 1u < p_end) issue(q + 1u);
             panel_barrier();
         }
@@ -253,7 +365,6 @@ void spmm_panel_kernel(const PanelArgs pa)
     // to its predecessor, which may lie in another chunk)
     uint32_t first_jump = t1 > t0 ? as_const(pa.step_panel)[t0] - p_begin : 0u;
 
-    typedef PanelOps<TT> Ops;
     f32x4 live[Ops::kLive];
 #pragma unroll
     for (int i = 0; i < Ops::kLive; ++i) live[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -277,13 +388,14 @@ void spmm_panel_kernel(const PanelArgs pa)
     panel_barrier();                                                // panel p_begin is in its buffer
     --owed;
     // the lane's bytes of a row, in the buffer of the current panel
-    uint32_t img = (p_begin & 1u) * kPanelBytes + Ops::lane_bytes(L);
+    uint32_t img = (p_begin & 1u) * kImage + Ops::lane_bytes(L);
+    const uint32_t img_both = kImage + 2u * Ops::lane_bytes(L);     // img of one buffer + img of the other
 
     // One step: first the barriers that lie between it and the step in front of it.
     auto step = [&](const Idx &I, const AVec &A, const uint32_t jump) __attribute__((always_inline)) {
         for (uint32_t n = jump; n && owed; --n) {                   // never more barriers than the producers pass
             panel_barrier();
-            img ^= kPanelBytes;
+            img = img_both - img;
             --owed;
         }
         Ops::step(L, smem, img, I, A, live);
