@@ -302,12 +302,20 @@ void spmm_panel_kernel(const PanelArgs pa)
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // blockIdx.x = (row block * feature blocks + feature block) * chunks + chunk
+    // The hardware hands consecutive workgroups to the eight XCDs in turn, and every XCD has an L2 of
+    // its own.  The workgroups of one row block and chunk - one per feature block - read the same
+    // tiles and ids: they get numbers that are equal mod 8 and adjacent in the launch order, so that
+    // one of them fetches the tile stream into its XCD's L2 and the others hit it.
+    //   position in launch order: XCD x = blockIdx % 8 runs blocks x, x + 8, ...; the work items
+    //   (row block, chunk, feature block), feature block fastest, are dealt out XCD by XCD.
+    constexpr uint32_t kXcds = 8;
+    const uint32_t n_blocks = gridDim.x, xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+    const uint32_t item = xcd * (n_blocks / kXcds) + umin32(xcd, n_blocks % kXcds) + slot;
     const uint32_t per_rb = pa.n_feat_blocks * pa.n_chunks;
-    const uint32_t rb = blockIdx.x / per_rb;
-    const uint32_t rest = blockIdx.x - rb * per_rb;
-    const uint32_t fb = rest / pa.n_chunks;
-    const uint32_t chunk = rest - fb * pa.n_chunks;
+    const uint32_t rb = item / per_rb;
+    const uint32_t rest = item - rb * per_rb;
+    const uint32_t chunk = rest / pa.n_feat_blocks;
+    const uint32_t fb = rest - chunk * pa.n_feat_blocks;
     const uint32_t p_begin = chunk * pa.panels_per_chunk;
     const uint32_t p_end = umin32(p_begin + pa.panels_per_chunk, pa.n_panels);
     const size_t row_bytes = size_t(pa.N) * TT::kElem;
