@@ -97,6 +97,8 @@ def load_library():
     L.hspmm_get_plan_info.argtypes = [vp, C.POINTER(PlanInfo)]
     L.hspmm_get_partition.argtypes = [vp, vp, u32]
     L.hspmm_partition_preview.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
+    L.hspmm_partition_preview_grouped.argtypes = [u32, vp, u32, u32, vp, u32, C.POINTER(u32), C.POINTER(u32),
+                                                  C.POINTER(u32)]
     L.hspmm_mtx_load.argtypes = [C.c_char_p, i, C.POINTER(_Csr)]
     L.hspmm_csr_free.argtypes = [C.POINTER(_Csr)]
     L.hspmm_csr_free.restype = None
@@ -276,16 +278,25 @@ def bitmap_to_grouped(bitmap, min_len=32):
     return out
 
 
-def partition_preview(rowOffset, target_ranges):
-    """The work partition hspmm_create would build (host only)."""
+def partition_preview(rowOffset, target_ranges, group=1):
+    """The work partition hspmm_create would build (host only).  group > 1: the partition
+    for workgroups whose waves add the partial sums of one window among themselves
+    (ranges then have a sixth word, "combine")."""
     L = load_library()
     rowOffset = np.ascontiguousarray(rowOffset, np.uint32)
     W = rowOffset.size - 1
     n, ns, nslots = C.c_uint32(), C.c_uint32(), C.c_uint32()
-    _check(L.hspmm_partition_preview(W, _p(rowOffset), target_ranges, None, 0, C.byref(n), C.byref(ns),
-                                     C.byref(nslots)))
-    ranges = np.zeros((n.value, 5), np.uint32)
-    _check(L.hspmm_partition_preview(W, _p(rowOffset), target_ranges, _p(ranges), n.value, None, None, None))
+    if group == 1:
+        _check(L.hspmm_partition_preview(W, _p(rowOffset), target_ranges, None, 0, C.byref(n), C.byref(ns),
+                                         C.byref(nslots)))
+        ranges = np.zeros((n.value, 5), np.uint32)
+        _check(L.hspmm_partition_preview(W, _p(rowOffset), target_ranges, _p(ranges), n.value, None, None, None))
+    else:
+        _check(L.hspmm_partition_preview_grouped(W, _p(rowOffset), target_ranges, group, None, 0, C.byref(n),
+                                                 C.byref(ns), C.byref(nslots)))
+        ranges = np.zeros((n.value, 6), np.uint32)
+        _check(L.hspmm_partition_preview_grouped(W, _p(rowOffset), target_ranges, group, _p(ranges), n.value, None,
+                                                 None, None))
     return dict(ranges=ranges, n_split_windows=ns.value, n_partial_slots=nslots.value)
 
 

@@ -89,7 +89,7 @@ struct hspmm_plan {
         hspmm::Partition part;
         uint32_t *d_ranges = nullptr, *d_split = nullptr, *d_fix_slots = nullptr;
     };
-    DevPartition parts[3];
+    DevPartition parts[4];              // [0..2]: fewer ranges per level; [3]: level 0 with sums added per workgroup
     std::vector<uint32_t> h_unitOffset;
     // LDS-panel kernels (matrices whose windows touch a large share of the columns):
     // the unit stream re-tiled panel by panel, built by hspmm_create when it pays
@@ -167,9 +167,9 @@ int choose_ranges(const hspmm_plan *p)
     return int(g);
 }
 
-int build_and_upload_partition(hspmm_plan *p, int level)
+int build_and_upload_partition(hspmm_plan *p, int level, uint32_t group = 1)
 {
-    hspmm_plan::DevPartition &dp = p->parts[level];
+    hspmm_plan::DevPartition &dp = p->parts[group > 1 ? 3 : level];
     if (dp.built || p->W == 0) return HSPMM_OK;
     double window_cost = 1.5, slack = 0.35, margin = 32.0;
     if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);   // tuning overrides
@@ -178,7 +178,7 @@ int build_and_upload_partition(hspmm_plan *p, int level)
     uint32_t target = uint32_t(choose_ranges(p)) >> level;
     const uint32_t floor_ranges = uint32_t(p->compute_units) * 4u;       // at least one range per SIMD
     if (target < floor_ranges) target = std::min<uint32_t>(floor_ranges, uint32_t(choose_ranges(p)));
-    dp.part = hspmm::build_partition(p->n_units, p->h_unitOffset.data(), target, window_cost, slack, margin);
+    dp.part = hspmm::build_partition(p->n_units, p->h_unitOffset.data(), target, window_cost, slack, margin, group);
     const auto &part = dp.part;
     std::vector<uint32_t> rw(part.ranges.size() * hspmm::kRangeWords, 0u);
     for (size_t i = 0; i < part.ranges.size(); ++i) {
@@ -186,6 +186,7 @@ int build_and_upload_partition(hspmm_plan *p, int level)
         d[0] = part.ranges[i].tile_begin; d[1] = part.ranges[i].tile_end; d[2] = part.ranges[i].first_window;
         d[3] = part.ranges[i].head_slot; d[4] = part.ranges[i].tail_slot;
         d[5] = part.ranges[i].head_split; d[6] = part.ranges[i].tail_split;
+        d[7] = part.ranges[i].combine;
     }
     std::vector<uint32_t> sw(part.split.size() * hspmm::kFixWords, 0u);
     for (size_t i = 0; i < part.split.size(); ++i) {
@@ -611,27 +612,47 @@ int hspmm_set_window_pairing(int mode)
     return HSPMM_OK;
 }
 
-int hspmm_partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
-                            uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges,
-                            uint32_t *n_split_windows, uint32_t *n_partial_slots)
+static int partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
+                             uint32_t group, uint32_t words, uint32_t *ranges, uint32_t capacity_ranges,
+                             uint32_t *n_ranges, uint32_t *n_split_windows, uint32_t *n_partial_slots)
 {
     if (eff_row_windows && !rowOffset) return fail(HSPMM_ERR_INVALID, "null rowOffset");
+    if (group < 1 || group > uint32_t(hspmm::kMaxWavesPerGroup))
+        return fail(HSPMM_ERR_INVALID, "group %u outside 1..%d", group, hspmm::kMaxWavesPerGroup);
     for (uint32_t w = 0; w < eff_row_windows; ++w)
         if (rowOffset[w + 1] <= rowOffset[w] || rowOffset[0] != 0)
             return fail(HSPMM_ERR_INVALID, "rowOffset must start at 0 and increase strictly");
-    const hspmm::Partition part = hspmm::build_partition(eff_row_windows, rowOffset, target_ranges);
+    const hspmm::Partition part = hspmm::build_partition(eff_row_windows, rowOffset, target_ranges, 1.5, 0.35, 32.0, group);
     if (n_ranges) *n_ranges = uint32_t(part.ranges.size());
     if (n_split_windows) *n_split_windows = uint32_t(part.split.size());
     if (n_partial_slots) *n_partial_slots = part.n_slots;
     if (ranges) {
         const size_t n = part.ranges.size() < capacity_ranges ? part.ranges.size() : capacity_ranges;
         for (size_t i = 0; i < n; ++i) {
-            ranges[5 * i + 0] = part.ranges[i].tile_begin; ranges[5 * i + 1] = part.ranges[i].tile_end;
-            ranges[5 * i + 2] = part.ranges[i].first_window;
-            ranges[5 * i + 3] = part.ranges[i].head_slot; ranges[5 * i + 4] = part.ranges[i].tail_slot;
+            uint32_t *d = ranges + words * i;
+            d[0] = part.ranges[i].tile_begin; d[1] = part.ranges[i].tile_end;
+            d[2] = part.ranges[i].first_window;
+            d[3] = part.ranges[i].head_slot; d[4] = part.ranges[i].tail_slot;
+            if (words > 5) d[5] = part.ranges[i].combine;
         }
     }
     return HSPMM_OK;
+}
+
+int hspmm_partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
+                            uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges,
+                            uint32_t *n_split_windows, uint32_t *n_partial_slots)
+{
+    return partition_preview(eff_row_windows, rowOffset, target_ranges, 1, 5, ranges, capacity_ranges, n_ranges,
+                             n_split_windows, n_partial_slots);
+}
+
+int hspmm_partition_preview_grouped(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
+                                    uint32_t group, uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges,
+                                    uint32_t *n_split_windows, uint32_t *n_partial_slots)
+{
+    return partition_preview(eff_row_windows, rowOffset, target_ranges, group, 6, ranges, capacity_ranges, n_ranges,
+                             n_split_windows, n_partial_slots);
 }
 
 int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
@@ -883,9 +904,13 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
         const double steps_per_range = double(p->n_steps) / double(p->parts[0].part.ranges.size());
         if (steps_per_unit >= 8.0 * steps_per_range) level = ka.n_feat_blocks >= 4 ? 2 : ka.n_feat_blocks >= 2 ? 1 : 0;
     }
-    int rc = build_and_upload_partition(p, level);
+    // One feature block: the waves of a workgroup walk consecutive ranges and add the partial sums of
+    // one unit among themselves.
+    const int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
+    const bool combine = level == 0 && ka.n_feat_blocks == 1 && wpg > 1 && !p->cfg.fused_fixup;
+    int rc = build_and_upload_partition(p, level, combine ? uint32_t(wpg) : 1u);
     if (rc) return rc;
-    const hspmm_plan::DevPartition &dp = p->parts[level];
+    const hspmm_plan::DevPartition &dp = p->parts[combine ? 3 : level];
     ka.ranges = dp.d_ranges; ka.split = dp.d_split; ka.fix_slots = dp.d_fix_slots;
     ka.n_ranges = uint32_t(dp.part.ranges.size());
     ka.n_split = uint32_t(dp.part.split.size());
@@ -902,7 +927,6 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage
                          : p->dtype == HSPMM_TF32 ? (p->G == 2 && c.V == 4 ? 3 : 4)
                          : (p->G == 2 && c.V == 4 ? 2 : 3);
-    const int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
     HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, c.layout, p->G, ka, c.V, prefetch, c.narrow, wpg, s, mid));
     return HSPMM_OK;
 }

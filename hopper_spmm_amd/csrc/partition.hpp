@@ -24,6 +24,7 @@ struct Range {
     uint32_t first_window;            // effective window holding tile_begin
     uint32_t head_slot, tail_slot;    // partial-sum slots (kNoSlot = none)
     uint32_t head_split, tail_split;  // index of the cut window's entry in Partition::split
+    uint32_t combine;                 // 1: the ranges of this range's group add their sums before they leave the chip
 };
 
 struct SplitWindow {
@@ -47,8 +48,12 @@ struct Partition {
 // tiles, every cut moves onto a boundary and no window is cut: halving so short a
 // window saves less time than the second launch that adds its partial sums costs
 // (measured: about 6 us against 0.4 us per tile of one wave).
+// group: ranges group * k .. group * k + group - 1 are walked by the waves of one workgroup.  Where all
+// of them lie inside one window, the workgroup adds their partial sums itself (in range order) and
+// the group takes one slot, that of its first range, instead of one per range.
 inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t target_ranges,
-                                 double window_cost = 1.5, double slack = 0.35, double whole_window_margin = 32.0)
+                                 double window_cost = 1.5, double slack = 0.35, double whole_window_margin = 32.0,
+                                 uint32_t group = 1)
 {
     Partition P;
     if (W == 0) return P;
@@ -96,7 +101,17 @@ inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t
         g.first_window = win;
         g.head_slot = g.tail_slot = kNoSlot;
         g.head_split = g.tail_split = kNoSlot;
+        g.combine = 0;
     }
+    if (group > 1)
+        for (size_t r0 = 0; r0 + group <= R; r0 += group) {
+            const uint32_t w = P.ranges[r0].first_window;
+            bool inside = true;
+            for (uint32_t k = 0; k < group; ++k)
+                inside = inside && P.ranges[r0 + k].first_window == w && P.ranges[r0 + k].tile_end <= rowOffset[w + 1];
+            // two or more ranges inside one window: none of them is the whole window
+            if (inside) for (uint32_t k = 0; k < group; ++k) P.ranges[r0 + k].combine = 1;
+        }
     // Partial segments: only the first and the last window segment of a range can
     // be incomplete.  The kernel's rule: an incomplete segment that starts at the
     // range's first tile uses head_slot, any other incomplete segment tail_slot.
@@ -109,7 +124,9 @@ inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t
             const uint32_t ws = rowOffset[wv], we = rowOffset[wv + 1];
             const uint32_t se = std::min(we, g.tile_end);
             const bool complete = (t == ws) && (se == we);
-            if (!complete) {
+            if (!complete && g.combine && r % group != 0) {
+                // the group's first range, in front of this one in the same window, holds the slot
+            } else if (!complete) {
                 const uint32_t slot = P.n_slots++;
                 if (cur_split != wv) {
                     P.split.push_back(SplitWindow{wv, uint32_t(P.fix_slots.size()), 0});

@@ -490,6 +490,9 @@ void spmm_mfma_kernel(const KernelArgs ka)
     const uint32_t t0 = rd[0], t1 = rd[1];
     const uint32_t head_slot = rd[3], tail_slot = rd[4];
     const uint32_t head_split = rd[5], tail_split = rd[6];
+    // 1 (for every wave of the workgroup alike): the range is one piece of a unit, as are those of the
+    // other waves, and the workgroup adds the pieces in LDS before one sum goes to the slot of wave 0
+    const uint32_t combine = rd[7];
     const uint32_t U = ka.n_units, rows = ka.rows;
 
     typename TT::Lane L;
@@ -555,7 +558,7 @@ void spmm_mfma_kernel(const KernelArgs ka)
             } else {
                 const bool head = ww.seg_start == t0;
                 const uint32_t slot = head ? head_slot : tail_slot;
-                if (slot != kIdxMax) {
+                if (slot != kIdxMax && !combine) {
                     f32x4 *dst = reinterpret_cast<f32x4 *>(ka.scratch) +
                                  (size_t(slot) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
                     if (!ka.arrive) {
@@ -604,8 +607,10 @@ void spmm_mfma_kernel(const KernelArgs ka)
                 const uint32_t gap_begin = row0 + (paired ? 2u * kRowWindow : kRowWindow);
                 if (gap_begin < ww.next_row) TT::zero_rows(L, c_lane, row_bytes, gap_begin, ww.next_row, active);
             }
+            if (!combine) {                     // (a combining wave ends here and still needs its sums)
 #pragma unroll
-            for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+                for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
             // next unit (the reads are clamped; values past the end are not used)
             ++ww.u;
             ww.ustart = ww.uend;
@@ -637,6 +642,25 @@ void spmm_mfma_kernel(const KernelArgs ka)
             TT::load_tile(L, t + k + P, I##k, gat, HSPMM_REGS(k)); \
             I##k = TT::load_idx(L, umin32(t + k + 2u * P, tlast)); } }
         HSPMM_FOR_STAGES(HSPMM_DRAIN)
+    }
+    if (combine) {
+        // every wave of the workgroup is here with the sums of its piece: wave 0 adds them in range order
+        __shared__ f32x4 pieces[(kMaxWavesPerGroup - 1) * NACC * 64];
+        const uint32_t wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+        if (wave) {
+#pragma unroll
+            for (int p = 0; p < NACC; ++p) pieces[((wave - 1u) * NACC + p) * 64u + lane] = acc[p];
+        }
+        __syncthreads();
+        if (wave == 0u) {
+            for (uint32_t w = 1; w < n_waves; ++w) {
+#pragma unroll
+                for (int p = 0; p < NACC; ++p) acc[p] += pieces[((w - 1u) * NACC + p) * 64u + lane];
+            }
+            f32x4 *dst = reinterpret_cast<f32x4 *>(ka.scratch) + size_t(head_slot) * (NACC * 64u) + lane;
+#pragma unroll
+            for (int p = 0; p < NACC; ++p) dst[p * 64] = acc[p];
+        }
     }
 #undef HSPMM_DRAIN
 #undef HSPMM_STEADY

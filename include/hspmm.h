@@ -144,6 +144,16 @@ int hspmm_partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset,
                             uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges,
                             uint32_t *n_split_windows, uint32_t *n_partial_slots);
 
+/* No reference counterpart: the same for the case that the waves of a workgroup
+ * walk `group` consecutive ranges (1..4) and add the partial sums of one window
+ * among themselves before one sum leaves the chip (what hspmm_run does when one
+ * wave covers the whole feature dimension).  ranges: n_ranges x 6 words, the five
+ * above and {combine}: 1 for the ranges of a group that lies inside one window;
+ * only the group's first range then has a slot. */
+int hspmm_partition_preview_grouped(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
+                                    uint32_t group, uint32_t *ranges, uint32_t capacity_ranges,
+                                    uint32_t *n_ranges, uint32_t *n_split_windows, uint32_t *n_partial_slots);
+
 /* ---- host format functions ---------------------------------------------- */
 
 typedef struct {

@@ -83,3 +83,63 @@ def test_partition_rejects_bad_offsets(hs):
         hs.partition_preview(np.array([0, 5, 5], np.uint32), 4)
     with pytest.raises(hs.HspmmError):
         hs.partition_preview(np.array([1, 5], np.uint32), 4)
+
+
+def simulate_grouped(ranges, ro, group):
+    """The kernel's rule with workgroups of `group` waves: a wave whose range has the combine
+    mark keeps its sums; wave 0 of the workgroup stores the workgroup's total in its head slot."""
+    partial, direct = {}, []
+    for i, (t0, t1, w, head, tail, combine) in enumerate(ranges.tolist()):
+        assert ro[w] <= t0 < ro[w + 1]
+        if combine:
+            mates = ranges[i - i % group: i - i % group + group]
+            assert len(mates) == group and np.all(mates[:, 5] == 1) and np.all(mates[:, 2] == w)
+            assert ro[w] <= t0 and t1 <= ro[w + 1] and (t0, t1) != (ro[w], ro[w + 1])   # one piece of one window
+            assert tail == NO
+            if i % group == 0:
+                assert head != NO
+                partial.setdefault(w, []).append(head)
+            else:
+                assert head == NO
+            continue
+        t = t0
+        while t < t1:
+            ws, we = int(ro[w]), int(ro[w + 1])
+            se = min(we, t1)
+            if t == ws and se == we:
+                direct.append(w)
+            else:
+                slot = head if t == t0 else tail
+                assert slot != NO
+                partial.setdefault(w, []).append(slot)
+            t = se
+            if se == we:
+                w += 1
+    return partial, direct
+
+
+@pytest.mark.parametrize("group", [2, 3, 4])
+def test_partition_with_sums_added_per_workgroup(hs, group):
+    rng = np.random.default_rng(group)
+    cases = [np.array([0, 100]), np.array([0, 1, 2, 400, 401]), np.arange(0, 1001),
+             np.concatenate([[0], np.cumsum(rng.integers(1, 600, 64))]),
+             np.concatenate([[0], np.cumsum(np.minimum(5000, np.floor(rng.pareto(1.2, 300)) + 1).astype(np.int64))])]
+    for ro in cases:
+        ro = np.asarray(ro, np.uint32)
+        for target in (1, 5, 16, 64, 255):
+            plain = hs.partition_preview(ro, target)
+            p = hs.partition_preview(ro, target, group=group)
+            r = p["ranges"]
+            assert np.array_equal(r[:, :3], plain["ranges"][:, :3])                   # the same cuts
+            partial, direct = simulate_grouped(r, ro, group)
+            slots = [s for w in sorted(partial) for s in partial[w]]
+            assert sorted(slots) == list(range(p["n_partial_slots"]))
+            assert p["n_split_windows"] == len(partial)
+            assert sorted(direct + list(partial)) == list(range(ro.size - 1))
+            assert p["n_partial_slots"] <= plain["n_partial_slots"]
+            # slots of a window appear in range order
+            for w, sl in partial.items():
+                assert sl == sorted(sl)
+    # a long window cut into many pieces: whole workgroups inside it share one slot each
+    p = hs.partition_preview(np.array([0, 4096], np.uint32), 64, group=4)
+    assert p["n_partial_slots"] == 16 and np.all(p["ranges"][:, 5] == 1)
