@@ -152,8 +152,20 @@ def get_config():
     return tuple(x.value for x in v)
 
 
+_kernel_mode = 0
+
+
 def set_kernel_mode(mode):
+    """hspmm_set_kernel_mode: 0 automatic, 1 scalar kernel, 2 wide loads, 3 word loads, 4 LDS-staging
+    kernels for every matrix, 5 the same with fp32 products for HSPMM_TF32."""
+    global _kernel_mode
     _check(load_library().hspmm_set_kernel_mode(mode))
+    _kernel_mode = mode
+
+
+def get_kernel_mode():
+    """The mode last set through set_kernel_mode of this module."""
+    return _kernel_mode
 
 
 def set_window_pairing(mode):

@@ -100,6 +100,7 @@ struct hspmm_plan {
         void *d_tiles = nullptr;
         uint32_t *d_split = nullptr, *d_fix_slots = nullptr;    // one split entry per unit, for the chunk sums
         bool quad = false;                                       // ids in the format of the 4x4x1 fp32 tile
+        bool split = false;                                      // fp32 stream in the bf16 hi / lo form (Fp32Split)
         uint32_t split_chunks = 0;                               // chunk count d_split was built for
         size_t fix_slot_count = 0;
     } panel;
@@ -316,6 +317,50 @@ std::vector<uint32_t> lane_order_wide_steps(const StepStream &st, const uint32_t
     return out;
 }
 
+// fp32 value -> its upper 16 bits (bf16, cut) in the low half, bf16(value - that) (nearest even) in the
+// high half; the same split the producer waves apply to B (write_piece of Fp32Split in spmm_panel_kernel.hpp).
+uint32_t split_bf16_host(float v)
+{
+    uint32_t bits;
+    std::memcpy(&bits, &v, 4);
+    const uint32_t hi = bits & 0xFFFF0000u;
+    if ((bits & 0x7F800000u) == 0x7F800000u) return hi >> 16;            // infinite or NaN: hi carries it
+    float hf;
+    std::memcpy(&hf, &hi, 4);
+    const float rest = v - hf;                                            // exact
+    uint32_t rb;
+    std::memcpy(&rb, &rest, 4);
+    rb += 0x7FFFu + ((rb >> 16) & 1u);                                    // nearest even (rest is finite and small)
+    return (hi >> 16) | (rb & 0xFFFF0000u);
+}
+
+// fp32 steps of 32 columns in the split form (Fp32Split): a re-tiled step of a window is [row r][32 floats];
+// lane l = (g, m) gets 32 bytes: the 8 hi halves, then the 8 lo halves of a[m][8g .. 8g + 7].
+std::vector<uint32_t> lane_order_split_steps(const StepStream &st, const uint32_t *rowOffset, const void *data)
+{
+    const float *vals = static_cast<const float *>(data);            // a step of a window is 8 x 32 floats
+    std::vector<uint32_t> out(size_t(st.n_steps) * 512u, 0u);
+    for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
+        const uint32_t w0 = st.unitWindow[u];
+        const int nwin = (st.unitRow[u] & 1u) ? 2 : 1;
+        for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
+            uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * 512u);
+            for (int w = 0; w < nwin; ++w) {
+                const float *src = vals + size_t(rowOffset[w0 + w] + i) * 256u;
+                for (uint32_t r = 0; r < 8; ++r)
+                    for (uint32_t g = 0; g < 4; ++g)
+                        for (uint32_t c = 0; c < 8; ++c) {
+                            const uint32_t sp = split_bf16_host(src[r * 32u + 8u * g + c]);
+                            uint16_t *lane = dst + (g * 16u + 8u * w + r) * 16u;
+                            lane[c] = uint16_t(sp & 0xFFFFu);
+                            lane[8 + c] = uint16_t(sp >> 16);
+                        }
+            }
+        }
+    }
+    return out;
+}
+
 // Re-tiles the matrix panel by panel for the LDS-panel kernels (spmm_panel_kernel.hpp):
 // inside every window the columns of one panel of kPanelRows columns get tiles of
 // their own.  Every step carries the number of panels it lies behind the step in
@@ -326,17 +371,20 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
 {
     *rc_out = HSPMM_OK;
     const uint32_t cw = p->cw, W = p->W;
-    const uint32_t KP = hspmm::kPanelRows;
+    // fp32: products of bf16 hi / lo parts (Fp32Split) unless the caller asked for fp32 products
+    const bool split = p->dtype == HSPMM_TF32 && p->cfg.kernel_mode != 5;
+    const uint32_t KP = (cw == 16 || split) ? hspmm::kPanelRowsWide : hspmm::kPanelRowsFp32;
     const uint32_t NP = (p->cols + KP - 1) / KP;
     const uint32_t U = uint32_t(st.unitRow.size());
     constexpr uint32_t kMaxJump = 15;
     if (U == 0 || NP == 0) return false;
-    // worth it when a unit has a few steps in every panel it meets: the panel image is
+    // worth it when a unit has a few steps in every 128 columns it meets: the panel image is
     // then read from LDS several times per load from the L2
-    if (!forced && double(st.n_steps) < 2.0 * double(U) * double(NP)) return false;
+    if (!forced && double(st.n_steps) < 2.0 * double(U) * double((p->cols + 127u) / 128u)) return false;
     if (uint64_t(U) * (NP + 1) > (1ull << 28)) return false;
-    // columns per re-tiled step: the 16-bit kernels contract 32 columns per step, fp32 a tile's 8
-    const uint32_t rw = cw == 16 ? 32u : cw;
+    // columns per re-tiled step: the kernels built on 16-bit MFMAs contract 32 columns per step, the fp32
+    // MFMA kernels a tile's 8
+    const uint32_t rw = (cw == 16 || split) ? 32u : cw;
     const size_t es = p->elem, src_tile_bytes = size_t(8) * cw * es, tile_bytes = size_t(8) * rw * es;
     std::vector<uint32_t> rt_rowOffset(size_t(W) + 1, 0u), rt_ids, rt_panel;
     std::vector<uint8_t> rt_data;
@@ -423,11 +471,10 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     // each) and in bits 28..31 the panels the step lies behind its predecessor.
     // 16-bit types, per step one word per lane (g = l / 16, i = l % 16): 9 x the panel rows of columns
     // 8g + i / 4 (bits 4..14) and 8g + 4 + i / 4 (bits 16..26); bits 0..3: the panel count.
-    const uint32_t id_words = cw == 16 ? 64u : 4u;
+    const uint32_t id_words = rw == 32 ? 64u : 4u;
     std::vector<uint32_t> ids(size_t(ps.n_steps) * id_words);
     // fp32 single windows run through the 4x4x1 instruction, which wants row offsets (see Fp32Quad)
-    bool quad = p->dtype == HSPMM_TF32 && st.G == 1;
-    if (const char *e = std::getenv("HSPMM_PANEL_QUAD")) quad = quad && std::atoi(e) != 0;       // tuning override
+    const bool quad = p->dtype == HSPMM_TF32 && !split && st.G == 1;
     for (uint32_t u = 0; u < U; ++u) {
         const uint32_t t0 = rt_rowOffset[st.unitWindow[u]], n = ps.unitOffset[u + 1] - ps.unitOffset[u];
         uint32_t *po = poff.data() + size_t(u) * (NP + 1);
@@ -441,7 +488,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
             uint32_t *dst = ids.data() + size_t(ps.unitOffset[u] + i) * id_words;
             const uint32_t jump = i ? rt_panel[t0 + i] - rt_panel[t0 + i - 1] : 0u;     // <= kMaxJump by construction
             step_panel[ps.unitOffset[u] + i] = rt_panel[t0 + i];
-            if (cw == 16) {
+            if (rw == 32) {
                 for (uint32_t l = 0; l < 64; ++l) {
                     const uint32_t c0 = 8u * (l >> 4) + ((l & 15u) >> 2);
                     dst[l] = jump | (src[c0] * 9u) << 4 | (src[c0 + 4] * 9u) << 16;
@@ -462,13 +509,14 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     if ((rc = upload(&pl.d_step_panel, step_panel.data(), step_panel.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     if ((rc = upload(&pl.d_ids, ids.data(), ids.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     {
-        const std::vector<uint32_t> tiles = cw == 16 ? lane_order_wide_steps(ps, rt_rowOffset.data(), rt_data.data())
-                                                     : lane_order_tiles(ps, p->dtype, rt_rowOffset.data(), rt_data.data());
+        const std::vector<uint32_t> tiles = split      ? lane_order_split_steps(ps, rt_rowOffset.data(), rt_data.data())
+                                            : cw == 16 ? lane_order_wide_steps(ps, rt_rowOffset.data(), rt_data.data())
+                                                       : lane_order_tiles(ps, p->dtype, rt_rowOffset.data(), rt_data.data());
         uint32_t *dt = nullptr;
         if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
         pl.d_tiles = dt;
     }
-    pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.built = true;
+    pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.split = split; pl.built = true;
     return true;
 }
 
@@ -598,7 +646,7 @@ void hspmm_get_config(int *buffer_stage, int *consumer_warp_num, int *producer_w
 
 int hspmm_set_kernel_mode(int mode)
 {
-    if (mode < 0 || mode > 4) return fail(HSPMM_ERR_INVALID, "kernel mode %d outside 0..4", mode);
+    if (mode < 0 || mode > 5) return fail(HSPMM_ERR_INVALID, "kernel mode %d outside 0..5", mode);
     std::lock_guard<std::mutex> lk(g_cfg_mutex);
     g_cfg.kernel_mode = mode;
     return HSPMM_OK;
@@ -723,9 +771,9 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         }
         p->h_unitOffset = st.unitOffset;
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
-        if (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 4) {
+        if (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4) {
             int prc = HSPMM_OK;
-            (void)build_panel_stream(p, st, rowOffset, tcA2B, data, p->cfg.kernel_mode == 4, &prc);
+            (void)build_panel_stream(p, st, rowOffset, tcA2B, data, p->cfg.kernel_mode >= 4, &prc);
             if (prc) return bail(prc);
         }
     }
@@ -815,20 +863,37 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     pa.n_units = p->n_units; pa.rows = p->rows; pa.cols = p->cols; pa.N = N;
     pa.n_feat_blocks = N / (hspmm::kPanelRowBytes / p->elem);
     pa.n_panels = pl.n_panels;
-    // 16 waves per workgroup fill a compute unit (two workgroups with 64 KB of LDS each
-    // do not become resident together): 14 units where the LDS reads bind (paired
-    // units), 12 otherwise, which spreads the consumer waves evenly over the SIMDs.
-    // (code 13 = 12 units and four producer waves: few enough registers for two workgroups per
-    // compute unit, which the 4x4x1 fp32 kernel needs to keep its short MFMAs fed)
-    int units = pl.quad ? 13 : (p->G == 2 || p->dtype != HSPMM_TF32) ? 14 : 12;
+    // The workgroup shape: code 14 / 12 = that many consumer waves and two producers, 13 = 12 consumers and
+    // four producers (few enough registers for two workgroups per compute unit, which the 4x4x1 fp32 kernel
+    // needs to keep its short MFMAs fed).  Of the consumer waves any number may be given a unit.
+    const bool wide = p->dtype != HSPMM_TF32 || pl.split;          // panels of 256 rows: always 12 + 4 waves
+    int units = (pl.quad || wide) ? 13 : p->G == 2 ? 14 : 12;
+    int forced_units = 0;
     if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) {                                      // tuning overrides
         units = std::atoi(e) == 14 ? 14 : std::atoi(e) == 13 ? 13 : 12;
+        forced_units = units == 13 ? 12 : units;
+        if (wide) { units = 13; forced_units = std::min(forced_units, 12); }
     }
-    // chunks of panels: as many as keep the workgroups within one round over the compute units
-    const int units_per_group = units == 13 ? 12 : units;
-    const uint64_t row_blocks = (uint64_t(p->n_units) + units_per_group - 1) / units_per_group;
+    const int max_units = units == 13 ? 12 : units;
+    const uint64_t slots = uint64_t(p->compute_units) * (pl.quad ? 2u : 1u);     // workgroups resident at a time
+    // Units per workgroup and chunks of panels: the workgroups should fill the compute units in whole
+    // rounds.  Cost of a shape = rounds x panels per chunk x (units + 3: a panel costs its LDS reads, which
+    // go with the units, plus its copy and barrier), plus the second launch when there are chunk sums.
+    uint64_t chunks = 1;
+    int best_units = max_units;
+    double best_cost = 0.0;
+    for (int nc = forced_units ? forced_units : std::max(4, max_units / 2); nc <= (forced_units ? forced_units : max_units); ++nc) {
+        const uint64_t rbs = (uint64_t(p->n_units) + nc - 1) / nc, base = rbs * pa.n_feat_blocks;
+        uint64_t ch = base >= slots ? 1 : std::min<uint64_t>(slots / base, pl.n_panels);
+        const uint64_t ppc = (pl.n_panels + ch - 1) / ch;
+        ch = (pl.n_panels + ppc - 1) / ppc;
+        const uint64_t rounds = (base * ch + slots - 1) / slots;
+        const double cost = double(rounds) * double(ppc) * (nc + 3.0) + (ch > 1 ? 80.0 : 0.0);
+        if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best_units = nc; chunks = ch; }
+    }
+    pa.units_per_group = uint32_t(best_units);
+    const uint64_t row_blocks = (uint64_t(p->n_units) + best_units - 1) / best_units;
     const uint64_t base = row_blocks * pa.n_feat_blocks;
-    uint64_t chunks = uint64_t(p->compute_units) / base;
     if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) chunks = uint64_t(std::atoi(e));
     if (chunks < 1) chunks = 1;
     if (chunks > pl.n_panels) chunks = pl.n_panels;
@@ -840,7 +905,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     if (pa.n_chunks > 1) {
         int rc = ensure_panel_split(p, pa.n_chunks);
         if (rc) return rc;
-        const size_t nacc = pl.quad ? 2u : p->dtype != HSPMM_TF32 ? 8u : 4u * size_t(p->G);
+        const size_t nacc = pl.quad ? 2u : pl.split ? 4u : p->dtype != HSPMM_TF32 ? 8u : 4u * size_t(p->G);
         const size_t need = size_t(p->n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
         if ((rc = ensure_scratch(p, need))) return rc;
         pa.scratch = p->d_scratch;
@@ -850,7 +915,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         ka.n_split = p->n_units; ka.n_units = p->n_units; ka.rows = p->rows; ka.N = N;
         ka.n_feat_blocks = pa.n_feat_blocks;
     }
-    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : p->G, pa, ka, units, s, mid));
+    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : p->G, pl.split, pa, ka, units, s, mid));
     return HSPMM_OK;
 }
 
@@ -877,7 +942,7 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
         HSPMM_HIP(hspmm::launch_fill_zero(dC, size_t(p->rows) * N * p->elem, s));
         return HSPMM_OK;
     }
-    if (p->panel.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 4)) {
+    if (p->panel.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4)) {
         // LDS-panel kernels: a workgroup covers 256 bytes of every B row with 16-byte accesses
         const uint32_t block_feat = hspmm::kPanelRowBytes / p->elem;
         const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);

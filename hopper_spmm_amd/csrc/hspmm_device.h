@@ -53,9 +53,10 @@ hipError_t launch_spmm_mfma(int dtype, int layout, int G, const KernelArgs &ka, 
 hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s);
 
 // LDS-panel kernels (spmm_panel_kernel.hpp).
-constexpr uint32_t kPanelRows = 128;           // B rows per panel
 constexpr uint32_t kPanelRowBytes = 256;       // bytes of a B row one workgroup covers (128 halves / 64 floats)
-constexpr uint32_t kPanelBytes = kPanelRows * kPanelRowBytes;
+// B rows per panel: 256 for the kernels built on the transposing LDS read (16-bit types, fp32 in bf16
+// parts), 128 for the fp32 MFMA forms
+constexpr uint32_t kPanelRowsWide = 256, kPanelRowsFp32 = 128;
 
 struct PanelArgs {
     const uint32_t *unitRow;     // n_units: first matrix row of the unit | 1 if it is a pair of windows
@@ -69,13 +70,16 @@ struct PanelArgs {
     const void     *B;
     void           *C;
     uint32_t n_units, n_steps, rows, cols, N, n_feat_blocks, n_panels, n_chunks, panels_per_chunk;
+    uint32_t units_per_group;    // consumer waves of a workgroup that get a unit (<= those the kernel has); the
+                                 // others only keep the barriers company
 };
 
 // units: 12 or 14 units (consumer waves) per workgroup, 2 more waves copy B to LDS; 13 = 12 units and 4 such waves.
-// G: windows per unit; 0 = fp32 single windows with ids in the format of the 4x4x1 tile.  ka: arguments of the kernel that adds
-// the chunk sums (split table with one entry per unit), used when pa.n_chunks > 1.
-hipError_t launch_spmm_panel(int dtype, int G, const PanelArgs &pa, const KernelArgs &ka, int units, hipStream_t s,
-                             hipEvent_t mid);
+// G: windows per unit; 0 = fp32 single windows with ids in the format of the 4x4x1 tile.  split (fp32): the plan's
+// stream is in the bf16 hi / lo form.  ka: arguments of the kernel that adds the chunk sums (split table with one
+// entry per unit), used when pa.n_chunks > 1.
+hipError_t launch_spmm_panel(int dtype, int G, bool split, const PanelArgs &pa, const KernelArgs &ka, int units,
+                             hipStream_t s, hipEvent_t mid);
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
 
 }  // namespace hspmm

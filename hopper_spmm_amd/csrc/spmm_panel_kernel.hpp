@@ -93,7 +93,13 @@ struct Fp32Quad {
 template <class TT>
 struct PanelOps {
     static_assert(TT::kElem == 4, "the 16-bit types have ops of their own");
+    static constexpr uint32_t kRows = kPanelRowsFp32;             // B rows per panel
     static constexpr uint32_t kPitch = kPanelRowBytes;            // bytes from one row of the LDS image to the next
+    // a producer's 16 bytes of a B row: column piece c of the image row
+    __device__ static __forceinline__ void write_piece(char *row, uint32_t c, const u32x4 x)
+    {
+        *reinterpret_cast<u32x4 *>(row + c * 16u) = x;
+    }
     static constexpr uint32_t kRing = 6;                          // steps of tiles and ids in flight
     static constexpr int kLive = TT::G * TT::V;                   // accumulator registers the step loop keeps
     __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
@@ -139,8 +145,8 @@ struct PanelOps {
 // The rows of the LDS image are 288 bytes apart: the four rows one block of lanes reads
 // lie in different banks when their numbers differ mod 4, and the plan orders the
 // columns of a step accordingly (hspmm_capi.hip, build_panel_stream).
-//   ids per step: 64 words, one per lane: bits 4..14 = 9 x (panel row of column
-//     8g + i / 4), bits 16..26 = 9 x (panel row of column 8g + 4 + i / 4) (i = l % 16;
+//   ids per step: 64 words, one per lane: bits 4..15 = 9 x (panel row of column
+//     8g + i / 4), bits 16..27 = 9 x (panel row of column 8g + 4 + i / 4) (i = l % 16;
 //     x 32 = byte offset in the image); bits 0..3: the panel jump.
 typedef short tr16x4 __attribute__((ext_vector_type(4)));
 typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
@@ -195,7 +201,12 @@ struct Fp16Tr {
 template <int G_, bool BF>
 struct PanelOps<Fp16Tr<G_, BF>> {
     typedef Fp16Tr<G_, BF> TT;
+    static constexpr uint32_t kRows = kPanelRowsWide;
     static constexpr uint32_t kPitch = kPanelRowBytes + 32u;
+    __device__ static __forceinline__ void write_piece(char *row, uint32_t c, const u32x4 x)
+    {
+        *reinterpret_cast<u32x4 *>(row + c * 16u) = x;
+    }
     static constexpr uint32_t kRing = 6;
     static constexpr int kLive = 8;
     __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
@@ -216,8 +227,8 @@ struct PanelOps<Fp16Tr<G_, BF>> {
     {
         typedef __attribute__((address_space(3))) char *lds_char_ptr;
         const lds_char_ptr base = (lds_char_ptr)smem + img;
-        const lds_char_ptr a0 = base + (__builtin_amdgcn_ubfe(I, 4, 11) << 5);
-        const lds_char_ptr a1 = base + (__builtin_amdgcn_ubfe(I, 16, 11) << 5);
+        const lds_char_ptr a0 = base + (__builtin_amdgcn_ubfe(I, 4, 12) << 5);
+        const lds_char_ptr a1 = base + (__builtin_amdgcn_ubfe(I, 16, 12) << 5);
 #pragma unroll
         for (int p = 0; p < 8; ++p) {
             const tr16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a0 + 32 * p));
@@ -231,9 +242,153 @@ struct PanelOps<Fp16Tr<G_, BF>> {
     __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return (L.j & 3u) * 8u; }
 };
 
+// fp32 storage through the 16-bit MFMA: gfx950 has no tf32 / xf32 matrix instruction, its fp32
+// MFMA runs at 1/16 of the bf16 rate, and the reference's "tf32" arithmetic keeps 10 mantissa bits
+// of each factor (reference src/ptx/wgmma.h:42-58).  Here every fp32 value v is taken as
+// hi + lo with hi = v cut to bf16 (its upper 16 bits: same sign, never overflows) and
+// lo = bf16(v - hi) (the difference is exact, its rounding leaves |v - hi - lo| <= 2^-16 |v|), and
+// a * b = a_hi b_hi + a_hi b_lo + a_lo b_hi + a_lo b_lo with fp32 accumulation: four
+// v_mfma_f32_16x16x32_bf16 where fp32 inputs would need eight 16x16x4 instructions of twice the
+// length, and 16 mantissa bits per factor where tf32 keeps 10.  The sparse values are split by
+// the plan, the rows of B by the producer waves on their way into LDS: an image row is
+// [64 hi halves][64 lo halves], read through the transposing LDS read like the 16-bit types.
+// An infinite or NaN v has lo = 0 (hi carries it).
+//   ids per step: as Fp16Tr.  tiles per step: per lane 8 hi halves then 8 lo halves of
+//   A[row l % 16][columns 8g .. 8g + 7] (32 bytes).
+//   accumulator p (of 4): features 16 p .. 16 p + 15 of the block of 64.
+template <int G_>
+struct Fp32Split {
+    static constexpr int G = G_, V = 4 / G_;       // G * V = 4 accumulators
+    static constexpr int kBlockFeat = 64;
+    static constexpr int kLaneFeat = 1;
+    static constexpr int kElem = 4;
+    typedef u32x8 AVec;
+    struct Lane {
+        uint32_t g, j;
+        const uint32_t *a_src;
+        const uint32_t *idx_src;
+        __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
+        {
+            g = lane >> 4; j = lane & 15u;
+            a_src = reinterpret_cast<const uint32_t *>(tiles) + lane * 8u;
+            idx_src = ids + lane;
+        }
+    };
+    template <int W0>
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[4], char *c_lane,
+                                                        size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
+    {
+        if ((L.g >> 1) != uint32_t(W0)) return;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t row = row0 + 4u * (L.g & 1u) + e;
+            if (active && row < rows) {
+                float *dst = reinterpret_cast<float *>(c_lane + size_t(row) * row_bytes);
+#pragma unroll
+                for (int p = 0; p < 4; ++p) { const float v = acc[p][e]; stream_store(dst + 16 * p, v); }
+            }
+        }
+    }
+    __device__ static __forceinline__ void zero_rows(const Lane &L, char *c_lane, size_t row_bytes, uint32_t r_begin,
+                                                     uint32_t r_end, bool active)
+    {
+        if (!active) return;
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) {
+            float *dst = reinterpret_cast<float *>(c_lane + size_t(r) * row_bytes);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) stream_store(dst + 16 * p, 0.f);
+        }
+    }
+};
+
+// v - (v cut to bf16): exact; 0 where v is infinite or NaN (hi carries those)
+__device__ __forceinline__ float split_rest(const uint32_t v)
+{
+    const float f = __builtin_bit_cast(float, v);
+    const float rest = f - __builtin_bit_cast(float, v & 0xFFFF0000u);
+    return __builtin_isfinite(f) ? rest : 0.f;
+}
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16_rn(const float a, const float b)
+{
+    bf16x2_t r;
+    r[0] = (__bf16)a; r[1] = (__bf16)b;
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+template <int G_>
+struct PanelOps<Fp32Split<G_>> {
+    typedef Fp32Split<G_> TT;
+    static constexpr uint32_t kRows = kPanelRowsWide;
+    static constexpr uint32_t kPitch = kPanelRowBytes + 32u;
+    // four floats of a row -> four hi halves at [4c .. 4c + 3], four lo halves 128 bytes further on
+    __device__ static __forceinline__ void write_piece(char *row, uint32_t c, const u32x4 x)
+    {
+        u32x2 hi, lo;
+        hi[0] = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);       // the upper halves
+        hi[1] = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
+        lo[0] = pack_bf16_rn(split_rest(x[0]), split_rest(x[1]));
+        lo[1] = pack_bf16_rn(split_rest(x[2]), split_rest(x[3]));
+        *reinterpret_cast<u32x2 *>(row + c * 8u) = hi;
+        *reinterpret_cast<u32x2 *>(row + 128u + c * 8u) = lo;
+    }
+    static constexpr uint32_t kRing = 4;
+    static constexpr int kLive = 4;
+    __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
+    typedef uint32_t Idx;
+    typedef u32x8 AVec;
+    __device__ static __forceinline__ Idx load_idx(const typename TT::Lane &L, const uint32_t *, uint32_t step)
+    {
+        return L.idx_src[size_t(step) * 64u];
+    }
+    __device__ static __forceinline__ AVec load_a(const typename TT::Lane &L, uint32_t step)
+    {
+        return *reinterpret_cast<const u32x8 *>(L.a_src + size_t(step) * 512u);
+    }
+    __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) & 15u; }
+    typedef tr16x4 __attribute__((address_space(3))) *lds_tr_ptr;
+    __device__ static __forceinline__ u32x4 operand(const __attribute__((address_space(3))) char *a0,
+                                                    const __attribute__((address_space(3))) char *a1, int off)
+    {
+        const tr16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a0 + off));
+        const tr16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a1 + off));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        u32x4 b;
+        b[0] = l2[0]; b[1] = l2[1]; b[2] = h2[0]; b[3] = h2[1];
+        return b;
+    }
+    __device__ static __forceinline__ void step(const typename TT::Lane &, const char *smem, uint32_t img, const Idx I,
+                                                const AVec &A, f32x4 (&acc)[kLive])
+    {
+        typedef __attribute__((address_space(3))) char *lds_char_ptr;
+        const lds_char_ptr base = (lds_char_ptr)smem + img;
+        const lds_char_ptr a0 = base + (__builtin_amdgcn_ubfe(I, 4, 12) << 5);
+        const lds_char_ptr a1 = base + (__builtin_amdgcn_ubfe(I, 16, 12) << 5);
+        u32x4 a_hi, a_lo;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { a_hi[i] = A[i]; a_lo[i] = A[4 + i]; }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const u32x4 b_hi = operand(a0, a1, 32 * p);
+            const u32x4 b_lo = operand(a0, a1, 128 + 32 * p);
+            // small terms first
+            f32x4 c = HalfOps<true>::mfma(a_lo, b_lo, acc[p]);
+            c = HalfOps<true>::mfma(a_lo, b_hi, c);
+            c = HalfOps<true>::mfma(a_hi, b_lo, c);
+            acc[p] = HalfOps<true>::mfma(a_hi, b_hi, c);
+        }
+    }
+    __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return (L.j & 3u) * 8u; }
+};
+
 template <>
 struct PanelOps<Fp32Quad> {
+    static constexpr uint32_t kRows = kPanelRowsFp32;
     static constexpr uint32_t kPitch = kPanelRowBytes;
+    __device__ static __forceinline__ void write_piece(char *row, uint32_t c, const u32x4 x)
+    {
+        *reinterpret_cast<u32x4 *>(row + c * 16u) = x;
+    }
     static constexpr uint32_t kRing = 3;                          // few registers: two workgroups per compute unit
     // Two accumulators per 32-feature half, used in turn: an MFMA then never reads the result of
     // the one two instructions in front of it.  fold() adds the pairs once, at the end of the unit.
@@ -295,8 +450,10 @@ void spmm_panel_kernel(const PanelArgs pa)
 {
     constexpr int G = TT::G, V = TT::V, NACC = G * V;
     typedef PanelOps<TT> Ops;
+    constexpr uint32_t kPanelRows = Ops::kRows, kPanelBytes = kPanelRows * kPanelRowBytes;
     constexpr int kPieces = int(kPanelBytes / 16u) / (NPW * 64);   // 16-byte pieces of a panel per producer thread
     static_assert(kPieces * NPW * 64 * 16 == int(kPanelBytes), "panel must divide among the producers");
+    static_assert(kPieces <= 16, "a producer thread holds a panel's pieces in registers");
     constexpr uint32_t kPitch = Ops::kPitch, kImage = kPanelRows * kPitch;   // one panel image in LDS
     __shared__ __attribute__((aligned(16))) char smem[2 * kImage];
 
@@ -342,10 +499,9 @@ void spmm_panel_kernel(const PanelArgs pa)
         };
         issue(p_begin);
         for (uint32_t q = p_begin; q < p_end; ++q) {
-            char *img = smem + (q & 1u) * kImage + piece_row0 * kPitch + (pt & 15u) * 16u;
+            char *img = smem + (q & 1u) * kImage + piece_row0 * kPitch;
 #pragma unroll
-            for (int i = 0; i < kPieces; ++i)
-                *reinterpret_cast<u32x4 *>(img + uint32_t(i) * (NPW * 4) * kPitch) = X[i];
+            for (int i = 0; i < kPieces; ++i) Ops::write_piece(img + uint32_t(i) * (NPW * 4) * kPitch, pt & 15u, X[i]);
             if (q + 1u < p_end) issue(q + 1u);
             panel_barrier();
         }
@@ -353,8 +509,8 @@ void spmm_panel_kernel(const PanelArgs pa)
     }
 
     // ---- consumer
-    const uint32_t u = rb * NC + wave;
-    const bool has_unit = u < pa.n_units;
+    const uint32_t u = rb * pa.units_per_group + wave;
+    const bool has_unit = wave < pa.units_per_group && u < pa.n_units;
     const const_u32_ptr poff = as_const(pa.poff) + size_t(has_unit ? u : 0u) * (pa.n_panels + 1u);
 
     typename TT::Lane L;
@@ -471,7 +627,8 @@ void spmm_panel_kernel(const PanelArgs pa)
 template <class TT, int NC, int NPW>
 static hipError_t launch_panel_tt(const PanelArgs &pa, const KernelArgs &ka, hipStream_t s, hipEvent_t mid)
 {
-    const uint32_t row_blocks = (pa.n_units + NC - 1) / NC;
+    if (pa.units_per_group < 1u || pa.units_per_group > uint32_t(NC)) return hipErrorInvalidValue;
+    const uint32_t row_blocks = (pa.n_units + pa.units_per_group - 1u) / pa.units_per_group;
     const dim3 grid(row_blocks * pa.n_feat_blocks * pa.n_chunks), block((NC + NPW) * 64);
     spmm_panel_kernel<TT, NC, NPW><<<grid, block, 0, s>>>(pa);
     hipError_t e = hipGetLastError();
@@ -485,9 +642,13 @@ static hipError_t launch_panel_tt(const PanelArgs &pa, const KernelArgs &ka, hip
 template <class TT>
 static hipError_t launch_panel_nw(const PanelArgs &pa, const KernelArgs &ka, int units, hipStream_t s, hipEvent_t mid)
 {
-    if (units == 14) return launch_panel_tt<TT, 14, 2>(pa, ka, s, mid);
-    if (units == 13) return launch_panel_tt<TT, 12, 4>(pa, ka, s, mid);      // 12 units, four producer waves
-    return launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
+    // panels of 256 rows need four producer waves to hold one in registers
+    if constexpr (PanelOps<TT>::kRows > 128u) return launch_panel_tt<TT, 12, 4>(pa, ka, s, mid);
+    else {
+        if (units == 14) return launch_panel_tt<TT, 14, 2>(pa, ka, s, mid);
+        if (units == 13) return launch_panel_tt<TT, 12, 4>(pa, ka, s, mid);      // 12 units, four producer waves
+        return launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
+    }
 }
 
 }  // namespace hspmm
