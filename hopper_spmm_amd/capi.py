@@ -38,10 +38,11 @@ def build_library(force=True):
         cmd.insert(1, "-B")
     subprocess.check_call(cmd, stdout=subprocess.DEVNULL)
     # the command-line drivers (fp16_test / tf32_test) link against the library
+    # (not with -B: it would also remake their prerequisite, the library, once per driver)
     cli = ["make", "-C", os.path.join(_HERE, "host")]
     if force:
-        cli.insert(1, "-B")
-    subprocess.check_call(cli + ["fp16_test", "bf16_test", "tf32_test"], stdout=subprocess.DEVNULL)
+        subprocess.check_call(cli + ["clean"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(cli + ["-j3", "fp16_test", "bf16_test", "tf32_test"], stdout=subprocess.DEVNULL)
     return _LIB
 
 
