@@ -391,13 +391,22 @@ static uint32_t window_columns(const uint32_t *row_ptr, const uint32_t *col_idx,
     return uint32_t(uniq.size());
 }
 
+// Windows a worker should get at least: what holds about 64 K stored entries (a matrix of few wide
+// windows, like block-clustered weights, still spreads over the cores).
+static size_t windows_per_worker(size_t nwin, size_t nnz)
+{
+    if (nnz == 0 || nwin == 0) return 2048;
+    const size_t per_window = (nnz + nwin - 1) / nwin;
+    return std::max<size_t>(1, std::min<size_t>(2048, (size_t(1) << 16) / std::max<size_t>(1, per_window)));
+}
+
 // tiles[w] = number of tiles of window w (0 for a window without entries).
 static void count_tiles(uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx, uint32_t cw,
                         std::vector<uint32_t> &tiles)
 {
     const size_t nwin = (size_t(rows) + HSPMM_ROW_WINDOW - 1) / HSPMM_ROW_WINDOW;
     tiles.assign(nwin, 0u);
-    parallel_blocks(nwin, 2048, [&](size_t wb, size_t we) {
+    parallel_blocks(nwin, windows_per_worker(nwin, row_ptr[rows]), [&](size_t wb, size_t we) {
         std::vector<uint32_t> uniq;
         for (size_t w = wb; w < we; ++w) {
             const uint32_t r0 = uint32_t(w * HSPMM_ROW_WINDOW);
@@ -455,7 +464,7 @@ int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uin
         set_error("null argument");
         return HSPMM_ERR_INVALID;
     }
-    parallel_blocks(nwin, 2048, [&](size_t wb, size_t we) {
+    parallel_blocks(nwin, windows_per_worker(nwin, row_ptr[rows]), [&](size_t wb, size_t we) {
         std::vector<uint32_t> uniq;
         for (size_t w = wb; w < we; ++w) {
             if (!tiles[w]) continue;
@@ -575,7 +584,7 @@ int hspmm_bitmap_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const u
         }
     };
     if (shared_words) convert_windows(0, nwin);
-    else parallel_blocks(nwin, 2048, convert_windows);
+    else parallel_blocks(nwin, windows_per_worker(nwin, row_ptr[rows]), convert_windows);
     return HSPMM_OK;
 }
 
