@@ -556,8 +556,9 @@ int ensure_panel_split(hspmm_plan *p, uint32_t chunks)
 // Two vertically adjacent windows whose column lists overlap a lot are rewritten to share the
 // union of the two lists (absent entries become stored zeros): they then form a pair (build_units),
 // whose steps feed all 16 MFMA rows from one set of B rows.  Worth it where the union has at most
-// 0.85 x the tiles of the two lists together - pruned dense weights at 10 % density: 6.5 instead of
-// 2 x 4.6 tiles per 256 columns.  Returns false (out unused) when no two windows qualify.
+// 0.85 x the columns and 0.85 x the tiles of the two lists together - pruned dense weights at 10 %
+// density: 6.5 instead of 2 x 4.6 tiles per 256 columns; the windows of a graph share too few columns.
+// Returns false (out unused) when no two windows qualify.
 struct Unioned {
     std::vector<uint32_t> rowOffset, tcA2B;
     std::vector<uint8_t> data;
@@ -595,7 +596,8 @@ bool union_adjacent_windows(uint32_t W, uint32_t cw, uint32_t elem, const uint32
         merged.resize(size_t(na) + nb);
         const uint32_t nu = uint32_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin());
         const uint32_t tu = (nu + cw - 1) / cw;
-        if (double(tu) <= 0.85 * double(tiles[w] + tiles[w + 1])) {
+        // fewer tiles, and because columns are shared, not because two short lists fit one tile
+        if (double(tu) <= 0.85 * double(tiles[w] + tiles[w + 1]) && double(nu) <= 0.85 * double(na + nb)) {
             join[w] = 1; tiles[w] = tiles[w + 1] = tu; any = true;
             w += 2;
         } else {
