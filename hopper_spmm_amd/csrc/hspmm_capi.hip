@@ -103,6 +103,7 @@ struct hspmm_plan {
         uint32_t *d_split = nullptr, *d_fix_slots = nullptr;    // one split entry per unit, for the chunk sums
         bool quad = false;                                       // ids in the format of the 4x4x1 fp32 tile
         bool split = false;                                      // fp32 stream in the bf16 hi / lo form (Fp32Split)
+        double density = 0.0;                                    // steps per unit and 128 columns of the gather stream
         uint32_t split_chunks = 0;                               // chunk count d_split was built for
         size_t fix_slot_count = 0;
     } panel;
@@ -381,8 +382,11 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     constexpr uint32_t kMaxJump = 15;
     if (U == 0 || NP == 0) return false;
     // worth it when a unit has a few steps in every 128 columns it meets: the panel image is
-    // then read from LDS several times per load from the L2
-    if (!forced && double(st.n_steps) < 2.0 * double(U) * double((p->cols + 127u) / 128u)) return false;
+    // then read from LDS several times per load from the L2.  Measured break-even against the gather
+    // kernels on uniformly random matrices: 16-bit types 1.2 tiles per 128 columns at N >= 256 and
+    // about 2 at N = 128 (hspmm_run looks at N), fp32 about 2.
+    const double density = double(st.n_steps) / (double(U) * double((p->cols + 127u) / 128u));
+    if (!forced && density < (cw == 16 ? 1.2 : 2.0)) return false;
     if (uint64_t(U) * (NP + 1) > (1ull << 28)) return false;
     // columns per re-tiled step: the kernels built on 16-bit MFMAs contract 32 columns per step, the fp32
     // MFMA kernels a tile's 8
@@ -466,7 +470,8 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     }
     ps.n_steps = ps.unitOffset.back();
     // padding inside every panel must not eat the gain
-    if (!forced && double(ps.n_steps) * double(rw / cw) > 1.35 * double(st.n_steps)) return false;
+    // (fp32 MFMA forms only: the measurements above include the padding of the 32-column steps)
+    if (!forced && rw == cw && double(ps.n_steps) > 1.35 * double(st.n_steps)) return false;
     // poff[u][pn]: first step of unit u at or behind panel pn; step_panel[s]: panel of step s
     std::vector<uint32_t> poff(size_t(U) * (NP + 1)), step_panel(ps.n_steps ? ps.n_steps : 1, 0u);
     // fp32, per step four words: word g packs the panel rows quarter-wave g reads (ids g and g + 4, 7 bits
@@ -518,7 +523,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
         if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
         pl.d_tiles = dt;
     }
-    pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.split = split; pl.built = true;
+    pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.split = split; pl.density = density; pl.built = true;
     return true;
 }
 
@@ -1053,7 +1058,9 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
         // LDS-panel kernels: a workgroup covers 256 bytes of every B row with 16-byte accesses
         const uint32_t block_feat = hspmm::kPanelRowBytes / p->elem;
         const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
-        if (N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid);
+        // a sparse 16-bit matrix is served faster by the gather kernels while one wave covers all of N
+        const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.0 || N >= 256u;
+        if (pays && N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid);
     }
     const Choice c = choose_kernel(p, dB, dC, N);
     hspmm::KernelArgs ka{};
