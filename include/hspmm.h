@@ -113,9 +113,12 @@ void hspmm_get_config(int *buffer_stage, int *consumer_warp_num,
 int hspmm_set_kernel_mode(int mode);
 
 /* No reference counterpart.  Two vertically adjacent windows with the same
- * column list (block-clustered weights) can share one gather of B.  Read by the
- * next hspmm_create: 0 = pair when at least a quarter of the tiles would be in
- * pairs, 1 = never, 2 = whenever any two windows qualify. */
+ * column list (block-clustered weights) can share one gather of B; two whose
+ * lists overlap (the union has at most 0.85 x the columns and tiles of both) are
+ * given the union of the lists by the plan, absent entries as zeros, and then
+ * qualify as well.  Read by the next hspmm_create: 0 = pair when at least a
+ * quarter of the tiles would be in pairs, 1 = never (and no unions), 2 = whenever
+ * any two windows qualify. */
 int hspmm_set_window_pairing(int mode);
 
 typedef struct {
