@@ -62,7 +62,8 @@ class PlanInfo(C.Structure):
                 ("total_tiles", C.c_uint32), ("dtype", C.c_int32), ("n_ranges", C.c_uint32),
                 ("n_split_windows", C.c_uint32), ("n_partial_slots", C.c_uint32),
                 ("compute_units", C.c_uint32), ("n_units", C.c_uint32), ("n_paired_units", C.c_uint32),
-                ("device_bytes", C.c_uint64), ("n_panels", C.c_uint32), ("n_panel_steps", C.c_uint32)]
+                ("device_bytes", C.c_uint64), ("n_panels", C.c_uint32), ("n_panel_steps", C.c_uint32),
+                ("n_panel_units", C.c_uint32), ("n_panel_paired_units", C.c_uint32)]
 
 
 def load_library():

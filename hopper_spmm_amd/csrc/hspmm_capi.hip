@@ -74,7 +74,6 @@ struct hspmm_plan {
     // device copies of the format arrays as given: scalar kernel
     uint32_t *d_rowOffset = nullptr, *d_rowIdx = nullptr;
     uint32_t *d_a2b_raw = nullptr;
-    uint32_t src_T = 0;                 // the caller's tile count (T: the plan's own, after windows were given common lists)
     void *d_data = nullptr;
     // the step stream of the MFMA kernels
     int G = 1;                          // windows per unit: 2 when windows were paired
@@ -101,6 +100,9 @@ struct hspmm_plan {
         uint32_t *d_poff = nullptr, *d_ids = nullptr, *d_step_panel = nullptr;
         void *d_tiles = nullptr;
         uint32_t *d_split = nullptr, *d_fix_slots = nullptr;    // one split entry per unit, for the chunk sums
+        uint32_t *d_unitRow = nullptr;                           // the units of this stream (first row | paired bit)
+        uint32_t n_units = 0, n_paired = 0;
+        int G = 1;
         bool quad = false;                                       // ids in the format of the 4x4x1 fp32 tile
         bool split = false;                                      // fp32 stream in the bf16 hi / lo form (Fp32Split)
         double density = 0.0;                                    // steps per unit and 128 columns of the gather stream
@@ -364,13 +366,115 @@ std::vector<uint32_t> lane_order_split_steps(const StepStream &st, const uint32_
     return out;
 }
 
+// For the LDS-panel kernels built on the 16-bit MFMA a step multiplies 16 rows, so two vertically
+// adjacent windows should share their steps: they are rewritten to carry the union of their column
+// lists (absent entries become stored zeros) and then form a pair (build_units).  A pair's step costs
+// what a single window's costs there, so the union pays whenever it has fewer steps of 32 columns,
+// panel by panel, than the two lists apart - pruned dense weights at 10 % density: 6.5 instead of
+// 2 x 4.6; sparser matrices still save the half-empty last step of every panel.  Returns false (out
+// unused) when no two windows qualify.
+struct Unioned {
+    std::vector<uint32_t> rowOffset, tcA2B;
+    std::vector<uint8_t> data;
+    uint32_t T = 0;
+};
+
+bool union_adjacent_windows(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, uint32_t step_cols,
+                            const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data, const uint32_t *rowIdx,
+                            Unioned &out)
+{
+    // steps of step_cols columns an ascending list needs when no step straddles a panel of panel_cols
+    auto panel_steps = [&](const uint32_t *c, uint32_t n) {
+        uint32_t steps = 0;
+        for (uint32_t i = 0; i < n;) {
+            const uint32_t pn = c[i] / panel_cols, a = i;
+            while (i < n && c[i] / panel_cols == pn) ++i;
+            steps += (i - a + step_cols - 1) / step_cols;
+        }
+        return steps;
+    };
+    const size_t tile_bytes = size_t(8) * cw * elem;
+    const uint8_t *src = static_cast<const uint8_t *>(data);
+    auto real_ids = [&](uint32_t w) {
+        uint32_t n = (rowOffset[w + 1] - rowOffset[w]) * cw;
+        const uint32_t *c = tcA2B + size_t(rowOffset[w]) * cw;
+        while (n && c[n - 1] == HSPMM_IDX_MAX) --n;
+        return n;
+    };
+    // first pass: which windows join their successor, and the new tile counts
+    std::vector<uint8_t> join(W, 0);
+    std::vector<uint32_t> tiles(W);
+    bool any = false;
+    for (uint32_t w = 0; w < W; ++w) tiles[w] = rowOffset[w + 1] - rowOffset[w];
+    std::vector<uint32_t> merged;
+    for (uint32_t w = 0; w + 1 < W;) {
+        if (rowIdx[w + 1] != rowIdx[w] + HSPMM_ROW_WINDOW) { ++w; continue; }
+        const uint32_t *a = tcA2B + size_t(rowOffset[w]) * cw, *b = tcA2B + size_t(rowOffset[w + 1]) * cw;
+        const uint32_t na = real_ids(w), nb = real_ids(w + 1);
+        if (na == nb && std::memcmp(a, b, size_t(na) * 4) == 0) { w += 2; continue; }      // a pair already
+        // (the converters write ascending lists; a caller's list in another order is left alone)
+        auto ascending = [](const uint32_t *c, uint32_t n) {
+            for (uint32_t i = 1; i < n; ++i) if (c[i] <= c[i - 1]) return false;
+            return true;
+        };
+        if (!ascending(a, na) || !ascending(b, nb)) { ++w; continue; }
+        merged.resize(size_t(na) + nb);
+        const uint32_t nu = uint32_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin());
+        const uint32_t tu = (nu + cw - 1) / cw;
+        if (panel_steps(merged.data(), nu) < panel_steps(a, na) + panel_steps(b, nb)) {
+            join[w] = 1; tiles[w] = tiles[w + 1] = tu; any = true;
+            w += 2;
+        } else {
+            ++w;
+        }
+    }
+    if (!any) return false;
+    out.rowOffset.assign(size_t(W) + 1, 0u);
+    for (uint32_t w = 0; w < W; ++w) out.rowOffset[w + 1] = out.rowOffset[w] + tiles[w];
+    out.T = out.rowOffset[W];
+    out.tcA2B.assign(size_t(out.T) * cw, HSPMM_IDX_MAX);
+    out.data.assign(size_t(out.T) * tile_bytes, 0);
+    // second pass: copy, or spread a window's tile columns over the union's columns
+    auto spread = [&](uint32_t w, const uint32_t *ids, uint32_t n_ids) {
+        const uint32_t *c = tcA2B + size_t(rowOffset[w]) * cw;
+        const uint32_t n = real_ids(w);
+        uint32_t *dst_ids = out.tcA2B.data() + size_t(out.rowOffset[w]) * cw;
+        std::memcpy(dst_ids, ids, size_t(n_ids) * 4);
+        uint32_t j = 0;                                         // position in the union (both lists ascend)
+        for (uint32_t i = 0; i < n; ++i) {
+            while (ids[j] != c[i]) ++j;
+            const uint8_t *st = src + size_t(rowOffset[w] + i / cw) * tile_bytes;
+            uint8_t *dt = out.data.data() + size_t(out.rowOffset[w] + j / cw) * tile_bytes;
+            for (uint32_t r = 0; r < 8; ++r)
+                std::memcpy(dt + (size_t(r) * cw + j % cw) * elem, st + (size_t(r) * cw + i % cw) * elem, elem);
+        }
+    };
+    for (uint32_t w = 0; w < W; ++w) {
+        if (join[w]) {
+            const uint32_t *a = tcA2B + size_t(rowOffset[w]) * cw, *b = tcA2B + size_t(rowOffset[w + 1]) * cw;
+            const uint32_t na = real_ids(w), nb = real_ids(w + 1);
+            merged.resize(size_t(na) + nb);
+            const uint32_t nu = uint32_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin());
+            spread(w, merged.data(), nu);
+            spread(w + 1, merged.data(), nu);
+            ++w;
+        } else {
+            std::memcpy(out.tcA2B.data() + size_t(out.rowOffset[w]) * cw, tcA2B + size_t(rowOffset[w]) * cw,
+                        size_t(tiles[w]) * cw * 4);
+            std::memcpy(out.data.data() + size_t(out.rowOffset[w]) * tile_bytes, src + size_t(rowOffset[w]) * tile_bytes,
+                        size_t(tiles[w]) * tile_bytes);
+        }
+    }
+    return true;
+}
+
 // Re-tiles the matrix panel by panel for the LDS-panel kernels (spmm_panel_kernel.hpp):
 // inside every window the columns of one panel of kPanelRows columns get tiles of
 // their own.  Every step carries the number of panels it lies behind the step in
 // front of it (4 bits; a longer run of panels without a step gets an all-zero step
 // every 15 panels).  Returns false when the kernels would not pay (criteria inside).
-bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *rowOffset, const uint32_t *tcA2B,
-                        const void *data, bool forced, int *rc_out)
+bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32_t *rowOffset, const uint32_t *tcA2B,
+                        const void *data, const uint32_t *rowIdx, bool forced, int *rc_out)
 {
     *rc_out = HSPMM_OK;
     const uint32_t cw = p->cw, W = p->W;
@@ -378,25 +482,42 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     const bool split = p->dtype == HSPMM_TF32 && p->cfg.kernel_mode != 5;
     const uint32_t KP = (cw == 16 || split) ? hspmm::kPanelRowsWide : hspmm::kPanelRowsFp32;
     const uint32_t NP = (p->cols + KP - 1) / KP;
-    const uint32_t U = uint32_t(st.unitRow.size());
     constexpr uint32_t kMaxJump = 15;
-    if (U == 0 || NP == 0) return false;
+    if (gather_st.unitRow.empty() || NP == 0) return false;
     // worth it when a unit has a few steps in every 128 columns it meets: the panel image is
     // then read from LDS several times per load from the L2.  Measured break-even against the gather
-    // kernels on uniformly random matrices: 16-bit types 1.2 tiles per 128 columns at N >= 256 and
-    // about 2 at N = 128 (hspmm_run looks at N), fp32 about 2.
-    const double density = double(st.n_steps) / (double(U) * double((p->cols + 127u) / 128u));
-    if (!forced && density < (cw == 16 ? 1.2 : 2.0)) return false;
-    if (uint64_t(U) * (NP + 1) > (1ull << 28)) return false;
+    // kernels on uniformly random matrices: 1.2 tiles per 128 columns for the kernels built on the
+    // 16-bit MFMA (8192 x 8192 at 2 %, fp16: 31 against 34 us at N = 128, 56 against 110 at N = 512; at
+    // 1 %: 29 against 16 and 48 against 42), about 2 for the fp32 MFMA forms.
+    const double density = double(gather_st.n_steps) / (double(gather_st.unitRow.size()) * double((p->cols + 127u) / 128u));
+    if (!forced && density < ((cw == 16 || split) ? 1.2 : 2.0)) return false;
+    if (uint64_t(gather_st.unitRow.size()) * (NP + 1) > (1ull << 28)) return false;
     // columns per re-tiled step: the kernels built on 16-bit MFMAs contract 32 columns per step, the fp32
     // MFMA kernels a tile's 8
     const uint32_t rw = (cw == 16 || split) ? 32u : cw;
+    // The units of this stream.  The kernels built on the 16-bit MFMA pair adjacent windows through
+    // the union of their column lists wherever that saves steps, and pair whatever can be paired
+    // (a pair costs them nothing); the fp32 MFMA forms walk the units of the gather kernels.
+    Unioned un;
+    StepStream st = gather_st;
+    if (rw == 32 && p->cfg.pairing != 1 && W > 1) {
+        if (union_adjacent_windows(W, cw, uint32_t(p->elem), KP, rw, rowOffset, tcA2B, data, rowIdx, un)) {
+            rowOffset = un.rowOffset.data(); tcA2B = un.tcA2B.data(); data = un.data.data();
+        }
+        const size_t n_ids = size_t(rowOffset[W]) * cw;
+        std::vector<uint32_t> clean(tcA2B, tcA2B + n_ids);
+        for (size_t i = 1; i < n_ids; ++i)
+            if (clean[i] == HSPMM_IDX_MAX) clean[i] = clean[i - 1];
+        st = build_units(W, cw, rowOffset, rowIdx, clean, 2);
+    }
+    const uint32_t U = uint32_t(st.unitRow.size());
+    const uint32_t T = rowOffset[W];
     const size_t es = p->elem, src_tile_bytes = size_t(8) * cw * es, tile_bytes = size_t(8) * rw * es;
     std::vector<uint32_t> rt_rowOffset(size_t(W) + 1, 0u), rt_ids, rt_panel;
     std::vector<uint8_t> rt_data;
-    rt_ids.reserve(size_t(p->T) * cw * 5 / 4);
-    rt_panel.reserve(size_t(p->T) * 5 / 4);
-    rt_data.reserve(size_t(p->T) * src_tile_bytes * 5 / 4);
+    rt_ids.reserve(size_t(T) * cw * 5 / 4);
+    rt_panel.reserve(size_t(T) * 5 / 4);
+    rt_data.reserve(size_t(T) * src_tile_bytes * 5 / 4);
     const uint8_t *src_data = static_cast<const uint8_t *>(data);
     for (uint32_t w = 0; w < W; ++w) {
         const uint32_t t0 = rowOffset[w], t1 = rowOffset[w + 1];
@@ -460,7 +581,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
         }
         rt_rowOffset[w + 1] = rt_rowOffset[w] + tiles;
     }
-    // the same units as the gather kernels walk, with the re-tiled step counts
+    // the units with the re-tiled step counts
     StepStream ps;
     ps.G = st.G; ps.unitRow = st.unitRow; ps.unitWindow = st.unitWindow; ps.n_paired = st.n_paired;
     ps.unitOffset.assign(1, 0u);
@@ -471,7 +592,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
     ps.n_steps = ps.unitOffset.back();
     // padding inside every panel must not eat the gain
     // (fp32 MFMA forms only: the measurements above include the padding of the 32-column steps)
-    if (!forced && rw == cw && double(ps.n_steps) > 1.35 * double(st.n_steps)) return false;
+    if (!forced && rw == cw && double(ps.n_steps) > 1.35 * double(gather_st.n_steps)) return false;
     // poff[u][pn]: first step of unit u at or behind panel pn; step_panel[s]: panel of step s
     std::vector<uint32_t> poff(size_t(U) * (NP + 1)), step_panel(ps.n_steps ? ps.n_steps : 1, 0u);
     // fp32, per step four words: word g packs the panel rows quarter-wave g reads (ids g and g + 4, 7 bits
@@ -523,6 +644,8 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
         if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
         pl.d_tiles = dt;
     }
+    if ((rc = upload(&pl.d_unitRow, st.unitRow.data(), st.unitRow.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
+    pl.n_units = U; pl.G = st.G; pl.n_paired = st.n_paired;
     pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.split = split; pl.density = density; pl.built = true;
     return true;
 }
@@ -532,7 +655,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &st, const uint32_t *row
 int ensure_panel_split(hspmm_plan *p, uint32_t chunks)
 {
     hspmm_plan::Panel &pl = p->panel;
-    const size_t slots = size_t(p->n_units) * chunks;
+    const size_t slots = size_t(pl.n_units) * chunks;
     if (slots > pl.fix_slot_count) {
         if (pl.d_fix_slots) { HSPMM_HIP(hipFree(pl.d_fix_slots)); pl.d_fix_slots = nullptr; pl.fix_slot_count = 0; }
         std::vector<uint32_t> ident(slots);
@@ -544,8 +667,8 @@ int ensure_panel_split(hspmm_plan *p, uint32_t chunks)
     }
     if (pl.split_chunks != chunks) {
         if (pl.d_split) { HSPMM_HIP(hipFree(pl.d_split)); pl.d_split = nullptr; pl.split_chunks = 0; }
-        std::vector<uint32_t> sp(size_t(p->n_units) * hspmm::kFixWords, 0u);
-        for (uint32_t u = 0; u < p->n_units; ++u) {
+        std::vector<uint32_t> sp(size_t(pl.n_units) * hspmm::kFixWords, 0u);
+        for (uint32_t u = 0; u < pl.n_units; ++u) {
             sp[size_t(u) * hspmm::kFixWords + 0] = u;
             sp[size_t(u) * hspmm::kFixWords + 1] = u * chunks;
             sp[size_t(u) * hspmm::kFixWords + 2] = chunks;
@@ -556,97 +679,6 @@ int ensure_panel_split(hspmm_plan *p, uint32_t chunks)
         pl.split_chunks = chunks;
     }
     return HSPMM_OK;
-}
-
-// Two vertically adjacent windows whose column lists overlap a lot are rewritten to share the
-// union of the two lists (absent entries become stored zeros): they then form a pair (build_units),
-// whose steps feed all 16 MFMA rows from one set of B rows.  Worth it where the union has at most
-// 0.85 x the columns and 0.85 x the tiles of the two lists together - pruned dense weights at 10 %
-// density: 6.5 instead of 2 x 4.6 tiles per 256 columns; the windows of a graph share too few columns.
-// Returns false (out unused) when no two windows qualify.
-struct Unioned {
-    std::vector<uint32_t> rowOffset, tcA2B;
-    std::vector<uint8_t> data;
-    uint32_t T = 0;
-};
-
-bool union_adjacent_windows(uint32_t W, uint32_t cw, uint32_t elem, const uint32_t *rowOffset, const uint32_t *tcA2B,
-                            const void *data, const uint32_t *rowIdx, Unioned &out)
-{
-    const size_t tile_bytes = size_t(8) * cw * elem;
-    const uint8_t *src = static_cast<const uint8_t *>(data);
-    auto real_ids = [&](uint32_t w) {
-        uint32_t n = (rowOffset[w + 1] - rowOffset[w]) * cw;
-        const uint32_t *c = tcA2B + size_t(rowOffset[w]) * cw;
-        while (n && c[n - 1] == HSPMM_IDX_MAX) --n;
-        return n;
-    };
-    // first pass: which windows join their successor, and the new tile counts
-    std::vector<uint8_t> join(W, 0);
-    std::vector<uint32_t> tiles(W);
-    bool any = false;
-    for (uint32_t w = 0; w < W; ++w) tiles[w] = rowOffset[w + 1] - rowOffset[w];
-    std::vector<uint32_t> merged;
-    for (uint32_t w = 0; w + 1 < W;) {
-        if (rowIdx[w + 1] != rowIdx[w] + HSPMM_ROW_WINDOW) { ++w; continue; }
-        const uint32_t *a = tcA2B + size_t(rowOffset[w]) * cw, *b = tcA2B + size_t(rowOffset[w + 1]) * cw;
-        const uint32_t na = real_ids(w), nb = real_ids(w + 1);
-        if (na == nb && std::memcmp(a, b, size_t(na) * 4) == 0) { w += 2; continue; }      // a pair already
-        // (the converters write ascending lists; a caller's list in another order is left alone)
-        auto ascending = [](const uint32_t *c, uint32_t n) {
-            for (uint32_t i = 1; i < n; ++i) if (c[i] <= c[i - 1]) return false;
-            return true;
-        };
-        if (!ascending(a, na) || !ascending(b, nb)) { ++w; continue; }
-        merged.resize(size_t(na) + nb);
-        const uint32_t nu = uint32_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin());
-        const uint32_t tu = (nu + cw - 1) / cw;
-        // fewer tiles, and because columns are shared, not because two short lists fit one tile
-        if (double(tu) <= 0.85 * double(tiles[w] + tiles[w + 1]) && double(nu) <= 0.85 * double(na + nb)) {
-            join[w] = 1; tiles[w] = tiles[w + 1] = tu; any = true;
-            w += 2;
-        } else {
-            ++w;
-        }
-    }
-    if (!any) return false;
-    out.rowOffset.assign(size_t(W) + 1, 0u);
-    for (uint32_t w = 0; w < W; ++w) out.rowOffset[w + 1] = out.rowOffset[w] + tiles[w];
-    out.T = out.rowOffset[W];
-    out.tcA2B.assign(size_t(out.T) * cw, HSPMM_IDX_MAX);
-    out.data.assign(size_t(out.T) * tile_bytes, 0);
-    // second pass: copy, or spread a window's tile columns over the union's columns
-    auto spread = [&](uint32_t w, const uint32_t *ids, uint32_t n_ids) {
-        const uint32_t *c = tcA2B + size_t(rowOffset[w]) * cw;
-        const uint32_t n = real_ids(w);
-        uint32_t *dst_ids = out.tcA2B.data() + size_t(out.rowOffset[w]) * cw;
-        std::memcpy(dst_ids, ids, size_t(n_ids) * 4);
-        uint32_t j = 0;                                         // position in the union (both lists ascend)
-        for (uint32_t i = 0; i < n; ++i) {
-            while (ids[j] != c[i]) ++j;
-            const uint8_t *st = src + size_t(rowOffset[w] + i / cw) * tile_bytes;
-            uint8_t *dt = out.data.data() + size_t(out.rowOffset[w] + j / cw) * tile_bytes;
-            for (uint32_t r = 0; r < 8; ++r)
-                std::memcpy(dt + (size_t(r) * cw + j % cw) * elem, st + (size_t(r) * cw + i % cw) * elem, elem);
-        }
-    };
-    for (uint32_t w = 0; w < W; ++w) {
-        if (join[w]) {
-            const uint32_t *a = tcA2B + size_t(rowOffset[w]) * cw, *b = tcA2B + size_t(rowOffset[w + 1]) * cw;
-            const uint32_t na = real_ids(w), nb = real_ids(w + 1);
-            merged.resize(size_t(na) + nb);
-            const uint32_t nu = uint32_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin());
-            spread(w, merged.data(), nu);
-            spread(w + 1, merged.data(), nu);
-            ++w;
-        } else {
-            std::memcpy(out.tcA2B.data() + size_t(out.rowOffset[w]) * cw, tcA2B + size_t(rowOffset[w]) * cw,
-                        size_t(tiles[w]) * cw * 4);
-            std::memcpy(out.data.data() + size_t(out.rowOffset[w]) * tile_bytes, src + size_t(rowOffset[w]) * tile_bytes,
-                        size_t(tiles[w]) * tile_bytes);
-        }
-    }
-    return true;
 }
 
 struct Choice {
@@ -817,23 +849,9 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
     hspmm_plan *p = new (std::nothrow) hspmm_plan;
     if (!p) return fail(HSPMM_ERR_ALLOC, "out of host memory");
     p->dtype = dtype; p->rows = rows; p->cols = cols; p->W = eff_row_windows; p->T = total_tiles;
-    p->src_T = total_tiles;
     p->cw = cw; p->elem = elem;
     { std::lock_guard<std::mutex> lk(g_cfg_mutex); p->cfg = g_cfg; }
     if (const char *e = std::getenv("HSPMM_FUSED_FIXUP")) p->cfg.fused_fixup = std::atoi(e);     // tuning override
-
-    // adjacent windows with much the same columns get one column list (and so become pairs)
-    Unioned un;
-    if (p->cfg.pairing != 1 && eff_row_windows > 1) {
-        bool use = false;
-        try { use = union_adjacent_windows(eff_row_windows, cw, elem, rowOffset, tcA2B, data, rowIdx, un); }
-        catch (const std::bad_alloc &) { delete p; return fail(HSPMM_ERR_ALLOC, "out of host memory"); }
-        if (use) {
-            rowOffset = un.rowOffset.data(); tcA2B = un.tcA2B.data(); data = un.data.data();
-            total_tiles = un.T;
-            p->T = un.T;
-        }
-    }
 
     auto bail = [&](int code) { hspmm_destroy(p); return code; };
     hipError_t e = hipGetDevice(&p->device);
@@ -885,7 +903,8 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
         if (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4) {
             int prc = HSPMM_OK;
-            (void)build_panel_stream(p, st, rowOffset, tcA2B, data, p->cfg.kernel_mode >= 4, &prc);
+            try { (void)build_panel_stream(p, st, rowOffset, tcA2B, data, rowIdx, p->cfg.kernel_mode >= 4, &prc); }
+            catch (const std::bad_alloc &) { return bail(fail(HSPMM_ERR_ALLOC, "out of host memory")); }
             if (prc) return bail(prc);
         }
     }
@@ -950,6 +969,7 @@ void hspmm_destroy(hspmm_plan *p)
     (void)hipFree(p->d_data); (void)hipFree(p->d_unitOffset); (void)hipFree(p->d_unitRow); (void)hipFree(p->d_ids);
     for (auto &dp : p->parts) { (void)hipFree(dp.d_ranges); (void)hipFree(dp.d_split); (void)hipFree(dp.d_fix_slots); }
     (void)hipFree(p->panel.d_poff); (void)hipFree(p->panel.d_ids); (void)hipFree(p->panel.d_tiles);
+    (void)hipFree(p->panel.d_unitRow);
     (void)hipFree(p->panel.d_step_panel);
     (void)hipFree(p->panel.d_split); (void)hipFree(p->panel.d_fix_slots);
     (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive);
@@ -969,17 +989,17 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
 {
     const hspmm_plan::Panel &pl = p->panel;
     hspmm::PanelArgs pa{};
-    pa.unitRow = p->d_unitRow; pa.poff = pl.d_poff; pa.step_panel = pl.d_step_panel; pa.ids = pl.d_ids;
+    pa.unitRow = pl.d_unitRow; pa.poff = pl.d_poff; pa.step_panel = pl.d_step_panel; pa.ids = pl.d_ids;
     pa.tiles = pl.d_tiles; pa.n_steps = pl.n_steps;
     pa.B = dB; pa.C = dC;
-    pa.n_units = p->n_units; pa.rows = p->rows; pa.cols = p->cols; pa.N = N;
+    pa.n_units = pl.n_units; pa.rows = p->rows; pa.cols = p->cols; pa.N = N;
     pa.n_feat_blocks = N / (hspmm::kPanelRowBytes / p->elem);
     pa.n_panels = pl.n_panels;
     // The workgroup shape: code 14 / 12 = that many consumer waves and two producers, 13 = 12 consumers and
     // four producers (few enough registers for two workgroups per compute unit, which the 4x4x1 fp32 kernel
     // needs to keep its short MFMAs fed).  Of the consumer waves any number may be given a unit.
     const bool wide = p->dtype != HSPMM_TF32 || pl.split;          // panels of 256 rows: always 12 + 4 waves
-    int units = (pl.quad || wide) ? 13 : p->G == 2 ? 14 : 12;
+    int units = (pl.quad || wide) ? 13 : pl.G == 2 ? 14 : 12;
     int forced_units = 0;
     if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) {                                      // tuning overrides
         units = std::atoi(e) == 14 ? 14 : std::atoi(e) == 13 ? 13 : 12;
@@ -995,7 +1015,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     int best_units = max_units;
     double best_cost = 0.0;
     for (int nc = forced_units ? forced_units : std::max(4, max_units / 2); nc <= (forced_units ? forced_units : max_units); ++nc) {
-        const uint64_t rbs = (uint64_t(p->n_units) + nc - 1) / nc, base = rbs * pa.n_feat_blocks;
+        const uint64_t rbs = (uint64_t(pl.n_units) + nc - 1) / nc, base = rbs * pa.n_feat_blocks;
         uint64_t ch = base >= slots ? 1 : std::min<uint64_t>(slots / base, pl.n_panels);
         const uint64_t ppc = (pl.n_panels + ch - 1) / ch;
         ch = (pl.n_panels + ppc - 1) / ppc;
@@ -1004,7 +1024,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best_units = nc; chunks = ch; }
     }
     pa.units_per_group = uint32_t(best_units);
-    const uint64_t row_blocks = (uint64_t(p->n_units) + best_units - 1) / best_units;
+    const uint64_t row_blocks = (uint64_t(pl.n_units) + best_units - 1) / best_units;
     const uint64_t base = row_blocks * pa.n_feat_blocks;
     if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) chunks = uint64_t(std::atoi(e));
     if (chunks < 1) chunks = 1;
@@ -1017,17 +1037,17 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     if (pa.n_chunks > 1) {
         int rc = ensure_panel_split(p, pa.n_chunks);
         if (rc) return rc;
-        const size_t nacc = pl.quad ? 2u : pl.split ? 4u : p->dtype != HSPMM_TF32 ? 8u : 4u * size_t(p->G);
-        const size_t need = size_t(p->n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
+        const size_t nacc = pl.quad ? 2u : pl.split ? 4u : p->dtype != HSPMM_TF32 ? 8u : 4u * size_t(pl.G);
+        const size_t need = size_t(pl.n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
         if ((rc = ensure_scratch(p, need))) return rc;
         pa.scratch = p->d_scratch;
-        ka.unitRow = p->d_unitRow; ka.ids = pl.d_ids; ka.tiles = pl.d_tiles;
+        ka.unitRow = pl.d_unitRow; ka.ids = pl.d_ids; ka.tiles = pl.d_tiles;
         ka.split = pl.d_split; ka.fix_slots = pl.d_fix_slots; ka.scratch = p->d_scratch;
         ka.C = dC; ka.B = dB;
-        ka.n_split = p->n_units; ka.n_units = p->n_units; ka.rows = p->rows; ka.N = N;
+        ka.n_split = pl.n_units; ka.n_units = pl.n_units; ka.rows = p->rows; ka.N = N;
         ka.n_feat_blocks = pa.n_feat_blocks;
     }
-    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : p->G, pl.split, pa, ka, units, s, mid));
+    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : pl.G, pl.split, pa, ka, units, s, mid));
     return HSPMM_OK;
 }
 
@@ -1058,8 +1078,9 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
         // LDS-panel kernels: a workgroup covers 256 bytes of every B row with 16-byte accesses
         const uint32_t block_feat = hspmm::kPanelRowBytes / p->elem;
         const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
-        // a sparse 16-bit matrix is served faster by the gather kernels while one wave covers all of N
-        const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.0 || N >= 256u;
+        // (a 16-bit matrix near the break-even is served as fast or faster by the gather kernels while
+        // one wave of theirs covers all of N)
+        const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 1.5 || N >= 256u;
         if (pays && N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid);
     }
     const Choice c = choose_kernel(p, dB, dC, N);
@@ -1170,7 +1191,7 @@ int hspmm_bench(hspmm_plan *p, const void *dB, void *dC, uint32_t N, int warmup,
 int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
 {
     if (!p || !info) return fail(HSPMM_ERR_INVALID, "null argument");
-    info->rows = p->rows; info->cols = p->cols; info->eff_row_windows = p->W; info->total_tiles = p->src_T;
+    info->rows = p->rows; info->cols = p->cols; info->eff_row_windows = p->W; info->total_tiles = p->T;
     info->dtype = p->dtype;
     info->n_ranges = uint32_t(p->parts[0].part.ranges.size());
     info->n_split_windows = uint32_t(p->parts[0].part.split.size());
@@ -1181,6 +1202,8 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->device_bytes = uint64_t(p->fixed_bytes) + uint64_t(p->scratch_bytes);
     info->n_panels = p->panel.built ? p->panel.n_panels : 0u;
     info->n_panel_steps = p->panel.built ? p->panel.n_steps : 0u;
+    info->n_panel_units = p->panel.built ? p->panel.n_units : 0u;
+    info->n_panel_paired_units = p->panel.built ? p->panel.n_paired : 0u;
     return HSPMM_OK;
 }
 

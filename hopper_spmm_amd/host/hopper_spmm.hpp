@@ -386,8 +386,11 @@ inline PERF_RESULT tf32_spmm(SPARSE_MTX &btcf_a, DENSE_MTX &dense_b, DENSE_MTX &
 // Element-wise comparison of two dense matrices.  The reference's helper counts
 // |a - b| > 1 (src/utils/verify.h:28); here the bound is the relative / absolute
 // form of its tile checks (src/tf32.cu:46-70): relative `tol` when |b| > 1e-6,
-// absolute 1e-5 * scale otherwise.
-inline bool verify_dense_matrix(const DENSE_MTX *A, const DENSE_MTX *B, double tol = 1e-2)
+// absolute 1e-5 otherwise - plus, where the caller knows it, abs_tol x sum |a||b| of
+// the element (what a sum that cancels may be off by: rounding errors scale with
+// the terms, not with the result).
+inline bool verify_dense_matrix(const DENSE_MTX *A, const DENSE_MTX *B, double tol = 1e-2,
+                                const double *sum_abs = nullptr, double abs_tol = 0.0)
 {
     const size_t total = size_t(A->rows) * A->cols;
     size_t failed = 0;
@@ -395,7 +398,8 @@ inline bool verify_dense_matrix(const DENSE_MTX *A, const DENSE_MTX *B, double t
     for (size_t i = 0; i < total; ++i) {
         const double a = double(A->values[i]), b = double(B->values[i]);
         const double err = std::fabs(a - b), ref = std::fabs(b);
-        const bool bad = ref > 1e-6 ? !(err / ref <= tol) : !(err <= 1e-5);
+        const double slack = sum_abs ? abs_tol * sum_abs[i] : 0.0;
+        const bool bad = ref > 1e-6 ? !(err <= tol * ref + slack) : !(err <= 1e-5 + slack);
         if (bad) {
             ++failed;
             if (printed++ < 20)

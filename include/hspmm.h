@@ -113,12 +113,13 @@ void hspmm_get_config(int *buffer_stage, int *consumer_warp_num,
 int hspmm_set_kernel_mode(int mode);
 
 /* No reference counterpart.  Two vertically adjacent windows with the same
- * column list (block-clustered weights) can share one gather of B; two whose
- * lists overlap (the union has at most 0.85 x the columns and tiles of both) are
- * given the union of the lists by the plan, absent entries as zeros, and then
- * qualify as well.  Read by the next hspmm_create: 0 = pair when at least a
- * quarter of the tiles would be in pairs, 1 = never (and no unions), 2 = whenever
- * any two windows qualify. */
+ * column list (block-clustered weights) can share one gather of B.  Read by the
+ * next hspmm_create: 0 = pair when at least a quarter of the tiles would be in
+ * pairs, 1 = never, 2 = whenever any two windows qualify.  The LDS-staging
+ * kernels built on the 16-bit MFMA (a step of theirs multiplies 16 rows) go
+ * further unless the mode is 1: in their copy of the matrix two adjacent windows
+ * carry the union of their column lists, absent entries as zeros, wherever that
+ * saves steps. */
 int hspmm_set_window_pairing(int mode);
 
 typedef struct {
@@ -133,6 +134,8 @@ typedef struct {
     uint64_t device_bytes;      /* bytes of device memory the plan holds right now */
     uint32_t n_panels;          /* column panels of the LDS-staging kernels; 0: the plan does not use them */
     uint32_t n_panel_steps;     /* steps of the unit stream re-tiled panel by panel */
+    uint32_t n_panel_units;     /* units of that stream: it pairs windows through the union of their columns */
+    uint32_t n_panel_paired_units;
 } hspmm_plan_info;
 
 /* No reference counterpart (the reference prints its statistics from main,
