@@ -101,7 +101,7 @@ struct hspmm_plan {
         void *d_tiles = nullptr;
         uint32_t *d_split = nullptr, *d_fix_slots = nullptr;    // one split entry per unit, for the chunk sums
         uint32_t *d_unitRow = nullptr;                           // the units of this stream (first row | paired bit)
-        uint32_t n_units = 0, n_paired = 0;
+        uint32_t n_units = 0, n_paired = 0, n_wide = 0;          // units of two or more / three or four windows
         int G = 1;
         bool quad = false;                                       // ids in the format of the 4x4x1 fp32 tile
         bool split = false;                                      // fp32 stream in the bf16 hi / lo form (Fp32Split)
@@ -214,6 +214,7 @@ struct StepStream {
     int G = 1;
     std::vector<uint32_t> unitOffset, unitRow, unitWindow;   // unitWindow: first effective window of the unit
     uint32_t n_paired = 0, n_steps = 0;
+    uint32_t n_wide = 0;                                     // units of three or four windows (LDS-panel stream only)
 };
 
 StepStream build_units(uint32_t W, uint32_t cw, const uint32_t *rowOffset, const uint32_t *rowIdx,
@@ -302,20 +303,23 @@ std::vector<uint32_t> lane_order_tiles(const StepStream &st, int dtype, const ui
 // 16-bit steps of 32 columns for the LDS-panel kernels (Fp16Tr in spmm_panel_kernel.hpp): a re-tiled
 // step of a window is [row r][32 halves]; lane l = (g, m) of the step's 1 KB gets the 16 bytes
 // a[m][8g .. 8g + 7], m = row of the unit's 16 rows (rows 8..15: the second window of a pair, else zero).
+// A stream with units of up to four windows (G = 4) has a second KB per step for windows 2 and 3.
 std::vector<uint32_t> lane_order_wide_steps(const StepStream &st, const uint32_t *rowOffset, const void *data)
 {
     const uint16_t *halves = static_cast<const uint16_t *>(data);   // a step of a window is 8 x 32 halves
-    std::vector<uint32_t> out(size_t(st.n_steps) * 256u, 0u);
+    const size_t step_words = st.G == 4 ? 512u : 256u;
+    std::vector<uint32_t> out(size_t(st.n_steps) * step_words, 0u);
     for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
         const uint32_t w0 = st.unitWindow[u];
-        const int nwin = (st.unitRow[u] & 1u) ? 2 : 1;
+        const uint32_t nwin = (st.unitRow[u] & 3u) + 1u;
         for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
-            uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * 256u);
-            for (int w = 0; w < nwin; ++w) {
+            uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * step_words);
+            for (uint32_t w = 0; w < nwin; ++w) {
                 const uint16_t *src = halves + size_t(rowOffset[w0 + w] + i) * 256u;
+                uint16_t *half = dst + (w >> 1) * 512u;
                 for (uint32_t r = 0; r < 8; ++r)
                     for (uint32_t g = 0; g < 4; ++g)
-                        std::memcpy(dst + ((g * 16u + 8u * w + r) * 8u), src + r * 32u + 8u * g, 16);
+                        std::memcpy(half + ((g * 16u + 8u * (w & 1u) + r) * 8u), src + r * 32u + 8u * g, 16);
             }
         }
     }
@@ -340,23 +344,26 @@ uint32_t split_bf16_host(float v)
 }
 
 // fp32 steps of 32 columns in the split form (Fp32Split): a re-tiled step of a window is [row r][32 floats];
-// lane l = (g, m) gets 32 bytes: the 8 hi halves, then the 8 lo halves of a[m][8g .. 8g + 7].
+// lane l = (g, m) gets 32 bytes: the 8 hi halves, then the 8 lo halves of a[m][8g .. 8g + 7].  A stream with
+// units of up to four windows (G = 4) has a second 2 KB per step for windows 2 and 3.
 std::vector<uint32_t> lane_order_split_steps(const StepStream &st, const uint32_t *rowOffset, const void *data)
 {
     const float *vals = static_cast<const float *>(data);            // a step of a window is 8 x 32 floats
-    std::vector<uint32_t> out(size_t(st.n_steps) * 512u, 0u);
+    const size_t step_words = st.G == 4 ? 1024u : 512u;
+    std::vector<uint32_t> out(size_t(st.n_steps) * step_words, 0u);
     for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
         const uint32_t w0 = st.unitWindow[u];
-        const int nwin = (st.unitRow[u] & 1u) ? 2 : 1;
+        const uint32_t nwin = (st.unitRow[u] & 3u) + 1u;
         for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
-            uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * 512u);
-            for (int w = 0; w < nwin; ++w) {
+            uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * step_words);
+            for (uint32_t w = 0; w < nwin; ++w) {
                 const float *src = vals + size_t(rowOffset[w0 + w] + i) * 256u;
+                uint16_t *half = dst + (w >> 1) * 1024u;
                 for (uint32_t r = 0; r < 8; ++r)
                     for (uint32_t g = 0; g < 4; ++g)
                         for (uint32_t c = 0; c < 8; ++c) {
                             const uint32_t sp = split_bf16_host(src[r * 32u + 8u * g + c]);
-                            uint16_t *lane = dst + (g * 16u + 8u * w + r) * 16u;
+                            uint16_t *lane = half + (g * 16u + 8u * (w & 1u) + r) * 16u;
                             lane[c] = uint16_t(sp & 0xFFFFu);
                             lane[8 + c] = uint16_t(sp >> 16);
                         }
@@ -366,22 +373,27 @@ std::vector<uint32_t> lane_order_split_steps(const StepStream &st, const uint32_
     return out;
 }
 
-// For the LDS-panel kernels built on the 16-bit MFMA a step multiplies 16 rows, so two vertically
-// adjacent windows should share their steps: they are rewritten to carry the union of their column
-// lists (absent entries become stored zeros) and then form a pair (build_units).  A pair's step costs
-// what a single window's costs there, so the union pays whenever it has fewer steps of 32 columns,
-// panel by panel, than the two lists apart - pruned dense weights at 10 % density: 6.5 instead of
-// 2 x 4.6; sparser matrices still save the half-empty last step of every panel.  Returns false (out
-// unused) when no two windows qualify.
+// For the LDS-panel kernels built on the 16-bit MFMA a step multiplies 16 rows, and a wave can run one
+// second operand (the gathered rows of B, read from LDS - what binds these kernels) against two first
+// operands, 32 rows.  So vertically adjacent windows should share their steps: groups of up to four
+// windows are rewritten to carry the union of their column lists (absent entries become stored zeros)
+// and run as one unit.  merge_groups is one pass over neighbouring groups: two groups whose windows
+// number at most max_windows are merged when cost x steps(union) < steps(a) + steps(b), steps counted
+// in panels of panel_cols columns and steps of step_cols (no step straddles a panel); cost = 1 for a
+// pair (its step costs what a single window's costs), wide_cost for three and four windows (the same
+// LDS reads, twice the MFMAs).  Pruned dense weights at 10 % density: 4.6 steps per 256 columns for a
+// window, 6.5 for a pair, 7.7 for four; sparser matrices still save the half-empty last step of every
+// panel.  Returns false (outputs unused) when no two groups merge.
 struct Unioned {
     std::vector<uint32_t> rowOffset, tcA2B;
     std::vector<uint8_t> data;
     uint32_t T = 0;
 };
 
-bool union_adjacent_windows(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, uint32_t step_cols,
-                            const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data, const uint32_t *rowIdx,
-                            Unioned &out)
+bool merge_groups(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, uint32_t step_cols, uint32_t max_windows,
+                  double wide_cost, const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
+                  const uint32_t *rowIdx, const std::vector<uint32_t> &first, const std::vector<uint32_t> &count,
+                  Unioned &out, std::vector<uint32_t> &out_first, std::vector<uint32_t> &out_count)
 {
     // steps of step_cols columns an ascending list needs when no step straddles a panel of panel_cols
     auto panel_steps = [&](const uint32_t *c, uint32_t n) {
@@ -401,31 +413,42 @@ bool union_adjacent_windows(uint32_t W, uint32_t cw, uint32_t elem, uint32_t pan
         while (n && c[n - 1] == HSPMM_IDX_MAX) --n;
         return n;
     };
-    // first pass: which windows join their successor, and the new tile counts
-    std::vector<uint8_t> join(W, 0);
+    // (the converters write ascending lists; a caller's list in another order is only merged with an equal one)
+    auto ascending = [](const uint32_t *c, uint32_t n) {
+        for (uint32_t i = 1; i < n; ++i) if (c[i] <= c[i - 1]) return false;
+        return true;
+    };
+    // the column list of the merged group (all windows of a group carry their group's list)
+    std::vector<uint32_t> merged;
+    auto merged_list = [&](uint32_t wa, uint32_t wb) {
+        const uint32_t *a = tcA2B + size_t(rowOffset[wa]) * cw, *b = tcA2B + size_t(rowOffset[wb]) * cw;
+        const uint32_t na = real_ids(wa), nb = real_ids(wb);
+        if (na == nb && std::memcmp(a, b, size_t(na) * 4) == 0) { merged.assign(a, a + na); return; }
+        merged.resize(size_t(na) + nb);
+        merged.resize(size_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin()));
+    };
+    // first pass: which groups join their successor, and the new tile counts
+    const size_t NG = first.size();
+    std::vector<uint8_t> join(NG, 0);
     std::vector<uint32_t> tiles(W);
     bool any = false;
     for (uint32_t w = 0; w < W; ++w) tiles[w] = rowOffset[w + 1] - rowOffset[w];
-    std::vector<uint32_t> merged;
-    for (uint32_t w = 0; w + 1 < W;) {
-        if (rowIdx[w + 1] != rowIdx[w] + HSPMM_ROW_WINDOW) { ++w; continue; }
-        const uint32_t *a = tcA2B + size_t(rowOffset[w]) * cw, *b = tcA2B + size_t(rowOffset[w + 1]) * cw;
-        const uint32_t na = real_ids(w), nb = real_ids(w + 1);
-        if (na == nb && std::memcmp(a, b, size_t(na) * 4) == 0) { w += 2; continue; }      // a pair already
-        // (the converters write ascending lists; a caller's list in another order is left alone)
-        auto ascending = [](const uint32_t *c, uint32_t n) {
-            for (uint32_t i = 1; i < n; ++i) if (c[i] <= c[i - 1]) return false;
-            return true;
-        };
-        if (!ascending(a, na) || !ascending(b, nb)) { ++w; continue; }
-        merged.resize(size_t(na) + nb);
-        const uint32_t nu = uint32_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin());
-        const uint32_t tu = (nu + cw - 1) / cw;
-        if (panel_steps(merged.data(), nu) < panel_steps(a, na) + panel_steps(b, nb)) {
-            join[w] = 1; tiles[w] = tiles[w + 1] = tu; any = true;
-            w += 2;
+    for (size_t g = 0; g + 1 < NG;) {
+        const uint32_t wa = first[g], wb = first[g + 1], nw = count[g] + count[g + 1];
+        if (rowIdx[wb] != rowIdx[wa] + HSPMM_ROW_WINDOW * count[g] || nw > max_windows) { ++g; continue; }
+        const uint32_t *a = tcA2B + size_t(rowOffset[wa]) * cw, *b = tcA2B + size_t(rowOffset[wb]) * cw;
+        const uint32_t na = real_ids(wa), nb = real_ids(wb);
+        const bool same = na == nb && std::memcmp(a, b, size_t(na) * 4) == 0;
+        if (!same && (!ascending(a, na) || !ascending(b, nb))) { ++g; continue; }
+        merged_list(wa, wb);
+        const uint32_t nu = uint32_t(merged.size());
+        const double cost = nw > 2 ? wide_cost : 1.0;
+        if (same || cost * double(panel_steps(merged.data(), nu)) < double(panel_steps(a, na) + panel_steps(b, nb))) {
+            join[g] = 1; any = true;
+            for (uint32_t w = wa; w < wa + nw; ++w) tiles[w] = (nu + cw - 1) / cw;
+            g += 2;
         } else {
-            ++w;
+            ++g;
         }
     }
     if (!any) return false;
@@ -434,13 +457,13 @@ bool union_adjacent_windows(uint32_t W, uint32_t cw, uint32_t elem, uint32_t pan
     out.T = out.rowOffset[W];
     out.tcA2B.assign(size_t(out.T) * cw, HSPMM_IDX_MAX);
     out.data.assign(size_t(out.T) * tile_bytes, 0);
-    // second pass: copy, or spread a window's tile columns over the union's columns
+    // second pass: copy, or spread a window's tile columns over the merged list's columns
     auto spread = [&](uint32_t w, const uint32_t *ids, uint32_t n_ids) {
         const uint32_t *c = tcA2B + size_t(rowOffset[w]) * cw;
         const uint32_t n = real_ids(w);
         uint32_t *dst_ids = out.tcA2B.data() + size_t(out.rowOffset[w]) * cw;
         std::memcpy(dst_ids, ids, size_t(n_ids) * 4);
-        uint32_t j = 0;                                         // position in the union (both lists ascend)
+        uint32_t j = 0;                                         // position in the merged list (same order)
         for (uint32_t i = 0; i < n; ++i) {
             while (ids[j] != c[i]) ++j;
             const uint8_t *st = src + size_t(rowOffset[w] + i / cw) * tile_bytes;
@@ -449,20 +472,23 @@ bool union_adjacent_windows(uint32_t W, uint32_t cw, uint32_t elem, uint32_t pan
                 std::memcpy(dt + (size_t(r) * cw + j % cw) * elem, st + (size_t(r) * cw + i % cw) * elem, elem);
         }
     };
-    for (uint32_t w = 0; w < W; ++w) {
-        if (join[w]) {
-            const uint32_t *a = tcA2B + size_t(rowOffset[w]) * cw, *b = tcA2B + size_t(rowOffset[w + 1]) * cw;
-            const uint32_t na = real_ids(w), nb = real_ids(w + 1);
-            merged.resize(size_t(na) + nb);
-            const uint32_t nu = uint32_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin());
-            spread(w, merged.data(), nu);
-            spread(w + 1, merged.data(), nu);
-            ++w;
+    out_first.clear(); out_count.clear();
+    for (size_t g = 0; g < NG; ++g) {
+        out_first.push_back(first[g]);
+        if (join[g]) {
+            const uint32_t wa = first[g], nw = count[g] + count[g + 1];
+            merged_list(wa, first[g + 1]);
+            for (uint32_t w = wa; w < wa + nw; ++w) spread(w, merged.data(), uint32_t(merged.size()));
+            out_count.push_back(nw);
+            ++g;
         } else {
-            std::memcpy(out.tcA2B.data() + size_t(out.rowOffset[w]) * cw, tcA2B + size_t(rowOffset[w]) * cw,
-                        size_t(tiles[w]) * cw * 4);
-            std::memcpy(out.data.data() + size_t(out.rowOffset[w]) * tile_bytes, src + size_t(rowOffset[w]) * tile_bytes,
-                        size_t(tiles[w]) * tile_bytes);
+            for (uint32_t w = first[g]; w < first[g] + count[g]; ++w) {
+                std::memcpy(out.tcA2B.data() + size_t(out.rowOffset[w]) * cw, tcA2B + size_t(rowOffset[w]) * cw,
+                            size_t(tiles[w]) * cw * 4);
+                std::memcpy(out.data.data() + size_t(out.rowOffset[w]) * tile_bytes, src + size_t(rowOffset[w]) * tile_bytes,
+                            size_t(tiles[w]) * tile_bytes);
+            }
+            out_count.push_back(count[g]);
         }
     }
     return true;
@@ -495,20 +521,54 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     // columns per re-tiled step: the kernels built on 16-bit MFMAs contract 32 columns per step, the fp32
     // MFMA kernels a tile's 8
     const uint32_t rw = (cw == 16 || split) ? 32u : cw;
-    // The units of this stream.  The kernels built on the 16-bit MFMA pair adjacent windows through
-    // the union of their column lists wherever that saves steps, and pair whatever can be paired
-    // (a pair costs them nothing); the fp32 MFMA forms walk the units of the gather kernels.
-    Unioned un;
+    // The units of this stream.  The kernels built on the 16-bit MFMA run groups of up to four adjacent
+    // windows with one column list as one unit, and give neighbours the union of their lists wherever
+    // that saves work (merge_groups); the fp32 MFMA forms walk the units of the gather kernels.
+    Unioned un1, un2;
     StepStream st = gather_st;
     if (rw == 32 && p->cfg.pairing != 1 && W > 1) {
-        if (union_adjacent_windows(W, cw, uint32_t(p->elem), KP, rw, rowOffset, tcA2B, data, rowIdx, un)) {
-            rowOffset = un.rowOffset.data(); tcA2B = un.tcA2B.data(); data = un.data.data();
+        // Units of three and four windows halve the LDS reads per row but leave half as many, twice as
+        // long waves: measured on pruned and block-clustered 16-bit matrices they pay once the units
+        // still fill the compute units at small N (16384 rows: 1.0 - 1.2 x, 28672 rows: 1.2 - 1.3 x;
+        // 8192 and 11008 rows: 0.93 - 1.1 x up to N = 512, 1.2 - 1.3 x only from N = 2048 on), and for
+        // fp32 storage in bf16 parts, with twice the MFMAs per LDS read, they gain nothing (0.82 - 1.2 x).
+        // Pairing mode 2 takes them wherever windows qualify.
+        double wide_cost = 1.25;
+        uint32_t max_windows = (p->cfg.pairing == 2 || cw == 16) ? 4u : 2u;
+        size_t min_wide_units = p->cfg.pairing == 2 ? 0u : size_t(p->compute_units) * 3u / 2u;
+        if (const char *e = std::getenv("HSPMM_PANEL_WIDE_COST")) wide_cost = std::atof(e);       // tuning overrides
+        if (const char *e = std::getenv("HSPMM_PANEL_MAX_WINDOWS")) {
+            max_windows = std::atoi(e) >= 4 ? 4u : 2u;
+            min_wide_units = 0;
         }
-        const size_t n_ids = size_t(rowOffset[W]) * cw;
-        std::vector<uint32_t> clean(tcA2B, tcA2B + n_ids);
-        for (size_t i = 1; i < n_ids; ++i)
-            if (clean[i] == HSPMM_IDX_MAX) clean[i] = clean[i - 1];
-        st = build_units(W, cw, rowOffset, rowIdx, clean, 2);
+        std::vector<uint32_t> first(W), count(W, 1u), f2, c2;
+        for (uint32_t w = 0; w < W; ++w) first[w] = w;
+        if (merge_groups(W, cw, uint32_t(p->elem), KP, rw, 2, 1.0, rowOffset, tcA2B, data, rowIdx, first, count, un1, f2, c2)) {
+            rowOffset = un1.rowOffset.data(); tcA2B = un1.tcA2B.data(); data = un1.data.data();
+            first.swap(f2); count.swap(c2);
+        }
+        if (max_windows > 2 && first.size() / 2u >= min_wide_units &&
+            merge_groups(W, cw, uint32_t(p->elem), KP, rw, max_windows, wide_cost, rowOffset, tcA2B, data, rowIdx, first,
+                         count, un2, f2, c2) &&
+            f2.size() >= min_wide_units) {
+            rowOffset = un2.rowOffset.data(); tcA2B = un2.tcA2B.data(); data = un2.data.data();
+            first.swap(f2); count.swap(c2);
+            un1 = Unioned();
+        }
+        st = StepStream();
+        st.unitOffset.push_back(0);
+        uint32_t widest = 1;
+        for (size_t g = 0; g < first.size(); ++g) {
+            const uint32_t w = first[g];
+            st.unitWindow.push_back(w);
+            st.unitRow.push_back(rowIdx[w] | (count[g] - 1u));
+            st.unitOffset.push_back(st.unitOffset.back() + (rowOffset[w + 1] - rowOffset[w]));
+            st.n_paired += count[g] >= 2u;
+            st.n_wide += count[g] >= 3u;
+            widest = std::max(widest, count[g]);
+        }
+        st.n_steps = st.unitOffset.back();
+        st.G = widest >= 3u ? 4 : int(widest);
     }
     const uint32_t U = uint32_t(st.unitRow.size());
     const uint32_t T = rowOffset[W];
@@ -583,7 +643,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     }
     // the units with the re-tiled step counts
     StepStream ps;
-    ps.G = st.G; ps.unitRow = st.unitRow; ps.unitWindow = st.unitWindow; ps.n_paired = st.n_paired;
+    ps.G = st.G; ps.unitRow = st.unitRow; ps.unitWindow = st.unitWindow; ps.n_paired = st.n_paired; ps.n_wide = st.n_wide;
     ps.unitOffset.assign(1, 0u);
     for (uint32_t u = 0; u < U; ++u) {
         const uint32_t w = st.unitWindow[u];
@@ -645,7 +705,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
         pl.d_tiles = dt;
     }
     if ((rc = upload(&pl.d_unitRow, st.unitRow.data(), st.unitRow.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
-    pl.n_units = U; pl.G = st.G; pl.n_paired = st.n_paired;
+    pl.n_units = U; pl.G = st.G; pl.n_paired = st.n_paired; pl.n_wide = st.n_wide;
     pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.split = split; pl.density = density; pl.built = true;
     return true;
 }
@@ -1006,7 +1066,9 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         forced_units = units == 13 ? 12 : units;
         if (wide) { units = 13; forced_units = std::min(forced_units, 12); }
     }
-    const int max_units = units == 13 ? 12 : units;
+    // (units of up to four windows: eight consumer waves with twice the accumulators)
+    const int max_units = pl.G == 4 ? 8 : units == 13 ? 12 : units;
+    if (forced_units) forced_units = std::min(forced_units, max_units);
     const uint64_t slots = uint64_t(p->compute_units) * (pl.quad ? 2u : 1u);     // workgroups resident at a time
     // Units per workgroup and chunks of panels: the workgroups should fill the compute units in whole
     // rounds.  Cost of a shape = rounds x panels per chunk x (units + 3: a panel costs its LDS reads, which
@@ -1037,7 +1099,8 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     if (pa.n_chunks > 1) {
         int rc = ensure_panel_split(p, pa.n_chunks);
         if (rc) return rc;
-        const size_t nacc = pl.quad ? 2u : pl.split ? 4u : p->dtype != HSPMM_TF32 ? 8u : 4u * size_t(pl.G);
+        const size_t wide = pl.G == 4 ? 2u : 1u;
+        const size_t nacc = pl.quad ? 2u : pl.split ? 4u * wide : p->dtype != HSPMM_TF32 ? 8u * wide : 4u * size_t(pl.G);
         const size_t need = size_t(pl.n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
         if ((rc = ensure_scratch(p, need))) return rc;
         pa.scratch = p->d_scratch;
@@ -1204,6 +1267,7 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_panel_steps = p->panel.built ? p->panel.n_steps : 0u;
     info->n_panel_units = p->panel.built ? p->panel.n_units : 0u;
     info->n_panel_paired_units = p->panel.built ? p->panel.n_paired : 0u;
+    info->n_panel_wide_units = p->panel.built ? p->panel.n_wide : 0u;
     return HSPMM_OK;
 }
 

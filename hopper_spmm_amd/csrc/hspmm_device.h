@@ -23,7 +23,7 @@ struct KernelArgs {
     const uint32_t *rowIdx;
     // the step stream the MFMA kernels walk
     const uint32_t *unitOffset;  // n_units + 1: first step of every unit
-    const uint32_t *unitRow;     // n_units: first matrix row of the unit | 1 if it is a pair of windows
+    const uint32_t *unitRow;     // n_units: first matrix row of the unit | its windows less one (1: a pair)
     const uint32_t *ids;         // per step, lane order, padding ids renamed
     const void     *tiles;       // per step, lane order
     // partition
@@ -59,7 +59,7 @@ constexpr uint32_t kPanelRowBytes = 256;       // bytes of a B row one workgroup
 constexpr uint32_t kPanelRowsWide = 256, kPanelRowsFp32 = 128;
 
 struct PanelArgs {
-    const uint32_t *unitRow;     // n_units: first matrix row of the unit | 1 if it is a pair of windows
+    const uint32_t *unitRow;     // n_units: first matrix row of the unit | its windows less one (0..3)
     const uint32_t *poff;        // n_units x (n_panels + 1): first step of the unit at or behind every panel
     const uint32_t *step_panel;  // per step: its panel
     const uint32_t *ids;         // per step: the rows (inside the panel) each quarter-wave reads and the panels
@@ -75,7 +75,7 @@ struct PanelArgs {
 };
 
 // units: 12 or 14 units (consumer waves) per workgroup, 2 more waves copy B to LDS; 13 = 12 units and 4 such waves.
-// G: windows per unit; 0 = fp32 single windows with ids in the format of the 4x4x1 tile.  split (fp32): the plan's
+// G: windows per unit at most (1, 2, 4); 0 = fp32 single windows with ids in the format of the 4x4x1 tile.  split (fp32): the plan's
 // stream is in the bf16 hi / lo form.  ka: arguments of the kernel that adds the chunk sums (split table with one
 // entry per unit), used when pa.n_chunks > 1.
 hipError_t launch_spmm_panel(int dtype, int G, bool split, const PanelArgs &pa, const KernelArgs &ka, int units,

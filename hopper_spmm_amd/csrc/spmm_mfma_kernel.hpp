@@ -671,6 +671,24 @@ void spmm_mfma_kernel(const KernelArgs ka)
 #undef HSPMM_FOR_STAGES
 }
 
+// Windows of a unit: the low bits of its row word hold the count less one (1: a pair; the
+// LDS-panel kernels also have units of three and four windows).
+template <class TT>
+__device__ __forceinline__ uint32_t unit_windows(const uint32_t row_word)
+{
+    return TT::G > 1 ? (row_word & 3u) + 1u : 1u;
+}
+
+// Stores the windows W0 .. of a unit (window w covers rows row0 + 8 w .. + 7).
+template <class TT, int W0 = 0, int NACC>
+__device__ __forceinline__ void store_unit(const typename TT::Lane &L, const f32x4 (&acc)[NACC], char *c_lane,
+                                           size_t row_bytes, uint32_t row0, uint32_t nwin, uint32_t rows, bool active)
+{
+    if (uint32_t(W0) < nwin)
+        TT::template store_window<W0>(L, acc, c_lane, row_bytes, row0 + uint32_t(W0) * kRowWindow, rows, active);
+    if constexpr (W0 + 1 < TT::G) store_unit<TT, W0 + 1>(L, acc, c_lane, row_bytes, row0, nwin, rows, active);
+}
+
 // ---------------------------------------------------------------------------
 // Second kernel: adds, in range order, the fp32 partial sums of every unit
 // whose steps were cut across ranges, and stores its window(s).
@@ -708,10 +726,7 @@ void spmm_fixup_kernel(const KernelArgs ka)
         for (int p = 0; p < NACC; ++p) acc[p] += src[p * 64];
     }
     const uint32_t row = ka.unitRow[u];
-    TT::template store_window<0>(L, acc, c_lane, row_bytes, row & ~7u, ka.rows, active);
-    if constexpr (G > 1) {
-        if (row & 1u) TT::template store_window<G - 1>(L, acc, c_lane, row_bytes, (row & ~7u) + kRowWindow, ka.rows, active);
-    }
+    store_unit<TT>(L, acc, c_lane, row_bytes, row & ~7u, unit_windows<TT>(row), ka.rows, active);
 }
 
 // ---------------------------------------------------------------------------

@@ -8,6 +8,7 @@ template <int G> using PanelTile = Fp16Tr<G, false>;
 
 hipError_t launch_panel_f16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid)
 {
+    if (G == 4) return launch_panel_nw<PanelTile<4>>(pa, ka, waves, s, mid);
     return G == 2 ? launch_panel_nw<PanelTile<2>>(pa, ka, waves, s, mid)
                   : launch_panel_nw<PanelTile<1>>(pa, ka, waves, s, mid);
 }

@@ -7,10 +7,11 @@ namespace hspmm {
 template <int G> using PanelTile = Fp32Tile<4, G>;
 
 // G = 0: single windows through the 4x4x1 instruction (the plan's ids are in that tile's format);
-// G = 1, 2 with split: the bf16 hi / lo form (the plan's ids and tiles are in that form).
+// G = 1, 2, 4 with split: the bf16 hi / lo form (the plan's ids and tiles are in that form).
 hipError_t launch_panel_f32(int G, bool split, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s,
                             hipEvent_t mid)
 {
+    if (split && G == 4) return launch_panel_nw<Fp32Split<4>>(pa, ka, waves, s, mid);
     if (split)
         return G == 2 ? launch_panel_nw<Fp32Split<2>>(pa, ka, waves, s, mid)
                       : launch_panel_nw<Fp32Split<1>>(pa, ka, waves, s, mid);

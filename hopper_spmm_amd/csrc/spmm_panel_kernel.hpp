@@ -6,20 +6,19 @@
 // and what the reference sketches with its producer / consumer shared-memory ring
 // (src/fp16.cu:56-175).
 //
-//   * Columns are cut into panels of kPanelRows.  The plan re-tiles every unit (a
-//     window, or a pair of windows with one column list) panel by panel: the
-//     unit's columns inside a panel are condensed into tiles of their own, so no
-//     tile straddles a panel; ids are row numbers inside the panel (one byte each,
-//     the four - fp32: two - ids of a lane in one word).  poff[u][p] is the first
-//     step of unit u in panel p.
-//   * A workgroup owns NC consecutive units (one per consumer wave), one block of
-//     256 bytes of every B row (128 halves / 64 floats of the feature dimension)
-//     and a contiguous chunk of panels.  Per panel its producer waves copy the
-//     panel's slice of B (kPanelRows x 256 bytes, coalesced 16-byte loads) to LDS;
-//     every consumer wave then runs the steps its unit has in the panel, reading
-//     its four (two for fp32) B rows per step from LDS with 16-byte reads: the 16
-//     lanes of a quarter-wave read one whole 256-byte row, so the reads of a
-//     quarter never share a bank.
+//   * Columns are cut into panels (256 columns for the kernels built on the 16-bit
+//     MFMA, 128 for the fp32 MFMA forms).  The plan re-tiles every unit (a window,
+//     or a group of adjacent windows with one column list) panel by panel: the
+//     unit's columns inside a panel are condensed into steps of their own, so no
+//     step straddles a panel; ids are row numbers inside the panel, packed the way
+//     the tile type's address arithmetic wants them (PanelOps below).  poff[u][p]
+//     is the first step of unit u in panel p.
+//   * A workgroup owns up to NC consecutive units (one per consumer wave), one
+//     block of 256 bytes of every B row (128 halves / 64 floats of the feature
+//     dimension) and a contiguous chunk of panels.  Per panel its producer waves
+//     copy the panel's slice of B (coalesced 16-byte loads) to LDS; every consumer
+//     wave then runs the steps its unit has in the panel, reading the B rows of
+//     its columns from LDS.
 //   * Two LDS buffers and one barrier per panel: the producers fill the buffer of
 //     panel p+1 while the consumers multiply panel p.
 //   * The unit's tiles and ids stream from global memory through a small register
@@ -142,9 +141,13 @@ struct PanelOps {
 //     pair, zero for a single window);
 //   * accumulator p (of 8): features 16 p .. 16 p + 15 of the block; register e of lane
 //     (g, j): unit row 4g + e, feature 16 p + j.
-// The rows of the LDS image are 288 bytes apart: the four rows one block of lanes reads
-// lie in different banks when their numbers differ mod 4, and the plan orders the
-// columns of a step accordingly (hspmm_capi.hip, build_panel_stream).
+// The rows of the LDS image are 288 bytes apart and the LDS serves two blocks of lanes at a
+// time: the eight rows they read lie in different banks when their numbers differ mod 8,
+// and the plan orders the columns of a step accordingly (hspmm_capi.hip, build_panel_stream).
+// Units of three and four windows (G = 4; the third and fourth in a second KB of the step's
+// tile copy) run every second operand against two first operands: half the LDS reads per
+// row, which is what binds these kernels, with eight consumer waves of twice the
+// accumulators.
 //   ids per step: 64 words, one per lane: bits 4..15 = 9 x (panel row of column
 //     8g + i / 4), bits 16..27 = 9 x (panel row of column 8g + 4 + i / 4) (i = l % 16;
 //     x 32 = byte offset in the image); bits 0..3: the panel jump.
@@ -153,7 +156,9 @@ typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
 
 template <int G_, bool BF>
 struct Fp16Tr {
-    static constexpr int G = G_, V = 8 / G_;       // G * V = 8 accumulators
+    // G * V accumulators: 8 for the 16 rows of one or two windows; units of up to four windows
+    // (G = 4) run every step's second operand against two first operands, rows 0..15 and 16..31
+    static constexpr int G = G_, V = G_ == 4 ? 4 : 8 / G_;
     static constexpr int kBlockFeat = 128;
     static constexpr int kLaneFeat = 1;            // lane's feature = j (+ 16 per accumulator)
     static constexpr int kElem = 2;
@@ -170,19 +175,20 @@ struct Fp16Tr {
             idx_src = ids + lane;
         }
     };
-    // Window W0 of the unit is held by quarter-waves 2 W0 and 2 W0 + 1.
+    // Window W0 of the unit is held by quarter-waves 2 (W0 % 2) and 2 (W0 % 2) + 1 of accumulators
+    // 8 (W0 / 2) .. + 7.
     template <int W0>
-    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[8], char *c_lane,
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[G * V], char *c_lane,
                                                         size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
     {
-        if ((L.g >> 1) != uint32_t(W0)) return;
+        if ((L.g >> 1) != uint32_t(W0 & 1)) return;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const uint32_t row = row0 + 4u * (L.g & 1u) + e;
             if (active && row < rows) {
                 elem_t *dst = reinterpret_cast<elem_t *>(c_lane + size_t(row) * row_bytes);
 #pragma unroll
-                for (int p = 0; p < 8; ++p) stream_store(dst + 16 * p, (elem_t)acc[p][e]);
+                for (int p = 0; p < 8; ++p) stream_store(dst + 16 * p, (elem_t)acc[8 * (W0 >> 1) + p][e]);
             }
         }
     }
@@ -207,18 +213,25 @@ struct PanelOps<Fp16Tr<G_, BF>> {
     {
         *reinterpret_cast<u32x4 *>(row + c * 16u) = x;
     }
-    static constexpr uint32_t kRing = 6;
-    static constexpr int kLive = 8;
+    static constexpr bool kFour = G_ == 4;                        // units of up to four windows
+    static constexpr int kConsumers = kFour ? 8 : 12;             // twice the accumulators: fewer, larger waves
+    static constexpr uint32_t kRing = kFour ? 4 : 6;
+    static constexpr int kLive = TT::G * TT::V;
     __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
     typedef uint32_t Idx;
-    typedef u32x4 AVec;
+    // the lane's 16 bytes of the step's first 1 KB (rows 0..15), with four windows also of the second (rows 16..31)
+    struct AVec { u32x4 r[kFour ? 2 : 1]; };
     __device__ static __forceinline__ Idx load_idx(const typename TT::Lane &L, const uint32_t *, uint32_t step)
     {
         return L.idx_src[size_t(step) * 64u];
     }
     __device__ static __forceinline__ AVec load_a(const typename TT::Lane &L, uint32_t step)
     {
-        return *reinterpret_cast<const u32x4 *>(L.a_src + size_t(step) * 256u);
+        AVec a;
+        const uint32_t *src = L.a_src + size_t(step) * (kFour ? 512u : 256u);
+        a.r[0] = *reinterpret_cast<const u32x4 *>(src);
+        if constexpr (kFour) a.r[1] = *reinterpret_cast<const u32x4 *>(src + 256);
+        return a;
     }
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) & 15u; }
     typedef tr16x4 __attribute__((address_space(3))) *lds_tr_ptr;
@@ -236,7 +249,8 @@ struct PanelOps<Fp16Tr<G_, BF>> {
             u32x4 b;
             const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
             b[0] = l2[0]; b[1] = l2[1]; b[2] = h2[0]; b[3] = h2[1];
-            acc[p] = HalfOps<BF>::mfma(A, b, acc[p]);
+            acc[p] = HalfOps<BF>::mfma(A.r[0], b, acc[p]);
+            if constexpr (kFour) acc[8 + p] = HalfOps<BF>::mfma(A.r[1], b, acc[8 + p]);
         }
     }
     __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return (L.j & 3u) * 8u; }
@@ -258,7 +272,7 @@ struct PanelOps<Fp16Tr<G_, BF>> {
 //   accumulator p (of 4): features 16 p .. 16 p + 15 of the block of 64.
 template <int G_>
 struct Fp32Split {
-    static constexpr int G = G_, V = 4 / G_;       // G * V = 4 accumulators
+    static constexpr int G = G_, V = G_ == 4 ? 2 : 4 / G_;   // G * V = 4 accumulators, 8 for up to four windows
     static constexpr int kBlockFeat = 64;
     static constexpr int kLaneFeat = 1;
     static constexpr int kElem = 4;
@@ -275,17 +289,17 @@ struct Fp32Split {
         }
     };
     template <int W0>
-    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[4], char *c_lane,
+    __device__ static __forceinline__ void store_window(const Lane &L, const f32x4 (&acc)[G * V], char *c_lane,
                                                         size_t row_bytes, uint32_t row0, uint32_t rows, bool active)
     {
-        if ((L.g >> 1) != uint32_t(W0)) return;
+        if ((L.g >> 1) != uint32_t(W0 & 1)) return;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const uint32_t row = row0 + 4u * (L.g & 1u) + e;
             if (active && row < rows) {
                 float *dst = reinterpret_cast<float *>(c_lane + size_t(row) * row_bytes);
 #pragma unroll
-                for (int p = 0; p < 4; ++p) { const float v = acc[p][e]; stream_store(dst + 16 * p, v); }
+                for (int p = 0; p < 4; ++p) { const float v = acc[4 * (W0 >> 1) + p][e]; stream_store(dst + 16 * p, v); }
             }
         }
     }
@@ -332,18 +346,25 @@ struct PanelOps<Fp32Split<G_>> {
         *reinterpret_cast<u32x2 *>(row + c * 8u) = hi;
         *reinterpret_cast<u32x2 *>(row + 128u + c * 8u) = lo;
     }
-    static constexpr uint32_t kRing = 4;
-    static constexpr int kLive = 4;
+    static constexpr bool kFour = G_ == 4;
+    static constexpr int kConsumers = kFour ? 8 : 12;
+    static constexpr uint32_t kRing = kFour ? 3 : 4;
+    static constexpr int kLive = TT::G * TT::V;
     __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
     typedef uint32_t Idx;
-    typedef u32x8 AVec;
+    // the lane's 32 bytes of the step's first 2 KB (rows 0..15), with four windows also of the second
+    struct AVec { u32x8 r[kFour ? 2 : 1]; };
     __device__ static __forceinline__ Idx load_idx(const typename TT::Lane &L, const uint32_t *, uint32_t step)
     {
         return L.idx_src[size_t(step) * 64u];
     }
     __device__ static __forceinline__ AVec load_a(const typename TT::Lane &L, uint32_t step)
     {
-        return *reinterpret_cast<const u32x8 *>(L.a_src + size_t(step) * 512u);
+        AVec a;
+        const uint32_t *src = L.a_src + size_t(step) * (kFour ? 1024u : 512u);
+        a.r[0] = *reinterpret_cast<const u32x8 *>(src);
+        if constexpr (kFour) a.r[1] = *reinterpret_cast<const u32x8 *>(src + 512);
+        return a;
     }
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) & 15u; }
     typedef tr16x4 __attribute__((address_space(3))) *lds_tr_ptr;
@@ -364,18 +385,24 @@ struct PanelOps<Fp32Split<G_>> {
         const lds_char_ptr base = (lds_char_ptr)smem + img;
         const lds_char_ptr a0 = base + (__builtin_amdgcn_ubfe(I, 4, 12) << 5);
         const lds_char_ptr a1 = base + (__builtin_amdgcn_ubfe(I, 16, 12) << 5);
-        u32x4 a_hi, a_lo;
+        constexpr int kHalves = kFour ? 2 : 1;
+        u32x4 a_hi[kHalves], a_lo[kHalves];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { a_hi[i] = A[i]; a_lo[i] = A[4 + i]; }
+        for (int h = 0; h < kHalves; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { a_hi[h][i] = A.r[h][i]; a_lo[h][i] = A.r[h][4 + i]; }
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const u32x4 b_hi = operand(a0, a1, 32 * p);
             const u32x4 b_lo = operand(a0, a1, 128 + 32 * p);
-            // small terms first
-            f32x4 c = HalfOps<true>::mfma(a_lo, b_lo, acc[p]);
-            c = HalfOps<true>::mfma(a_lo, b_hi, c);
-            c = HalfOps<true>::mfma(a_hi, b_lo, c);
-            acc[p] = HalfOps<true>::mfma(a_hi, b_hi, c);
+#pragma unroll
+            for (int h = 0; h < kHalves; ++h) {
+                // small terms first
+                f32x4 c = HalfOps<true>::mfma(a_lo[h], b_lo, acc[4 * h + p]);
+                c = HalfOps<true>::mfma(a_lo[h], b_hi, c);
+                c = HalfOps<true>::mfma(a_hi[h], b_lo, c);
+                acc[4 * h + p] = HalfOps<true>::mfma(a_hi[h], b_hi, c);
+            }
         }
     }
     __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return (L.j & 3u) * 8u; }
@@ -597,12 +624,9 @@ void spmm_panel_kernel(const PanelArgs pa)
     for (int i = 0; i < NACC; ++i) acc[i] = live[i];
     const uint32_t row = pa.unitRow[u];
     const uint32_t row0 = row & ~7u;
-    const bool paired = (G > 1) && (row & 1u);
+    const uint32_t nwin = unit_windows<TT>(row);
     if (pa.n_chunks == 1u) {
-        TT::template store_window<0>(L, acc, c_lane, row_bytes, row0, pa.rows, true);
-        if constexpr (G > 1) {
-            if (paired) TT::template store_window<G - 1>(L, acc, c_lane, row_bytes, row0 + kRowWindow, pa.rows, true);
-        }
+        store_unit<TT>(L, acc, c_lane, row_bytes, row0, nwin, pa.rows, true);
     } else {
         f32x4 *dst = reinterpret_cast<f32x4 *>(pa.scratch) +
                      ((size_t(u) * pa.n_chunks + chunk) * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
@@ -612,15 +636,16 @@ void spmm_panel_kernel(const PanelArgs pa)
     if (chunk == 0u) {
         // rows of the windows without entries behind this unit, and in front of the first one
         const uint32_t next_row = (u + 1u < pa.n_units) ? (pa.unitRow[u + 1u] & ~7u) : pa.rows;
-        const uint32_t gap_begin = row0 + (paired ? 2u * kRowWindow : kRowWindow);
+        const uint32_t gap_begin = row0 + nwin * kRowWindow;
         if (gap_begin < next_row) TT::zero_rows(L, c_lane, row_bytes, gap_begin, next_row, true);
         if (u == 0u) TT::zero_rows(L, c_lane, row_bytes, 0u, row0, true);
     }
 }
 
-// Units (consumer waves) per workgroup: 12 or 14; two more waves are producers (four in
-// the shape the 4x4x1 fp32 kernel uses).  Waves go to the four SIMDs of a compute unit
-// round-robin, so 12 consumers spread evenly.
+// Units (consumer waves) per workgroup: 12 or 14 and two producer waves for panels of 128
+// rows (12 + 4 in the shape the 4x4x1 fp32 kernel uses); 12 + 4, or 8 + 4 for units of up
+// to four windows, for panels of 256 rows.  Waves go to the four SIMDs of a compute unit
+// round-robin, so 8 and 12 consumers spread evenly.
 
 // ka: the arguments of spmm_fixup_kernel for the chunk sums (split table with one
 // entry per unit); used only when pa.n_chunks > 1.
@@ -643,7 +668,7 @@ template <class TT>
 static hipError_t launch_panel_nw(const PanelArgs &pa, const KernelArgs &ka, int units, hipStream_t s, hipEvent_t mid)
 {
     // panels of 256 rows need four producer waves to hold one in registers
-    if constexpr (PanelOps<TT>::kRows > 128u) return launch_panel_tt<TT, 12, 4>(pa, ka, s, mid);
+    if constexpr (PanelOps<TT>::kRows > 128u) return launch_panel_tt<TT, PanelOps<TT>::kConsumers, 4>(pa, ka, s, mid);
     else {
         if (units == 14) return launch_panel_tt<TT, 14, 2>(pa, ka, s, mid);
         if (units == 13) return launch_panel_tt<TT, 12, 4>(pa, ka, s, mid);      // 12 units, four producer waves

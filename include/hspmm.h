@@ -116,10 +116,10 @@ int hspmm_set_kernel_mode(int mode);
  * column list (block-clustered weights) can share one gather of B.  Read by the
  * next hspmm_create: 0 = pair when at least a quarter of the tiles would be in
  * pairs, 1 = never, 2 = whenever any two windows qualify.  The LDS-staging
- * kernels built on the 16-bit MFMA (a step of theirs multiplies 16 rows) go
- * further unless the mode is 1: in their copy of the matrix two adjacent windows
- * carry the union of their column lists, absent entries as zeros, wherever that
- * saves steps. */
+ * kernels built on the 16-bit MFMA (a step of theirs multiplies 16 or 32 rows)
+ * go further unless the mode is 1: in their copy of the matrix groups of up to
+ * four adjacent windows carry the union of their column lists, absent entries
+ * as zeros, wherever that saves work. */
 int hspmm_set_window_pairing(int mode);
 
 typedef struct {
@@ -134,8 +134,9 @@ typedef struct {
     uint64_t device_bytes;      /* bytes of device memory the plan holds right now */
     uint32_t n_panels;          /* column panels of the LDS-staging kernels; 0: the plan does not use them */
     uint32_t n_panel_steps;     /* steps of the unit stream re-tiled panel by panel */
-    uint32_t n_panel_units;     /* units of that stream: it pairs windows through the union of their columns */
-    uint32_t n_panel_paired_units;
+    uint32_t n_panel_units;     /* units of that stream: groups of up to four adjacent windows that share, or were given, one column list */
+    uint32_t n_panel_paired_units;  /* of those: units of two or more windows */
+    uint32_t n_panel_wide_units;    /* of those: units of three or four windows */
 } hspmm_plan_info;
 
 /* No reference counterpart (the reference prints its statistics from main,

@@ -330,8 +330,8 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
             per_step = 1 if mode == 5 else 4 if dtype == 1 else 2
             panel_rows = 128 if mode == 5 else 256      # the fp32 MFMA forms keep panels of 128 columns
             assert info["n_panels"] == (cols + panel_rows - 1) // panel_rows
-            # (adjacent windows with much the same columns may have been given one list: two windows per step)
-            assert info["n_panel_steps"] >= info["total_tiles"] // (2 * per_step)
+            # (adjacent windows with much the same columns may have been given one list: up to four windows per step)
+            assert info["n_panel_steps"] >= info["total_tiles"] // (4 * per_step)
             for N in (block, 2 * block, 5 * block):
                 B = make_b(rng, cols, N, dtype)
                 got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
@@ -402,14 +402,17 @@ def test_lds_panel_kernels_are_chosen_for_dense_windows_only(torch_cuda, hs):
 
 
 @pytest.mark.parametrize("dtype", [0, 1, 2])
-def test_adjacent_windows_with_overlapping_columns_become_pairs(torch_cuda, hs, oracle, dtype):
+def test_adjacent_windows_with_overlapping_columns_share_units(torch_cuda, hs, oracle, dtype):
     """In the LDS-panel kernels' copy of the matrix adjacent windows are given the union of their
-    column lists and run as pairs: same product (the added entries are zeros); the other kernel
-    families keep the caller's windows."""
+    column lists and run as one unit - pairs, and with pairing mode 2 (or on matrices large enough
+    to fill the GPU that way) groups of three and four windows: same product (the added entries are
+    zeros), also when the panels are cut into chunks whose sums a second kernel adds; the other
+    kernel families keep the caller's windows."""
     rng = np.random.default_rng(40 + dtype)
     rows, cols = 203, 1500
     D = rng.integers(-3, 4, (rows, cols)) * (rng.random((rows, cols)) < 0.25)
     D[64:80] = 0                                        # two empty windows in the middle
+    D[136:144] = 0                                      # and one that leaves seven windows in a row: 4 + 3
     D[100, :] = rng.integers(1, 3, cols)                # a full row
     rp = np.zeros(rows + 1, np.uint32)
     ci, vv = [], []
@@ -432,14 +435,48 @@ def test_adjacent_windows_with_overlapping_columns_become_pairs(torch_cuda, hs, 
                 hs.set_window_pairing(0)
             info = plan.info()
             assert info["total_tiles"] == b["total_tiles"] and info["n_paired_units"] == 0
-            if mode in (0, 4) or (mode == 5 and dtype != 1):    # a panel stream built on the 16-bit MFMA
+            grouped = mode in (0, 4) or (mode == 5 and dtype != 1)     # a panel stream built on the 16-bit MFMA
+            if grouped:
                 assert info["n_panels"] > 0
                 assert (info["n_panel_paired_units"] > 0) == (pairing != 1), (mode, pairing, info)
-            for N in (block, 2 * block, 24):
-                Bm = rng.integers(-4, 5, (cols, N))
-                got = gpu_spmm(torch_cuda, hs, b, encode(Bm, dtype), N, plan=plan)
-                assert np.array_equal(got, encode(D @ Bm, dtype)), (mode, pairing, N)
+                assert (info["n_panel_wide_units"] > 0) == (pairing == 2), (mode, pairing, info)
+                if pairing == 2:        # 8, 7 and 8 windows between the gaps: two fours, a four and a three, two fours
+                    assert info["n_panel_units"] == 6 and info["n_panel_wide_units"] == 6, info
+            for chunks in (None, "2") if grouped else (None,):
+                if chunks:
+                    os.environ["HSPMM_PANEL_CHUNKS"] = chunks
+                try:
+                    for N in (block, 2 * block, 24):
+                        Bm = rng.integers(-4, 5, (cols, N))
+                        got = gpu_spmm(torch_cuda, hs, b, encode(Bm, dtype), N, plan=plan)
+                        assert np.array_equal(got, encode(D @ Bm, dtype)), (mode, pairing, chunks, N)
+                finally:
+                    os.environ.pop("HSPMM_PANEL_CHUNKS", None)
             plan.close()
+
+
+@pytest.mark.parametrize("dtype", [0, 2])
+def test_units_of_four_windows_are_chosen_for_large_pruned_matrices(torch_cuda, hs, oracle, dtype):
+    """A 16-bit matrix with dense windows and enough rows to fill the GPU with units of 32 rows gets
+    them without being asked; a smaller one, and fp32 storage, keep pairs."""
+    from hopper_spmm_amd import generators as G
+    rows, cols, N = 13312, 1024, 256                     # 416 units of four windows >= 1.5 x 256 compute units
+    A = G.pruned_weight(rows, cols, 0.10, 77, dtype=dtype)
+    b = convert(hs, A)
+    plan = hs.Plan(b)
+    info = plan.info()
+    assert info["n_panels"] == 4 and info["n_panel_units"] == rows // 32 == info["n_panel_wide_units"], info
+    rng = np.random.default_rng(5)
+    B = make_b(rng, cols, N, dtype)
+    got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+    plan.close()
+    ref, mag = oracle_spmm(oracle, A, B, N)
+    assert_parity(got, ref, mag, dtype, "units of four windows")
+    small = G.pruned_weight(4096, cols, 0.10, 78, dtype=dtype)
+    assert hs.Plan(convert(hs, small)).info()["n_panel_wide_units"] == 0
+    f32 = G.pruned_weight(rows, cols, 0.10, 77, dtype=1)
+    info = hs.Plan(convert(hs, f32)).info()
+    assert info["n_panels"] > 0 and info["n_panel_paired_units"] > 0 and info["n_panel_wide_units"] == 0
 
 
 @pytest.mark.parametrize("seed", [11, 12, 13])
