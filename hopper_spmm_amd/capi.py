@@ -102,6 +102,8 @@ def load_library():
     L.hspmm_partition_preview.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
     L.hspmm_partition_preview_grouped.argtypes = [u32, vp, u32, u32, vp, u32, C.POINTER(u32), C.POINTER(u32),
                                                   C.POINTER(u32)]
+    L.hspmm_panel_units_preview.argtypes = [i, u32, u32, u32, u32, vp, vp, vp, vp, u32, C.POINTER(u32), vp, vp, vp,
+                                            C.POINTER(u32), u32, vp, vp]
     L.hspmm_mtx_load.argtypes = [C.c_char_p, i, C.POINTER(_Csr)]
     L.hspmm_csr_free.argtypes = [C.POINTER(_Csr)]
     L.hspmm_csr_free.restype = None
@@ -313,6 +315,32 @@ def partition_preview(rowOffset, target_ranges, group=1):
         _check(L.hspmm_partition_preview_grouped(W, _p(rowOffset), target_ranges, group, _p(ranges), n.value, None,
                                                  None, None))
     return dict(ranges=ranges, n_split_windows=ns.value, n_partial_slots=nslots.value)
+
+
+def panel_units_preview(btcf, max_windows=4):
+    """How the LDS-staging kernels built on the 16-bit MFMA group adjacent windows into units
+    (host only): dict with group_first, group_count and the rewritten matrix (rowOffset, tcA2B,
+    data, total_tiles) whose windows carry their group's union of column lists."""
+    L = load_library()
+    dtype = btcf["dtype"]
+    vt = _val_dtype(dtype)
+    cw = 8 if dtype == TF32 else 16
+    ro = np.ascontiguousarray(btcf["rowOffset"], np.uint32)
+    a2b = np.ascontiguousarray(btcf["tcA2B"], np.uint32)
+    data = np.ascontiguousarray(btcf["data"], vt)
+    ri = np.ascontiguousarray(btcf["rowIdx"], np.uint32)
+    W, T = int(btcf["eff_row_windows"]), int(btcf["total_tiles"])
+    ng, nt = C.c_uint32(), C.c_uint32()
+    first = np.zeros(max(W, 1), np.uint32)
+    count = np.zeros(max(W, 1), np.uint32)
+    new_ro = np.zeros(W + 1, np.uint32)
+    args = (dtype, int(btcf["rows"]), int(btcf["cols"]), W, T, _p(ro), _p(a2b), _p(data), _p(ri), max_windows)
+    _check(L.hspmm_panel_units_preview(*args, C.byref(ng), _p(first), _p(count), _p(new_ro), C.byref(nt), 0, None, None))
+    new_a2b = np.zeros(nt.value * cw, np.uint32)
+    new_data = np.zeros(nt.value * 8 * cw, vt)
+    _check(L.hspmm_panel_units_preview(*args, None, None, None, None, None, nt.value, _p(new_a2b), _p(new_data)))
+    return dict(group_first=first[:ng.value].copy(), group_count=count[:ng.value].copy(), rowOffset=new_ro,
+                tcA2B=new_a2b, data=new_data, total_tiles=nt.value)
 
 
 class Plan:

@@ -494,6 +494,34 @@ bool merge_groups(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, u
     return true;
 }
 
+// The two passes of merge_groups: windows into pairs, then neighbouring groups into units of up to
+// max_windows (2 or 4) windows, the second pass only when it leaves at least min_wide_units units.
+// On return rowOffset / tcA2B / data point to the arrays the groups refer to: the caller's, or those
+// of `un` when anything was merged.
+void group_windows(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, uint32_t step_cols, uint32_t max_windows,
+                   double wide_cost, size_t min_wide_units, const uint32_t *&rowOffset, const uint32_t *&tcA2B,
+                   const void *&data, const uint32_t *rowIdx, Unioned &un, std::vector<uint32_t> &first,
+                   std::vector<uint32_t> &count)
+{
+    first.resize(W); count.assign(W, 1u);
+    for (uint32_t w = 0; w < W; ++w) first[w] = w;
+    if (max_windows < 2 || W < 2) return;
+    std::vector<uint32_t> f2, c2;
+    if (merge_groups(W, cw, elem, panel_cols, step_cols, 2, 1.0, rowOffset, tcA2B, data, rowIdx, first, count, un, f2, c2)) {
+        rowOffset = un.rowOffset.data(); tcA2B = un.tcA2B.data(); data = un.data.data();
+        first.swap(f2); count.swap(c2);
+    }
+    Unioned un2;
+    if (max_windows > 2 && first.size() / 2u >= min_wide_units &&
+        merge_groups(W, cw, elem, panel_cols, step_cols, max_windows, wide_cost, rowOffset, tcA2B, data, rowIdx, first,
+                     count, un2, f2, c2) &&
+        f2.size() >= min_wide_units) {
+        un = std::move(un2);
+        rowOffset = un.rowOffset.data(); tcA2B = un.tcA2B.data(); data = un.data.data();
+        first.swap(f2); count.swap(c2);
+    }
+}
+
 // Re-tiles the matrix panel by panel for the LDS-panel kernels (spmm_panel_kernel.hpp):
 // inside every window the columns of one panel of kPanelRows columns get tiles of
 // their own.  Every step carries the number of panels it lies behind the step in
@@ -524,7 +552,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     // The units of this stream.  The kernels built on the 16-bit MFMA run groups of up to four adjacent
     // windows with one column list as one unit, and give neighbours the union of their lists wherever
     // that saves work (merge_groups); the fp32 MFMA forms walk the units of the gather kernels.
-    Unioned un1, un2;
+    Unioned un;
     StepStream st = gather_st;
     if (rw == 32 && p->cfg.pairing != 1 && W > 1) {
         // Units of three and four windows halve the LDS reads per row but leave half as many, twice as
@@ -541,20 +569,9 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
             max_windows = std::atoi(e) >= 4 ? 4u : 2u;
             min_wide_units = 0;
         }
-        std::vector<uint32_t> first(W), count(W, 1u), f2, c2;
-        for (uint32_t w = 0; w < W; ++w) first[w] = w;
-        if (merge_groups(W, cw, uint32_t(p->elem), KP, rw, 2, 1.0, rowOffset, tcA2B, data, rowIdx, first, count, un1, f2, c2)) {
-            rowOffset = un1.rowOffset.data(); tcA2B = un1.tcA2B.data(); data = un1.data.data();
-            first.swap(f2); count.swap(c2);
-        }
-        if (max_windows > 2 && first.size() / 2u >= min_wide_units &&
-            merge_groups(W, cw, uint32_t(p->elem), KP, rw, max_windows, wide_cost, rowOffset, tcA2B, data, rowIdx, first,
-                         count, un2, f2, c2) &&
-            f2.size() >= min_wide_units) {
-            rowOffset = un2.rowOffset.data(); tcA2B = un2.tcA2B.data(); data = un2.data.data();
-            first.swap(f2); count.swap(c2);
-            un1 = Unioned();
-        }
+        std::vector<uint32_t> first, count;
+        group_windows(W, cw, uint32_t(p->elem), KP, rw, max_windows, wide_cost, min_wide_units, rowOffset, tcA2B, data,
+                      rowIdx, un, first, count);
         st = StepStream();
         st.unitOffset.push_back(0);
         uint32_t widest = 1;
@@ -891,6 +908,44 @@ int hspmm_partition_preview_grouped(uint32_t eff_row_windows, const uint32_t *ro
 {
     return partition_preview(eff_row_windows, rowOffset, target_ranges, group, 6, ranges, capacity_ranges, n_ranges,
                              n_split_windows, n_partial_slots);
+}
+
+int hspmm_panel_units_preview(int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows, uint32_t total_tiles,
+                              const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data, const uint32_t *rowIdx,
+                              uint32_t max_windows, uint32_t *n_groups, uint32_t *group_first, uint32_t *group_count,
+                              uint32_t *new_rowOffset, uint32_t *new_total_tiles, uint32_t capacity_tiles,
+                              uint32_t *new_tcA2B, void *new_data)
+{
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16)
+        return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
+    if (max_windows != 1 && max_windows != 2 && max_windows != 4)
+        return fail(HSPMM_ERR_INVALID, "max_windows %u: 1, 2 or 4", max_windows);
+    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u, elem = dtype == HSPMM_TF32 ? 4u : 2u;
+    const int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx);
+    if (rc) return rc;
+    const uint32_t W = eff_row_windows;
+    Unioned un;
+    std::vector<uint32_t> first, count;
+    const void *d = data;
+    try {
+        group_windows(W, cw, elem, hspmm::kPanelRowsWide, 32u, max_windows, 1.25, 0, rowOffset, tcA2B, d, rowIdx, un, first,
+                      count);
+    } catch (const std::bad_alloc &) { return fail(HSPMM_ERR_ALLOC, "out of host memory"); }
+    const uint32_t T = W ? rowOffset[W] : 0u;
+    if (n_groups) *n_groups = uint32_t(first.size());
+    if (new_total_tiles) *new_total_tiles = T;
+    for (size_t g = 0; g < first.size(); ++g) {
+        if (group_first) group_first[g] = first[g];
+        if (group_count) group_count[g] = count[g];
+    }
+    if (new_rowOffset && W) std::memcpy(new_rowOffset, rowOffset, (size_t(W) + 1) * 4);
+    if (new_tcA2B || new_data) {
+        if (T > capacity_tiles)
+            return fail(HSPMM_ERR_INVALID, "the grouped matrix has %u tiles, the output arrays hold %u", T, capacity_tiles);
+        if (new_tcA2B && T) std::memcpy(new_tcA2B, tcA2B, size_t(T) * cw * 4);
+        if (new_data && T) std::memcpy(new_data, d, size_t(T) * 8u * cw * elem);
+    }
+    return HSPMM_OK;
 }
 
 int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,

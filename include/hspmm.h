@@ -122,6 +122,24 @@ int hspmm_set_kernel_mode(int mode);
  * as zeros, wherever that saves work. */
 int hspmm_set_window_pairing(int mode);
 
+/* No reference counterpart; host only (no device needed).  The grouping that the
+ * LDS-staging kernels built on the 16-bit MFMA apply to their copy of the
+ * matrix, for tests and for sizing: adjacent windows are merged into units of up
+ * to max_windows (1, 2 or 4) windows that carry the union of their column lists
+ * wherever that saves steps of 32 columns inside panels of 256 columns (a step of
+ * three or four windows counted as 1.25).  Outputs, each optional: the groups
+ * (first window and window count; at most eff_row_windows of them), the tile
+ * offsets of the rewritten matrix (eff_row_windows + 1 words), its tile count,
+ * and its tcA2B / data arrays when they fit capacity_tiles tiles
+ * (HSPMM_ERR_INVALID otherwise; *new_total_tiles then says how many are needed).
+ * All windows of a group carry the same column list; added entries are zeros. */
+int hspmm_panel_units_preview(int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows, uint32_t total_tiles,
+                              const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
+                              const uint32_t *rowIdx, uint32_t max_windows, uint32_t *n_groups,
+                              uint32_t *group_first, uint32_t *group_count, uint32_t *new_rowOffset,
+                              uint32_t *new_total_tiles, uint32_t capacity_tiles, uint32_t *new_tcA2B,
+                              void *new_data);
+
 typedef struct {
     uint32_t rows, cols, eff_row_windows, total_tiles;
     int32_t  dtype;
