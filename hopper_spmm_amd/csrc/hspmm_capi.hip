@@ -1121,6 +1121,8 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         forced_units = units == 13 ? 12 : units;
         if (wide) { units = 13; forced_units = std::min(forced_units, 12); }
     }
+    if (const char *e = std::getenv("HSPMM_PANEL_UNITS_PER_GROUP"))      // fewer units than the shape has consumer waves
+        forced_units = std::max(1, std::min(std::atoi(e), units == 13 ? 12 : units));
     // (units of up to four windows: eight consumer waves with twice the accumulators)
     const int max_units = pl.G == 4 ? 8 : units == 13 ? 12 : units;
     if (forced_units) forced_units = std::min(forced_units, max_units);
