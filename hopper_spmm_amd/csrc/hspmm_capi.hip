@@ -18,6 +18,7 @@
 #include "../../include/hspmm.h"
 #include "hspmm_device.h"
 #include "partition.hpp"
+#include "host_parallel.hpp"
 
 namespace {
 
@@ -309,20 +310,22 @@ std::vector<uint32_t> lane_order_wide_steps(const StepStream &st, const uint32_t
     const uint16_t *halves = static_cast<const uint16_t *>(data);   // a step of a window is 8 x 32 halves
     const size_t step_words = st.G == 4 ? 512u : 256u;
     std::vector<uint32_t> out(size_t(st.n_steps) * step_words, 0u);
-    for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
-        const uint32_t w0 = st.unitWindow[u];
-        const uint32_t nwin = (st.unitRow[u] & 3u) + 1u;
-        for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
-            uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * step_words);
-            for (uint32_t w = 0; w < nwin; ++w) {
-                const uint16_t *src = halves + size_t(rowOffset[w0 + w] + i) * 256u;
-                uint16_t *half = dst + (w >> 1) * 512u;
-                for (uint32_t r = 0; r < 8; ++r)
-                    for (uint32_t g = 0; g < 4; ++g)
-                        std::memcpy(half + ((g * 16u + 8u * (w & 1u) + r) * 8u), src + r * 32u + 8u * g, 16);
+    hspmm_host::parallel_blocks(st.unitRow.size(), 16, [&](size_t ub, size_t ue) {
+        for (size_t u = ub; u < ue; ++u) {
+            const uint32_t w0 = st.unitWindow[u];
+            const uint32_t nwin = (st.unitRow[u] & 3u) + 1u;
+            for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
+                uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * step_words);
+                for (uint32_t w = 0; w < nwin; ++w) {
+                    const uint16_t *src = halves + size_t(rowOffset[w0 + w] + i) * 256u;
+                    uint16_t *half = dst + (w >> 1) * 512u;
+                    for (uint32_t r = 0; r < 8; ++r)
+                        for (uint32_t g = 0; g < 4; ++g)
+                            std::memcpy(half + ((g * 16u + 8u * (w & 1u) + r) * 8u), src + r * 32u + 8u * g, 16);
+                }
             }
         }
-    }
+    });
     return out;
 }
 
@@ -351,25 +354,27 @@ std::vector<uint32_t> lane_order_split_steps(const StepStream &st, const uint32_
     const float *vals = static_cast<const float *>(data);            // a step of a window is 8 x 32 floats
     const size_t step_words = st.G == 4 ? 1024u : 512u;
     std::vector<uint32_t> out(size_t(st.n_steps) * step_words, 0u);
-    for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
-        const uint32_t w0 = st.unitWindow[u];
-        const uint32_t nwin = (st.unitRow[u] & 3u) + 1u;
-        for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
-            uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * step_words);
-            for (uint32_t w = 0; w < nwin; ++w) {
-                const float *src = vals + size_t(rowOffset[w0 + w] + i) * 256u;
-                uint16_t *half = dst + (w >> 1) * 1024u;
-                for (uint32_t r = 0; r < 8; ++r)
-                    for (uint32_t g = 0; g < 4; ++g)
-                        for (uint32_t c = 0; c < 8; ++c) {
-                            const uint32_t sp = split_bf16_host(src[r * 32u + 8u * g + c]);
-                            uint16_t *lane = half + (g * 16u + 8u * (w & 1u) + r) * 16u;
-                            lane[c] = uint16_t(sp & 0xFFFFu);
-                            lane[8 + c] = uint16_t(sp >> 16);
-                        }
+    hspmm_host::parallel_blocks(st.unitRow.size(), 16, [&](size_t ub, size_t ue) {
+        for (size_t u = ub; u < ue; ++u) {
+            const uint32_t w0 = st.unitWindow[u];
+            const uint32_t nwin = (st.unitRow[u] & 3u) + 1u;
+            for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
+                uint16_t *dst = reinterpret_cast<uint16_t *>(out.data() + size_t(st.unitOffset[u] + i) * step_words);
+                for (uint32_t w = 0; w < nwin; ++w) {
+                    const float *src = vals + size_t(rowOffset[w0 + w] + i) * 256u;
+                    uint16_t *half = dst + (w >> 1) * 1024u;
+                    for (uint32_t r = 0; r < 8; ++r)
+                        for (uint32_t g = 0; g < 4; ++g)
+                            for (uint32_t c = 0; c < 8; ++c) {
+                                const uint32_t sp = split_bf16_host(src[r * 32u + 8u * g + c]);
+                                uint16_t *lane = half + (g * 16u + 8u * (w & 1u) + r) * 16u;
+                                lane[c] = uint16_t(sp & 0xFFFFu);
+                                lane[8 + c] = uint16_t(sp >> 16);
+                            }
+                }
             }
         }
-    }
+    });
     return out;
 }
 
@@ -419,37 +424,43 @@ bool merge_groups(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, u
         return true;
     };
     // the column list of the merged group (all windows of a group carry their group's list)
-    std::vector<uint32_t> merged;
-    auto merged_list = [&](uint32_t wa, uint32_t wb) {
+    auto merged_list = [&](uint32_t wa, uint32_t wb, std::vector<uint32_t> &merged) {
         const uint32_t *a = tcA2B + size_t(rowOffset[wa]) * cw, *b = tcA2B + size_t(rowOffset[wb]) * cw;
         const uint32_t na = real_ids(wa), nb = real_ids(wb);
         if (na == nb && std::memcmp(a, b, size_t(na) * 4) == 0) { merged.assign(a, a + na); return; }
         merged.resize(size_t(na) + nb);
         merged.resize(size_t(std::set_union(a, a + na, b, b + nb, merged.begin()) - merged.begin()));
     };
-    // first pass: which groups join their successor, and the new tile counts
+    // first pass: which groups could join their successor (all candidates, in parallel), then the
+    // greedy choice from the top, and the new tile counts
     const size_t NG = first.size();
-    std::vector<uint8_t> join(NG, 0);
-    std::vector<uint32_t> tiles(W);
+    std::vector<uint8_t> can(NG, 0), join(NG, 0);
+    std::vector<uint32_t> union_tiles(NG, 0u), tiles(W);
+    hspmm_host::parallel_blocks(NG - 1, 256, [&](size_t gb, size_t ge) {
+        std::vector<uint32_t> merged;
+        for (size_t g = gb; g < ge; ++g) {
+            const uint32_t wa = first[g], wb = first[g + 1], nw = count[g] + count[g + 1];
+            if (rowIdx[wb] != rowIdx[wa] + HSPMM_ROW_WINDOW * count[g] || nw > max_windows) continue;
+            const uint32_t *a = tcA2B + size_t(rowOffset[wa]) * cw, *b = tcA2B + size_t(rowOffset[wb]) * cw;
+            const uint32_t na = real_ids(wa), nb = real_ids(wb);
+            const bool same = na == nb && std::memcmp(a, b, size_t(na) * 4) == 0;
+            if (!same && (!ascending(a, na) || !ascending(b, nb))) continue;
+            merged_list(wa, wb, merged);
+            const uint32_t nu = uint32_t(merged.size());
+            const double cost = nw > 2 ? wide_cost : 1.0;
+            if (same || cost * double(panel_steps(merged.data(), nu)) < double(panel_steps(a, na) + panel_steps(b, nb))) {
+                can[g] = 1;
+                union_tiles[g] = (nu + cw - 1) / cw;
+            }
+        }
+    });
     bool any = false;
     for (uint32_t w = 0; w < W; ++w) tiles[w] = rowOffset[w + 1] - rowOffset[w];
     for (size_t g = 0; g + 1 < NG;) {
-        const uint32_t wa = first[g], wb = first[g + 1], nw = count[g] + count[g + 1];
-        if (rowIdx[wb] != rowIdx[wa] + HSPMM_ROW_WINDOW * count[g] || nw > max_windows) { ++g; continue; }
-        const uint32_t *a = tcA2B + size_t(rowOffset[wa]) * cw, *b = tcA2B + size_t(rowOffset[wb]) * cw;
-        const uint32_t na = real_ids(wa), nb = real_ids(wb);
-        const bool same = na == nb && std::memcmp(a, b, size_t(na) * 4) == 0;
-        if (!same && (!ascending(a, na) || !ascending(b, nb))) { ++g; continue; }
-        merged_list(wa, wb);
-        const uint32_t nu = uint32_t(merged.size());
-        const double cost = nw > 2 ? wide_cost : 1.0;
-        if (same || cost * double(panel_steps(merged.data(), nu)) < double(panel_steps(a, na) + panel_steps(b, nb))) {
-            join[g] = 1; any = true;
-            for (uint32_t w = wa; w < wa + nw; ++w) tiles[w] = (nu + cw - 1) / cw;
-            g += 2;
-        } else {
-            ++g;
-        }
+        if (!can[g]) { ++g; continue; }
+        join[g] = 1; any = true;
+        for (uint32_t w = first[g]; w < first[g] + count[g] + count[g + 1]; ++w) tiles[w] = union_tiles[g];
+        g += 2;
     }
     if (!any) return false;
     out.rowOffset.assign(size_t(W) + 1, 0u);
@@ -473,24 +484,30 @@ bool merge_groups(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, u
         }
     };
     out_first.clear(); out_count.clear();
+    std::vector<uint32_t> second;                               // first window of the group that joined, or IDX_MAX
     for (size_t g = 0; g < NG; ++g) {
         out_first.push_back(first[g]);
-        if (join[g]) {
-            const uint32_t wa = first[g], nw = count[g] + count[g + 1];
-            merged_list(wa, first[g + 1]);
-            for (uint32_t w = wa; w < wa + nw; ++w) spread(w, merged.data(), uint32_t(merged.size()));
-            out_count.push_back(nw);
-            ++g;
-        } else {
-            for (uint32_t w = first[g]; w < first[g] + count[g]; ++w) {
-                std::memcpy(out.tcA2B.data() + size_t(out.rowOffset[w]) * cw, tcA2B + size_t(rowOffset[w]) * cw,
-                            size_t(tiles[w]) * cw * 4);
-                std::memcpy(out.data.data() + size_t(out.rowOffset[w]) * tile_bytes, src + size_t(rowOffset[w]) * tile_bytes,
-                            size_t(tiles[w]) * tile_bytes);
-            }
-            out_count.push_back(count[g]);
-        }
+        out_count.push_back(join[g] ? count[g] + count[g + 1] : count[g]);
+        second.push_back(join[g] ? first[g + 1] : HSPMM_IDX_MAX);
+        if (join[g]) ++g;
     }
+    hspmm_host::parallel_blocks(out_first.size(), 64, [&](size_t gb, size_t ge) {
+        std::vector<uint32_t> merged;
+        for (size_t g = gb; g < ge; ++g) {
+            const uint32_t wa = out_first[g], nw = out_count[g];
+            if (second[g] != HSPMM_IDX_MAX) {
+                merged_list(wa, second[g], merged);
+                for (uint32_t w = wa; w < wa + nw; ++w) spread(w, merged.data(), uint32_t(merged.size()));
+            } else {
+                for (uint32_t w = wa; w < wa + nw; ++w) {
+                    std::memcpy(out.tcA2B.data() + size_t(out.rowOffset[w]) * cw, tcA2B + size_t(rowOffset[w]) * cw,
+                                size_t(tiles[w]) * cw * 4);
+                    std::memcpy(out.data.data() + size_t(out.rowOffset[w]) * tile_bytes,
+                                src + size_t(rowOffset[w]) * tile_bytes, size_t(tiles[w]) * tile_bytes);
+                }
+            }
+        }
+    });
     return true;
 }
 
@@ -590,74 +607,93 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     const uint32_t U = uint32_t(st.unitRow.size());
     const uint32_t T = rowOffset[W];
     const size_t es = p->elem, src_tile_bytes = size_t(8) * cw * es, tile_bytes = size_t(8) * rw * es;
+    // Two passes over the windows, both on all cores: the steps every window gets, then the steps.
     std::vector<uint32_t> rt_rowOffset(size_t(W) + 1, 0u), rt_ids, rt_panel;
     std::vector<uint8_t> rt_data;
-    rt_ids.reserve(size_t(T) * cw * 5 / 4);
-    rt_panel.reserve(size_t(T) * 5 / 4);
-    rt_data.reserve(size_t(T) * src_tile_bytes * 5 / 4);
     const uint8_t *src_data = static_cast<const uint8_t *>(data);
-    for (uint32_t w = 0; w < W; ++w) {
-        const uint32_t t0 = rowOffset[w], t1 = rowOffset[w + 1];
-        const uint32_t *col = tcA2B + size_t(t0) * cw;
-        uint32_t nreal = (t1 - t0) * cw;
+    auto real_columns = [&](uint32_t w) {
+        const uint32_t *col = tcA2B + size_t(rowOffset[w]) * cw;
+        uint32_t nreal = (rowOffset[w + 1] - rowOffset[w]) * cw;
         while (nreal && col[nreal - 1] == HSPMM_IDX_MAX) --nreal;
-        uint32_t i = 0, tiles = 0, last_pn = 0;
-        while (i < nreal) {
-            const uint32_t pn = col[i] / KP, a = i;
-            while (i < nreal && col[i] / KP == pn) ++i;
-            while (tiles && pn - last_pn > kMaxJump) {           // all-zero step that only carries the jump
-                last_pn += kMaxJump;
-                rt_ids.resize(rt_ids.size() + rw, 0u);
-                rt_data.resize(rt_data.size() + tile_bytes, 0);
-                rt_panel.push_back(last_pn);
-                ++tiles;
+        return nreal;
+    };
+    const size_t windows_per_worker = std::max<size_t>(1, (size_t(1) << 14) / std::max<uint32_t>(1u, T / W));
+    hspmm_host::parallel_blocks(W, windows_per_worker, [&](size_t wb, size_t we) {
+        for (size_t w = wb; w < we; ++w) {
+            const uint32_t *col = tcA2B + size_t(rowOffset[w]) * cw;
+            const uint32_t nreal = real_columns(uint32_t(w));
+            uint32_t i = 0, tiles = 0, last_pn = 0;
+            while (i < nreal) {
+                const uint32_t pn = col[i] / KP, a = i;
+                while (i < nreal && col[i] / KP == pn) ++i;
+                while (tiles && pn - last_pn > kMaxJump) { last_pn += kMaxJump; ++tiles; }
+                tiles += (i - a + rw - 1) / rw;
+                last_pn = pn;
             }
-            const uint32_t nt = (i - a + rw - 1) / rw;
-            const size_t id_at = rt_ids.size(), data_at = rt_data.size();
-            rt_ids.resize(id_at + size_t(nt) * rw);
-            rt_data.resize(data_at + size_t(nt) * tile_bytes, 0);
-            rt_panel.resize(rt_panel.size() + nt, pn);
-            for (uint32_t tl = 0; tl < nt; ++tl) {
-                // The columns of the step.  16-bit types: one LDS instruction reads, in each block of 16
-                // lanes, the rows of four consecutive columns of the step (block g, instruction h: columns
-                // 8g + 4h .. + 3), the LDS serves two blocks (g = 0, 1 or g = 2, 3) at a time, and rows
-                // whose numbers differ mod 8 lie in different banks: columns ordered by row number mod 8
-                // (stable) and dealt out over the four sets of eight that are read together put
-                // different remainders into a set wherever the step has them.
-                const uint32_t first = a + tl * rw, n = std::min(rw, i - first);
-                uint32_t order[32];
-                if (rw == 32) {
-                    uint32_t sorted[32], m = 0;
-                    for (uint32_t res = 0; res < 8; ++res)
-                        for (uint32_t k = 0; k < rw; ++k) {
-                            // padding takes the row of the last real column (its tile column stays zero)
-                            const uint32_t c = col[first + std::min(k, n - 1)] - pn * KP;
-                            if ((c & 7u) == res) sorted[m++] = k;
-                        }
-                    for (uint32_t k = 0; k < rw; ++k) {
-                        const uint32_t set = k % 4, e = k / 4;          // set = 2 * (g / 2) + h
-                        const uint32_t g = 2 * (set / 2) + e / 4, h = set % 2;
-                        order[8 * g + 4 * h + e % 4] = sorted[k];
-                    }
-                } else {
-                    for (uint32_t k = 0; k < rw; ++k) order[k] = k;
-                }
-                uint8_t *dt_tile = rt_data.data() + data_at + size_t(tl) * tile_bytes;
-                for (uint32_t k = 0; k < rw; ++k) {
-                    const uint32_t from = order[k];
-                    const uint32_t srci = first + std::min(from, n - 1);
-                    rt_ids[id_at + size_t(tl) * rw + k] = col[srci] - pn * KP;      // row inside the panel
-                    if (from >= n) continue;
-                    const uint8_t *st_tile = src_data + size_t(t0 + srci / cw) * src_tile_bytes;
-                    for (uint32_t r = 0; r < 8; ++r)
-                        std::memcpy(dt_tile + (size_t(r) * rw + k) * es, st_tile + (size_t(r) * cw + srci % cw) * es, es);
-                }
-            }
-            tiles += nt;
-            last_pn = pn;
+            rt_rowOffset[w + 1] = tiles;
         }
-        rt_rowOffset[w + 1] = rt_rowOffset[w] + tiles;
-    }
+    });
+    for (uint32_t w = 0; w < W; ++w) rt_rowOffset[w + 1] += rt_rowOffset[w];
+    const size_t RT = rt_rowOffset[W];
+    rt_ids.assign(RT * rw, 0u);
+    rt_panel.assign(RT, 0u);
+    rt_data.assign(RT * tile_bytes, 0);
+    hspmm_host::parallel_blocks(W, windows_per_worker, [&](size_t wb, size_t we) {
+        for (size_t w = wb; w < we; ++w) {
+            const uint32_t t0 = rowOffset[w];
+            const uint32_t *col = tcA2B + size_t(t0) * cw;
+            const uint32_t nreal = real_columns(uint32_t(w));
+            uint32_t i = 0, last_pn = 0;
+            size_t at = rt_rowOffset[w];                             // next step of the window
+            while (i < nreal) {
+                const uint32_t pn = col[i] / KP, a = i;
+                while (i < nreal && col[i] / KP == pn) ++i;
+                while (at > rt_rowOffset[w] && pn - last_pn > kMaxJump) {   // all-zero step that only carries the jump
+                    last_pn += kMaxJump;
+                    rt_panel[at++] = last_pn;
+                }
+                const uint32_t nt = (i - a + rw - 1) / rw;
+                for (uint32_t tl = 0; tl < nt; ++tl, ++at) {
+                    rt_panel[at] = pn;
+                    // The columns of the step.  16-bit types: one LDS instruction reads, in each block of 16
+                    // lanes, the rows of four consecutive columns of the step (block g, instruction h: columns
+                    // 8g + 4h .. + 3), the LDS serves two blocks (g = 0, 1 or g = 2, 3) at a time, and rows
+                    // whose numbers differ mod 8 lie in different banks: columns ordered by row number mod 8
+                    // (stable) and dealt out over the four sets of eight that are read together put
+                    // different remainders into a set wherever the step has them.
+                    const uint32_t first_col = a + tl * rw, n = std::min(rw, i - first_col);
+                    uint32_t order[32];
+                    if (rw == 32) {
+                        uint32_t sorted[32], m = 0;
+                        for (uint32_t res = 0; res < 8; ++res)
+                            for (uint32_t k = 0; k < rw; ++k) {
+                                // padding takes the row of the last real column (its tile column stays zero)
+                                const uint32_t c = col[first_col + std::min(k, n - 1)] - pn * KP;
+                                if ((c & 7u) == res) sorted[m++] = k;
+                            }
+                        for (uint32_t k = 0; k < rw; ++k) {
+                            const uint32_t set = k % 4, e = k / 4;          // set = 2 * (g / 2) + h
+                            const uint32_t g = 2 * (set / 2) + e / 4, h = set % 2;
+                            order[8 * g + 4 * h + e % 4] = sorted[k];
+                        }
+                    } else {
+                        for (uint32_t k = 0; k < rw; ++k) order[k] = k;
+                    }
+                    uint8_t *dt_tile = rt_data.data() + at * tile_bytes;
+                    for (uint32_t k = 0; k < rw; ++k) {
+                        const uint32_t from = order[k];
+                        const uint32_t srci = first_col + std::min(from, n - 1);
+                        rt_ids[at * rw + k] = col[srci] - pn * KP;      // row inside the panel
+                        if (from >= n) continue;
+                        const uint8_t *st_tile = src_data + size_t(t0 + srci / cw) * src_tile_bytes;
+                        for (uint32_t r = 0; r < 8; ++r)
+                            std::memcpy(dt_tile + (size_t(r) * rw + k) * es, st_tile + (size_t(r) * cw + srci % cw) * es, es);
+                    }
+                }
+                last_pn = pn;
+            }
+        }
+    });
     // the units with the re-tiled step counts
     StepStream ps;
     ps.G = st.G; ps.unitRow = st.unitRow; ps.unitWindow = st.unitWindow; ps.n_paired = st.n_paired; ps.n_wide = st.n_wide;
@@ -680,34 +716,36 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     std::vector<uint32_t> ids(size_t(ps.n_steps) * id_words);
     // fp32 single windows run through the 4x4x1 instruction, which wants row offsets (see Fp32Quad)
     const bool quad = p->dtype == HSPMM_TF32 && !split && st.G == 1;
-    for (uint32_t u = 0; u < U; ++u) {
-        const uint32_t t0 = rt_rowOffset[st.unitWindow[u]], n = ps.unitOffset[u + 1] - ps.unitOffset[u];
-        uint32_t *po = poff.data() + size_t(u) * (NP + 1);
-        uint32_t at = 0;
-        for (uint32_t pn = 0; pn <= NP; ++pn) {
-            while (at < n && rt_panel[t0 + at] < pn) ++at;
-            po[pn] = ps.unitOffset[u] + at;
-        }
-        for (uint32_t i = 0; i < n; ++i) {
-            const uint32_t *src = rt_ids.data() + size_t(t0 + i) * rw;
-            uint32_t *dst = ids.data() + size_t(ps.unitOffset[u] + i) * id_words;
-            const uint32_t jump = i ? rt_panel[t0 + i] - rt_panel[t0 + i - 1] : 0u;     // <= kMaxJump by construction
-            step_panel[ps.unitOffset[u] + i] = rt_panel[t0 + i];
-            if (rw == 32) {
-                for (uint32_t l = 0; l < 64; ++l) {
-                    const uint32_t c0 = 8u * (l >> 4) + ((l & 15u) >> 2);
-                    dst[l] = jump | (src[c0] * 9u) << 4 | (src[c0 + 4] * 9u) << 16;
+    hspmm_host::parallel_blocks(U, 16, [&](size_t ub, size_t ue) {
+        for (size_t u = ub; u < ue; ++u) {
+            const uint32_t t0 = rt_rowOffset[st.unitWindow[u]], n = ps.unitOffset[u + 1] - ps.unitOffset[u];
+            uint32_t *po = poff.data() + size_t(u) * (NP + 1);
+            uint32_t at = 0;
+            for (uint32_t pn = 0; pn <= NP; ++pn) {
+                while (at < n && rt_panel[t0 + at] < pn) ++at;
+                po[pn] = ps.unitOffset[u] + at;
+            }
+            for (uint32_t i = 0; i < n; ++i) {
+                const uint32_t *src = rt_ids.data() + size_t(t0 + i) * rw;
+                uint32_t *dst = ids.data() + size_t(ps.unitOffset[u] + i) * id_words;
+                const uint32_t jump = i ? rt_panel[t0 + i] - rt_panel[t0 + i - 1] : 0u;     // <= kMaxJump by construction
+                step_panel[ps.unitOffset[u] + i] = rt_panel[t0 + i];
+                if (rw == 32) {
+                    for (uint32_t l = 0; l < 64; ++l) {
+                        const uint32_t c0 = 8u * (l >> 4) + ((l & 15u) >> 2);
+                        dst[l] = jump | (src[c0] * 9u) << 4 | (src[c0 + 4] * 9u) << 16;
+                    }
+                    continue;
                 }
-                continue;
-            }
-            for (uint32_t g = 0; g < 4; ++g) {
-                if (quad)   // byte offsets of rows g and g + 4 inside the panel image; the jump in bits 0..3 of word 0
-                    dst[g] = (src[g] << 8 | (g == 0 ? jump : 0u)) | (src[g + 4] << 8) << 16;
-                else
-                    dst[g] = (src[g] | src[g + 4] << 7) | jump << 28;
+                for (uint32_t g = 0; g < 4; ++g) {
+                    if (quad)   // byte offsets of rows g and g + 4 inside the panel image; the jump in bits 0..3 of word 0
+                        dst[g] = (src[g] << 8 | (g == 0 ? jump : 0u)) | (src[g + 4] << 8) << 16;
+                    else
+                        dst[g] = (src[g] | src[g + 4] << 7) | jump << 28;
+                }
             }
         }
-    }
+    });
     hspmm_plan::Panel &pl = p->panel;
     int rc;
     if ((rc = upload(&pl.d_poff, poff.data(), poff.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }

@@ -21,6 +21,7 @@
 #include <vector>
 
 #include "../../include/hspmm.h"
+#include "host_parallel.hpp"
 
 namespace hspmm_host {
 
@@ -62,30 +63,6 @@ static uint16_t float_to_bf16_bits(float f)
     std::memcpy(&x, &f, 4);
     if ((x & 0x7FFFFFFFu) > 0x7F800000u) return uint16_t((x >> 16) | 0x0040u);    // NaN stays NaN (quiet)
     return uint16_t((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
-}
-
-static unsigned worker_count(size_t work_items, size_t min_per_worker)
-{
-    unsigned hw = std::thread::hardware_concurrency();
-    if (hw == 0) hw = 1;
-    if (hw > 16) hw = 16;
-    size_t by_work = work_items / (min_per_worker ? min_per_worker : 1);
-    if (by_work < 1) by_work = 1;
-    return unsigned(std::min<size_t>(hw, by_work));
-}
-
-template <class F>
-static void parallel_blocks(size_t n, size_t min_per_worker, F &&fn)
-{
-    const unsigned nw = worker_count(n, min_per_worker);
-    if (nw <= 1) { fn(size_t(0), n); return; }
-    std::vector<std::thread> th;
-    th.reserve(nw);
-    for (unsigned i = 0; i < nw; ++i) {
-        const size_t b = n * i / nw, e = n * (i + 1) / nw;
-        th.emplace_back([&fn, b, e] { fn(b, e); });
-    }
-    for (auto &t : th) t.join();
 }
 
 // ---------------------------------------------------------------------------
