@@ -710,9 +710,9 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     std::vector<uint32_t> poff(size_t(U) * (NP + 1)), step_panel(ps.n_steps ? ps.n_steps : 1, 0u);
     // fp32, per step four words: word g packs the panel rows quarter-wave g reads (ids g and g + 4, 7 bits
     // each) and in bits 28..31 the panels the step lies behind its predecessor.
-    // 16-bit types, per step one word per lane (g = l / 16, i = l % 16): 9 x the panel rows of columns
-    // 8g + i / 4 (bits 4..14) and 8g + 4 + i / 4 (bits 16..26); bits 0..3: the panel count.
-    const uint32_t id_words = rw == 32 ? 64u : 4u;
+    // 16-bit types, per step one word per four lanes (word q = l / 4, g = q / 4): 9 x the panel rows of
+    // columns 8g + q % 4 (bits 4..15) and 8g + 4 + q % 4 (bits 16..27); bits 0..3: the panel count.
+    const uint32_t id_words = rw == 32 ? 16u : 4u;
     std::vector<uint32_t> ids(size_t(ps.n_steps) * id_words);
     // fp32 single windows run through the 4x4x1 instruction, which wants row offsets (see Fp32Quad)
     const bool quad = p->dtype == HSPMM_TF32 && !split && st.G == 1;
@@ -731,9 +731,9 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
                 const uint32_t jump = i ? rt_panel[t0 + i] - rt_panel[t0 + i - 1] : 0u;     // <= kMaxJump by construction
                 step_panel[ps.unitOffset[u] + i] = rt_panel[t0 + i];
                 if (rw == 32) {
-                    for (uint32_t l = 0; l < 64; ++l) {
-                        const uint32_t c0 = 8u * (l >> 4) + ((l & 15u) >> 2);
-                        dst[l] = jump | (src[c0] * 9u) << 4 | (src[c0 + 4] * 9u) << 16;
+                    for (uint32_t q = 0; q < 16; ++q) {
+                        const uint32_t c0 = 8u * (q >> 2) + (q & 3u);
+                        dst[q] = jump | (src[c0] * 9u) << 4 | (src[c0 + 4] * 9u) << 16;
                     }
                     continue;
                 }

@@ -148,9 +148,9 @@ struct PanelOps {
 // tile copy) run every second operand against two first operands: half the LDS reads per
 // row, which is what binds these kernels, with eight consumer waves of twice the
 // accumulators.
-//   ids per step: 64 words, one per lane: bits 4..15 = 9 x (panel row of column
-//     8g + i / 4), bits 16..27 = 9 x (panel row of column 8g + 4 + i / 4) (i = l % 16;
-//     x 32 = byte offset in the image); bits 0..3: the panel jump.
+//   ids per step: 16 words, one per four lanes (word l / 4): bits 4..15 = 9 x (panel row
+//     of column 8g + i / 4), bits 16..27 = 9 x (panel row of column 8g + 4 + i / 4)
+//     (i = l % 16; x 32 = byte offset in the image); bits 0..3: the panel jump.
 typedef short tr16x4 __attribute__((ext_vector_type(4)));
 typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
 
@@ -172,7 +172,7 @@ struct Fp16Tr {
         {
             g = lane >> 4; j = lane & 15u;
             a_src = reinterpret_cast<const uint32_t *>(tiles) + lane * 4u;
-            idx_src = ids + lane;
+            idx_src = ids + (lane >> 2);           // four neighbouring lanes read one word
         }
     };
     // Window W0 of the unit is held by quarter-waves 2 (W0 % 2) and 2 (W0 % 2) + 1 of accumulators
@@ -223,7 +223,7 @@ struct PanelOps<Fp16Tr<G_, BF>> {
     struct AVec { u32x4 r[kFour ? 2 : 1]; };
     __device__ static __forceinline__ Idx load_idx(const typename TT::Lane &L, const uint32_t *, uint32_t step)
     {
-        return L.idx_src[size_t(step) * 64u];
+        return L.idx_src[size_t(step) * 16u];
     }
     __device__ static __forceinline__ AVec load_a(const typename TT::Lane &L, uint32_t step)
     {
@@ -285,7 +285,7 @@ struct Fp32Split {
         {
             g = lane >> 4; j = lane & 15u;
             a_src = reinterpret_cast<const uint32_t *>(tiles) + lane * 8u;
-            idx_src = ids + lane;
+            idx_src = ids + (lane >> 2);           // four neighbouring lanes read one word
         }
     };
     template <int W0>
@@ -356,7 +356,7 @@ struct PanelOps<Fp32Split<G_>> {
     struct AVec { u32x8 r[kFour ? 2 : 1]; };
     __device__ static __forceinline__ Idx load_idx(const typename TT::Lane &L, const uint32_t *, uint32_t step)
     {
-        return L.idx_src[size_t(step) * 64u];
+        return L.idx_src[size_t(step) * 16u];
     }
     __device__ static __forceinline__ AVec load_a(const typename TT::Lane &L, uint32_t step)
     {
