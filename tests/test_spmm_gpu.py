@@ -569,6 +569,42 @@ def test_plan_reuse_is_deterministic(torch_cuda, hs, oracle):
     plan.close()
 
 
+def test_plans_on_different_streams_do_not_disturb_each_other(torch_cuda, hs, oracle):
+    """Different plans may run at the same time: each owns its scratch memory.  Three plans
+    (cut units with partial sums, the LDS-panel kernel with chunk sums, fp32 storage) are
+    launched round robin on three streams without waiting; every output must be bit-identical
+    to what the same plan gives alone."""
+    torch = torch_cuda
+    rng = np.random.default_rng(21)
+    cases = []
+    for dtype, dens, heavy, N in ((0, 0.003, (3, 200), 64), (2, 0.1, (), 128), (1, 0.1, (), 64)):
+        A = random_csr(rng, 400, 4000, dens, dtype, 0.1, heavy)
+        b = convert(hs, A)
+        hs.configure(producer_warp_group_num=16)
+        try:
+            plan = hs.Plan(b)
+        finally:
+            hs.configure()
+        B = make_b(rng, 4000, N, dtype)
+        alone = gpu_spmm(torch, hs, b, B, N, plan=plan)
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        assert_parity(alone, ref, mag, dtype, "alone, dtype %d" % dtype)
+        tt = torch.float32 if dtype == 1 else torch.int16
+        dB = torch.from_numpy(B if dtype == 1 else B.view(np.int16)).cuda()
+        dC = torch.empty((400, N), dtype=tt, device="cuda")
+        cases.append((plan, dB, dC, N, alone, dtype, torch.cuda.Stream()))
+    torch.cuda.synchronize()
+    for _ in range(20):
+        for plan, dB, dC, N, _, _, stream in cases:
+            plan.run(dB.data_ptr(), dC.data_ptr(), N, stream.cuda_stream)
+    torch.cuda.synchronize()
+    for plan, dB, dC, N, alone, dtype, _ in cases:
+        got = dC.cpu().numpy()
+        got = got if dtype == 1 else got.view(np.uint16)
+        assert np.array_equal(got, alone), "dtype %d" % dtype
+        plan.close()
+
+
 def test_run_captured_in_a_hip_graph_replays_correctly(torch_cuda, hs, oracle):
     """After one eager call (which sizes the plan's scratch memory) hspmm_run only
     launches kernels, so a stream capture records it; every replay, with eager work
