@@ -60,10 +60,15 @@ int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
 
 /* Replaces one launch of fp16_spmm_kernel (reference src/fp16.cu:256): computes
  * all of C = A*B for feature dimension N.  dB (cols x N) and dC (rows x N) are
- * DEVICE pointers, row-major, 4-byte aligned; every element of C is written
- * (rows without nonzeros become 0).  Asynchronous on `stream` (a hipStream_t,
- * NULL = default stream).  A plan owns scratch memory, so launches of one plan
- * must not overlap in time; different plans may run concurrently. */
+ * DEVICE pointers, row-major, aligned to the element size (the MFMA kernels want
+ * 4 bytes and an even N for the 16-bit types, the LDS-staging kernels 16 bytes;
+ * anything else runs through the all-shapes kernel); every element of C is
+ * written (rows without nonzeros become 0).  Asynchronous on `stream` (a
+ * hipStream_t, NULL = default stream).  A plan owns scratch memory, so launches
+ * of one plan must not overlap in time; different plans may run concurrently.
+ * The first call for a feature dimension may allocate that memory and build a
+ * second work partition; later calls with the same or a smaller N only launch
+ * kernels and can be captured in a HIP graph. */
 int hspmm_run(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stream);
 
 /* Replaces the warm-up + timed loop of fp16_spmm (reference src/fp16.cu:254-268,
