@@ -67,8 +67,8 @@ int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
  * hipStream_t, NULL = default stream).  A plan owns scratch memory, so launches
  * of one plan must not overlap in time; different plans may run concurrently.
  * The first call for a feature dimension may allocate that memory and build a
- * second work partition; later calls with the same or a smaller N only launch
- * kernels and can be captured in a HIP graph. */
+ * work partition for it; later calls with the same N only launch kernels and
+ * can be captured in a HIP graph. */
 int hspmm_run(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stream);
 
 /* Replaces the warm-up + timed loop of fp16_spmm (reference src/fp16.cu:254-268,
