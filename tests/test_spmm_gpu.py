@@ -479,17 +479,23 @@ def test_units_of_four_windows_are_chosen_for_large_pruned_matrices(torch_cuda, 
     assert info["n_panels"] > 0 and info["n_panel_paired_units"] > 0 and info["n_panel_wide_units"] == 0
 
 
-@pytest.mark.parametrize("seed", [11, 12, 13])
-def test_seeded_sweep_of_shapes_formats_and_kernel_choices(torch_cuda, hs, oracle, seed):
-    """150 seeded combinations per seed of element type, shape, density, empty and heavy rows,
+@pytest.mark.parametrize("seed,large", [(11, False), (12, False), (13, False), (14, True)])
+def test_seeded_sweep_of_shapes_formats_and_kernel_choices(torch_cuda, hs, oracle, seed, large):
+    """Seeded combinations (150 per seed; 80 for the sweep over larger shapes, whose matrices span
+    many column panels and several workgroups) of element type, shape, density, empty and heavy rows,
     kernel mode, window pairing, input format (plain / bitmap / grouped), prefetch depth,
     partition granularity and feature dimension, each compared with the oracle."""
     rng = np.random.default_rng(seed)
-    for case in range(150):
+    for case in range(80 if large else 150):
         dtype = int(rng.integers(0, 3))
-        rows = int(rng.choice([1, 7, 8, 9, 31, 64, 129, 300, 777]))
-        cols = int(rng.choice([1, 5, 16, 17, 127, 128, 129, 500, 2049, 6000]))
-        dens = float(rng.choice([0.002, 0.02, 0.1, 0.4, 0.9]))
+        if large:
+            rows = int(rng.choice([513, 1000, 2049, 4100]))
+            cols = int(rng.choice([255, 1025, 4097, 9000, 20001]))
+            dens = float(rng.choice([0.001, 0.01, 0.05, 0.2]))
+        else:
+            rows = int(rng.choice([1, 7, 8, 9, 31, 64, 129, 300, 777]))
+            cols = int(rng.choice([1, 5, 16, 17, 127, 128, 129, 500, 2049, 6000]))
+            dens = float(rng.choice([0.002, 0.02, 0.1, 0.4, 0.9]))
         erp = float(rng.choice([0.0, 0.3, 0.8]))
         heavy = tuple(int(x) for x in rng.integers(0, rows, int(rng.integers(0, 3)))) if rows > 8 else ()
         A = random_csr(rng, rows, cols, dens, dtype, erp, heavy)
@@ -498,7 +504,9 @@ def test_seeded_sweep_of_shapes_formats_and_kernel_choices(torch_cuda, hs, oracl
         fmt = int(rng.integers(0, 3))
         stages = int(rng.choice([0, 0, 1, 2, 4]))
         ranges_per_simd = int(rng.choice([0, 0, 1, 16]))
-        if mode >= 4:
+        if mode >= 4 and large:
+            N = int(rng.choice([64, 128, 320, 512])) if dtype == 1 else int(rng.choice([128, 256, 640, 1024]))
+        elif mode >= 4:
             N = int(rng.choice([64, 128, 192, 256, 384])) if dtype == 1 else int(rng.choice([128, 256, 384]))
         else:
             N = int(rng.choice([1, 2, 3, 8, 16, 24, 32, 40, 64, 96, 128, 136, 256, 320]))
