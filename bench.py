@@ -178,8 +178,12 @@ def main():
         "roofline": {"bound": "hbm", "achieved": bytes_alg / (main_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": bytes_alg / (main_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": traffic,
-                     "kernel": "spmm_mfma_kernel", "kernel_ms": main_ms, "fixup_kernel_ms": fix_ms,
+                     "kernel": {1: "spmm_scalar_kernel", 2: "spmm_mfma_kernel", 3: "spmm_panel_kernel"}.get(
+                         plan.info()["last_kernel_family"], "none"),
+                     "kernel_ms": main_ms, "fixup_kernel_ms": fix_ms,
                      "algorithmic_bytes": bytes_alg, "gather_bytes": bytes_gather,
+                     # every gathered B row counted every time it is gathered, for comparison with the HBM peak
+                     "gathered_gbps": bytes_gather / (main_ms * 1e-3) / 1e9,
                      "mfma_frac_of_peak_useful_flops": flops / (main_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[dt]},
         "reference_convention_ms": ref_conv_ms,
         # one call of the host-buffer interface (fp16_spmm): plan + upload, one launch, download of C

@@ -115,6 +115,7 @@ struct hspmm_plan {
     uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
     size_t arrive_words = 0;
     size_t fixed_bytes = 0;
+    uint32_t last_family = 0;           // kernel family of the last hspmm_run: 0 none yet, 1 all-shapes, 2 gather, 3 LDS-panel, 4 clear
 };
 
 namespace {
@@ -1229,6 +1230,7 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (p->W == 0) {
+        p->last_family = 4;
         HSPMM_HIP(hspmm::launch_fill_zero(dC, size_t(p->rows) * N * p->elem, s));
         return HSPMM_OK;
     }
@@ -1239,7 +1241,7 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
         // (a 16-bit matrix near the break-even is served as fast or faster by the gather kernels while
         // one wave of theirs covers all of N)
         const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 1.5 || N >= 256u;
-        if (pays && N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid);
+        if (pays && N % block_feat == 0 && !(align & 15u)) { p->last_family = 3; return run_panel(p, dB, dC, N, s, mid); }
     }
     const Choice c = choose_kernel(p, dB, dC, N);
     hspmm::KernelArgs ka{};
@@ -1247,9 +1249,11 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     ka.B = dB; ka.C = dC;
     ka.eff_windows = p->W; ka.rows = p->rows; ka.N = N;
     if (c.scalar) {
+        p->last_family = 1;
         HSPMM_HIP(hspmm::launch_spmm_scalar(p->dtype, ka, s));
         return HSPMM_OK;
     }
+    p->last_family = 2;
     ka.unitOffset = p->d_unitOffset; ka.unitRow = p->d_unitRow; ka.ids = p->d_ids; ka.tiles = p->d_tiles;
     ka.n_units = p->n_units;
     ka.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
@@ -1363,6 +1367,7 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_panel_units = p->panel.built ? p->panel.n_units : 0u;
     info->n_panel_paired_units = p->panel.built ? p->panel.n_paired : 0u;
     info->n_panel_wide_units = p->panel.built ? p->panel.n_wide : 0u;
+    info->last_kernel_family = p->last_family;
     return HSPMM_OK;
 }
 

@@ -160,6 +160,8 @@ typedef struct {
     uint32_t n_panel_units;     /* units of that stream: groups of up to four adjacent windows that share, or were given, one column list */
     uint32_t n_panel_paired_units;  /* of those: units of two or more windows */
     uint32_t n_panel_wide_units;    /* of those: units of three or four windows */
+    uint32_t last_kernel_family;    /* what the last hspmm_run launched: 0 nothing yet, 1 all-shapes kernel, 2 gather (MFMA) kernels,
+                                       3 LDS-staging kernels, 4 clear only (matrix without entries) */
 } hspmm_plan_info;
 
 /* No reference counterpart (the reference prints its statistics from main,

@@ -337,11 +337,13 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
                 got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
                 ref, mag = oracle_spmm(oracle, A, B, N)
                 assert_parity(got, ref, mag, dtype, "panel mode %d units %s chunks %s shape %s N=%d" % (mode, units, chunks, shape[:2], N))
+                assert plan.info()["last_kernel_family"] == 3          # the LDS-staging kernels did run
             # a feature dimension the panel kernels do not take falls back to the gather kernels
             B = make_b(rng, cols, 24, dtype)
             got = gpu_spmm(torch_cuda, hs, b, B, 24, plan=plan)
             ref, mag = oracle_spmm(oracle, A, B, 24)
             assert_parity(got, ref, mag, dtype, "panel plan, N=24")
+            assert plan.info()["last_kernel_family"] == 2
             plan.close()
         finally:
             hs.set_kernel_mode(0)
@@ -539,20 +541,29 @@ def test_unaligned_and_odd_feature_dims_use_the_all_shapes_kernel(torch_cuda, hs
     for dt in (0, 2):
         A = random_csr(rng, 90, 120, 0.1, dt, 0.2)
         b = convert(hs, A)
+        plan = hs.Plan(b)
         for N in (1, 3, 7, 33, 129):
             B = make_b(rng, 120, N, dt)
-            got = gpu_spmm(torch_cuda, hs, b, B, N)
+            got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
             ref, mag = oracle_spmm(oracle, A, B, N)
             assert_parity(got, ref, mag, dt, "%s odd N=%d" % (DT[dt], N))
+            assert plan.info()["last_kernel_family"] == 1              # the all-shapes kernel
+        got = gpu_spmm(torch_cuda, hs, b, make_b(rng, 120, 34, dt), 34, plan=plan)
+        assert plan.info()["last_kernel_family"] == 2                  # an even N: MFMA kernels again
+        plan.close()
 
 
 def test_matrix_without_entries_gives_zeros(torch_cuda, hs):
     for dt in (0, 1, 2):
         vt = np.float32 if dt == 1 else np.uint16
         b = hs.csr_to_btcf(21, 9, np.zeros(22, np.uint32), np.zeros(0, np.uint32), np.zeros(0, vt), dt)
+        plan = hs.Plan(b)
+        assert plan.info()["last_kernel_family"] == 0
         for N in (1, 5, 64):
-            got = gpu_spmm(torch_cuda, hs, b, np.ones((9, N), vt), N)
+            got = gpu_spmm(torch_cuda, hs, b, np.ones((9, N), vt), N, plan=plan)
             assert got.shape == (21, N) and not got.any()
+            assert plan.info()["last_kernel_family"] == 4              # nothing but the clear kernel
+        plan.close()
 
 
 def test_plan_reuse_is_deterministic(torch_cuda, hs, oracle):
