@@ -13,6 +13,7 @@ constexpr uint32_t kRangeWordsDev = 8u;
 constexpr uint32_t kRangeWords = kRangeWordsDev;
 constexpr uint32_t kFixWords = 4u;
 constexpr int kMaxWavesPerGroup = 4;
+constexpr int kAlignedGroupWaves = 8;          // waves of a workgroup that walks one whole unit (aligned partition)
 
 struct KernelArgs {
     // the four format arrays exactly as given (device copies), reference

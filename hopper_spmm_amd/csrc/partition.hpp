@@ -24,7 +24,8 @@ struct Range {
     uint32_t first_window;            // effective window holding tile_begin
     uint32_t head_slot, tail_slot;    // partial-sum slots (kNoSlot = none)
     uint32_t head_split, tail_split;  // index of the cut window's entry in Partition::split
-    uint32_t combine;                 // 1: the ranges of this range's group add their sums before they leave the chip
+    uint32_t combine;                 // 1: the ranges of this range's group add their sums before they leave the chip;
+                                      // 2: they are a whole window, which the group stores itself
 };
 
 struct SplitWindow {
@@ -153,6 +154,28 @@ inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t
             } else {
                 t = se;
             }
+        }
+    }
+    return P;
+}
+
+// Every window cut into `group` ranges of (almost) equal length, walked by the waves of one workgroup,
+// which add their sums among themselves and store the window: no slot and no second kernel.  For
+// matrices whose windows are all long; the caller makes sure every window has at least `group` tiles.
+inline Partition build_aligned_partition(uint32_t W, const uint32_t *rowOffset, uint32_t group)
+{
+    Partition P;
+    P.ranges.resize(size_t(W) * group);
+    for (uint32_t w = 0; w < W; ++w) {
+        const uint64_t ws = rowOffset[w], n = rowOffset[w + 1] - rowOffset[w];
+        for (uint32_t k = 0; k < group; ++k) {
+            Range &g = P.ranges[size_t(w) * group + k];
+            g.tile_begin = uint32_t(ws + n * k / group);
+            g.tile_end = uint32_t(ws + n * (k + 1) / group);
+            g.first_window = w;
+            g.head_slot = g.tail_slot = kNoSlot;
+            g.head_split = g.tail_split = kNoSlot;
+            g.combine = 2;
         }
     }
     return P;

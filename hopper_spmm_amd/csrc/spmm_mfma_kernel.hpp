@@ -35,6 +35,7 @@
 //     ids, to the real column in front of them; their tile column is all zero.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <algorithm>
 #pragma once
 #include "hspmm_device.h"
 
@@ -474,8 +475,28 @@ struct UnitWalk {
     uint32_t seg_start, seg_end;   // part of the span inside this wave's range
 };
 
-template <class TT, int P, bool NARROW>
-__global__ __launch_bounds__(kMaxWavesPerGroup * 64, (P <= 4 ? 4 : 2))
+// Windows of a unit: the low bits of its row word hold the count less one (1: a pair; the
+// LDS-panel kernels also have units of three and four windows).
+template <class TT>
+__device__ __forceinline__ uint32_t unit_windows(const uint32_t row_word)
+{
+    return TT::G > 1 ? (row_word & 3u) + 1u : 1u;
+}
+
+// Stores the windows W0 .. of a unit (window w covers rows row0 + 8 w .. + 7).
+template <class TT, int W0 = 0, int NACC>
+__device__ __forceinline__ void store_unit(const typename TT::Lane &L, const f32x4 (&acc)[NACC], char *c_lane,
+                                           size_t row_bytes, uint32_t row0, uint32_t nwin, uint32_t rows, bool active)
+{
+    if (uint32_t(W0) < nwin)
+        TT::template store_window<W0>(L, acc, c_lane, row_bytes, row0 + uint32_t(W0) * kRowWindow, rows, active);
+    if constexpr (W0 + 1 < TT::G) store_unit<TT, W0 + 1>(L, acc, c_lane, row_bytes, row0, nwin, rows, active);
+}
+
+// WAVES: the largest workgroup the kernel is launched with (4, or 8 for the aligned partition); with
+// 8 waves half as many workgroups share a compute unit, the waves per SIMD stay what they are.
+template <class TT, int P, bool NARROW, int WAVES = kMaxWavesPerGroup>
+__global__ __launch_bounds__(WAVES * 64, (P <= 4 ? 4 : 2) * kMaxWavesPerGroup / WAVES)
 void spmm_mfma_kernel(const KernelArgs ka)
 {
     constexpr int G = TT::G, V = TT::V, NACC = G * V;
@@ -491,7 +512,8 @@ void spmm_mfma_kernel(const KernelArgs ka)
     const uint32_t head_slot = rd[3], tail_slot = rd[4];
     const uint32_t head_split = rd[5], tail_split = rd[6];
     // 1 (for every wave of the workgroup alike): the range is one piece of a unit, as are those of the
-    // other waves, and the workgroup adds the pieces in LDS before one sum goes to the slot of wave 0
+    // other waves, and the workgroup adds the pieces in LDS before one sum goes to the slot of wave 0;
+    // 2: the pieces are the whole unit, and wave 0 stores it
     const uint32_t combine = rd[7];
     const uint32_t U = ka.n_units, rows = ka.rows;
 
@@ -645,7 +667,7 @@ void spmm_mfma_kernel(const KernelArgs ka)
     }
     if (combine) {
         // every wave of the workgroup is here with the sums of its piece: wave 0 adds them in range order
-        __shared__ f32x4 pieces[(kMaxWavesPerGroup - 1) * NACC * 64];
+        __shared__ f32x4 pieces[(WAVES - 1) * NACC * 64];
         const uint32_t wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
         if (wave) {
 #pragma unroll
@@ -657,9 +679,14 @@ void spmm_mfma_kernel(const KernelArgs ka)
 #pragma unroll
                 for (int p = 0; p < NACC; ++p) acc[p] += pieces[((w - 1u) * NACC + p) * 64u + lane];
             }
-            f32x4 *dst = reinterpret_cast<f32x4 *>(ka.scratch) + size_t(head_slot) * (NACC * 64u) + lane;
+            if (combine == 2u) {
+                const uint32_t row = unitRow[rd[2]];
+                store_unit<TT>(L, acc, c_lane, row_bytes, row & ~7u, unit_windows<TT>(row), rows, active);
+            } else {
+                f32x4 *dst = reinterpret_cast<f32x4 *>(ka.scratch) + size_t(head_slot) * (NACC * 64u) + lane;
 #pragma unroll
-            for (int p = 0; p < NACC; ++p) dst[p * 64] = acc[p];
+                for (int p = 0; p < NACC; ++p) dst[p * 64] = acc[p];
+            }
         }
     }
 #undef HSPMM_DRAIN
@@ -669,24 +696,6 @@ void spmm_mfma_kernel(const KernelArgs ka)
 #undef HSPMM_REGS
 #undef HSPMM_DECL
 #undef HSPMM_FOR_STAGES
-}
-
-// Windows of a unit: the low bits of its row word hold the count less one (1: a pair; the
-// LDS-panel kernels also have units of three and four windows).
-template <class TT>
-__device__ __forceinline__ uint32_t unit_windows(const uint32_t row_word)
-{
-    return TT::G > 1 ? (row_word & 3u) + 1u : 1u;
-}
-
-// Stores the windows W0 .. of a unit (window w covers rows row0 + 8 w .. + 7).
-template <class TT, int W0 = 0, int NACC>
-__device__ __forceinline__ void store_unit(const typename TT::Lane &L, const f32x4 (&acc)[NACC], char *c_lane,
-                                           size_t row_bytes, uint32_t row0, uint32_t nwin, uint32_t rows, bool active)
-{
-    if (uint32_t(W0) < nwin)
-        TT::template store_window<W0>(L, acc, c_lane, row_bytes, row0 + uint32_t(W0) * kRowWindow, rows, active);
-    if constexpr (W0 + 1 < TT::G) store_unit<TT, W0 + 1>(L, acc, c_lane, row_bytes, row0, nwin, rows, active);
 }
 
 // ---------------------------------------------------------------------------
@@ -736,6 +745,16 @@ void spmm_fixup_kernel(const KernelArgs ka)
 template <class TT, bool NARROW>
 static hipError_t launch_main_p(const KernelArgs &ka, int prefetch, dim3 grid, dim3 block, hipStream_t s)
 {
+    if (block.x > 64u * kMaxWavesPerGroup) {
+        // workgroups of kAlignedGroupWaves waves (aligned partition): built for the default depths only
+        switch (prefetch) {
+        case 2: spmm_mfma_kernel<TT, 2, NARROW, kAlignedGroupWaves><<<grid, block, 0, s>>>(ka); break;
+        case 3: spmm_mfma_kernel<TT, 3, NARROW, kAlignedGroupWaves><<<grid, block, 0, s>>>(ka); break;
+        case 4: spmm_mfma_kernel<TT, 4, NARROW, kAlignedGroupWaves><<<grid, block, 0, s>>>(ka); break;
+        default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     switch (prefetch) {
     case 1: spmm_mfma_kernel<TT, 1, NARROW><<<grid, block, 0, s>>>(ka); break;
     case 2: spmm_mfma_kernel<TT, 2, NARROW><<<grid, block, 0, s>>>(ka); break;
@@ -759,8 +778,9 @@ static hipError_t launch_tt(const KernelArgs &ka, int prefetch, bool narrow, int
     if (e != hipSuccess || ka.n_split == 0 || ka.arrive) return e;
     if (mid && (e = hipEventRecord(mid, s)) != hipSuccess) return e;
     const uint32_t fitems = ka.n_split * ka.n_feat_blocks;
-    const dim3 fgrid((fitems + waves_per_group - 1) / waves_per_group);
-    spmm_fixup_kernel<TT><<<fgrid, block, 0, s>>>(ka);
+    const uint32_t fwaves = uint32_t(std::min(waves_per_group, kMaxWavesPerGroup));
+    const dim3 fgrid((fitems + fwaves - 1) / fwaves);
+    spmm_fixup_kernel<TT><<<fgrid, dim3(64u * fwaves), 0, s>>>(ka);
     return hipGetLastError();
 }
 

@@ -395,6 +395,50 @@ def test_lds_panel_kernels_exact_and_paired(torch_cuda, hs, oracle, dtype):
         hs.set_window_pairing(0)
 
 
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_long_units_are_walked_by_one_workgroup_each(torch_cuda, hs, oracle, dtype):
+    """Matrices whose units are all long (block-clustered weights at a small feature dimension): every
+    unit is cut into the ranges of one workgroup, which adds the partial sums itself and stores the
+    unit - one kernel, although the balanced partition of the same plan cuts every unit.  Exact
+    integers: the result must be the one rounding of the exact product, as from every other path."""
+    torch = torch_cuda
+    rng = np.random.default_rng(90 + dtype)
+    rows, cols = 75, 8192                                   # 10 windows (the last with 3 rows), 256-tile units
+    keep = rng.random((5, cols // 16)) < 0.5                # 16-row blocks: pairs of windows with one column list
+    D = np.zeros((rows, cols), np.int64)
+    for r in range(rows):
+        cols_kept = np.repeat(keep[r // 16], 16)
+        D[r, cols_kept] = rng.integers(-3, 4, int(cols_kept.sum()))
+    D[32:40] = 0                                            # an empty window: the pair around it is broken
+    rp = np.zeros(rows + 1, np.uint32)
+    ci, vv = [], []
+    for r in range(rows):
+        nz = np.nonzero(D[r])[0]
+        ci += nz.tolist(); vv += D[r, nz].tolist()
+        rp[r + 1] = len(ci)
+    A = dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=np.array(ci, np.uint32),
+             values=encode(np.array(vv, np.float32), dtype))
+    b = convert(hs, A)
+    for pairing in (0, 1):
+        hs.set_window_pairing(pairing)
+        try:
+            plan = hs.Plan(b)
+        finally:
+            hs.set_window_pairing(0)
+        assert plan.info()["n_split_windows"] > 0           # the balanced partition cuts units
+        for N in (8, 16, 48, 56 if dtype == 1 else 64):     # (fp32 at N = 64 would go to the LDS-staging kernels)
+            Bm = rng.integers(-4, 5, (cols, N))
+            got = gpu_spmm(torch, hs, b, encode(Bm, dtype), N, plan=plan)
+            assert np.array_equal(got, encode(D @ Bm, dtype)), (pairing, N)
+            assert plan.info()["last_kernel_family"] == 2
+            tt = torch.float32 if dtype == 1 else torch.int16
+            dB = torch.zeros((cols, N), dtype=tt, device="cuda")
+            dC = torch.empty((rows, N), dtype=tt, device="cuda")
+            main_ms, sum_ms = plan.profile(dB.data_ptr(), dC.data_ptr(), N, runs=2)
+            assert main_ms > 0 and sum_ms == 0, "a second kernel ran"
+        plan.close()
+
+
 def test_lds_panel_kernels_are_chosen_for_dense_windows_only(torch_cuda, hs):
     from hopper_spmm_amd import generators as G
     dense = G.make_config(4, 8)["A"]            # block-clustered: every window meets half of all columns
