@@ -93,7 +93,7 @@ struct hspmm_plan {
     };
     DevPartition parts[5];              // [0..2]: fewer ranges per level; [3]: level 0 with sums added per workgroup;
                                         // [4]: every unit cut into the ranges of one workgroup (aligned)
-    bool aligned_ok = false;            // every unit is long enough for [4]
+    int aligned_group = 0;              // waves of the workgroup that walks one unit in [4]; 0: units too short for it
     std::vector<uint32_t> h_unitOffset;
     // LDS-panel kernels (matrices whose windows touch a large share of the columns):
     // the unit stream re-tiled panel by panel, built by hspmm_create when it pays
@@ -1059,14 +1059,17 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         p->h_unitOffset = st.unitOffset;
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
         {
-            // all units long, and so long that the balanced partition cuts each of them eight ways or more
+            // all units long, and so long that the balanced partition cuts each of them several ways:
+            // eight ranges per unit where it would cut eight ways or more, four from `four_from` ways on
             uint32_t shortest = 0xFFFFFFFFu;
             for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u)
                 shortest = std::min(shortest, st.unitOffset[u + 1] - st.unitOffset[u]);
             const double steps_per_range = double(p->n_steps) / double(p->parts[0].part.ranges.size());
-            p->aligned_ok = shortest >= 8u * uint32_t(hspmm::kAlignedGroupWaves) &&
-                            double(p->n_steps) / double(p->n_units) >= 8.0 * steps_per_range &&
-                            uint64_t(p->n_units) * hspmm::kAlignedGroupWaves <= (1u << 24);
+            const double ways = double(p->n_steps) / double(p->n_units) / steps_per_range;
+            double four_from = 2.5;
+            if (const char *e = std::getenv("HSPMM_ALIGNED_FOUR_FROM")) four_from = std::atof(e);        // tuning override
+            const int group = ways >= 8.0 ? hspmm::kAlignedGroupWaves : ways >= four_from ? hspmm::kMaxWavesPerGroup : 0;
+            if (group && shortest >= 8u * uint32_t(group) && uint64_t(p->n_units) * group <= (1u << 24)) p->aligned_group = group;
         }
         if (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4) {
             int prc = HSPMM_OK;
@@ -1287,9 +1290,9 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     // the ranges of one workgroup of eight waves, which stores it itself - no partial sums leave the
     // chip and there is no second launch (block-clustered 4096 x 14336: 18.9 + 6.4 us -> see the
     // measurements).  With the default knobs only: the eight-wave kernels exist for the default depths.
-    const bool aligned = combine && p->aligned_ok && c.narrow && p->cfg.consumer_warp_num == 0 &&
+    const bool aligned = combine && p->aligned_group && c.narrow && p->cfg.consumer_warp_num == 0 &&
                          p->cfg.buffer_stage == 0 && p->cfg.producer_warp_group_num == 0 && p->cfg.kernel_mode == 0;
-    if (aligned) wpg = hspmm::kAlignedGroupWaves;
+    if (aligned) wpg = p->aligned_group;
     int rc = build_and_upload_partition(p, level, combine ? uint32_t(wpg) : 1u, aligned);
     if (rc) return rc;
     const hspmm_plan::DevPartition &dp = p->parts[aligned ? 4 : combine ? 3 : level];
