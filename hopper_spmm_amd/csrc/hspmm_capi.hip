@@ -1256,7 +1256,7 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
         const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
         // (a 16-bit matrix near the break-even is served as fast or faster by the gather kernels while
         // one wave of theirs covers all of N)
-        const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 1.5 || N >= 256u;
+        const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
         if (pays && N % block_feat == 0 && !(align & 15u)) { p->last_family = 3; return run_panel(p, dB, dC, N, s, mid); }
     }
     const Choice c = choose_kernel(p, dB, dC, N);
@@ -1291,7 +1291,7 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     // chip and there is no second launch (block-clustered 4096 x 14336: 18.9 + 6.4 us -> see the
     // measurements).  With the default knobs only: the eight-wave kernels exist for the default depths.
     const bool aligned = combine && p->aligned_group && c.narrow && p->cfg.consumer_warp_num == 0 &&
-                         p->cfg.buffer_stage == 0 && p->cfg.producer_warp_group_num == 0 && p->cfg.kernel_mode == 0;
+                         p->cfg.buffer_stage == 0 && p->cfg.producer_warp_group_num == 0;
     if (aligned) wpg = p->aligned_group;
     int rc = build_and_upload_partition(p, level, combine ? uint32_t(wpg) : 1u, aligned);
     if (rc) return rc;
