@@ -846,6 +846,7 @@ int ensure_arrive(hspmm_plan *p, size_t words)
     if (p->d_arrive) { HSPMM_HIP(hipFree(p->d_arrive)); p->d_arrive = nullptr; p->arrive_words = 0; }
     HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->d_arrive), words * 4));
     HSPMM_HIP(hipMemset(p->d_arrive, 0, words * 4));
+    HSPMM_HIP(hipStreamSynchronize(nullptr));       // the launch that follows may be on a stream that does not wait for this one
     p->arrive_words = words;
     return HSPMM_OK;
 }
@@ -1216,6 +1217,13 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         const size_t need = size_t(pl.n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
         if ((rc = ensure_scratch(p, need))) return rc;
         pa.scratch = p->d_scratch;
+        // (experiment, as in the gather kernels: the wave that brings a unit's last chunk adds the chunk sums
+        // itself; the device-scope accesses cost more than the second launch: 61.7 + 8.8 -> 76.8 us on the
+        // block-clustered configuration at N = 512)
+        if (p->cfg.fused_fixup) {
+            if ((rc = ensure_arrive(p, size_t(pl.n_units) * pa.n_feat_blocks))) return rc;
+            pa.arrive = p->d_arrive;
+        }
         ka.unitRow = pl.d_unitRow; ka.ids = pl.d_ids; ka.tiles = pl.d_tiles;
         ka.split = pl.d_split; ka.fix_slots = pl.d_fix_slots; ka.scratch = p->d_scratch;
         ka.C = dC; ka.B = dB;

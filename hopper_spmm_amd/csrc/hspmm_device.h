@@ -68,6 +68,8 @@ struct PanelArgs {
                                  // type (PanelOps in spmm_panel_kernel.hpp)
     const void     *tiles;       // per step, lane order
     float          *scratch;     // partial sums [unit * n_chunks + chunk][feature block][acc reg][lane]
+    uint32_t       *arrive;      // per (unit, feature block): chunks that have left their sums (zero between launches);
+                                 // null: a second kernel adds the sums
     const void     *B;
     void           *C;
     uint32_t n_units, n_steps, rows, cols, N, n_feat_blocks, n_panels, n_chunks, panels_per_chunk;

@@ -627,11 +627,37 @@ void spmm_panel_kernel(const PanelArgs pa)
     const uint32_t nwin = unit_windows<TT>(row);
     if (pa.n_chunks == 1u) {
         store_unit<TT>(L, acc, c_lane, row_bytes, row0, nwin, pa.rows, true);
-    } else {
+    } else if (!pa.arrive) {
         f32x4 *dst = reinterpret_cast<f32x4 *>(pa.scratch) +
                      ((size_t(u) * pa.n_chunks + chunk) * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
 #pragma unroll
         for (int i = 0; i < NACC; ++i) dst[i * 64] = acc[i];
+    } else {
+        // The wave that brings the last chunk's sums of a unit adds all of them, in chunk order (so the
+        // result does not depend on who is last), and stores the unit.  The sums cross the L2s of
+        // different XCDs: they are written and read with device-scope accesses, and the writes are
+        // waited for before the arrival is counted.
+        f32x4 *slot0 = reinterpret_cast<f32x4 *>(pa.scratch) +
+                       (size_t(u) * pa.n_chunks * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
+        const size_t chunk_stride = size_t(pa.n_feat_blocks) * (NACC * 64u);
+        f32x4 *dst = slot0 + chunk * chunk_stride;
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) store_device_scope(dst + i * 64, acc[i]);
+        __builtin_amdgcn_s_waitcnt(0x0F70);                        // vmcnt(0): the stores are acknowledged
+        uint32_t *ctr = pa.arrive + size_t(u) * pa.n_feat_blocks + fb;
+        uint32_t old = 0;
+        if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        old = __builtin_amdgcn_readfirstlane(old);
+        if (old + 1u == pa.n_chunks) {
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (uint32_t c = 0; c < pa.n_chunks; ++c) {
+#pragma unroll
+                for (int i = 0; i < NACC; ++i) acc[i] += load_device_scope(slot0 + c * chunk_stride + i * 64);
+            }
+            store_unit<TT>(L, acc, c_lane, row_bytes, row0, nwin, pa.rows, true);
+            if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     if (chunk == 0u) {
         // rows of the windows without entries behind this unit, and in front of the first one
@@ -657,7 +683,7 @@ static hipError_t launch_panel_tt(const PanelArgs &pa, const KernelArgs &ka, hip
     const dim3 grid(row_blocks * pa.n_feat_blocks * pa.n_chunks), block((NC + NPW) * 64);
     spmm_panel_kernel<TT, NC, NPW><<<grid, block, 0, s>>>(pa);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || pa.n_chunks == 1u) return e;
+    if (e != hipSuccess || pa.n_chunks == 1u || pa.arrive) return e;
     if (mid && (e = hipEventRecord(mid, s)) != hipSuccess) return e;
     const uint32_t fitems = ka.n_split * ka.n_feat_blocks;
     spmm_fixup_kernel<TT><<<dim3((fitems + 3u) / 4u), dim3(256), 0, s>>>(ka);

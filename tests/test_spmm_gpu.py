@@ -439,6 +439,51 @@ def test_long_units_are_walked_by_one_workgroup_each(torch_cuda, hs, oracle, dty
         plan.close()
 
 
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_partial_sums_added_inside_the_main_kernel(torch_cuda, hs, oracle, dtype):
+    """HSPMM_FUSED_FIXUP=1 (an experiment switch, slower than the second launch): the wave that brings
+    the last partial sum of a cut unit, or of a unit's chunks of panels, adds them in the fixed order and
+    stores the unit: the same bits launch after launch, whoever arrives last."""
+    torch = torch_cuda
+    rng = np.random.default_rng(33 + dtype)
+    block = 64 if dtype == 1 else 128
+    sparse = random_csr(rng, 300, 3000, 0.004, dtype, 0.2, (5, 100, 101, 299))     # heavy windows: cut units
+    dense = random_csr(rng, 300, 3000, 0.1, dtype, 0.1)                             # LDS-staging kernels
+    for A, N, family in ((sparse, 48 if dtype == 1 else 64, 2), (dense, block, 3)):   # (fp32, N = 64: LDS-staging kernels)
+        b = convert(hs, A)
+        B = make_b(rng, 3000, N, dtype)
+        hs.configure(producer_warp_group_num=16)
+        os.environ["HSPMM_PANEL_CHUNKS"] = "3"
+        try:
+            two = hs.Plan(b)
+            want = gpu_spmm(torch, hs, b, B, N, plan=two)
+            two.close()
+            os.environ["HSPMM_FUSED_FIXUP"] = "1"
+            try:
+                plan = hs.Plan(b)
+            finally:
+                os.environ.pop("HSPMM_FUSED_FIXUP", None)
+            ref, mag = oracle_spmm(oracle, A, B, N)
+            first = gpu_spmm(torch, hs, b, B, N, plan=plan)
+            assert_parity(first, ref, mag, dtype, "sums added in the main kernel")
+            if family == 3:             # the chunk order is the same in both paths; the gather kernels' two-kernel
+                assert np.array_equal(first, want)      # path adds four ranges per workgroup first
+            for _ in range(3):
+                assert np.array_equal(gpu_spmm(torch, hs, b, B, N, plan=plan), first)
+            assert plan.info()["last_kernel_family"] == family
+            tt = torch.float32 if dtype == 1 else torch.int16
+            dB = torch.zeros((3000, N), dtype=tt, device="cuda")
+            dC = torch.empty((300, N), dtype=tt, device="cuda")
+            main_ms, sum_ms = plan.profile(dB.data_ptr(), dC.data_ptr(), N, runs=2)
+            assert main_ms > 0 and sum_ms == 0
+            plan.close()
+        finally:
+            hs.configure()
+            os.environ.pop("HSPMM_PANEL_CHUNKS", None)
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        assert_parity(want, ref, mag, dtype, "two-kernel path")
+
+
 def test_lds_panel_kernels_are_chosen_for_dense_windows_only(torch_cuda, hs):
     from hopper_spmm_amd import generators as G
     dense = G.make_config(4, 8)["A"]            # block-clustered: every window meets half of all columns
