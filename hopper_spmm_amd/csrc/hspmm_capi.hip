@@ -1294,10 +1294,11 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     // one unit among themselves.
     int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
     const bool combine = level == 0 && ka.n_feat_blocks == 1 && wpg > 1 && !p->cfg.fused_fixup;
-    // Units that are all long (block-clustered or pruned weights at a small N): every unit is cut into
-    // the ranges of one workgroup of eight waves, which stores it itself - no partial sums leave the
-    // chip and there is no second launch (block-clustered 4096 x 14336: 18.9 + 6.4 us -> see the
-    // measurements).  With the default knobs only: the eight-wave kernels exist for the default depths.
+    // Units that are all long (block-clustered, pruned or dense-ish random matrices at a small N): every
+    // unit is cut into the ranges of one workgroup of four or eight waves, which stores it itself - no
+    // partial sums leave the chip and there is no second launch (block-clustered 4096 x 14336, N = 16:
+    // 18.9 + 6.4 us -> 19 us; random 8192 x 8192 at 2 %, N = 128: 26.8 + 7.1 -> 22.8 us).  With the default
+    // knobs only: the eight-wave kernels exist for the default depths.
     const bool aligned = combine && p->aligned_group && c.narrow && p->cfg.consumer_warp_num == 0 &&
                          p->cfg.buffer_stage == 0 && p->cfg.producer_warp_group_num == 0;
     if (aligned) wpg = p->aligned_group;
