@@ -642,6 +642,56 @@ def test_unaligned_and_odd_feature_dims_use_the_all_shapes_kernel(torch_cuda, hs
         plan.close()
 
 
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_pointer_alignment_selects_the_kernel_family(torch_cuda, hs, oracle, dtype):
+    """B and C need only be aligned to the element size: the LDS-staging kernels want 16 bytes, the
+    MFMA gather kernels 4 (8 and 16 for their wider loads), anything else runs through the all-shapes
+    kernel - with the same result (exact integers) whatever the offsets."""
+    torch = torch_cuda
+    rng = np.random.default_rng(61 + dtype)
+    rows, cols, N = 96, 1024, 128
+    D = rng.integers(-3, 4, (rows, cols)) * (rng.random((rows, cols)) < 0.2)
+    rp = np.zeros(rows + 1, np.uint32)
+    ci, vv = [], []
+    for r in range(rows):
+        nz = np.nonzero(D[r])[0]
+        ci += nz.tolist(); vv += D[r, nz].tolist()
+        rp[r + 1] = len(ci)
+    A = dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=np.array(ci, np.uint32),
+             values=encode(np.array(vv, np.float32), dtype))
+    plan = hs.Plan(convert(hs, A))
+    assert plan.info()["n_panels"] > 0
+    Bm = rng.integers(-4, 5, (cols, N))
+    want = encode(D @ Bm, dtype)
+    es = 4 if dtype == 1 else 2
+    tt = torch.float32 if dtype == 1 else torch.int16
+    host_b = torch.from_numpy(encode(Bm, dtype) if dtype == 1 else encode(Bm, dtype).view(np.int16))
+    seen = set()
+    for off_b, off_c in ((0, 0), (16, 32), (8, 0), (0, 4), (4, 4), (2, 0), (0, 2), (6, 10)):
+        if off_b % es or off_c % es:
+            continue
+        buf_b = torch.zeros(cols * N + 16, dtype=tt, device="cuda")
+        buf_c = torch.full((rows * N + 16,), 7, dtype=tt, device="cuda")
+        dB = buf_b[off_b // es: off_b // es + cols * N]
+        dC = buf_c[off_c // es: off_c // es + rows * N]
+        dB.copy_(host_b.reshape(-1))
+        assert dB.data_ptr() % 16 == off_b % 16 and dC.data_ptr() % 16 == off_c % 16
+        plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        got = dC.cpu().numpy().reshape(rows, N)
+        got = got if dtype == 1 else got.view(np.uint16)
+        assert np.array_equal(got, want), (off_b, off_c)
+        # nothing outside C was written
+        edge = buf_c.cpu().numpy()
+        assert (edge[:off_c // es] == 7).all() and (edge[off_c // es + rows * N:] == 7).all()
+        family = plan.info()["last_kernel_family"]
+        seen.add(family)
+        worst = (off_b | off_c) % 16
+        assert family == (3 if worst == 0 else 2 if worst % 4 == 0 else 1), (off_b, off_c, family)
+    assert seen == ({3, 2} if dtype == 1 else {3, 2, 1})
+    plan.close()
+
+
 def test_matrix_without_entries_gives_zeros(torch_cuda, hs):
     for dt in (0, 1, 2):
         vt = np.float32 if dt == 1 else np.uint16
