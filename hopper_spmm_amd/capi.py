@@ -102,6 +102,7 @@ def load_library():
     L.hspmm_partition_preview.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
     L.hspmm_partition_preview_grouped.argtypes = [u32, vp, u32, u32, vp, u32, C.POINTER(u32), C.POINTER(u32),
                                                   C.POINTER(u32)]
+    L.hspmm_partition_preview_aligned.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32)]
     L.hspmm_panel_units_preview.argtypes = [i, u32, u32, u32, u32, vp, vp, vp, vp, u32, C.POINTER(u32), vp, vp, vp,
                                             C.POINTER(u32), u32, vp, vp]
     L.hspmm_mtx_load.argtypes = [C.c_char_p, i, C.POINTER(_Csr)]
@@ -293,6 +294,19 @@ def bitmap_to_grouped(bitmap, min_len=32):
     out.update(total_groups=n, tgl=tgl.value, groupOffset=groupOffset, rowIdx=groupRowIdx, atomic=atomic,
                total_row_windows=n + 1, eff_row_windows=n + 1)
     return out
+
+
+def partition_preview_aligned(rowOffset, group):
+    """The partition for plans whose units are all long: every window cut into `group` ranges that
+    one workgroup walks (host only).  Ranges have six words; the sixth is 2."""
+    L = load_library()
+    rowOffset = np.ascontiguousarray(rowOffset, np.uint32)
+    W = rowOffset.size - 1
+    n = C.c_uint32()
+    _check(L.hspmm_partition_preview_aligned(W, _p(rowOffset), group, None, 0, C.byref(n)))
+    ranges = np.zeros((n.value, 6), np.uint32)
+    _check(L.hspmm_partition_preview_aligned(W, _p(rowOffset), group, _p(ranges), n.value, None))
+    return ranges
 
 
 def partition_preview(rowOffset, target_ranges, group=1):

@@ -953,6 +953,28 @@ int hspmm_partition_preview_grouped(uint32_t eff_row_windows, const uint32_t *ro
                              n_split_windows, n_partial_slots);
 }
 
+int hspmm_partition_preview_aligned(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t group,
+                                    uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges)
+{
+    if (eff_row_windows && !rowOffset) return fail(HSPMM_ERR_INVALID, "null rowOffset");
+    if (group != uint32_t(hspmm::kMaxWavesPerGroup) && group != uint32_t(hspmm::kAlignedGroupWaves))
+        return fail(HSPMM_ERR_INVALID, "group %u: %d or %d", group, hspmm::kMaxWavesPerGroup, hspmm::kAlignedGroupWaves);
+    for (uint32_t w = 0; w < eff_row_windows; ++w)
+        if (rowOffset[0] != 0 || rowOffset[w + 1] < rowOffset[w] + group)
+            return fail(HSPMM_ERR_INVALID, "rowOffset must start at 0 and every window needs at least %u tiles", group);
+    const hspmm::Partition part = hspmm::build_aligned_partition(eff_row_windows, rowOffset, group);
+    if (n_ranges) *n_ranges = uint32_t(part.ranges.size());
+    if (ranges) {
+        const size_t n = part.ranges.size() < capacity_ranges ? part.ranges.size() : capacity_ranges;
+        for (size_t i = 0; i < n; ++i) {
+            uint32_t *d = ranges + 6 * i;
+            d[0] = part.ranges[i].tile_begin; d[1] = part.ranges[i].tile_end; d[2] = part.ranges[i].first_window;
+            d[3] = part.ranges[i].head_slot; d[4] = part.ranges[i].tail_slot; d[5] = part.ranges[i].combine;
+        }
+    }
+    return HSPMM_OK;
+}
+
 int hspmm_panel_units_preview(int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows, uint32_t total_tiles,
                               const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data, const uint32_t *rowIdx,
                               uint32_t max_windows, uint32_t *n_groups, uint32_t *group_first, uint32_t *group_count,

@@ -190,6 +190,15 @@ int hspmm_partition_preview_grouped(uint32_t eff_row_windows, const uint32_t *ro
                                     uint32_t group, uint32_t *ranges, uint32_t capacity_ranges,
                                     uint32_t *n_ranges, uint32_t *n_split_windows, uint32_t *n_partial_slots);
 
+/* No reference counterpart; host only.  The partition used where every unit is
+ * long (the balanced partition would cut each of them 2.5 ways or more, and one
+ * wave covers the feature dimension): every window is cut into `group` (4 or 8)
+ * ranges of about equal length, walked by the waves of one workgroup, which adds
+ * their sums itself and stores the window - no slots and no second kernel.
+ * Ranges as in hspmm_partition_preview_grouped (six words; the sixth is 2). */
+int hspmm_partition_preview_aligned(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t group,
+                                    uint32_t *ranges, uint32_t capacity_ranges, uint32_t *n_ranges);
+
 /* ---- host format functions ---------------------------------------------- */
 
 typedef struct {

@@ -143,3 +143,26 @@ def test_partition_with_sums_added_per_workgroup(hs, group):
     # a long window cut into many pieces: whole workgroups inside it share one slot each
     p = hs.partition_preview(np.array([0, 4096], np.uint32), 64, group=4)
     assert p["n_partial_slots"] == 16 and np.all(p["ranges"][:, 5] == 1)
+
+
+def test_aligned_partition_cuts_every_window_into_the_ranges_of_one_workgroup(hs):
+    """Every window becomes `group` contiguous ranges of nearly equal length that cover it exactly; no
+    range has a slot (the workgroup stores the window itself); windows too short for it are refused."""
+    rng = np.random.default_rng(4)
+    for group in (4, 8):
+        tiles = rng.integers(group, 700, 300)
+        ro = np.concatenate([[0], np.cumsum(tiles)]).astype(np.uint32)
+        r = hs.partition_preview_aligned(ro, group)
+        assert r.shape == (300 * group, 6)
+        assert (r[:, 5] == 2).all() and (r[:, 3] == 0xFFFFFFFF).all() and (r[:, 4] == 0xFFFFFFFF).all()
+        assert r[0, 0] == 0 and r[-1, 1] == ro[-1]
+        assert np.array_equal(r[1:, 0], r[:-1, 1])                      # contiguous, nothing skipped
+        per = r.reshape(300, group, 6)
+        assert np.array_equal(per[:, 0, 0], ro[:-1]) and np.array_equal(per[:, -1, 1], ro[1:])
+        assert (per[:, :, 2] == np.arange(300)[:, None]).all()
+        lengths = (per[:, :, 1] - per[:, :, 0]).astype(np.int64)
+        assert lengths.min() >= 1 and (lengths.max(axis=1) - lengths.min(axis=1) <= 1).all()
+    with pytest.raises(hs.HspmmError):
+        hs.partition_preview_aligned(np.array([0, 3, 40], np.uint32), 4)    # a window of three tiles
+    with pytest.raises(hs.HspmmError):
+        hs.partition_preview_aligned(np.array([0, 30, 60], np.uint32), 3)
