@@ -12,6 +12,7 @@
 #include <string>
 #include <vector>
 #include <mutex>
+#include <atomic>
 #include <new>
 #include <algorithm>
 
@@ -53,6 +54,29 @@ struct Config {
     int kernel_mode = 0;
     int fused_fixup = 0;                // 1: the last wave of a cut unit adds its partial sums; 0: second kernel
     int pairing = 0;                    // 0 automatic, 1 never, 2 whenever two windows share a column list
+    // Tuning overrides from the environment (HSPMM_*), read once by hspmm_create: a plan's behaviour does
+    // not change with the environment afterwards and the launch path reads no variable.
+    double window_cost = 1.5, slack = 0.35, whole_window_margin = 32.0;     // cost model of partition.hpp
+    double aligned_four_from = 2.5;     // ways the balanced partition must cut every unit before one workgroup walks it
+    double panel_wide_cost = 1.25;      // a step of three or four windows, in steps of two
+    int panel_units = 0;                // workgroup shape of the LDS-panel kernels: 12, 13, 14 (0: by tile type)
+    int panel_units_per_group = 0;      // consumer waves of a workgroup that get a unit (0: searched per N)
+    int panel_chunks = 0;               // chunks of panels (0: searched per N)
+    int panel_max_windows = 0;          // 2 or 4: windows per unit of the panel stream (0: by matrix size)
+
+    void read_environment()
+    {
+        if (const char *e = std::getenv("HSPMM_FUSED_FIXUP")) fused_fixup = std::atoi(e);
+        if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);
+        if (const char *e = std::getenv("HSPMM_SLACK")) slack = std::atof(e);
+        if (const char *e = std::getenv("HSPMM_WHOLE_WINDOW_MARGIN")) whole_window_margin = std::atof(e);
+        if (const char *e = std::getenv("HSPMM_ALIGNED_FOUR_FROM")) aligned_four_from = std::atof(e);
+        if (const char *e = std::getenv("HSPMM_PANEL_WIDE_COST")) panel_wide_cost = std::atof(e);
+        if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) panel_units = std::atoi(e) == 14 ? 14 : std::atoi(e) == 13 ? 13 : 12;
+        if (const char *e = std::getenv("HSPMM_PANEL_UNITS_PER_GROUP")) panel_units_per_group = std::max(1, std::atoi(e));
+        if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) panel_chunks = std::max(1, std::atoi(e));
+        if (const char *e = std::getenv("HSPMM_PANEL_MAX_WINDOWS")) panel_max_windows = std::atoi(e) >= 4 ? 4 : 2;
+    }
 };
 std::mutex g_cfg_mutex;
 Config g_cfg;
@@ -102,22 +126,29 @@ struct hspmm_plan {
         uint32_t n_panels = 0, n_steps = 0;
         uint32_t *d_poff = nullptr, *d_ids = nullptr, *d_step_panel = nullptr;
         void *d_tiles = nullptr;
-        uint32_t *d_split = nullptr, *d_fix_slots = nullptr;    // one split entry per unit, for the chunk sums
         uint32_t *d_unitRow = nullptr;                           // the units of this stream (first row | paired bit)
         uint32_t n_units = 0, n_paired = 0, n_wide = 0;          // units of two or more / three or four windows
         int G = 1;
         bool quad = false;                                       // ids in the format of the 4x4x1 fp32 tile
         bool split = false;                                      // fp32 stream in the bf16 hi / lo form (Fp32Split)
         double density = 0.0;                                    // steps per unit and 128 columns of the gather stream
-        uint32_t split_chunks = 0;                               // chunk count d_split was built for
-        size_t fix_slot_count = 0;
     } panel;
     float *d_scratch = nullptr;
     size_t scratch_bytes = 0;
     uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
     size_t arrive_words = 0;
     size_t fixed_bytes = 0;
-    uint32_t last_family = 0;           // kernel family of the last hspmm_run: 0 none yet, 1 all-shapes, 2 gather, 3 LDS-panel, 4 clear
+    // Every real column list strictly ascending and padding only behind a window's last column: what the
+    // reference's converters write (reference src/utils/convert.h:166-181).  The gather and all-shapes
+    // kernels take any list; merging windows and the LDS-panel stream need this order.
+    bool canonical = true;
+    // What a launch may still have to build (a partition for a wider N, larger scratch) is built under
+    // this mutex; everything else in the plan is immutable after hspmm_create.
+    std::mutex mu;
+    // Superseded scratch buffers stay allocated until hspmm_destroy: launches recorded earlier (HIP
+    // graphs) carry their addresses.
+    std::vector<void *> retired;
+    std::atomic<uint32_t> last_family{0};   // kernel family of the last hspmm_run: 0 none yet, 1 all-shapes, 2 gather, 3 LDS-panel, 4 clear
 };
 
 namespace {
@@ -132,9 +163,13 @@ int upload(T **dst, const T *src, size_t n, size_t *acc_bytes)
     return HSPMM_OK;
 }
 
+// canonical (optional): whether every window's real column ids ascend strictly with padding only behind
+// the window's last column, as the reference's converter writes them (src/utils/convert.h:166-181).
 int validate_format(uint32_t rows, uint32_t cols, uint32_t W, uint32_t T, uint32_t cw,
-                    const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data, const uint32_t *rowIdx)
+                    const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data, const uint32_t *rowIdx,
+                    bool *canonical = nullptr)
 {
+    if (canonical) *canonical = true;
     if (W == 0) {
         if (T != 0) return fail(HSPMM_ERR_INVALID, "total_tiles = %u with no effective row window", T);
         return HSPMM_OK;
@@ -164,6 +199,21 @@ int validate_format(uint32_t rows, uint32_t cols, uint32_t W, uint32_t T, uint32
             if (ids[k] >= cols) return fail(HSPMM_ERR_INVALID, "tile %u: column id %u >= cols %u", t, ids[k], cols);
         }
     }
+    if (canonical) {
+        std::atomic<bool> ok{true};
+        hspmm_host::parallel_blocks(W, 4096, [&](size_t wb, size_t we) {
+            for (size_t w = wb; w < we && ok.load(std::memory_order_relaxed); ++w) {
+                const uint32_t *c = tcA2B + size_t(rowOffset[w]) * cw;
+                const size_t n = size_t(rowOffset[w + 1] - rowOffset[w]) * cw;
+                size_t real = n;
+                while (real && c[real - 1] == HSPMM_IDX_MAX) --real;
+                bool good = n - real < cw;                      // padding only in the window's last tile
+                for (size_t i = 1; i < real && good; ++i) good = c[i] != HSPMM_IDX_MAX && c[i] > c[i - 1];
+                if (!good) ok.store(false, std::memory_order_relaxed);
+            }
+        });
+        *canonical = ok.load();
+    }
     return HSPMM_OK;
 }
 
@@ -181,10 +231,7 @@ int build_and_upload_partition(hspmm_plan *p, int level, uint32_t group = 1, boo
 {
     hspmm_plan::DevPartition &dp = p->parts[aligned ? 4 : group > 1 ? 3 : level];
     if (dp.built || p->W == 0) return HSPMM_OK;
-    double window_cost = 1.5, slack = 0.35, margin = 32.0;
-    if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);   // tuning overrides
-    if (const char *e = std::getenv("HSPMM_SLACK")) slack = std::atof(e);
-    if (const char *e = std::getenv("HSPMM_WHOLE_WINDOW_MARGIN")) margin = std::atof(e);
+    const double window_cost = p->cfg.window_cost, slack = p->cfg.slack, margin = p->cfg.whole_window_margin;
     uint32_t target = uint32_t(choose_ranges(p)) >> level;
     const uint32_t floor_ranges = uint32_t(p->compute_units) * 4u;       // at least one range per SIMD
     if (target < floor_ranges) target = std::min<uint32_t>(floor_ranges, uint32_t(choose_ranges(p)));
@@ -582,12 +629,11 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
         // 8192 and 11008 rows: 0.93 - 1.1 x up to N = 512, 1.2 - 1.3 x only from N = 2048 on), and for
         // fp32 storage in bf16 parts, with twice the MFMAs per LDS read, they gain nothing (0.82 - 1.2 x).
         // Pairing mode 2 takes them wherever windows qualify.
-        double wide_cost = 1.25;
+        const double wide_cost = p->cfg.panel_wide_cost;
         uint32_t max_windows = (p->cfg.pairing == 2 || cw == 16) ? 4u : 2u;
         size_t min_wide_units = p->cfg.pairing == 2 ? 0u : size_t(p->compute_units) * 3u / 2u;
-        if (const char *e = std::getenv("HSPMM_PANEL_WIDE_COST")) wide_cost = std::atof(e);       // tuning overrides
-        if (const char *e = std::getenv("HSPMM_PANEL_MAX_WINDOWS")) {
-            max_windows = std::atoi(e) >= 4 ? 4u : 2u;
+        if (p->cfg.panel_max_windows) {                                                           // tuning override
+            max_windows = uint32_t(p->cfg.panel_max_windows);
             min_wide_units = 0;
         }
         std::vector<uint32_t> first, count;
@@ -769,37 +815,6 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     return true;
 }
 
-// Split table for the chunk sums of the panel kernels: unit u owns slots
-// u * chunks .. u * chunks + chunks - 1, added in that order.
-int ensure_panel_split(hspmm_plan *p, uint32_t chunks)
-{
-    hspmm_plan::Panel &pl = p->panel;
-    const size_t slots = size_t(pl.n_units) * chunks;
-    if (slots > pl.fix_slot_count) {
-        if (pl.d_fix_slots) { HSPMM_HIP(hipFree(pl.d_fix_slots)); pl.d_fix_slots = nullptr; pl.fix_slot_count = 0; }
-        std::vector<uint32_t> ident(slots);
-        for (size_t i = 0; i < slots; ++i) ident[i] = uint32_t(i);
-        size_t dummy = 0;
-        int rc = upload(&pl.d_fix_slots, ident.data(), ident.size(), &dummy);
-        if (rc) return rc;
-        pl.fix_slot_count = slots;
-    }
-    if (pl.split_chunks != chunks) {
-        if (pl.d_split) { HSPMM_HIP(hipFree(pl.d_split)); pl.d_split = nullptr; pl.split_chunks = 0; }
-        std::vector<uint32_t> sp(size_t(pl.n_units) * hspmm::kFixWords, 0u);
-        for (uint32_t u = 0; u < pl.n_units; ++u) {
-            sp[size_t(u) * hspmm::kFixWords + 0] = u;
-            sp[size_t(u) * hspmm::kFixWords + 1] = u * chunks;
-            sp[size_t(u) * hspmm::kFixWords + 2] = chunks;
-        }
-        size_t dummy = 0;
-        int rc = upload(&pl.d_split, sp.data(), sp.size(), &dummy);
-        if (rc) return rc;
-        pl.split_chunks = chunks;
-    }
-    return HSPMM_OK;
-}
-
 struct Choice {
     bool scalar;
     int layout, V, block_feat;
@@ -840,29 +855,49 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
     return c;
 }
 
-int ensure_arrive(hspmm_plan *p, size_t words)
+// How a launch gets the memory it needs beyond the plan's fixed arrays.
+//   kLaunch:  hspmm_run - may build a partition and grow the plan's scratch buffer (under the plan's mutex)
+//   kPrepare: hspmm_prepare - builds and grows exactly like kLaunch and launches nothing
+enum class RunMode { kLaunch, kPrepare };
+
+// Arrival counters of the in-kernel reduction (an experiment switch).
+// Called with the plan's mutex held.
+int ensure_arrive(hspmm_plan *p, size_t words, uint32_t **out)
 {
-    if (words <= p->arrive_words) return HSPMM_OK;
-    if (p->d_arrive) { HSPMM_HIP(hipFree(p->d_arrive)); p->d_arrive = nullptr; p->arrive_words = 0; }
-    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->d_arrive), words * 4));
-    HSPMM_HIP(hipMemset(p->d_arrive, 0, words * 4));
-    HSPMM_HIP(hipStreamSynchronize(nullptr));       // the launch that follows may be on a stream that does not wait for this one
-    p->arrive_words = words;
+    if (words > p->arrive_words) {
+        uint32_t *fresh = nullptr;
+        HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&fresh), words * 4));
+        HSPMM_HIP(hipMemset(fresh, 0, words * 4));
+        HSPMM_HIP(hipStreamSynchronize(nullptr));   // the launch that follows may be on a stream that does not wait for this one
+        if (p->d_arrive) p->retired.push_back(p->d_arrive);
+        p->d_arrive = fresh;
+        p->arrive_words = words;
+    }
+    *out = p->d_arrive;
     return HSPMM_OK;
 }
 
-int ensure_scratch(hspmm_plan *p, size_t bytes)
+// The buffer for `bytes` of partial sums: the plan's buffer, grown when too small (sizes are powers of two, so the superseded buffers, which stay
+// allocated until hspmm_destroy, never add up to more than the current one).  Called with the plan's mutex held.
+int scratch_for(hspmm_plan *p, size_t bytes, RunMode mode, float **out)
 {
-    if (bytes <= p->scratch_bytes) return HSPMM_OK;
-    if (p->d_scratch) { HSPMM_HIP(hipFree(p->d_scratch)); p->d_scratch = nullptr; p->scratch_bytes = 0; }
-    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->d_scratch), bytes));
-    p->scratch_bytes = bytes;
+    (void)mode;
+    if (bytes > p->scratch_bytes) {
+        size_t cap = size_t(1) << 16;
+        while (cap < bytes) cap <<= 1;
+        float *fresh = nullptr;
+        HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&fresh), cap));
+        if (p->d_scratch) p->retired.push_back(p->d_scratch);
+        p->d_scratch = fresh;
+        p->scratch_bytes = cap;
+    }
+    *out = p->d_scratch;
     return HSPMM_OK;
 }
 
 }  // namespace
 
-static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream, hipEvent_t mid);
+static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream, hipEvent_t mid, RunMode mode);
 
 extern "C" {
 
@@ -986,15 +1021,17 @@ int hspmm_panel_units_preview(int dtype, uint32_t rows, uint32_t cols, uint32_t 
     if (max_windows != 1 && max_windows != 2 && max_windows != 4)
         return fail(HSPMM_ERR_INVALID, "max_windows %u: 1, 2 or 4", max_windows);
     const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u, elem = dtype == HSPMM_TF32 ? 4u : 2u;
-    const int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx);
+    bool canonical = true;
+    const int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx, &canonical);
     if (rc) return rc;
     const uint32_t W = eff_row_windows;
     Unioned un;
     std::vector<uint32_t> first, count;
     const void *d = data;
     try {
-        group_windows(W, cw, elem, hspmm::kPanelRowsWide, 32u, max_windows, 1.25, 0, rowOffset, tcA2B, d, rowIdx, un, first,
-                      count);
+        // column lists that do not ascend strictly, or with padding inside a window, are never merged
+        group_windows(W, cw, elem, hspmm::kPanelRowsWide, 32u, canonical ? max_windows : 1u, 1.25, 0, rowOffset, tcA2B, d,
+                      rowIdx, un, first, count);
     } catch (const std::bad_alloc &) { return fail(HSPMM_ERR_ALLOC, "out of host memory"); }
     const uint32_t T = W ? rowOffset[W] : 0u;
     if (n_groups) *n_groups = uint32_t(first.size());
@@ -1023,15 +1060,16 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
     const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
     const uint32_t elem = dtype == HSPMM_TF32 ? 4u : 2u;
-    int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx);
+    bool canonical = true;
+    int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx, &canonical);
     if (rc) return rc;
 
     hspmm_plan *p = new (std::nothrow) hspmm_plan;
     if (!p) return fail(HSPMM_ERR_ALLOC, "out of host memory");
     p->dtype = dtype; p->rows = rows; p->cols = cols; p->W = eff_row_windows; p->T = total_tiles;
-    p->cw = cw; p->elem = elem;
+    p->cw = cw; p->elem = elem; p->canonical = canonical;
     { std::lock_guard<std::mutex> lk(g_cfg_mutex); p->cfg = g_cfg; }
-    if (const char *e = std::getenv("HSPMM_FUSED_FIXUP")) p->cfg.fused_fixup = std::atoi(e);     // tuning override
+    p->cfg.read_environment();                      // tuning overrides, once per plan
 
     auto bail = [&](int code) { hspmm_destroy(p); return code; };
     hipError_t e = hipGetDevice(&p->device);
@@ -1089,12 +1127,13 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
                 shortest = std::min(shortest, st.unitOffset[u + 1] - st.unitOffset[u]);
             const double steps_per_range = double(p->n_steps) / double(p->parts[0].part.ranges.size());
             const double ways = double(p->n_steps) / double(p->n_units) / steps_per_range;
-            double four_from = 2.5;
-            if (const char *e = std::getenv("HSPMM_ALIGNED_FOUR_FROM")) four_from = std::atof(e);        // tuning override
+            const double four_from = p->cfg.aligned_four_from;
             const int group = ways >= 8.0 ? hspmm::kAlignedGroupWaves : ways >= four_from ? hspmm::kMaxWavesPerGroup : 0;
             if (group && shortest >= 8u * uint32_t(group) && uint64_t(p->n_units) * group <= (1u << 24)) p->aligned_group = group;
         }
-        if (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4) {
+        // (the LDS-panel stream re-tiles ascending column lists; a caller's lists in another order stay
+        // with the gather and all-shapes kernels)
+        if ((p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4) && p->canonical) {
             int prc = HSPMM_OK;
             try { (void)build_panel_stream(p, st, rowOffset, tcA2B, data, rowIdx, p->cfg.kernel_mode >= 4, &prc); }
             catch (const std::bad_alloc &) { return bail(fail(HSPMM_ERR_ALLOC, "out of host memory")); }
@@ -1164,21 +1203,34 @@ void hspmm_destroy(hspmm_plan *p)
     (void)hipFree(p->panel.d_poff); (void)hipFree(p->panel.d_ids); (void)hipFree(p->panel.d_tiles);
     (void)hipFree(p->panel.d_unitRow);
     (void)hipFree(p->panel.d_step_panel);
-    (void)hipFree(p->panel.d_split); (void)hipFree(p->panel.d_fix_slots);
     (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive);
+    for (void *old : p->retired) (void)hipFree(old);
     delete p;
 }
 
 int hspmm_run(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream)
 {
-    return hspmm_run_marked(p, dB, dC, N, stream, nullptr);
+    return run_impl(p, dB, dC, N, stream, nullptr, RunMode::kLaunch);
+}
+
+int hspmm_prepare(hspmm_plan *p, uint32_t N)
+{
+    // B and C at the three alignments that select different load widths (and so different partitions and
+    // amounts of partial sums); nothing is launched and the pointers are never dereferenced
+    for (uintptr_t align : {uintptr_t(16), uintptr_t(8), uintptr_t(4)}) {
+        const int rc = run_impl(p, reinterpret_cast<const void *>(align), reinterpret_cast<void *>(align), N, nullptr,
+                                nullptr, RunMode::kPrepare);
+        if (rc) return rc;
+    }
+    return HSPMM_OK;
 }
 
 }  // extern "C"
 
 // Launch through the LDS-panel kernels.  Grid = row blocks x feature blocks x chunks of
 // panels; the chunk count is what it takes to have about two workgroups per compute unit.
-static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStream_t s, hipEvent_t mid)
+// The launch shape is a function of the plan and N alone.
+static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStream_t s, hipEvent_t mid, RunMode mode)
 {
     const hspmm_plan::Panel &pl = p->panel;
     hspmm::PanelArgs pa{};
@@ -1194,13 +1246,13 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     const bool wide = p->dtype != HSPMM_TF32 || pl.split;          // panels of 256 rows: always 12 + 4 waves
     int units = (pl.quad || wide) ? 13 : pl.G == 2 ? 14 : 12;
     int forced_units = 0;
-    if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) {                                      // tuning overrides
-        units = std::atoi(e) == 14 ? 14 : std::atoi(e) == 13 ? 13 : 12;
+    if (p->cfg.panel_units) {                                                                    // tuning overrides
+        units = p->cfg.panel_units;
         forced_units = units == 13 ? 12 : units;
         if (wide) { units = 13; forced_units = std::min(forced_units, 12); }
     }
-    if (const char *e = std::getenv("HSPMM_PANEL_UNITS_PER_GROUP"))      // fewer units than the shape has consumer waves
-        forced_units = std::max(1, std::min(std::atoi(e), units == 13 ? 12 : units));
+    if (p->cfg.panel_units_per_group)          // fewer units than the shape has consumer waves
+        forced_units = std::min(p->cfg.panel_units_per_group, units == 13 ? 12 : units);
     // (units of up to four windows: eight consumer waves with twice the accumulators)
     const int max_units = pl.G == 4 ? 8 : units == 13 ? 12 : units;
     if (forced_units) forced_units = std::min(forced_units, max_units);
@@ -1223,7 +1275,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     pa.units_per_group = uint32_t(best_units);
     const uint64_t row_blocks = (uint64_t(pl.n_units) + best_units - 1) / best_units;
     const uint64_t base = row_blocks * pa.n_feat_blocks;
-    if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) chunks = uint64_t(std::atoi(e));
+    if (p->cfg.panel_chunks) chunks = uint64_t(p->cfg.panel_chunks);
     if (chunks < 1) chunks = 1;
     if (chunks > pl.n_panels) chunks = pl.n_panels;
     pa.panels_per_chunk = uint32_t((pl.n_panels + chunks - 1) / chunks);
@@ -1232,33 +1284,40 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many workgroups", N);
     hspmm::KernelArgs ka{};
     if (pa.n_chunks > 1) {
-        int rc = ensure_panel_split(p, pa.n_chunks);
-        if (rc) return rc;
-        const size_t wide = pl.G == 4 ? 2u : 1u;
-        const size_t nacc = pl.quad ? 2u : pl.split ? 4u * wide : p->dtype != HSPMM_TF32 ? 8u * wide : 4u * size_t(pl.G);
+        const size_t wide_acc = pl.G == 4 ? 2u : 1u;
+        const size_t nacc = pl.quad ? 2u : pl.split ? 4u * wide_acc : p->dtype != HSPMM_TF32 ? 8u * wide_acc : 4u * size_t(pl.G);
         const size_t need = size_t(pl.n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
-        if ((rc = ensure_scratch(p, need))) return rc;
-        pa.scratch = p->d_scratch;
-        // (experiment, as in the gather kernels: the wave that brings a unit's last chunk adds the chunk sums
-        // itself; the device-scope accesses cost more than the second launch: 61.7 + 8.8 -> 76.8 us on the
-        // block-clustered configuration at N = 512)
-        if (p->cfg.fused_fixup) {
-            if ((rc = ensure_arrive(p, size_t(pl.n_units) * pa.n_feat_blocks))) return rc;
-            pa.arrive = p->d_arrive;
+        if (uint64_t(pl.n_units) * pa.n_chunks > 0xFFFFFFFFull)
+            return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many partial sums", N);
+        {
+            std::lock_guard<std::mutex> lk(p->mu);
+            int rc = scratch_for(p, need, mode, &pa.scratch);
+            if (rc) return rc;
+            // (experiment, as in the gather kernels: the wave that brings a unit's last chunk adds the chunk sums
+            // itself; the device-scope accesses cost more than the second launch: 61.7 + 8.8 -> 76.8 us on the
+            // block-clustered configuration at N = 512)
+            if (p->cfg.fused_fixup &&
+                (rc = ensure_arrive(p, size_t(pl.n_units) * pa.n_feat_blocks, &pa.arrive)))
+                return rc;
         }
+        // the chunk sums of unit u are slots u * chunks .. + chunks - 1: no table
         ka.unitRow = pl.d_unitRow; ka.ids = pl.d_ids; ka.tiles = pl.d_tiles;
-        ka.split = pl.d_split; ka.fix_slots = pl.d_fix_slots; ka.scratch = p->d_scratch;
+        ka.scratch = pa.scratch;
         ka.C = dC; ka.B = dB;
         ka.n_split = pl.n_units; ka.n_units = pl.n_units; ka.rows = p->rows; ka.N = N;
         ka.n_feat_blocks = pa.n_feat_blocks;
+        ka.uniform_chunks = pa.n_chunks;
     }
+    if (mode == RunMode::kPrepare) return HSPMM_OK;
+    p->last_family.store(3, std::memory_order_relaxed);
     HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : pl.G, pl.split, pa, ka, units, s, mid));
     return HSPMM_OK;
 }
 
-// mid: when not null, an event recorded between the main kernel and the kernel
-// that adds the partial sums of split windows.
-static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream, hipEvent_t mid)
+// One launch (or, kPrepare, everything a launch with this N and these pointer alignments would build).
+// mid: when not null, an event recorded between the main kernel and the kernel that adds the partial
+// sums of split windows.
+static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream, hipEvent_t mid, RunMode mode)
 {
     if (!p) return fail(HSPMM_ERR_INVALID, "null plan");
     if (N == 0) return fail(HSPMM_ERR_INVALID, "feature dimension N = 0");
@@ -1274,9 +1333,11 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
         if (dev != p->device)
             return fail(HSPMM_ERR_INVALID, "the plan was created on device %d, the current device is %d", p->device, dev);
     }
+    const bool launch = mode != RunMode::kPrepare;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (p->W == 0) {
-        p->last_family = 4;
+        if (!launch) return HSPMM_OK;
+        p->last_family.store(4, std::memory_order_relaxed);
         HSPMM_HIP(hspmm::launch_fill_zero(dC, size_t(p->rows) * N * p->elem, s));
         return HSPMM_OK;
     }
@@ -1287,7 +1348,7 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
         // (a 16-bit matrix near the break-even is served as fast or faster by the gather kernels while
         // one wave of theirs covers all of N)
         const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
-        if (pays && N % block_feat == 0 && !(align & 15u)) { p->last_family = 3; return run_panel(p, dB, dC, N, s, mid); }
+        if (pays && N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
     }
     const Choice c = choose_kernel(p, dB, dC, N);
     hspmm::KernelArgs ka{};
@@ -1295,11 +1356,11 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     ka.B = dB; ka.C = dC;
     ka.eff_windows = p->W; ka.rows = p->rows; ka.N = N;
     if (c.scalar) {
-        p->last_family = 1;
+        if (!launch) return HSPMM_OK;
+        p->last_family.store(1, std::memory_order_relaxed);
         HSPMM_HIP(hspmm::launch_spmm_scalar(p->dtype, ka, s));
         return HSPMM_OK;
     }
-    p->last_family = 2;
     ka.unitOffset = p->d_unitOffset; ka.unitRow = p->d_unitRow; ka.ids = p->d_ids; ka.tiles = p->d_tiles;
     ka.n_units = p->n_units;
     ka.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
@@ -1315,6 +1376,7 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     // One feature block: the waves of a workgroup walk consecutive ranges and add the partial sums of
     // one unit among themselves.
     int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
+    const bool fused = p->cfg.fused_fixup != 0;
     const bool combine = level == 0 && ka.n_feat_blocks == 1 && wpg > 1 && !p->cfg.fused_fixup;
     // Units that are all long (block-clustered, pruned or dense-ish random matrices at a small N): every
     // unit is cut into the ranges of one workgroup of four or eight waves, which stores it itself - no
@@ -1324,21 +1386,25 @@ static int hspmm_run_marked(hspmm_plan *p, const void *dB, void *dC, uint32_t N,
     const bool aligned = combine && p->aligned_group && c.narrow && p->cfg.consumer_warp_num == 0 &&
                          p->cfg.buffer_stage == 0 && p->cfg.producer_warp_group_num == 0;
     if (aligned) wpg = p->aligned_group;
-    int rc = build_and_upload_partition(p, level, combine ? uint32_t(wpg) : 1u, aligned);
-    if (rc) return rc;
-    const hspmm_plan::DevPartition &dp = p->parts[aligned ? 4 : combine ? 3 : level];
-    ka.ranges = dp.d_ranges; ka.split = dp.d_split; ka.fix_slots = dp.d_fix_slots;
-    ka.n_ranges = uint32_t(dp.part.ranges.size());
-    ka.n_split = uint32_t(dp.part.split.size());
-    if (uint64_t(ka.n_ranges) * ka.n_feat_blocks > 0x7FFFFFFFull)
-        return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many work items", N);
-    const size_t need = size_t(dp.part.n_slots) * ka.n_feat_blocks * size_t(c.V) * size_t(p->G) * 64u * 16u;
-    if ((rc = ensure_scratch(p, need))) return rc;
-    ka.scratch = p->d_scratch;
-    if (p->cfg.fused_fixup && ka.n_split) {
-        if ((rc = ensure_arrive(p, size_t(ka.n_split) * ka.n_feat_blocks))) return rc;
-        ka.arrive = p->d_arrive;
+    hspmm_plan::DevPartition &dp = p->parts[aligned ? 4 : combine ? 3 : level];
+    {
+        std::lock_guard<std::mutex> lk(p->mu);
+        if (!dp.built) {
+            const int rc = build_and_upload_partition(p, level, combine ? uint32_t(wpg) : 1u, aligned);
+            if (rc) return rc;
+        }
+        ka.n_ranges = uint32_t(dp.part.ranges.size());
+        ka.n_split = uint32_t(dp.part.split.size());
+        if (uint64_t(ka.n_ranges) * ka.n_feat_blocks > 0x7FFFFFFFull)
+            return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many work items", N);
+        const size_t need = size_t(dp.part.n_slots) * ka.n_feat_blocks * size_t(c.V) * size_t(p->G) * 64u * 16u;
+        int rc = scratch_for(p, need, mode, &ka.scratch);
+        if (rc) return rc;
+        if (fused && ka.n_split && (rc = ensure_arrive(p, size_t(ka.n_split) * ka.n_feat_blocks, &ka.arrive))) return rc;
     }
+    ka.ranges = dp.d_ranges; ka.split = dp.d_split; ka.fix_slots = dp.d_fix_slots;
+    if (!launch) return HSPMM_OK;
+    p->last_family.store(2, std::memory_order_relaxed);
     // default depth: what fits 128 registers per lane without spilling
     const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage
                          : p->dtype == HSPMM_TF32 ? (p->G == 2 && c.V == 4 ? 3 : 4)
@@ -1355,30 +1421,37 @@ int hspmm_profile(hspmm_plan *p, const void *dB, void *dC, uint32_t N, int runs,
     if (!main_ms || !fixup_ms) return fail(HSPMM_ERR_INVALID, "null output");
     if (runs < 1 || runs > 1000) return fail(HSPMM_ERR_INVALID, "runs %d outside 1..1000", runs);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    std::vector<hipEvent_t> ev(size_t(runs) * 3);
-    for (auto &e : ev) HSPMM_HIP(hipEventCreate(&e));
-    int rc = HSPMM_OK;
-    for (int i = 0; i < runs && !rc; ++i) {
+    // the events are destroyed on every way out
+    struct Events {
+        std::vector<hipEvent_t> ev;
+        ~Events() { for (hipEvent_t e : ev) (void)hipEventDestroy(e); }
+    } events;
+    events.ev.reserve(size_t(runs) * 3);
+    for (int i = 0; i < runs * 3; ++i) {
+        hipEvent_t e;
+        HSPMM_HIP(hipEventCreate(&e));
+        events.ev.push_back(e);
+    }
+    const std::vector<hipEvent_t> &ev = events.ev;
+    for (int i = 0; i < runs; ++i) {
         HSPMM_HIP(hipEventRecord(ev[3 * i], s));
-        rc = hspmm_run_marked(p, dB, dC, N, stream, ev[3 * i + 1]);
+        const int rc = run_impl(p, dB, dC, N, stream, ev[3 * i + 1], RunMode::kLaunch);
+        if (rc) return rc;
         HSPMM_HIP(hipEventRecord(ev[3 * i + 2], s));
     }
-    if (!rc) {
-        HSPMM_HIP(hipStreamSynchronize(s));
-        *main_ms = 0.f; *fixup_ms = 0.f;
-        for (int i = 0; i < runs; ++i) {
-            float a = 0.f, b = 0.f;
-            if (hipEventQuery(ev[3 * i + 1]) == hipSuccess && hipEventElapsedTime(&a, ev[3 * i], ev[3 * i + 1]) == hipSuccess) {
-                HSPMM_HIP(hipEventElapsedTime(&b, ev[3 * i + 1], ev[3 * i + 2]));
-            } else {                          // no split windows (or scalar kernel): one kernel only
-                (void)hipGetLastError();
-                HSPMM_HIP(hipEventElapsedTime(&a, ev[3 * i], ev[3 * i + 2]));
-            }
-            *main_ms += a; *fixup_ms += b;
+    HSPMM_HIP(hipStreamSynchronize(s));
+    *main_ms = 0.f; *fixup_ms = 0.f;
+    for (int i = 0; i < runs; ++i) {
+        float a = 0.f, b = 0.f;
+        if (hipEventQuery(ev[3 * i + 1]) == hipSuccess && hipEventElapsedTime(&a, ev[3 * i], ev[3 * i + 1]) == hipSuccess) {
+            HSPMM_HIP(hipEventElapsedTime(&b, ev[3 * i + 1], ev[3 * i + 2]));
+        } else {                          // no split windows (or scalar kernel): one kernel only
+            (void)hipGetLastError();
+            HSPMM_HIP(hipEventElapsedTime(&a, ev[3 * i], ev[3 * i + 2]));
         }
+        *main_ms += a; *fixup_ms += b;
     }
-    for (auto &e : ev) (void)hipEventDestroy(e);
-    return rc;
+    return HSPMM_OK;
 }
 
 int hspmm_bench(hspmm_plan *p, const void *dB, void *dC, uint32_t N, int warmup, int runs, void *stream,
@@ -1390,17 +1463,18 @@ int hspmm_bench(hspmm_plan *p, const void *dB, void *dC, uint32_t N, int warmup,
     int rc;
     for (int i = 0; i < warmup; ++i)
         if ((rc = hspmm_run(p, dB, dC, N, stream))) return rc;
-    hipEvent_t a, b;
-    HSPMM_HIP(hipEventCreate(&a));
-    HSPMM_HIP(hipEventCreate(&b));
-    HSPMM_HIP(hipEventRecord(a, s));
+    struct Pair {
+        hipEvent_t a = nullptr, b = nullptr;
+        ~Pair() { if (a) (void)hipEventDestroy(a); if (b) (void)hipEventDestroy(b); }
+    } ev;
+    HSPMM_HIP(hipEventCreate(&ev.a));
+    HSPMM_HIP(hipEventCreate(&ev.b));
+    HSPMM_HIP(hipEventRecord(ev.a, s));
     for (int i = 0; i < runs; ++i)
-        if ((rc = hspmm_run(p, dB, dC, N, stream))) { (void)hipEventDestroy(a); (void)hipEventDestroy(b); return rc; }
-    HSPMM_HIP(hipEventRecord(b, s));
-    HSPMM_HIP(hipEventSynchronize(b));
-    HSPMM_HIP(hipEventElapsedTime(total_ms, a, b));
-    HSPMM_HIP(hipEventDestroy(a));
-    HSPMM_HIP(hipEventDestroy(b));
+        if ((rc = hspmm_run(p, dB, dC, N, stream))) return rc;
+    HSPMM_HIP(hipEventRecord(ev.b, s));
+    HSPMM_HIP(hipEventSynchronize(ev.b));
+    HSPMM_HIP(hipEventElapsedTime(total_ms, ev.a, ev.b));
     return HSPMM_OK;
 }
 
@@ -1421,7 +1495,7 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_panel_units = p->panel.built ? p->panel.n_units : 0u;
     info->n_panel_paired_units = p->panel.built ? p->panel.n_paired : 0u;
     info->n_panel_wide_units = p->panel.built ? p->panel.n_wide : 0u;
-    info->last_kernel_family = p->last_family;
+    info->last_kernel_family = p->last_family.load(std::memory_order_relaxed);
     return HSPMM_OK;
 }
 

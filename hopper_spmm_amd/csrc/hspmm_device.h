@@ -37,6 +37,8 @@ struct KernelArgs {
     const void     *B;           // cols x N
     void           *C;           // rows x N
     uint32_t n_ranges, n_split, eff_windows, n_units, rows, N, n_feat_blocks;
+    uint32_t uniform_chunks;     // != 0 (LDS-panel kernels): no split table - entry e is unit e, whose partial sums
+                                 // are slots e * uniform_chunks .. + uniform_chunks - 1, in that order
 };
 
 // dtype: 0 = fp16 tiles 8x16, 1 = fp32 tiles 8x8, 2 = bf16 tiles 8x16.  V = 32-bit words a lane loads

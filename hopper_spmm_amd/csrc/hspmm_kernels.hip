@@ -61,12 +61,19 @@ void spmm_scalar_kernel(const KernelArgs ka)
         for (uint32_t r = 0; r < row0; ++r) C[size_t(r) * N + f] = from_f32<T>(0.f);
 }
 
-// Whole-matrix clear for a matrix without any stored entry (every row of C is 0).
-__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t *dst, size_t n_words, uint16_t *tail, int tail_halves)
+// Whole-matrix clear for a matrix without any stored entry (every row of C is 0).  dst is aligned to
+// two bytes: one half in front of the first whole word when dst starts inside one, whole words, one half behind.
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint16_t *dst, size_t n_halves)
 {
+    const size_t head = (reinterpret_cast<uintptr_t>(dst) & 2u) ? 1u : 0u;
+    const size_t n_words = (n_halves - head) / 2u;
+    uint32_t *words = reinterpret_cast<uint32_t *>(dst + head);
     const size_t stride = size_t(gridDim.x) * blockDim.x;
-    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n_words; i += stride) dst[i] = 0u;
-    if (blockIdx.x == 0 && threadIdx.x < (unsigned)tail_halves) tail[threadIdx.x] = 0;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n_words; i += stride) words[i] = 0u;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        if (head) dst[0] = 0;
+        if (head + 2u * n_words < n_halves) dst[n_halves - 1u] = 0;
+    }
 }
 
 #define HSPMM_DECLARE_LAUNCH(name) \
@@ -114,14 +121,13 @@ hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s)
 
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s)
 {
-    // bytes is a multiple of 2 (fp16) or 4 (fp32); dst is at least 4-byte aligned.
-    const size_t words = bytes / 4;
-    const int tail = int((bytes % 4) / 2);
-    size_t blocks = (words + 255) / 256;
+    // bytes is a multiple of the element size (2 or 4) and dst is aligned to it
+    const size_t halves = bytes / 2;
+    if (halves == 0) return hipSuccess;
+    size_t blocks = (halves / 2 + 255) / 256;
     if (blocks > 4096) blocks = 4096;
     if (blocks == 0) blocks = 1;
-    fill_zero_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(reinterpret_cast<uint32_t *>(dst), words,
-                                                          reinterpret_cast<uint16_t *>(dst) + words * 2, tail);
+    fill_zero_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(reinterpret_cast<uint16_t *>(dst), halves);
     return hipGetLastError();
 }
 

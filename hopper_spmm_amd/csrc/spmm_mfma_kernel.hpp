@@ -712,8 +712,12 @@ void spmm_fixup_kernel(const KernelArgs ka)
     if (item >= ka.n_split * ka.n_feat_blocks) return;
     const uint32_t entry = item / ka.n_feat_blocks;
     const uint32_t fb = item - entry * ka.n_feat_blocks;
-    const uint32_t *fx = ka.split + size_t(entry) * kFixWords;
-    const uint32_t u = fx[0], sb = fx[1], sc = fx[2];
+    // one table entry per cut unit, or (uniform_chunks) every unit cut the same number of ways
+    const bool uniform = ka.uniform_chunks != 0u;
+    const uint32_t *fx = ka.split + size_t(uniform ? 0u : entry) * kFixWords;
+    const uint32_t u = uniform ? entry : fx[0];
+    const uint32_t sb = uniform ? entry * ka.uniform_chunks : fx[1];
+    const uint32_t sc = uniform ? ka.uniform_chunks : fx[2];
 
     typename TT::Lane L;
     L.init(lane, ka.tiles, ka.ids);
@@ -728,7 +732,7 @@ void spmm_fixup_kernel(const KernelArgs ka)
     // the additions keep the slot order; the loads of four slots are in flight together
 #pragma unroll 4
     for (uint32_t i = 0; i < sc; ++i) {
-        const uint32_t slot = ka.fix_slots[sb + i];
+        const uint32_t slot = uniform ? sb + i : ka.fix_slots[sb + i];
         const f32x4 *src = reinterpret_cast<const f32x4 *>(ka.scratch) +
                            (size_t(slot) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
 #pragma unroll

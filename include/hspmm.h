@@ -52,7 +52,14 @@ typedef struct hspmm_plan hspmm_plan;
  * src/fp16.cu:228-249) and create_tma_desc_A (src/fp16.cu:177-219): validates
  * the four format arrays (host pointers), copies them to the current HIP
  * device and builds the work partition the kernels walk.  `dtype` is
- * HSPMM_FP16, HSPMM_TF32 or HSPMM_BF16. */
+ * HSPMM_FP16, HSPMM_TF32 or HSPMM_BF16.
+ * Column lists: the reference's converter writes every window's real column
+ * ids strictly ascending, with padding only behind the window's last column
+ * (src/utils/convert.h:166-181).  Other orders are accepted (ids < cols,
+ * padding only at the end of a tile) and give the same product, but such a plan
+ * runs the gather and all-shapes kernels only: the LDS-staging kernels, and the
+ * merging of adjacent windows, need the ascending order.
+ * Tuning variables of the environment (HSPMM_*) are read here, once per plan. */
 int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
                  uint32_t eff_row_windows, uint32_t total_tiles,
                  const uint32_t *rowOffset, const uint32_t *tcA2B,
@@ -64,12 +71,26 @@ int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
  * 4 bytes and an even N for the 16-bit types, the LDS-staging kernels 16 bytes;
  * anything else runs through the all-shapes kernel); every element of C is
  * written (rows without nonzeros become 0).  Asynchronous on `stream` (a
- * hipStream_t, NULL = default stream).  A plan owns scratch memory, so launches
- * of one plan must not overlap in time; different plans may run concurrently.
- * The first call for a feature dimension may allocate that memory and build a
- * work partition for it; later calls with the same N only launch kernels and
- * can be captured in a HIP graph. */
+ * hipStream_t, NULL = default stream).
+ * Host side: a plan is immutable after hspmm_create except for what the first
+ * launch with a new N may add under the plan's own mutex - a work partition for
+ * that width and a larger buffer for partial sums (older buffers stay allocated
+ * until hspmm_destroy, so launches recorded earlier, e.g. in a HIP graph, stay
+ * valid whatever N is run afterwards).  hspmm_run may therefore be called from
+ * several threads; after hspmm_prepare(plan, N), or one earlier call with that
+ * N, it only launches kernels (no allocation, memset or copy) and can be
+ * captured in a HIP graph.
+ * Device side: launches of one plan share its partial-sum buffer, so two
+ * launches of one plan must not overlap in time (one stream per plan, or an
+ * event between them); different plans may run concurrently. */
 int hspmm_run(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stream);
+
+/* No reference counterpart (the reference allocates inside every call,
+ * src/fp16.cu:236-249): builds now what the first hspmm_run with feature
+ * dimension N would build - the work partition for that width and the buffer
+ * for partial sums, for every alignment of B and C - and launches nothing. */
+int hspmm_prepare(hspmm_plan *plan, uint32_t N);
+
 
 /* Replaces the warm-up + timed loop of fp16_spmm (reference src/fp16.cu:254-268,
  * WARMUP_RUNS / RUNS of src/common.h:48-49): `warmup` untimed launches, then

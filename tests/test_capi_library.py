@@ -114,3 +114,4 @@ def test_operator_fails_loudly_without_a_gfx950_device(hs):
     with pytest.raises(hs.HspmmError) as e:
         hs.Plan(ok)
     assert e.value.code == 2                              # HSPMM_ERR_DEVICE: no CPU fallback exists
+

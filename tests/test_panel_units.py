@@ -145,3 +145,37 @@ def test_preview_rejects_bad_arguments(hs):
     bad = dict(b, rowIdx=b["rowIdx"][::-1].copy())
     with pytest.raises(hs.HspmmError):
         hs.panel_units_preview(bad, 2)
+
+
+def test_lists_that_do_not_ascend_or_repeat_an_id_are_never_merged(hs):
+    """The gather and all-shapes kernels take any column order; merging windows and the LDS-staging
+    stream need strictly ascending lists with padding only behind a window's last column.  A matrix
+    that breaks that rule anywhere comes back from the preview unmerged and unchanged."""
+    def matrix(lists, cols=400):
+        W = len(lists)
+        a2b = np.full((W, 16), IDX_MAX, np.uint32)
+        data = np.zeros((W, 8, 16), np.uint16)
+        for w, ids in enumerate(lists):
+            a2b[w, :len(ids)] = ids
+            for k in range(len(ids)):
+                data[w, (w + k) % 8, k] = encode(np.array([1.0 + k]), 0)[0]
+        return dict(rows=8 * W, cols=cols, dtype=0, cw=16, eff_row_windows=W, total_tiles=W,
+                    rowOffset=np.arange(W + 1, dtype=np.uint32), rowIdx=8 * np.arange(W, dtype=np.uint32),
+                    tcA2B=a2b.ravel(), data=data.ravel())
+    for lists in ([[5, 5, 9, 300], [5, 5, 9, 300]],          # a repeated id, both windows alike
+                  [[9, 5, 300], [5, 9, 300]],                # descending
+                  [[5, 9, 300], [5, 9, 300], [7, 7]]):       # one bad window spoils the plan's merging altogether
+        b = matrix(lists)
+        g = hs.panel_units_preview(b, 4)
+        assert np.array_equal(g["group_count"], np.ones(len(lists), np.uint32)), lists
+        assert g["total_tiles"] == b["total_tiles"]
+        assert np.array_equal(g["tcA2B"], b["tcA2B"]) and np.array_equal(g["data"], b["data"])
+    # the same lists in canonical form do merge
+    g = hs.panel_units_preview(matrix([[5, 9, 300], [5, 9, 300]]), 4)
+    assert np.array_equal(g["group_count"], [2])
+    # padding inside a window (a tile that is not the window's last ends in padding) also keeps it unmerged
+    b = matrix([[1, 2, 3], [1, 2, 3]])
+    two = dict(b, eff_row_windows=1, total_tiles=2, rowOffset=np.array([0, 2], np.uint32), rowIdx=np.array([0], np.uint32),
+               rows=8)
+    g = hs.panel_units_preview(two, 4)
+    assert np.array_equal(g["group_count"], [1]) and g["total_tiles"] == 2

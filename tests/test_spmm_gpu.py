@@ -817,6 +817,58 @@ def test_run_captured_in_a_hip_graph_replays_correctly(torch_cuda, hs, oracle):
         plan.close()
 
 
+def test_graph_captured_at_one_width_survives_launches_at_another(torch_cuda, hs, oracle):
+    """A launch recorded in a HIP graph carries the addresses of the plan's partial-sum buffer and
+    tables.  Running the same plan eagerly at a wider N afterwards (more partial sums, another number
+    of chunks) must leave the recorded launch valid: replays stay bit-identical to the eager result."""
+    torch = torch_cuda
+    rng = np.random.default_rng(16)
+    for dtype, panels in ((0, False), (0, True), (1, True)):
+        if panels:
+            A = random_csr(rng, 400, 4000, 0.1, dtype, 0.1)
+            b = convert(hs, A)
+            plan = hs.Plan(b)
+            assert plan.info()["n_panels"] > 0
+            N1, N2 = 128, 1024
+        else:
+            A = random_csr(rng, 400, 4000, 0.003, dtype, 0.1, (3, 200))
+            b = convert(hs, A)
+            hs.configure(producer_warp_group_num=16)
+            try:
+                plan = hs.Plan(b)
+            finally:
+                hs.configure()
+            assert plan.info()["n_split_windows"] > 0
+            N1, N2 = 64, 512
+        B1, B2 = make_b(rng, 4000, N1, dtype), make_b(rng, 4000, N2, dtype)
+        want1 = gpu_spmm(torch, hs, b, B1, N1, plan=plan)         # eager: sizes the buffers for N1
+        tt = torch.int16 if dtype == 0 else torch.float32
+        as_t = (lambda x: torch.from_numpy(x.view(np.int16))) if dtype == 0 else torch.from_numpy
+        dB = as_t(B1).cuda()
+        dC = torch.empty((400, N1), dtype=tt, device="cuda")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            plan.run(dB.data_ptr(), dC.data_ptr(), N1, torch.cuda.current_stream().cuda_stream)
+        bytes_before = plan.info()["device_bytes"]
+        got2 = gpu_spmm(torch, hs, b, B2, N2, plan=plan)          # a wider launch on the same plan
+        assert plan.info()["device_bytes"] > bytes_before, "the wider launch was meant to need more partial sums"
+        ref2, mag2 = oracle_spmm(oracle, A, B2, N2)
+        assert_parity(got2, ref2, mag2, dtype, "wide launch")
+        for rep in range(3):
+            dC.fill_(0x7E01 if dtype == 0 else float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = dC.cpu().numpy()
+            got = got.view(np.uint16) if dtype == 0 else got
+            assert np.array_equal(got.view(np.uint8), want1.view(np.uint8)), "dtype %d panels %s replay %d" % (dtype, panels, rep)
+            gpu_spmm(torch, hs, b, B2, N2, plan=plan)             # and again something else in between
+        del graph
+        plan.close()
+
+
 def test_bench_entry_point_and_errors(torch_cuda, hs, oracle):
     torch = torch_cuda
     rng = np.random.default_rng(3)
