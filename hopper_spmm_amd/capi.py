@@ -88,6 +88,7 @@ def load_library():
     L.hspmm_last_error.restype = C.c_char_p
     L.hspmm_create.argtypes = [C.POINTER(vp), i, u32, u32, u32, u32, vp, vp, vp, vp]
     L.hspmm_run.argtypes = [vp, vp, vp, u32, vp]
+    L.hspmm_run_static.argtypes = [vp, vp, vp, u32, vp]
     L.hspmm_prepare.argtypes = [vp, u32]
     L.hspmm_bench.argtypes = [vp, vp, vp, u32, i, i, vp, C.POINTER(C.c_float)]
     L.hspmm_profile.argtypes = [vp, vp, vp, u32, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_float)]
@@ -396,6 +397,12 @@ class Plan:
     def run(self, dB_ptr, dC_ptr, N, stream=0):
         """dB_ptr / dC_ptr: integer device addresses (e.g. torch tensor .data_ptr())."""
         _check(load_library().hspmm_run(self._h, C.c_void_p(dB_ptr), C.c_void_p(dC_ptr), N, C.c_void_p(stream)))
+
+    def run_static(self, dB_ptr, dC_ptr, N, stream=0):
+        """hspmm_run_static: the same launch with its partial sums in the library's fixed device array
+        (no allocation; the partition for N must exist: prepare(N) or one run with N first)."""
+        _check(load_library().hspmm_run_static(self._h, C.c_void_p(dB_ptr), C.c_void_p(dC_ptr), N,
+                                               C.c_void_p(stream)))
 
     def prepare(self, N):
         """hspmm_prepare: builds what the first run with feature dimension N would build; launches nothing."""

@@ -21,6 +21,11 @@
 #include "partition.hpp"
 #include "host_parallel.hpp"
 
+// The fixed scratch array of hspmm_run_static (see static_scratch_address below): device memory the
+// library holds on every device it is loaded on, for callers that must not allocate.
+constexpr size_t kStaticScratchBytes = HSPMM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char hspmm_static_scratch[kStaticScratchBytes];
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -858,9 +863,33 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
 // How a launch gets the memory it needs beyond the plan's fixed arrays.
 //   kLaunch:  hspmm_run - may build a partition and grow the plan's scratch buffer (under the plan's mutex)
 //   kPrepare: hspmm_prepare - builds and grows exactly like kLaunch and launches nothing
-enum class RunMode { kLaunch, kPrepare };
+//   kStatic:  hspmm_run_static - partial sums go to the library's fixed device array; builds and allocates nothing
+enum class RunMode { kLaunch, kPrepare, kStatic };
 
-// Arrival counters of the in-kernel reduction (an experiment switch).
+// The fixed scratch array of hspmm_run_static: one copy per device, held from the moment the library is
+// loaded on that device until the process ends.  Host code never passes the array's name to a kernel (on
+// the host it names a stand-in, not device memory): the device address is looked up once per device with
+// hipGetSymbolAddress and that pointer is what launches carry.
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+void *g_static_scratch_ptr[kMaxDevices] = {};
+
+// `device` must be the current device.
+int static_scratch_address(int device, float **out)
+{
+    if (device < 0 || device >= kMaxDevices) return fail(HSPMM_ERR_UNSUPPORTED, "device %d: at most %d devices", device, kMaxDevices);
+    std::lock_guard<std::mutex> lk(g_static_mutex);
+    if (!g_static_scratch_ptr[device]) {
+        void *ptr = nullptr;
+        HSPMM_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(hspmm_static_scratch)));
+        if (!ptr) return fail(HSPMM_ERR_DEVICE, "hipGetSymbolAddress gave no address for the static scratch array");
+        g_static_scratch_ptr[device] = ptr;
+    }
+    *out = static_cast<float *>(g_static_scratch_ptr[device]);
+    return HSPMM_OK;
+}
+
+// Arrival counters of the in-kernel reduction (an experiment switch, never used by hspmm_run_static).
 // Called with the plan's mutex held.
 int ensure_arrive(hspmm_plan *p, size_t words, uint32_t **out)
 {
@@ -877,11 +906,18 @@ int ensure_arrive(hspmm_plan *p, size_t words, uint32_t **out)
     return HSPMM_OK;
 }
 
-// The buffer for `bytes` of partial sums: the plan's buffer, grown when too small (sizes are powers of two, so the superseded buffers, which stay
+// The buffer for `bytes` of partial sums.  kStatic: the device's fixed array (bytes must fit).  Else the
+// plan's buffer, grown when too small (sizes are powers of two, so the superseded buffers, which stay
 // allocated until hspmm_destroy, never add up to more than the current one).  Called with the plan's mutex held.
 int scratch_for(hspmm_plan *p, size_t bytes, RunMode mode, float **out)
 {
-    (void)mode;
+    if (mode == RunMode::kStatic) {
+        if (bytes > kStaticScratchBytes)
+            return fail(HSPMM_ERR_UNSUPPORTED,
+                        "hspmm_run_static: this launch needs %zu bytes of partial sums, the fixed array holds %zu "
+                        "(use hspmm_run)", bytes, kStaticScratchBytes);
+        return static_scratch_address(p->device, out);
+    }
     if (bytes > p->scratch_bytes) {
         size_t cap = size_t(1) << 16;
         while (cap < bytes) cap <<= 1;
@@ -1081,6 +1117,11 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         return bail(fail(HSPMM_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only", p->device,
                          prop.gcnArchName));
     p->compute_units = p->cfg.sm_num > 0 ? p->cfg.sm_num : prop.multiProcessorCount;
+    {
+        // the address of this device's fixed scratch array, for hspmm_run_static (which then looks nothing up)
+        float *unused = nullptr;
+        if ((rc = static_scratch_address(p->device, &unused))) return bail(rc);
+    }
 
     if (p->W) {
         const size_t n_ids = size_t(total_tiles) * cw;
@@ -1213,6 +1254,11 @@ int hspmm_run(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream)
     return run_impl(p, dB, dC, N, stream, nullptr, RunMode::kLaunch);
 }
 
+int hspmm_run_static(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream)
+{
+    return run_impl(p, dB, dC, N, stream, nullptr, RunMode::kStatic);
+}
+
 int hspmm_prepare(hspmm_plan *p, uint32_t N)
 {
     // B and C at the three alignments that select different load widths (and so different partitions and
@@ -1296,7 +1342,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
             // (experiment, as in the gather kernels: the wave that brings a unit's last chunk adds the chunk sums
             // itself; the device-scope accesses cost more than the second launch: 61.7 + 8.8 -> 76.8 us on the
             // block-clustered configuration at N = 512)
-            if (p->cfg.fused_fixup &&
+            if (p->cfg.fused_fixup && mode != RunMode::kStatic &&
                 (rc = ensure_arrive(p, size_t(pl.n_units) * pa.n_feat_blocks, &pa.arrive)))
                 return rc;
         }
@@ -1376,7 +1422,7 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     // One feature block: the waves of a workgroup walk consecutive ranges and add the partial sums of
     // one unit among themselves.
     int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
-    const bool fused = p->cfg.fused_fixup != 0;
+    const bool fused = p->cfg.fused_fixup && mode != RunMode::kStatic;
     const bool combine = level == 0 && ka.n_feat_blocks == 1 && wpg > 1 && !p->cfg.fused_fixup;
     // Units that are all long (block-clustered, pruned or dense-ish random matrices at a small N): every
     // unit is cut into the ranges of one workgroup of four or eight waves, which stores it itself - no
@@ -1390,6 +1436,10 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     {
         std::lock_guard<std::mutex> lk(p->mu);
         if (!dp.built) {
+            if (mode == RunMode::kStatic)
+                return fail(HSPMM_ERR_UNSUPPORTED,
+                            "hspmm_run_static: the work partition for N = %u is not built yet; call hspmm_prepare(plan, N) "
+                            "or hspmm_run once with this N first", N);
             const int rc = build_and_upload_partition(p, level, combine ? uint32_t(wpg) : 1u, aligned);
             if (rc) return rc;
         }

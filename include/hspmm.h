@@ -91,6 +91,19 @@ int hspmm_run(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stre
  * for partial sums, for every alignment of B and C - and launches nothing. */
 int hspmm_prepare(hspmm_plan *plan, uint32_t N);
 
+/* No reference counterpart; for callers that must not allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): hspmm_run with the partial sums of cut windows kept in a fixed
+ * array of device memory that the library holds on every device it is loaded
+ * on (HSPMM_STATIC_SCRATCH_BYTES, from library load until the process ends)
+ * instead of the plan's own buffer.  It calls no hipMalloc / hipFree and builds
+ * nothing: the work partition for this N must exist already (hspmm_prepare, or
+ * one hspmm_run with this N), else HSPMM_ERR_UNSUPPORTED; so does a launch whose
+ * partial sums exceed the array (the message says how much it needs).  Results
+ * are bit-identical to hspmm_run.  All calls on one device share the one array
+ * whatever their plan: two calls that overlap in time on one device race. */
+#define HSPMM_STATIC_SCRATCH_BYTES (32u << 20)
+int hspmm_run_static(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stream);
 
 /* Replaces the warm-up + timed loop of fp16_spmm (reference src/fp16.cu:254-268,
  * WARMUP_RUNS / RUNS of src/common.h:48-49): `warmup` untimed launches, then

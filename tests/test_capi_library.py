@@ -115,3 +115,24 @@ def test_operator_fails_loudly_without_a_gfx950_device(hs):
         hs.Plan(ok)
     assert e.value.code == 2                              # HSPMM_ERR_DEVICE: no CPU fallback exists
 
+
+def test_static_scratch_array_is_a_visible_symbol_of_the_device_code(hs):
+    """hspmm_run_static finds its fixed device array with hipGetSymbolAddress, which looks the array up
+    by name in the gfx950 code object: the symbol must be there with global binding (a file-scope
+    static that the compiler leaves local, e.g. one marked `used`, cannot be found at run time)."""
+    import shutil
+    import subprocess
+    import tempfile
+    tools = "/opt/rocm/llvm/bin"
+    obj = os.path.join(ROOT, "hopper_spmm_amd", "csrc", "build", "hspmm_capi.hip.o")
+    if not (os.path.exists(obj) and shutil.which(os.path.join(tools, "clang-offload-bundler"))):
+        pytest.skip("needs the object file of the last build and the ROCm llvm tools")
+    with tempfile.TemporaryDirectory() as d:
+        fat, dev = os.path.join(d, "fatbin"), os.path.join(d, "dev.o")
+        subprocess.check_call([os.path.join(tools, "llvm-objcopy"), "--dump-section", ".hip_fatbin=" + fat, obj])
+        subprocess.check_call([os.path.join(tools, "clang-offload-bundler"), "--unbundle", "--type=o", "--input=" + fat,
+                               "--targets=hipv4-amdgcn-amd-amdhsa--gfx950", "--output=" + dev])
+        table = subprocess.check_output([os.path.join(tools, "llvm-readelf"), "-s", dev], text=True)
+    rows = [l.split() for l in table.splitlines() if "hspmm_static_scratch" in l]
+    assert rows, "the static scratch array is not in the device code object"
+    assert all(r[4] == "GLOBAL" and int(r[2]) == 32 << 20 for r in rows), rows

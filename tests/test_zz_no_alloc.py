@@ -1,0 +1,116 @@
+"""hspmm_run_static - the entry point that allocates nothing: the partial sums of cut windows go to a
+fixed array of device memory that the library holds, not to a buffer of the plan.  Its output must be
+bit-identical to hspmm_run's, call after call, also when a later call is smaller than the one before
+(the array keeps the earlier call's contents).  Needs a real MI355X: run with -m gpu."""
+import numpy as np
+import pytest
+
+from util import random_csr
+from test_spmm_gpu import torch_cuda, convert, make_b, oracle_spmm, assert_parity  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+
+def _device_buffers(torch, B, rows, N, dtype):
+    if dtype != 1:
+        dB = torch.from_numpy(np.ascontiguousarray(B, np.uint16).view(np.int16)).cuda()
+        dC = torch.empty((rows, N), dtype=torch.int16, device="cuda")
+    else:
+        dB = torch.from_numpy(np.ascontiguousarray(B, np.float32)).cuda()
+        dC = torch.empty((rows, N), dtype=torch.float32, device="cuda")
+    return dB, dC
+
+
+def _poison(dC, dtype):
+    dC.fill_(0x7E01 if dtype != 1 else float("nan"))
+
+
+def _result(dC, dtype):
+    out = dC.cpu().numpy()
+    return out.view(np.uint16) if dtype != 1 else out
+
+
+def _cases(hs, rng, dtype):
+    """(name, CSR, N, configure keywords): first a large call, then a smaller one; both with windows cut
+    across waves (gather kernels, two kernels per call), then the LDS-staging kernels with chunk sums."""
+    heavy = dict(producer_warp_group_num=16)
+    yield "gather, large", random_csr(rng, 640, 6000, 0.004, dtype, 0.1, (5, 17, 300)), 128, heavy
+    yield "gather, small", random_csr(rng, 200, 3000, 0.004, dtype, 0.1, (9,)), 64, heavy
+    yield "panel, large", random_csr(rng, 480, 4000, 0.1, dtype, 0.05), 256, {}
+    yield "panel, small", random_csr(rng, 160, 2000, 0.1, dtype, 0.05), 128, {}
+
+
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_static_scratch_entry_point_matches_hspmm_run(torch_cuda, hs, oracle, dtype):
+    torch = torch_cuda
+    rng = np.random.default_rng(700 + dtype)
+    stream = torch.cuda.current_stream().cuda_stream
+    for name, A, N, knobs in _cases(hs, rng, dtype):
+        b = convert(hs, A)
+        hs.configure(**knobs)
+        try:
+            plan = hs.Plan(b)
+        finally:
+            hs.configure()
+        info = plan.info()
+        B = make_b(rng, A["cols"], N, dtype)
+        dB, dC = _device_buffers(torch, B, A["rows"], N, dtype)
+        # 16-bit types, one wave covers all of N: the launch wants the partition whose workgroups add their
+        # waves' sums, which hspmm_create has not built - the entry point must refuse instead of building it
+        if info["n_panels"] == 0 and dtype != 1:
+            with pytest.raises(hs.HspmmError) as e:
+                plan.run_static(dB.data_ptr(), dC.data_ptr(), N, stream)
+            assert "hspmm_prepare" in str(e.value)
+        plan.prepare(N)
+        before = torch.cuda.memory_allocated(), plan.info()["device_bytes"]
+        _poison(dC, dtype)
+        plan.run_static(dB.data_ptr(), dC.data_ptr(), N, stream)
+        torch.cuda.synchronize()
+        got = _result(dC, dtype)
+        assert plan.info()["device_bytes"] == before[1], name + ": the plan's device memory changed"
+        # the existing entry point, same plan, same inputs
+        _poison(dC, dtype)
+        plan.run(dB.data_ptr(), dC.data_ptr(), N, stream)
+        torch.cuda.synchronize()
+        want = _result(dC, dtype)
+        family = plan.info()["last_kernel_family"]
+        assert family == (3 if name.startswith("panel") else 2), (name, family)
+        if name.startswith("gather"):
+            assert info["n_split_windows"] > 0, name + ": no window is cut, nothing would use scratch memory"
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), name + ": differs from hspmm_run"
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        assert_parity(got, ref, mag, dtype, name)
+        # again, into the array the call above left its sums in
+        _poison(dC, dtype)
+        plan.run_static(dB.data_ptr(), dC.data_ptr(), N, stream)
+        torch.cuda.synchronize()
+        assert np.array_equal(_result(dC, dtype).view(np.uint8), want.view(np.uint8)), name + ": second call differs"
+        plan.close()
+
+
+def test_static_scratch_entry_point_rejects_what_does_not_fit(torch_cuda, hs):
+    """A launch whose partial sums exceed the fixed array is refused with a message that says so."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    # every window far longer than a range, many ranges, wide N: tens of MB of partial sums
+    A = random_csr(rng, 2048, 8192, 0.25, 0)
+    b = convert(hs, A)
+    hs.set_kernel_mode(3)
+    hs.configure(producer_warp_group_num=16)
+    try:
+        plan = hs.Plan(b)
+    finally:
+        hs.configure()
+        hs.set_kernel_mode(0)
+    N = 2048
+    plan.prepare(N)
+    assert plan.info()["device_bytes"] > 2 * (32 << 20)          # the plan's own buffer for this N is far larger
+    dB = torch.zeros((8192, N), dtype=torch.int16, device="cuda")
+    dC = torch.zeros((2048, N), dtype=torch.int16, device="cuda")
+    with pytest.raises(hs.HspmmError) as e:
+        plan.run_static(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)
+    assert "fixed array holds" in str(e.value), str(e.value)
+    plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)   # the allocating entry point serves it
+    torch.cuda.synchronize()
+    assert not dC.any().item()
+    plan.close()
