@@ -65,6 +65,10 @@ def cpu_baseline(A, B, N, flops_full):
     }
 
 
+def info_family(plan):
+    return plan.info()["last_kernel_family"]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -142,6 +146,29 @@ def main():
     # the reference's own convention: 3 warm-ups, 5 timed launches (src/common.h:48-49)
     ref_conv_ms = plan.bench(pB, pC, N, warmup=3, runs=5, stream=stream) / 5.0
 
+    # floor of the gather kernels: the same row gathers and nothing else, measured in this run
+    gather_floor = None
+    if info_family(plan) == 2 and (N * (2 if dt != 1 else 4)) % 128 == 0:
+        g_ms, g_bytes = plan.measure_gather(pB, N, runs=5, stream=stream)
+        gather_floor = {"ms": g_ms, "bytes": g_bytes}
+    # the fp32-storage variant has two arithmetic forms in the LDS-panel kernels: bf16 hi / lo parts in
+    # three products (default) and true fp32 MFMA products (kernel mode 5); both are timed
+    fp32_products = None
+    if dt == 1 and info_family(plan) == 3 and args.mode == 0:
+        hs.set_kernel_mode(5)
+        try:
+            plan5 = hs.Plan(b)
+        finally:
+            hs.set_kernel_mode(0)
+        for _ in range(args.warmup):
+            plan5.run(pB, pC, N, stream)
+        m5, f5 = plan5.profile(pB, pC, N, runs=args.steps, stream=stream)
+        fp32_products = {"kernel_ms": m5 / args.steps, "fixup_kernel_ms": f5 / args.steps,
+                         "arithmetic": "v_mfma_f32_4x4x1 / 16x16x4 on fp32 inputs (hspmm_set_kernel_mode(5))"}
+        plan5.close()
+        plan.run(pB, pC, N, stream)                  # the default plan is the last one that ran
+        torch.cuda.synchronize()
+
     if args.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")       # 1 GiB read + 1 GiB written
         dst = torch.empty_like(src)
@@ -161,6 +188,7 @@ def main():
         with open(tfile) as f:
             traffic = json.load(f).get("config%d_N%d" % (args.config, N))
 
+    kernels_ms = main_ms + fix_ms
     out = {
         "metric": "SpMM effective TFLOP/s (2*nnz*N)",
         "value": flops / (ms_per_step * 1e-3) / 1e12,
@@ -170,20 +198,24 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 in, f32 accumulate" if dt == hs.FP16 else "f32 (tf32 variant)",
         "data": "synthetic",
+        # seeded generators of hopper_spmm_amd/generators.py: bit-stable for a given numpy version
+        "data_generator": "numpy %s Philox" % np.__version__,
         "config": {"workload": "configs[%d]: %s, N=%d" % (args.config, cfg["name"], N),
                    "rows": A["rows"], "cols": A["cols"], "nnz": nnz, "tiles": int(b["total_tiles"]),
                    "eff_row_windows": int(b["eff_row_windows"]), "ranges": info["n_ranges"],
                    "split_windows": info["n_split_windows"]},
         "effective_gbps": bytes_alg / (ms_per_step * 1e-3) / 1e9,
-        "roofline": {"bound": "hbm", "achieved": bytes_alg / (main_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": bytes_alg / (main_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        # achieved: algorithmic bytes of one launch / (main kernel + partial-sum kernel), device events
+        "roofline": {"bound": "hbm", "achieved": bytes_alg / (kernels_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": bytes_alg / (kernels_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     # counter figures stored with the rocprofv3 summary they come from (not measured in this run)
                      "traffic": traffic,
                      "kernel": {1: "spmm_scalar_kernel", 2: "spmm_mfma_kernel", 3: "spmm_panel_kernel"}.get(
                          plan.info()["last_kernel_family"], "none"),
                      "kernel_ms": main_ms, "fixup_kernel_ms": fix_ms,
                      "algorithmic_bytes": bytes_alg, "gather_bytes": bytes_gather,
                      # every gathered B row counted every time it is gathered, for comparison with the HBM peak
-                     "gathered_gbps": bytes_gather / (main_ms * 1e-3) / 1e9,
+                     "gathered_gbps": bytes_gather / (kernels_ms * 1e-3) / 1e9,
                      "mfma_frac_of_peak_useful_flops": flops / (main_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[dt]},
         "reference_convention_ms": ref_conv_ms,
         # one call of the host-buffer interface (fp16_spmm): plan + upload, one launch, download of C
@@ -191,6 +223,15 @@ def main():
                              "tflops_including_transfers": flops / (t_h2d + t_d2h + ms_per_step * 1e-3) / 1e12},
         "setup_seconds": t_gen,
     }
+    if gather_floor:
+        # every (window, column) pair gathers one B row; this is what loading those rows alone takes
+        out["roofline"]["gather_ceiling_gbps"] = gather_floor["bytes"] / (gather_floor["ms"] * 1e-3) / 1e9
+        out["roofline"]["gather_only_ms"] = gather_floor["ms"]
+        out["roofline"]["frac_of_gather_ceiling"] = gather_floor["ms"] / kernels_ms
+    if fp32_products:
+        out["tf32_variant"] = {"default": {"kernel_ms": main_ms, "fixup_kernel_ms": fix_ms,
+                                           "arithmetic": "bf16 hi / lo parts, three v_mfma_f32_16x16x32_bf16 products"},
+                               "fp32_products": fp32_products}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(A, B, N, flops)
     plan.close()

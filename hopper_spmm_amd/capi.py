@@ -92,6 +92,7 @@ def load_library():
     L.hspmm_prepare.argtypes = [vp, u32]
     L.hspmm_bench.argtypes = [vp, vp, vp, u32, i, i, vp, C.POINTER(C.c_float)]
     L.hspmm_profile.argtypes = [vp, vp, vp, u32, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    L.hspmm_measure_gather.argtypes = [vp, vp, u32, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_uint64)]
     L.hspmm_destroy.argtypes = [vp]
     L.hspmm_destroy.restype = None
     L.hspmm_configure.argtypes = [i, i, i, i]
@@ -421,6 +422,13 @@ class Plan:
         _check(load_library().hspmm_profile(self._h, C.c_void_p(dB_ptr), C.c_void_p(dC_ptr), N, runs,
                                             C.c_void_p(stream), C.byref(a), C.byref(b)))
         return a.value, b.value
+
+    def measure_gather(self, dB_ptr, N, runs=5, stream=0):
+        """(ms per run, bytes loaded per run) of the plan's row gathers alone (measurement only)."""
+        ms, nbytes = C.c_float(), C.c_uint64()
+        _check(load_library().hspmm_measure_gather(self._h, C.c_void_p(dB_ptr), N, runs, C.c_void_p(stream),
+                                                   C.byref(ms), C.byref(nbytes)))
+        return ms.value, nbytes.value
 
     def info(self):
         inf = PlanInfo()

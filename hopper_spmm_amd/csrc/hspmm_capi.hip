@@ -68,6 +68,7 @@ struct Config {
     int panel_units_per_group = 0;      // consumer waves of a workgroup that get a unit (0: searched per N)
     int panel_chunks = 0;               // chunks of panels (0: searched per N)
     int panel_max_windows = 0;          // 2 or 4: windows per unit of the panel stream (0: by matrix size)
+    int xcd_split = -1;                 // gather kernels: two feature blocks dealt out by XCD half (-1: by matrix, 0 never, 1 always)
 
     void read_environment()
     {
@@ -81,6 +82,7 @@ struct Config {
         if (const char *e = std::getenv("HSPMM_PANEL_UNITS_PER_GROUP")) panel_units_per_group = std::max(1, std::atoi(e));
         if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) panel_chunks = std::max(1, std::atoi(e));
         if (const char *e = std::getenv("HSPMM_PANEL_MAX_WINDOWS")) panel_max_windows = std::atoi(e) >= 4 ? 4 : 2;
+        if (const char *e = std::getenv("HSPMM_XCD_SPLIT")) xcd_split = std::atoi(e) != 0;
     }
 };
 std::mutex g_cfg_mutex;
@@ -826,7 +828,9 @@ struct Choice {
     bool narrow;
 };
 
-Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32_t N)
+// split_features: prefer the load width of one 128-byte line per row and feature block (blocks with XCDs of their own, see
+// spmm_mfma_kernel), where the feature dimension allows it.
+Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32_t N, bool split_features = false)
 {
     Choice c{};
     const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
@@ -841,6 +845,8 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
         if (mode != 2 && (dw_ok || mode == 3) && N % 32 == 0) {
             c.layout = hspmm::kLayoutDW;
             c.V = (N % 128 == 0) ? 4 : (N % 64 == 0) ? 2 : 1;
+            // one 128-byte line per row and feature block while that gives at most eight blocks
+            if (split_features && (N == 128 || N == 256 || N == 512)) c.V = 2;
             c.block_feat = 32 * c.V;
             return c;
         }
@@ -1396,7 +1402,13 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
         if (pays && N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
     }
-    const Choice c = choose_kernel(p, dB, dC, N);
+    // Feature blocks with XCDs of their own (see spmm_mfma_kernel): pays when B is far larger than an
+    // XCD's 4 MB L2, so that what an L2 can keep of it decides the hit rate of the gathers (power-law
+    // graph 2^20, N = 128: 575 -> 535 us; uniform 65536^2: 39.7 -> 35.5 us), and costs a second pass over
+    // the tile stream.  Requests below a 128-byte line lose (N = 64 as two blocks of 32: 280 -> 510 us).
+    const bool want_split = p->cfg.xcd_split > 0 ||
+                             (p->cfg.xcd_split < 0 && uint64_t(p->cols) * N * p->elem >= (uint64_t(8) << 20));
+    const Choice c = choose_kernel(p, dB, dC, N, want_split);
     hspmm::KernelArgs ka{};
     ka.rowOffset = p->d_rowOffset; ka.data = p->d_data; ka.rowIdx = p->d_rowIdx; ka.tcA2B = p->d_a2b_raw;
     ka.B = dB; ka.C = dC;
@@ -1410,6 +1422,7 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     ka.unitOffset = p->d_unitOffset; ka.unitRow = p->d_unitRow; ka.ids = p->d_ids; ka.tiles = p->d_tiles;
     ka.n_units = p->n_units;
     ka.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
+    ka.xcd_split = (want_split && (ka.n_feat_blocks == 2u || ka.n_feat_blocks == 4u || ka.n_feat_blocks == 8u)) ? 1u : 0u;
     // Several feature blocks give several waves per range; fewer, longer ranges then keep
     // the number of waves, and pay off where units are long enough to be cut into many
     // pieces (each piece of a cut unit costs a partial sum).
@@ -1525,6 +1538,50 @@ int hspmm_bench(hspmm_plan *p, const void *dB, void *dC, uint32_t N, int warmup,
     HSPMM_HIP(hipEventRecord(ev.b, s));
     HSPMM_HIP(hipEventSynchronize(ev.b));
     HSPMM_HIP(hipEventElapsedTime(total_ms, ev.a, ev.b));
+    return HSPMM_OK;
+}
+
+int hspmm_measure_gather(hspmm_plan *p, const void *dB, uint32_t N, int runs, void *stream, float *ms,
+                         uint64_t *bytes_per_run)
+{
+    if (!p || !dB || !ms) return fail(HSPMM_ERR_INVALID, "null argument");
+    if (runs < 1 || runs > 1000) return fail(HSPMM_ERR_INVALID, "runs %d outside 1..1000", runs);
+    if (p->W == 0) return fail(HSPMM_ERR_INVALID, "the matrix has no stored entries");
+    const uint64_t row_bytes = uint64_t(N) * p->elem;
+    if (row_bytes % 128u || row_bytes > (1u << 24) || reinterpret_cast<uintptr_t>(dB) % 16u)
+        return fail(HSPMM_ERR_UNSUPPORTED, "rows of %llu bytes: a multiple of 128 bytes and a B aligned to 16 is needed",
+                    (unsigned long long)row_bytes);
+    int dev = -1;
+    HSPMM_HIP(hipGetDevice(&dev));
+    if (dev != p->device) return fail(HSPMM_ERR_INVALID, "the plan was created on device %d, the current device is %d", p->device, dev);
+    // the parts the gather kernels would read the rows in: one 128-byte line per XCD group where they deal
+    // feature blocks out by XCD (same rule as run_impl), else 256 bytes at a time
+    const bool split = p->cfg.xcd_split > 0 ||
+                       (p->cfg.xcd_split < 0 && uint64_t(p->cols) * row_bytes >= (uint64_t(8) << 20));
+    uint32_t part_bytes = 256u, parts = 1u, passes = uint32_t(row_bytes / 256u);
+    if (row_bytes % 256u) { part_bytes = 128u; passes = uint32_t(row_bytes / 128u); }
+    if (split && (row_bytes == 256u || row_bytes == 512u || row_bytes == 1024u)) {
+        part_bytes = 128u; parts = uint32_t(row_bytes / 128u); passes = 1u;
+    }
+    const uint64_t n_ids = uint64_t(p->n_steps) * p->cw;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    struct Pair {
+        hipEvent_t a = nullptr, b = nullptr;
+        ~Pair() { if (a) (void)hipEventDestroy(a); if (b) (void)hipEventDestroy(b); }
+    } ev;
+    HSPMM_HIP(hipEventCreate(&ev.a));
+    HSPMM_HIP(hipEventCreate(&ev.b));
+    for (int i = -1; i < runs; ++i) {                      // one untimed run first
+        if (i == 0) HSPMM_HIP(hipEventRecord(ev.a, s));
+        for (uint32_t pass = 0; pass < passes; ++pass)
+            HSPMM_HIP(hspmm::launch_gather_rate(p->d_ids, n_ids, static_cast<const char *>(dB) + size_t(pass) * part_bytes,
+                                                uint32_t(row_bytes), part_bytes, parts, p->compute_units, nullptr, s));
+    }
+    HSPMM_HIP(hipEventRecord(ev.b, s));
+    HSPMM_HIP(hipEventSynchronize(ev.b));
+    HSPMM_HIP(hipEventElapsedTime(ms, ev.a, ev.b));
+    *ms /= float(runs);
+    if (bytes_per_run) *bytes_per_run = n_ids * row_bytes;
     return HSPMM_OK;
 }
 

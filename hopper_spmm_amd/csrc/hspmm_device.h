@@ -37,6 +37,7 @@ struct KernelArgs {
     const void     *B;           // cols x N
     void           *C;           // rows x N
     uint32_t n_ranges, n_split, eff_windows, n_units, rows, N, n_feat_blocks;
+    uint32_t xcd_split;          // != 0 (gather kernels; 2, 4 or 8 feature blocks): every feature block has XCDs of its own
     uint32_t uniform_chunks;     // != 0 (LDS-panel kernels): no split table - entry e is unit e, whose partial sums
                                  // are slots e * uniform_chunks .. + uniform_chunks - 1, in that order
 };
@@ -86,5 +87,9 @@ struct PanelArgs {
 hipError_t launch_spmm_panel(int dtype, int G, bool split, const PanelArgs &pa, const KernelArgs &ka, int units,
                              hipStream_t s, hipEvent_t mid);
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
+// Measurement only (gather_rate_kernel in hspmm_kernels.hip): loads part_bytes (128 or 256) of row ids[i] of B for
+// every i < n_ids; parts > 1: `parts` parts of part_bytes each, dealt out by XCD, every part walking all ids.
+hipError_t launch_gather_rate(const uint32_t *ids, uint64_t n_ids, const void *B, uint32_t row_bytes, uint32_t part_bytes,
+                              uint32_t parts, int compute_units, uint32_t *sink, hipStream_t s);
 
 }  // namespace hspmm

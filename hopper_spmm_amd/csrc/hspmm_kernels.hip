@@ -119,6 +119,67 @@ hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s)
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Measurement only: the row gathers of a plan's step stream and nothing else.
+// Every wave walks a slice of the stream's column ids and loads, for each id,
+// PART bytes of that row of B (PART = 256: a quarter-wave per row, 16 bytes per
+// lane; PART = 128: 8 bytes per lane, the part chosen by the XCD the workgroup
+// runs on, as the gather kernels do with feature blocks dealt out by XCD), eight
+// loads per lane in flight, sixteen waves per compute unit.  The time is the
+// floor of any kernel that gathers these rows in this order: what the L2s, the
+// fabric and HBM deliver for this id stream.
+// ---------------------------------------------------------------------------
+template <int PART>
+__global__ __launch_bounds__(256)
+void gather_rate_kernel(const uint32_t *__restrict__ ids, uint64_t n_ids, uint64_t ids_per_wave, const char *__restrict__ B,
+                        uint32_t row_bytes, uint32_t parts, uint32_t *sink)
+{
+    typedef uint32_t vec_t __attribute__((ext_vector_type(PART / 64)));
+    const uint32_t lane = threadIdx.x & 63u, g = lane >> 4, j = lane & 15u;
+    uint32_t part = 0, wave;
+    if (parts > 1u) {
+        // workgroups dealt out as by spmm_mfma_kernel: XCD x = blockIdx % 8 serves part x / (8 / parts)
+        const uint32_t per_part = 8u / parts, xcd = blockIdx.x & 7u, set = blockIdx.x >> 3;
+        part = xcd / per_part;
+        wave = (set * per_part + (xcd - part * per_part)) * 4u + (threadIdx.x >> 6);
+    } else {
+        wave = blockIdx.x * 4u + (threadIdx.x >> 6);
+    }
+    const uint64_t begin = uint64_t(wave) * ids_per_wave;
+    const uint64_t end = begin + ids_per_wave < n_ids ? begin + ids_per_wave : n_ids;
+    const char *lane_base = B + size_t(part) * PART + j * (PART / 16);
+    vec_t acc = {};
+    for (uint64_t i = begin; i + 32u <= end; i += 32u) {
+        vec_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const uint32_t row = ids[i + 4u * u + g];
+            v[u] = *reinterpret_cast<const vec_t *>(lane_base + size_t(row) * row_bytes);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[u];
+    }
+    uint32_t x = 0;
+#pragma unroll
+    for (int k = 0; k < PART / 64; ++k) x ^= acc[k];
+    if (x == 0x9E3779B9u && sink) sink[0] = x;      // (keeps the loads; practically never taken)
+}
+
+hipError_t launch_gather_rate(const uint32_t *ids, uint64_t n_ids, const void *B, uint32_t row_bytes, uint32_t part_bytes,
+                              uint32_t parts, int compute_units, uint32_t *sink, hipStream_t s)
+{
+    const uint64_t waves = uint64_t(compute_units) * 16u;
+    uint64_t per_wave = ((n_ids + waves - 1u) / waves + 31u) & ~uint64_t(31);
+    if (per_wave < 32u) per_wave = 32u;
+    const uint64_t used = (n_ids + per_wave - 1u) / per_wave;             // waves with work
+    const uint64_t per_set = uint64_t(8u / parts) * 4u;
+    const uint64_t blocks = parts > 1u ? 8u * ((used + per_set - 1u) / per_set) : (used + 3u) / 4u;
+    const char *b = static_cast<const char *>(B);
+    if (part_bytes == 256u) gather_rate_kernel<256><<<dim3(unsigned(blocks)), 256, 0, s>>>(ids, n_ids, per_wave, b, row_bytes, parts, sink);
+    else gather_rate_kernel<128><<<dim3(unsigned(blocks)), 256, 0, s>>>(ids, n_ids, per_wave, b, row_bytes, parts, sink);
+    return hipGetLastError();
+}
+
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s)
 {
     // bytes is a multiple of the element size (2 or 4) and dst is aligned to it

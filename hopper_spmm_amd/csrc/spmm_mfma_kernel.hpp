@@ -501,10 +501,24 @@ void spmm_mfma_kernel(const KernelArgs ka)
 {
     constexpr int G = TT::G, V = TT::V, NACC = G * V;
     const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t item = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
-    if (item >= ka.n_ranges * ka.n_feat_blocks) return;
-    const uint32_t range = item / ka.n_feat_blocks;
-    const uint32_t fb = item - range * ka.n_feat_blocks;
+    uint32_t range, fb;
+    if (ka.xcd_split) {
+        // Two, four or eight feature blocks, each with XCDs of its own.  The hardware hands consecutive
+        // workgroups to the eight XCDs in turn and every XCD has an L2 of its own: with two feature blocks
+        // workgroups 0..3 mod 8 take block 0 and workgroups 4..7 mod 8 block 1, so that an L2 only ever
+        // holds one part of every B row it caches - that many more rows of a B that does not fit.
+        const uint32_t waves = blockDim.x >> 6, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const uint32_t per_fb = 8u / ka.n_feat_blocks;                  // XCDs per feature block: 4, 2, 1
+        const uint32_t xcd = blockIdx.x & 7u, set = blockIdx.x >> 3;
+        fb = xcd / per_fb;
+        range = (set * per_fb + (xcd - fb * per_fb)) * waves + wave;
+        if (range >= ka.n_ranges) return;
+    } else {
+        const uint32_t item = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+        if (item >= ka.n_ranges * ka.n_feat_blocks) return;
+        range = item / ka.n_feat_blocks;
+        fb = item - range * ka.n_feat_blocks;
+    }
     const const_u32_ptr rd = as_const(ka.ranges) + size_t(range) * kRangeWords;
     const const_u32_ptr unitOffset = as_const(ka.unitOffset);
     const const_u32_ptr unitRow = as_const(ka.unitRow);
@@ -776,7 +790,10 @@ static hipError_t launch_tt(const KernelArgs &ka, int prefetch, bool narrow, int
 {
     const uint32_t items = ka.n_ranges * ka.n_feat_blocks;
     const dim3 block(64u * waves_per_group);
-    const dim3 grid((items + waves_per_group - 1) / waves_per_group);
+    // (feature blocks dealt out by XCD: sets of eight workgroups, 8 / feature blocks of them per block)
+    const uint32_t per_set = (8u / (ka.xcd_split ? ka.n_feat_blocks : 1u)) * uint32_t(waves_per_group);
+    const dim3 grid(ka.xcd_split ? 8u * ((ka.n_ranges + per_set - 1u) / per_set)
+                                  : (items + waves_per_group - 1) / waves_per_group);
     hipError_t e = narrow ? launch_main_p<TT, true>(ka, prefetch, grid, block, s)
                           : launch_main_p<TT, false>(ka, prefetch, grid, block, s);
     if (e != hipSuccess || ka.n_split == 0 || ka.arrive) return e;

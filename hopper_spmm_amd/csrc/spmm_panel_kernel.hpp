@@ -261,9 +261,10 @@ struct PanelOps<Fp16Tr<G_, BF>> {
 // of each factor (reference src/ptx/wgmma.h:42-58).  Here every fp32 value v is taken as
 // hi + lo with hi = v cut to bf16 (its upper 16 bits: same sign, never overflows) and
 // lo = bf16(v - hi) (the difference is exact, its rounding leaves |v - hi - lo| <= 2^-16 |v|), and
-// a * b = a_hi b_hi + a_hi b_lo + a_lo b_hi + a_lo b_lo with fp32 accumulation: four
-// v_mfma_f32_16x16x32_bf16 where fp32 inputs would need eight 16x16x4 instructions of twice the
-// length, and 16 mantissa bits per factor where tf32 keeps 10.  The sparse values are split by
+// a * b = a_hi b_hi + a_hi b_lo + a_lo b_hi with fp32 accumulation (the fourth product, a_lo b_lo,
+// is below 2^-14 |a||b| and is left out): three v_mfma_f32_16x16x32_bf16 where fp32 inputs would
+// need eight 16x16x4 instructions of twice the length, and a product exact to 2^-14 where tf32,
+// with 10 mantissa bits per factor, is exact to 2^-10.  The sparse values are split by
 // the plan, the rows of B by the producer waves on their way into LDS: an image row is
 // [64 hi halves][64 lo halves], read through the transposing LDS read like the 16-bit types.
 // An infinite or NaN v has lo = 0 (hi carries it).
@@ -397,9 +398,8 @@ struct PanelOps<Fp32Split<G_>> {
             const u32x4 b_lo = operand(a0, a1, 128 + 32 * p);
 #pragma unroll
             for (int h = 0; h < kHalves; ++h) {
-                // small terms first
-                f32x4 c = HalfOps<true>::mfma(a_lo[h], b_lo, acc[4 * h + p]);
-                c = HalfOps<true>::mfma(a_lo[h], b_hi, c);
+                // small terms first; a_lo * b_lo (below 2^-14 |a||b|, 2^-16 on average) is left out
+                f32x4 c = HalfOps<true>::mfma(a_lo[h], b_hi, acc[4 * h + p]);
                 c = HalfOps<true>::mfma(a_hi[h], b_lo, c);
                 acc[4 * h + p] = HalfOps<true>::mfma(a_hi[h], b_hi, c);
             }

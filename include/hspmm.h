@@ -119,6 +119,17 @@ int hspmm_bench(hspmm_plan *plan, const void *dB, void *dC, uint32_t N,
 int hspmm_profile(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, int runs, void *stream,
                   float *main_ms, float *fixup_ms);
 
+/* No reference counterpart.  Measurement only: launches, `runs` times, a kernel that
+ * loads every row of B the plan's step stream gathers (each (window, column) pair
+ * once, in the stream's order, N elements per row, in the same parts and with the
+ * same assignment to XCDs as the gather kernels use) and does nothing else.  *ms
+ * receives the mean time of one run, *bytes_per_run (optional) the bytes its lanes
+ * load.  That time is a floor for any kernel that gathers these rows: bench.py
+ * reports it next to the SpMM kernel's time.  N * element size must be a multiple
+ * of 128 bytes and dB aligned to 16. */
+int hspmm_measure_gather(hspmm_plan *plan, const void *dB, uint32_t N, int runs, void *stream, float *ms,
+                         uint64_t *bytes_per_run);
+
 /* Replaces the cudaFree block of fp16_spmm (reference src/fp16.cu:274-279). */
 void hspmm_destroy(hspmm_plan *plan);
 
