@@ -64,7 +64,8 @@ class PlanInfo(C.Structure):
                 ("compute_units", C.c_uint32), ("n_units", C.c_uint32), ("n_paired_units", C.c_uint32),
                 ("device_bytes", C.c_uint64), ("n_panels", C.c_uint32), ("n_panel_steps", C.c_uint32),
                 ("n_panel_units", C.c_uint32), ("n_panel_paired_units", C.c_uint32),
-                ("n_panel_wide_units", C.c_uint32), ("last_kernel_family", C.c_uint32)]
+                ("n_panel_wide_units", C.c_uint32), ("last_kernel_family", C.c_uint32),
+                ("panel_stream_mode", C.c_uint32)]
 
 
 def load_library():
@@ -100,6 +101,7 @@ def load_library():
     L.hspmm_get_config.restype = None
     L.hspmm_set_kernel_mode.argtypes = [i]
     L.hspmm_set_window_pairing.argtypes = [i]
+    L.hspmm_set_panel_stream.argtypes = [i]
     L.hspmm_get_plan_info.argtypes = [vp, C.POINTER(PlanInfo)]
     L.hspmm_get_partition.argtypes = [vp, vp, u32]
     L.hspmm_partition_preview.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
@@ -180,6 +182,12 @@ def get_kernel_mode():
 def set_window_pairing(mode):
     """0 = automatic, 1 = never, 2 = whenever two adjacent windows share a column list."""
     _check(load_library().hspmm_set_window_pairing(mode))
+
+
+def set_panel_stream(mode):
+    """0 = uncompressed tiles (default), 1 = two units per consumer wave of the LDS-staging kernels,
+    2 = as 1 with the tiles kept on the device without their zeros (bitmap + stored values)."""
+    _check(load_library().hspmm_set_panel_stream(mode))
 
 
 def mtx_load(path, dtype):

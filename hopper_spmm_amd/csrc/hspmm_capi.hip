@@ -68,6 +68,8 @@ struct Config {
     int panel_units_per_group = 0;      // consumer waves of a workgroup that get a unit (0: searched per N)
     int panel_chunks = 0;               // chunks of panels (0: searched per N)
     int panel_max_windows = 0;          // 2 or 4: windows per unit of the panel stream (0: by matrix size)
+    int panel_tall = 0;                 // LDS-panel waves with two units each (1: whenever the stream allows)
+    int panel_packed = 0;               // ... and their tiles stored without zeros (1: whenever the stream allows)
     int xcd_split = -1;                 // gather kernels: two feature blocks dealt out by XCD half (-1: by matrix, 0 never, 1 always)
 
     void read_environment()
@@ -83,6 +85,8 @@ struct Config {
         if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) panel_chunks = std::max(1, std::atoi(e));
         if (const char *e = std::getenv("HSPMM_PANEL_MAX_WINDOWS")) panel_max_windows = std::atoi(e) >= 4 ? 4 : 2;
         if (const char *e = std::getenv("HSPMM_XCD_SPLIT")) xcd_split = std::atoi(e) != 0;
+        if (const char *e = std::getenv("HSPMM_PANEL_TALL")) panel_tall = std::atoi(e) != 0;
+        if (const char *e = std::getenv("HSPMM_PANEL_PACKED")) panel_packed = std::atoi(e) != 0;
     }
 };
 std::mutex g_cfg_mutex;
@@ -138,6 +142,12 @@ struct hspmm_plan {
         int G = 1;
         bool quad = false;                                       // ids in the format of the 4x4x1 fp32 tile
         bool split = false;                                      // fp32 stream in the bf16 hi / lo form (Fp32Split)
+        bool tall = false;                                       // two units per consumer wave: poff per pair of units,
+                                                                 // their steps merged panel by panel
+        bool packed = false;                                     // tiles without their zeros: masks, values, step_voff
+        uint64_t *d_masks = nullptr;
+        void *d_vals = nullptr;
+        uint32_t *d_step_voff = nullptr;
         double density = 0.0;                                    // steps per unit and 128 columns of the gather stream
     } panel;
     float *d_scratch = nullptr;
@@ -597,6 +607,101 @@ void group_windows(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, 
     }
 }
 
+// Two units per consumer wave of the LDS-panel kernels ("tall" streams): units 2q and 2q + 1 become one
+// sequence of steps, panel by panel the steps of the first, then those of the second (marked with bit 28 of
+// their id words; the panel counts in bits 0..3 are those of the merged sequence).  One image of a panel in
+// LDS then serves twice as many rows.  ids: 16 words per step; tiles: tile_words per step.
+void merge_unit_pairs(uint32_t U, uint32_t NP, size_t tile_words, const std::vector<uint32_t> &unitOffset,
+                      std::vector<uint32_t> &poff, std::vector<uint32_t> &step_panel, std::vector<uint32_t> &ids,
+                      std::vector<uint32_t> &tiles)
+{
+    const uint32_t Q = (U + 1u) / 2u;
+    const size_t n_steps = step_panel.size();
+    std::vector<uint32_t> n_poff(size_t(Q) * (NP + 1)), n_panel(n_steps), n_ids(ids.size()), n_tiles(tiles.size());
+    hspmm_host::parallel_blocks(Q, 8, [&](size_t qb, size_t qe) {
+        for (size_t q = qb; q < qe; ++q) {
+            const uint32_t a = uint32_t(2 * q), b = a + 1u;
+            const bool two = b < U;
+            const uint32_t *pa = poff.data() + size_t(a) * (NP + 1);
+            const uint32_t *pb = two ? poff.data() + size_t(b) * (NP + 1) : nullptr;
+            uint32_t at = unitOffset[a];                          // the pair's steps start where its first unit's did
+            uint32_t *po = n_poff.data() + q * (NP + 1);
+            uint32_t prev_panel = 0;
+            bool first = true;
+            for (uint32_t pn = 0; pn <= NP; ++pn) {
+                po[pn] = at;
+                if (pn == NP) break;
+                for (int which = 0; which < (two ? 2 : 1); ++which) {
+                    const uint32_t *src_off = which ? pb : pa;
+                    for (uint32_t t = src_off[pn]; t < src_off[pn + 1]; ++t, ++at) {
+                        const uint32_t jump = first ? 0u : pn - prev_panel;
+                        first = false;
+                        prev_panel = pn;
+                        n_panel[at] = pn;
+                        for (uint32_t w = 0; w < 16; ++w)
+                            n_ids[size_t(at) * 16 + w] = (ids[size_t(t) * 16 + w] & 0x0FFFFFF0u) | jump | (which ? 1u << 28 : 0u);
+                        std::memcpy(n_tiles.data() + size_t(at) * tile_words, tiles.data() + size_t(t) * tile_words,
+                                    tile_words * 4);
+                    }
+                }
+            }
+        }
+    });
+    poff.swap(n_poff); step_panel.swap(n_panel); ids.swap(n_ids); tiles.swap(n_tiles);
+}
+
+// The tiles of a stream of 16 x 32 steps without their zeros.  A lane-order step is [lane l][8 values] (16-bit
+// types: halves; fp32 in bf16 parts: 8 hi halves then 8 lo halves).  masks[8 s + i] has bit l set when lane l's
+// i-th value of step s is stored (any bit pattern but +0); the stored values follow in the order (i, l), one
+// half each (fp32 in parts: one word, hi | lo << 16), those of step s from position step_voff[s] on.  Position
+// 0 holds a zero, and a step's worth of zeros follows the last value.  This is the bitmap layout of the
+// reference's BTCF_MTX (nnzOffset / tcBit / packed data, reference src/utils/class.h:55-67 and
+// src/utils/convert.h:83-101) with one bitmap per step and the bits in the order the lanes need them.
+void pack_steps(size_t n_steps, bool split, const std::vector<uint32_t> &tiles, std::vector<uint64_t> &masks,
+                std::vector<uint8_t> &vals, std::vector<uint32_t> &step_voff)
+{
+    const size_t lane_halves = split ? 16 : 8, es = split ? 4 : 2;
+    const uint16_t *h = reinterpret_cast<const uint16_t *>(tiles.data());
+    masks.assign(n_steps * 8, 0);
+    step_voff.assign(n_steps + 1, 0);
+    auto stored = [&](size_t s, uint32_t l, uint32_t i) {
+        const uint16_t *lane = h + (s * 64 + l) * lane_halves;
+        return split ? (lane[i] | lane[8 + i]) != 0 : lane[i] != 0;
+    };
+    hspmm_host::parallel_blocks(n_steps, 1024, [&](size_t sb, size_t se) {
+        for (size_t s = sb; s < se; ++s) {
+            uint32_t count = 0;
+            for (uint32_t i = 0; i < 8; ++i) {
+                uint64_t m = 0;
+                for (uint32_t l = 0; l < 64; ++l) if (stored(s, l, i)) m |= uint64_t(1) << l;
+                masks[s * 8 + i] = m;
+                count += uint32_t(__builtin_popcountll(m));
+            }
+            step_voff[s + 1] = count;
+        }
+    });
+    step_voff[0] = 1;                                             // position 0: the zero
+    for (size_t s = 0; s < n_steps; ++s) step_voff[s + 1] += step_voff[s];
+    vals.assign((size_t(step_voff[n_steps]) + 512) * es, 0);
+    hspmm_host::parallel_blocks(n_steps, 1024, [&](size_t sb, size_t se) {
+        for (size_t s = sb; s < se; ++s) {
+            size_t at = step_voff[s];
+            for (uint32_t i = 0; i < 8; ++i)
+                for (uint32_t l = 0; l < 64; ++l) {
+                    if (!(masks[s * 8 + i] >> l & 1u)) continue;
+                    const uint16_t *lane = h + (s * 64 + l) * lane_halves;
+                    if (split) {
+                        const uint32_t w = uint32_t(lane[i]) | uint32_t(lane[8 + i]) << 16;
+                        std::memcpy(vals.data() + at * 4, &w, 4);
+                    } else {
+                        std::memcpy(vals.data() + at * 2, &lane[i], 2);
+                    }
+                    ++at;
+                }
+        }
+    });
+}
+
 // Re-tiles the matrix panel by panel for the LDS-panel kernels (spmm_panel_kernel.hpp):
 // inside every window the columns of one panel of kPanelRows columns get tiles of
 // their own.  Every step carries the number of panels it lies behind the step in
@@ -805,17 +910,45 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     });
     hspmm_plan::Panel &pl = p->panel;
     int rc;
+    std::vector<uint32_t> tiles = split      ? lane_order_split_steps(ps, rt_rowOffset.data(), rt_data.data())
+                                  : cw == 16 ? lane_order_wide_steps(ps, rt_rowOffset.data(), rt_data.data())
+                                             : lane_order_tiles(ps, p->dtype, rt_rowOffset.data(), rt_data.data());
+    // Two units per consumer wave, and tiles without their zeros (kernels built on the 16-bit MFMA, units of one
+    // or two windows): fewer 128-byte lines through the compute units' L1s (one copy of a panel in LDS serves
+    // twice the rows; a packed step is its stored values and 64 bytes of masks).  Measured, the lines go down
+    // by a third and by 60 % and the time does not: what binds these kernels is the LDS reads and MFMAs of a
+    // step, which a SIMD runs one after the other.  Both are therefore taken on request only
+    // (hspmm_set_panel_stream, HSPMM_PANEL_TALL / HSPMM_PANEL_PACKED).
+    bool tall = false, packed = false;
+    if (rw == 32 && ps.G <= 2 && U >= 2 && (p->cfg.panel_tall > 0 || p->cfg.panel_packed > 0)) {
+        tall = true;
+        const size_t tile_words = split ? 512u : 256u;
+        merge_unit_pairs(U, NP, tile_words, ps.unitOffset, poff, step_panel, ids, tiles);
+        packed = p->cfg.panel_packed > 0;
+    }
     if ((rc = upload(&pl.d_poff, poff.data(), poff.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     if ((rc = upload(&pl.d_step_panel, step_panel.data(), step_panel.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     if ((rc = upload(&pl.d_ids, ids.data(), ids.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
-    {
-        const std::vector<uint32_t> tiles = split      ? lane_order_split_steps(ps, rt_rowOffset.data(), rt_data.data())
-                                            : cw == 16 ? lane_order_wide_steps(ps, rt_rowOffset.data(), rt_data.data())
-                                                       : lane_order_tiles(ps, p->dtype, rt_rowOffset.data(), rt_data.data());
+    if (packed) {
+        std::vector<uint64_t> masks;
+        std::vector<uint8_t> vals;
+        std::vector<uint32_t> step_voff;
+        pack_steps(ps.n_steps, split, tiles, masks, vals, step_voff);
+        if (vals.size() >= (size_t(1) << 32)) packed = false;        // positions are 32-bit byte offsets in the kernel
+        else {
+            uint8_t *dv = nullptr;
+            if ((rc = upload(&pl.d_masks, masks.data(), masks.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
+            if ((rc = upload(&dv, vals.data(), vals.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
+            pl.d_vals = dv;
+            if ((rc = upload(&pl.d_step_voff, step_voff.data(), step_voff.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
+        }
+    }
+    if (!packed) {
         uint32_t *dt = nullptr;
         if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
         pl.d_tiles = dt;
     }
+    pl.tall = tall; pl.packed = packed;
     if ((rc = upload(&pl.d_unitRow, st.unitRow.data(), st.unitRow.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     pl.n_units = U; pl.G = st.G; pl.n_paired = st.n_paired; pl.n_wide = st.n_wide;
     pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.split = split; pl.density = density; pl.built = true;
@@ -984,6 +1117,15 @@ int hspmm_set_window_pairing(int mode)
     if (mode < 0 || mode > 2) return fail(HSPMM_ERR_INVALID, "pairing mode %d outside 0..2", mode);
     std::lock_guard<std::mutex> lk(g_cfg_mutex);
     g_cfg.pairing = mode;
+    return HSPMM_OK;
+}
+
+int hspmm_set_panel_stream(int mode)
+{
+    if (mode < 0 || mode > 2) return fail(HSPMM_ERR_INVALID, "panel stream mode %d outside 0..2", mode);
+    std::lock_guard<std::mutex> lk(g_cfg_mutex);
+    g_cfg.panel_tall = mode >= 1;
+    g_cfg.panel_packed = mode == 2;
     return HSPMM_OK;
 }
 
@@ -1250,6 +1392,7 @@ void hspmm_destroy(hspmm_plan *p)
     (void)hipFree(p->panel.d_poff); (void)hipFree(p->panel.d_ids); (void)hipFree(p->panel.d_tiles);
     (void)hipFree(p->panel.d_unitRow);
     (void)hipFree(p->panel.d_step_panel);
+    (void)hipFree(p->panel.d_masks); (void)hipFree(p->panel.d_vals); (void)hipFree(p->panel.d_step_voff);
     (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive);
     for (void *old : p->retired) (void)hipFree(old);
     delete p;
@@ -1288,6 +1431,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     hspmm::PanelArgs pa{};
     pa.unitRow = pl.d_unitRow; pa.poff = pl.d_poff; pa.step_panel = pl.d_step_panel; pa.ids = pl.d_ids;
     pa.tiles = pl.d_tiles; pa.n_steps = pl.n_steps;
+    pa.masks = pl.d_masks; pa.vals = pl.d_vals; pa.step_voff = pl.d_step_voff;
     pa.B = dB; pa.C = dC;
     pa.n_units = pl.n_units; pa.rows = p->rows; pa.cols = p->cols; pa.N = N;
     pa.n_feat_blocks = N / (hspmm::kPanelRowBytes / p->elem);
@@ -1307,25 +1451,29 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         forced_units = std::min(p->cfg.panel_units_per_group, units == 13 ? 12 : units);
     // (units of up to four windows: eight consumer waves with twice the accumulators)
     const int max_units = pl.G == 4 ? 8 : units == 13 ? 12 : units;
+    // what one consumer wave takes: a unit, or (tall streams) two
+    const uint32_t wave_units = pl.tall ? (pl.n_units + 1u) / 2u : pl.n_units;
     if (forced_units) forced_units = std::min(forced_units, max_units);
     const uint64_t slots = uint64_t(p->compute_units) * (pl.quad ? 2u : 1u);     // workgroups resident at a time
     // Units per workgroup and chunks of panels: the workgroups should fill the compute units in whole
-    // rounds.  Cost of a shape = rounds x panels per chunk x (units + 3: a panel costs its LDS reads, which
-    // go with the units, plus its copy and barrier), plus the second launch when there are chunk sums.
+    // rounds.  Cost of a shape = rounds x panels per chunk x (units + 3: a panel costs its LDS reads and
+    // MFMAs, which go with the units, plus its copy and barrier), plus the second launch when there are
+    // chunk sums.
     uint64_t chunks = 1;
     int best_units = max_units;
     double best_cost = 0.0;
     for (int nc = forced_units ? forced_units : std::max(4, max_units / 2); nc <= (forced_units ? forced_units : max_units); ++nc) {
-        const uint64_t rbs = (uint64_t(pl.n_units) + nc - 1) / nc, base = rbs * pa.n_feat_blocks;
+        const uint64_t rbs = (uint64_t(wave_units) + nc - 1) / nc, base = rbs * pa.n_feat_blocks;
         uint64_t ch = base >= slots ? 1 : std::min<uint64_t>(slots / base, pl.n_panels);
         const uint64_t ppc = (pl.n_panels + ch - 1) / ch;
         ch = (pl.n_panels + ppc - 1) / ppc;
         const uint64_t rounds = (base * ch + slots - 1) / slots;
-        const double cost = double(rounds) * double(ppc) * (nc + 3.0) + (ch > 1 ? 80.0 : 0.0);
+        const double units_here = double(nc) * (pl.tall ? 2.0 : 1.0);
+        const double cost = double(rounds) * double(ppc) * (units_here + 3.0) + (ch > 1 ? 80.0 : 0.0);
         if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best_units = nc; chunks = ch; }
     }
     pa.units_per_group = uint32_t(best_units);
-    const uint64_t row_blocks = (uint64_t(pl.n_units) + best_units - 1) / best_units;
+    const uint64_t row_blocks = (uint64_t(wave_units) + best_units - 1) / best_units;
     const uint64_t base = row_blocks * pa.n_feat_blocks;
     if (p->cfg.panel_chunks) chunks = uint64_t(p->cfg.panel_chunks);
     if (chunks < 1) chunks = 1;
@@ -1362,7 +1510,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     }
     if (mode == RunMode::kPrepare) return HSPMM_OK;
     p->last_family.store(3, std::memory_order_relaxed);
-    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : pl.G, pl.split, pa, ka, units, s, mid));
+    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : pl.G, pl.split, pl.tall, pl.packed, pa, ka, units, s, mid));
     return HSPMM_OK;
 }
 
@@ -1603,6 +1751,7 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_panel_paired_units = p->panel.built ? p->panel.n_paired : 0u;
     info->n_panel_wide_units = p->panel.built ? p->panel.n_wide : 0u;
     info->last_kernel_family = p->last_family.load(std::memory_order_relaxed);
+    info->panel_stream_mode = !p->panel.built ? 0u : p->panel.packed ? 2u : p->panel.tall ? 1u : 0u;
     return HSPMM_OK;
 }
 

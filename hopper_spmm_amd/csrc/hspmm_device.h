@@ -69,7 +69,12 @@ struct PanelArgs {
     const uint32_t *ids;         // per step: the rows (inside the panel) each quarter-wave reads and the panels
                                  // between the step and the one in front of it; the format depends on the element
                                  // type (PanelOps in spmm_panel_kernel.hpp)
-    const void     *tiles;       // per step, lane order
+    const void     *tiles;       // per step, lane order (null when the stream is packed)
+    // packed streams (tiles without their zeros): per step eight lane masks; the stored values, (mask, lane)
+    // order, values[0] = 0; per step the position of its first value
+    const uint64_t *masks;
+    const void     *vals;
+    const uint32_t *step_voff;
     float          *scratch;     // partial sums [unit * n_chunks + chunk][feature block][acc reg][lane]
     uint32_t       *arrive;      // per (unit, feature block): chunks that have left their sums (zero between launches);
                                  // null: a second kernel adds the sums
@@ -84,8 +89,10 @@ struct PanelArgs {
 // G: windows per unit at most (1, 2, 4); 0 = fp32 single windows with ids in the format of the 4x4x1 tile.  split (fp32): the plan's
 // stream is in the bf16 hi / lo form.  ka: arguments of the kernel that adds the chunk sums (split table with one
 // entry per unit), used when pa.n_chunks > 1.
-hipError_t launch_spmm_panel(int dtype, int G, bool split, const PanelArgs &pa, const KernelArgs &ka, int units,
-                             hipStream_t s, hipEvent_t mid);
+// tall: the stream gives every consumer wave two units (poff per pair of units, steps of the second unit marked);
+// packed: its tiles are stored without their zeros (tall streams only).
+hipError_t launch_spmm_panel(int dtype, int G, bool split, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka,
+                             int units, hipStream_t s, hipEvent_t mid);
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
 // Measurement only (gather_rate_kernel in hspmm_kernels.hip): loads part_bytes (128 or 256) of row ids[i] of B for
 // every i < n_ids; parts > 1: `parts` parts of part_bytes each, dealt out by XCD, every part walking all ids.

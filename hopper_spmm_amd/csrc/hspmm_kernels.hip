@@ -97,17 +97,19 @@ hipError_t launch_spmm_mfma(int dtype, int layout, int G, const KernelArgs &ka, 
                   : launch_mfma_f16_g1(layout, ka, V, prefetch, narrow, waves_per_group, s, mid);
 }
 
-hipError_t launch_panel_f16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid);
-hipError_t launch_panel_bf16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid);
-hipError_t launch_panel_f32(int G, bool split, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s,
+hipError_t launch_panel_f16(int G, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s,
+                           hipEvent_t mid);
+hipError_t launch_panel_bf16(int G, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s,
                             hipEvent_t mid);
+hipError_t launch_panel_f32(int G, bool split, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka, int waves,
+                            hipStream_t s, hipEvent_t mid);
 
-hipError_t launch_spmm_panel(int dtype, int G, bool split, const PanelArgs &pa, const KernelArgs &ka, int waves,
-                             hipStream_t s, hipEvent_t mid)
+hipError_t launch_spmm_panel(int dtype, int G, bool split, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka,
+                             int waves, hipStream_t s, hipEvent_t mid)
 {
-    if (dtype == kDtypeF32) return launch_panel_f32(G, split, pa, ka, waves, s, mid);
-    if (dtype == kDtypeBf16) return launch_panel_bf16(G, pa, ka, waves, s, mid);
-    return launch_panel_f16(G, pa, ka, waves, s, mid);
+    if (dtype == kDtypeF32) return launch_panel_f32(G, split, tall, packed, pa, ka, waves, s, mid);
+    if (dtype == kDtypeBf16) return launch_panel_bf16(G, tall, packed, pa, ka, waves, s, mid);
+    return launch_panel_f16(G, tall, packed, pa, ka, waves, s, mid);
 }
 
 hipError_t launch_spmm_scalar(int dtype, const KernelArgs &ka, hipStream_t s)

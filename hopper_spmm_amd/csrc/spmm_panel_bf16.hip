@@ -6,8 +6,12 @@ namespace hspmm {
 
 template <int G> using PanelTile = Fp16Tr<G, true>;
 
-hipError_t launch_panel_bf16(int G, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s, hipEvent_t mid)
+hipError_t launch_panel_bf16_tall(int G, bool packed, const PanelArgs &pa, const KernelArgs &ka, hipStream_t s, hipEvent_t mid);
+
+hipError_t launch_panel_bf16(int G, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s,
+                           hipEvent_t mid)
 {
+    if (tall) return launch_panel_bf16_tall(G, packed, pa, ka, s, mid);
     if (G == 4) return launch_panel_nw<PanelTile<4>>(pa, ka, waves, s, mid);
     return G == 2 ? launch_panel_nw<PanelTile<2>>(pa, ka, waves, s, mid)
                   : launch_panel_nw<PanelTile<1>>(pa, ka, waves, s, mid);

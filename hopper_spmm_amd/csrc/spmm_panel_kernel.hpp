@@ -234,6 +234,18 @@ struct PanelOps<Fp16Tr<G_, BF>> {
         return a;
     }
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) & 15u; }
+    // (waves with two units) the step belongs to the wave's second unit
+    __device__ static __forceinline__ bool second_unit(const Idx I) { return (__builtin_amdgcn_readfirstlane(I) >> 28) & 1u; }
+    static constexpr uint32_t kPackedRing = 2;                    // steps in flight when the tiles are packed
+    // the lane's eight halves from their positions in the packed values (position 0 holds a zero)
+    __device__ static __forceinline__ AVec gather_a(const void *vals, const uint32_t (&pos)[8])
+    {
+        const uint16_t *v = static_cast<const uint16_t *>(vals);
+        AVec a;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) a.r[0][k] = uint32_t(v[pos[2 * k]]) | uint32_t(v[pos[2 * k + 1]]) << 16;
+        return a;
+    }
     typedef tr16x4 __attribute__((address_space(3))) *lds_tr_ptr;
     __device__ static __forceinline__ void step(const typename TT::Lane &, const char *smem, uint32_t img, const Idx I,
                                                 const AVec &A, f32x4 (&acc)[kLive])
@@ -368,6 +380,22 @@ struct PanelOps<Fp32Split<G_>> {
         return a;
     }
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) & 15u; }
+    __device__ static __forceinline__ bool second_unit(const Idx I) { return (__builtin_amdgcn_readfirstlane(I) >> 28) & 1u; }
+    static constexpr uint32_t kPackedRing = 4;                    // steps in flight when the tiles are packed
+    // the lane's eight values (hi half | lo half << 16) from their positions in the packed values
+    // (position 0 holds a zero), rearranged to four words of hi halves and four of lo halves
+    __device__ static __forceinline__ AVec gather_a(const void *vals, const uint32_t (&pos)[8])
+    {
+        const uint32_t *v = static_cast<const uint32_t *>(vals);
+        AVec a;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t w0 = v[pos[2 * k]], w1 = v[pos[2 * k + 1]];
+            a.r[0][k] = __builtin_amdgcn_perm(w1, w0, 0x05040100u);
+            a.r[0][4 + k] = __builtin_amdgcn_perm(w1, w0, 0x07060302u);
+        }
+        return a;
+    }
     typedef tr16x4 __attribute__((address_space(3))) *lds_tr_ptr;
     __device__ static __forceinline__ u32x4 operand(const __attribute__((address_space(3))) char *a0,
                                                     const __attribute__((address_space(3))) char *a1, int off)
@@ -459,6 +487,18 @@ struct PanelOps<Fp32Quad> {
     __device__ static __forceinline__ uint32_t lane_bytes(const Fp32Quad::Lane &L) { return L.j * 4u; }
 };
 
+// The eight lane masks of a step whose tile is stored without its zeros (see spmm_panel_kernel).
+struct PackedHeader { uint64_t m[8]; };
+typedef const uint64_t __attribute__((address_space(4))) *const_u64_ptr;
+__device__ __forceinline__ PackedHeader load_packed_header(const uint64_t *masks, uint32_t step)
+{
+    const const_u64_ptr mp = (const_u64_ptr)(uintptr_t)masks + size_t(step) * 8u;   // uniform: scalar loads
+    PackedHeader h;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h.m[i] = mp[i];
+    return h;
+}
+
 // One barrier of the workgroup with the LDS writes in front of it visible behind it.
 __device__ __forceinline__ void panel_barrier()
 {
@@ -471,7 +511,7 @@ __device__ __forceinline__ void panel_barrier()
 // panel images to LDS: the consumers' register ring of tile / id loads then never
 // has to wait for a panel load (vector loads return in order, and a wave that had
 // both kinds in flight would drain its ring at every panel).
-template <class TT, int NC, int NPW>
+template <class TT, int NC, int NPW, bool TALL = false, bool PACKED = false>
 __global__ __launch_bounds__((NC + NPW) * 64)
 void spmm_panel_kernel(const PanelArgs pa)
 {
@@ -536,9 +576,12 @@ void spmm_panel_kernel(const PanelArgs pa)
     }
 
     // ---- consumer
-    const uint32_t u = rb * pa.units_per_group + wave;
+    // TALL: the wave owns two units, 2 su and 2 su + 1 (the second may not exist), with accumulators of
+    // their own; the plan has merged their steps panel by panel and marked those of the second unit.
+    const uint32_t su = rb * pa.units_per_group + wave;
+    const uint32_t u = TALL ? 2u * su : su;
     const bool has_unit = wave < pa.units_per_group && u < pa.n_units;
-    const const_u32_ptr poff = as_const(pa.poff) + size_t(has_unit ? u : 0u) * (pa.n_panels + 1u);
+    const const_u32_ptr poff = as_const(pa.poff) + size_t(has_unit ? su : 0u) * (pa.n_panels + 1u);
 
     typename TT::Lane L;
     L.init(lane, pa.tiles, pa.ids);
@@ -557,23 +600,64 @@ void spmm_panel_kernel(const PanelArgs pa)
     uint32_t first_jump = t1 > t0 ? as_const(pa.step_panel)[t0] - p_begin : 0u;
 
     f32x4 live[Ops::kLive];
+    f32x4 live2[TALL ? Ops::kLive : 1];
 #pragma unroll
     for (int i = 0; i < Ops::kLive; ++i) live[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < (TALL ? Ops::kLive : 1); ++i) live2[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     typedef typename Ops::AVec AVec;
     typedef typename Ops::Idx Idx;
     auto ring_idx = [&](uint32_t step) __attribute__((always_inline)) -> Idx {
         return Ops::load_idx(L, pa.ids, umin32(step, tlast));
     };
-    auto ring_a = [&](uint32_t step) __attribute__((always_inline)) -> AVec {
-        return Ops::load_a(L, umin32(step, tlast));
+    // PACKED: the step's tile is stored without its zeros.  masks[8 s + i] has bit l set when lane l's
+    // i-th value of step s (its column 8 (l / 16) + i of row l % 16) is stored; the stored values follow
+    // one another in the order (i, l), those of step s from vals[step_voff[s]] on, and vals[0] is zero
+    // (what a lane without the value reads).  The masks are uniform (scalar loads); a lane's position is
+    // a count of mask bits below it.  next_val: position of the first value of the next step to load.
+    PackedHeader H0 = {}, H1 = {};
+    uint32_t next_val = 0;
+    if constexpr (PACKED) next_val = as_const(pa.step_voff)[umin32(t0, tlast)];
+    auto request = [&](PackedHeader &H, uint32_t step) __attribute__((always_inline)) {
+        if constexpr (PACKED) H = load_packed_header(pa.masks, umin32(step, tlast));
+    };
+    auto ring_a = [&](const PackedHeader &H, uint32_t step) __attribute__((always_inline)) -> AVec {
+        if constexpr (PACKED) {
+            uint32_t pos[8], base = next_val;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t rank = __builtin_amdgcn_mbcnt_hi(uint32_t(H.m[i] >> 32),
+                                                                __builtin_amdgcn_mbcnt_lo(uint32_t(H.m[i]), base));
+                pos[i] = __builtin_amdgcn_inverse_ballot_w64(H.m[i]) ? rank : 0u;
+                base += uint32_t(__builtin_popcountll(H.m[i]));
+            }
+            if (step <= tlast) next_val = base;            // (a clamped load repeats the last step)
+            return Ops::gather_a(pa.vals, pos);
+        } else {
+            return Ops::load_a(L, umin32(step, tlast));
+        }
     };
     // register ring of kRing steps (separate variables: an array would go to scratch)
 #define HSPMM_RING(X) X(0) X(1) X(2) X(3) X(4) X(5)
-    constexpr uint32_t kRing = Ops::kRing;
+#define HSPMM_HEADER(k) ((k##u & 1u) ? H1 : H0)
+#define HSPMM_OTHER_HEADER(k) ((k##u & 1u) ? H0 : H1)
+    // (two sets of accumulators leave registers for four steps in flight; packed tiles: see Ops::kPackedRing)
+#ifdef HSPMM_PANEL_RING
+    constexpr uint32_t kRing = HSPMM_PANEL_RING;                    // (measurement builds)
+#else
+    constexpr uint32_t kRing = [] {
+        if constexpr (PACKED) return Ops::kPackedRing;
+        else return (TALL && Ops::kRing > 4u) ? 4u : Ops::kRing;
+    }();
+#endif
     static_assert(kRing >= 1 && kRing <= 6, "ring slots are named variables");
+    static_assert(!PACKED || kRing % 2u == 0u, "the two headers alternate with the ring slots");
+    // (PACKED: the header of a step is requested one slot ahead of the loads that need it)
+    request(H0, t0);
 #define HSPMM_RING_DECL(k) Idx I##k = {}; AVec A##k = {}; \
-    if constexpr (kRing > k) { I##k = ring_idx(t0 + k##u); A##k = ring_a(t0 + k##u); }
+    if constexpr (kRing > k) { request(HSPMM_OTHER_HEADER(k), t0 + k##u + 1u); \
+                               I##k = ring_idx(t0 + k##u); A##k = ring_a(HSPMM_HEADER(k), t0 + k##u); }
     HSPMM_RING(HSPMM_RING_DECL)
 #undef HSPMM_RING_DECL
     panel_barrier();                                                // panel p_begin is in its buffer
@@ -589,7 +673,12 @@ void spmm_panel_kernel(const PanelArgs pa)
             img = img_both - img;
             --owed;
         }
-        Ops::step(L, smem, img, I, A, live);
+        if constexpr (TALL) {
+            if (Ops::second_unit(I)) Ops::step(L, smem, img, I, A, live2);
+            else Ops::step(L, smem, img, I, A, live);
+        } else {
+            Ops::step(L, smem, img, I, A, live);
+        }
     };
     auto jump_of = [&](const Idx &I, const uint32_t t) __attribute__((always_inline)) -> uint32_t {
         const uint32_t stored = Ops::jump(I);
@@ -598,73 +687,85 @@ void spmm_panel_kernel(const PanelArgs pa)
 
     uint32_t t = t0;
     // Steady state: every slot runs its step and reloads its registers with the step kRing
-    // further on, without conditions on the loads.
+    // further on, without conditions on the loads.  (After the prologue the header of step
+    // t0 + kRing is in H0 / H1 by the parity of kRing, i.e. in slot 0's header.)
     for (; t + 2u * kRing <= t1; t += kRing) {
 #define HSPMM_PANEL_STEADY(k) if constexpr (kRing > k) { \
         step(I##k, A##k, jump_of(I##k, t + k##u)); \
-        I##k = ring_idx(t + k##u + kRing); A##k = ring_a(t + k##u + kRing); }
+        request(HSPMM_OTHER_HEADER(k), t + k##u + kRing + 1u); \
+        I##k = ring_idx(t + k##u + kRing); A##k = ring_a(HSPMM_HEADER(k), t + k##u + kRing); }
         HSPMM_RING(HSPMM_PANEL_STEADY)
 #undef HSPMM_PANEL_STEADY
     }
     for (; t < t1; t += kRing) {
 #define HSPMM_PANEL_DRAIN(k) if constexpr (kRing > k) { \
         if (t + k##u < t1) step(I##k, A##k, jump_of(I##k, t + k##u)); \
-        if (t + k##u + kRing < t1) { I##k = ring_idx(t + k##u + kRing); A##k = ring_a(t + k##u + kRing); } }
+        request(HSPMM_OTHER_HEADER(k), t + k##u + kRing + 1u); \
+        if (t + k##u + kRing < t1) { I##k = ring_idx(t + k##u + kRing); A##k = ring_a(HSPMM_HEADER(k), t + k##u + kRing); } }
         HSPMM_RING(HSPMM_PANEL_DRAIN)
 #undef HSPMM_PANEL_DRAIN
     }
 #undef HSPMM_RING
+#undef HSPMM_HEADER
+#undef HSPMM_OTHER_HEADER
     // the panels behind the unit's last step
     for (; owed; --owed) panel_barrier();
 
     if (!has_unit) return;
-    Ops::fold(live);
-    f32x4 acc[NACC];
+    // Stores unit `unit` from the sums in `sums` (or leaves them as this chunk's partial sums).
+    auto finish = [&](const uint32_t unit, f32x4 (&sums)[Ops::kLive]) __attribute__((always_inline)) {
+        Ops::fold(sums);
+        f32x4 acc[NACC];
 #pragma unroll
-    for (int i = 0; i < NACC; ++i) acc[i] = live[i];
-    const uint32_t row = pa.unitRow[u];
-    const uint32_t row0 = row & ~7u;
-    const uint32_t nwin = unit_windows<TT>(row);
-    if (pa.n_chunks == 1u) {
-        store_unit<TT>(L, acc, c_lane, row_bytes, row0, nwin, pa.rows, true);
-    } else if (!pa.arrive) {
-        f32x4 *dst = reinterpret_cast<f32x4 *>(pa.scratch) +
-                     ((size_t(u) * pa.n_chunks + chunk) * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
-#pragma unroll
-        for (int i = 0; i < NACC; ++i) dst[i * 64] = acc[i];
-    } else {
-        // The wave that brings the last chunk's sums of a unit adds all of them, in chunk order (so the
-        // result does not depend on who is last), and stores the unit.  The sums cross the L2s of
-        // different XCDs: they are written and read with device-scope accesses, and the writes are
-        // waited for before the arrival is counted.
-        f32x4 *slot0 = reinterpret_cast<f32x4 *>(pa.scratch) +
-                       (size_t(u) * pa.n_chunks * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
-        const size_t chunk_stride = size_t(pa.n_feat_blocks) * (NACC * 64u);
-        f32x4 *dst = slot0 + chunk * chunk_stride;
-#pragma unroll
-        for (int i = 0; i < NACC; ++i) store_device_scope(dst + i * 64, acc[i]);
-        __builtin_amdgcn_s_waitcnt(0x0F70);                        // vmcnt(0): the stores are acknowledged
-        uint32_t *ctr = pa.arrive + size_t(u) * pa.n_feat_blocks + fb;
-        uint32_t old = 0;
-        if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        old = __builtin_amdgcn_readfirstlane(old);
-        if (old + 1u == pa.n_chunks) {
-#pragma unroll
-            for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-            for (uint32_t c = 0; c < pa.n_chunks; ++c) {
-#pragma unroll
-                for (int i = 0; i < NACC; ++i) acc[i] += load_device_scope(slot0 + c * chunk_stride + i * 64);
-            }
+        for (int i = 0; i < NACC; ++i) acc[i] = sums[i];
+        const uint32_t row = pa.unitRow[unit];
+        const uint32_t row0 = row & ~7u;
+        const uint32_t nwin = unit_windows<TT>(row);
+        if (pa.n_chunks == 1u) {
             store_unit<TT>(L, acc, c_lane, row_bytes, row0, nwin, pa.rows, true);
-            if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (!pa.arrive) {
+            f32x4 *dst = reinterpret_cast<f32x4 *>(pa.scratch) +
+                         ((size_t(unit) * pa.n_chunks + chunk) * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) dst[i * 64] = acc[i];
+        } else {
+            // The wave that brings the last chunk's sums of a unit adds all of them, in chunk order (so the
+            // result does not depend on who is last), and stores the unit.  The sums cross the L2s of
+            // different XCDs: they are written and read with device-scope accesses, and the writes are
+            // waited for before the arrival is counted.
+            f32x4 *slot0 = reinterpret_cast<f32x4 *>(pa.scratch) +
+                           (size_t(unit) * pa.n_chunks * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
+            const size_t chunk_stride = size_t(pa.n_feat_blocks) * (NACC * 64u);
+            f32x4 *dst = slot0 + chunk * chunk_stride;
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) store_device_scope(dst + i * 64, acc[i]);
+            __builtin_amdgcn_s_waitcnt(0x0F70);                        // vmcnt(0): the stores are acknowledged
+            uint32_t *ctr = pa.arrive + size_t(unit) * pa.n_feat_blocks + fb;
+            uint32_t old = 0;
+            if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            old = __builtin_amdgcn_readfirstlane(old);
+            if (old + 1u == pa.n_chunks) {
+#pragma unroll
+                for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+                for (uint32_t c = 0; c < pa.n_chunks; ++c) {
+#pragma unroll
+                    for (int i = 0; i < NACC; ++i) acc[i] += load_device_scope(slot0 + c * chunk_stride + i * 64);
+                }
+                store_unit<TT>(L, acc, c_lane, row_bytes, row0, nwin, pa.rows, true);
+                if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
-    }
-    if (chunk == 0u) {
-        // rows of the windows without entries behind this unit, and in front of the first one
-        const uint32_t next_row = (u + 1u < pa.n_units) ? (pa.unitRow[u + 1u] & ~7u) : pa.rows;
-        const uint32_t gap_begin = row0 + nwin * kRowWindow;
-        if (gap_begin < next_row) TT::zero_rows(L, c_lane, row_bytes, gap_begin, next_row, true);
-        if (u == 0u) TT::zero_rows(L, c_lane, row_bytes, 0u, row0, true);
+        if (chunk == 0u) {
+            // rows of the windows without entries behind this unit, and in front of the first one
+            const uint32_t next_row = (unit + 1u < pa.n_units) ? (pa.unitRow[unit + 1u] & ~7u) : pa.rows;
+            const uint32_t gap_begin = row0 + nwin * kRowWindow;
+            if (gap_begin < next_row) TT::zero_rows(L, c_lane, row_bytes, gap_begin, next_row, true);
+            if (unit == 0u) TT::zero_rows(L, c_lane, row_bytes, 0u, row0, true);
+        }
+    };
+    finish(u, live);
+    if constexpr (TALL) {
+        if (u + 1u < pa.n_units) finish(u + 1u, live2);
     }
 }
 
@@ -675,13 +776,14 @@ void spmm_panel_kernel(const PanelArgs pa)
 
 // ka: the arguments of spmm_fixup_kernel for the chunk sums (split table with one
 // entry per unit); used only when pa.n_chunks > 1.
-template <class TT, int NC, int NPW>
+template <class TT, int NC, int NPW, bool TALL = false, bool PACKED = false>
 static hipError_t launch_panel_tt(const PanelArgs &pa, const KernelArgs &ka, hipStream_t s, hipEvent_t mid)
 {
     if (pa.units_per_group < 1u || pa.units_per_group > uint32_t(NC)) return hipErrorInvalidValue;
-    const uint32_t row_blocks = (pa.n_units + pa.units_per_group - 1u) / pa.units_per_group;
+    const uint32_t wave_units = TALL ? (pa.n_units + 1u) / 2u : pa.n_units;     // what one consumer wave takes
+    const uint32_t row_blocks = (wave_units + pa.units_per_group - 1u) / pa.units_per_group;
     const dim3 grid(row_blocks * pa.n_feat_blocks * pa.n_chunks), block((NC + NPW) * 64);
-    spmm_panel_kernel<TT, NC, NPW><<<grid, block, 0, s>>>(pa);
+    spmm_panel_kernel<TT, NC, NPW, TALL, PACKED><<<grid, block, 0, s>>>(pa);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || pa.n_chunks == 1u || pa.arrive) return e;
     if (mid && (e = hipEventRecord(mid, s)) != hipSuccess) return e;
@@ -700,6 +802,16 @@ static hipError_t launch_panel_nw(const PanelArgs &pa, const KernelArgs &ka, int
         if (units == 13) return launch_panel_tt<TT, 12, 4>(pa, ka, s, mid);      // 12 units, four producer waves
         return launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
     }
+}
+
+// Waves with two units each (kernels built on the 16-bit MFMA, units of one or two windows); packed: the
+// stream holds the tiles without their zeros.
+template <class TT>
+static hipError_t launch_panel_tall(const PanelArgs &pa, const KernelArgs &ka, bool packed, hipStream_t s, hipEvent_t mid)
+{
+    static_assert(PanelOps<TT>::kRows > 128u && TT::G <= 2, "two units per wave: 16 rows each");
+    return packed ? launch_panel_tt<TT, PanelOps<TT>::kConsumers, 4, true, true>(pa, ka, s, mid)
+                  : launch_panel_tt<TT, PanelOps<TT>::kConsumers, 4, true, false>(pa, ka, s, mid);
 }
 
 }  // namespace hspmm

@@ -172,6 +172,22 @@ int hspmm_set_kernel_mode(int mode);
  * as zeros, wherever that saves work. */
 int hspmm_set_window_pairing(int mode);
 
+/* Bitmap tiles on the device (the reference's CSR2BTCF format, src/utils/convert.h:22-139
+ * and BTCF_MTX of src/utils/class.h:55-67, which its kernel never reads).  Read by the
+ * next hspmm_create / hspmm_create_bitmap / hspmm_create_grouped.  mode 0 (default): the
+ * LDS-staging kernels stream their steps as uncompressed tiles.  mode 1: every consumer
+ * wave of theirs takes two units (one copy of a panel of B in LDS then serves twice the
+ * rows).  mode 2: as 1, and the tiles of the steps are kept on the device without their
+ * zeros - per step of 16 rows x 32 columns a 512-bit mask and the stored values - and
+ * expanded in registers (a lane finds its values by counting mask bits below it).
+ * Modes 1 and 2 apply to streams built on the 16-bit MFMA (fp16, bf16, fp32 in bf16
+ * parts) whose units have at most two windows; other plans ignore them.  Results are
+ * bit-identical in all three modes.  Both cut the bytes a launch moves (measured: a
+ * third and 60 % fewer 128-byte lines into the compute units) and neither makes it
+ * faster on the configurations measured: these kernels are bound by the LDS reads and
+ * MFMAs of a step, not by their traffic; hence the default. */
+int hspmm_set_panel_stream(int mode);
+
 /* No reference counterpart; host only (no device needed).  The grouping that the
  * LDS-staging kernels built on the 16-bit MFMA apply to their copy of the
  * matrix, for tests and for sizing: adjacent windows are merged into units of up
@@ -207,6 +223,8 @@ typedef struct {
     uint32_t n_panel_wide_units;    /* of those: units of three or four windows */
     uint32_t last_kernel_family;    /* what the last hspmm_run launched: 0 nothing yet, 1 all-shapes kernel, 2 gather (MFMA) kernels,
                                        3 LDS-staging kernels, 4 clear only (matrix without entries) */
+    uint32_t panel_stream_mode;     /* the LDS-staging stream as built (hspmm_set_panel_stream): 0 uncompressed tiles, 1 two units
+                                     * per consumer wave, 2 also tiles without their zeros; 0 when the plan has no such stream */
 } hspmm_plan_info;
 
 /* No reference counterpart (the reference prints its statistics from main,

@@ -1049,3 +1049,71 @@ def test_feature_blocks_dealt_out_by_xcd(torch_cuda, hs, oracle, dtype):
     got = gpu_spmm(torch_cuda, hs, bi, encode(Bm, dtype), 128, plan=plan)
     plan.close()
     assert np.array_equal(got, encode(D @ Bm, dtype))
+
+
+# ------------------------------------------------------------------ bitmap tiles on the device
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_panel_stream_with_two_units_per_wave_and_packed_tiles(torch_cuda, hs, oracle, dtype):
+    """hspmm_set_panel_stream: 1 = every consumer wave of the LDS-staging kernels takes two units,
+    2 = also the tiles of the steps without their zeros (masks + stored values, expanded in
+    registers).  The MFMA inputs are the same in all three modes, so with the same split into
+    chunks of panels the results are bit-identical; and exact-integer inputs are exact."""
+    rng = np.random.default_rng(70 + dtype)
+    feature_dims = (64, 128) if dtype == 1 else (128, 384)
+    cases = [
+        random_csr(rng, 300, 1000, 0.1, dtype, empty_row_prob=0.05),          # unions of overlapping column lists
+        random_csr(rng, 77, 530, 0.3, dtype),                                  # odd number of units, ragged last window
+        random_csr(rng, 24, 3000, 0.02, dtype, heavy_rows=(3,)),               # three windows, long runs of empty panels
+    ]
+    hs.set_kernel_mode(4)
+    try:
+        for ci, A in enumerate(cases):
+            b = convert(hs, A)
+            for N in feature_dims:
+                B = make_b(rng, A["cols"], N, dtype)
+                ref, mag = oracle_spmm(oracle, A, B, N)
+                for chunks in ("1", "3"):
+                    os.environ["HSPMM_PANEL_CHUNKS"] = chunks
+                    got = {}
+                    try:
+                        for mode in (0, 1, 2):
+                            hs.set_panel_stream(mode)
+                            plan = hs.Plan(b)
+                            got[mode] = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+                            info = plan.info()
+                            plan.close()
+                            assert info["last_kernel_family"] == 3
+                            assert info["panel_stream_mode"] == mode, (ci, N, mode, info)
+                    finally:
+                        hs.set_panel_stream(0)
+                        os.environ.pop("HSPMM_PANEL_CHUNKS", None)
+                    assert_parity(got[0], ref, mag, dtype, "case %d N=%d chunks=%s" % (ci, N, chunks))
+                    assert np.array_equal(got[1], got[0]), "two units per wave: case %d N=%d chunks=%s" % (ci, N, chunks)
+                    assert np.array_equal(got[2], got[0]), "packed tiles: case %d N=%d chunks=%s" % (ci, N, chunks)
+        # exact integers, with stored zeros, negative zeros and a dense window among sparse ones
+        rows, cols = 90, 700
+        D = rng.integers(-3, 4, (rows, cols)) * (rng.random((rows, cols)) < 0.12)
+        D[16:24] = rng.integers(1, 4, (8, cols))
+        rr, cc = np.nonzero(D)
+        rp = np.zeros(rows + 1, np.uint32)
+        rp[1:] = np.cumsum(np.bincount(rr, minlength=rows))
+        vals = D[rr, cc].astype(np.float32)
+        vals[::17] = 0.0                                                        # stored zeros
+        vals[5::29] = -0.0
+        D2 = np.zeros((rows, cols))
+        D2[rr, cc] = vals
+        Ai = dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=cc.astype(np.uint32), values=encode(vals, dtype))
+        bi = convert(hs, Ai)
+        N = feature_dims[0]
+        Bm = rng.integers(-4, 5, (cols, N))
+        for mode in (1, 2):
+            hs.set_panel_stream(mode)
+            plan = hs.Plan(bi)
+            got = gpu_spmm(torch_cuda, hs, bi, encode(Bm, dtype), N, plan=plan)
+            assert plan.info()["panel_stream_mode"] == mode
+            plan.close()
+            # (the sums are exact in fp32; the output is their one rounding to the storage type)
+            assert np.array_equal(decode(got, dtype), decode(encode(D2 @ Bm, dtype), dtype)), "mode %d" % mode
+    finally:
+        hs.set_panel_stream(0)
+        hs.set_kernel_mode(0)
