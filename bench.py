@@ -82,6 +82,8 @@ def main():
     ap.add_argument("--stages", type=int, default=0)
     ap.add_argument("--waves-per-group", type=int, default=0)
     ap.add_argument("--ranges-per-simd", type=int, default=0)
+    ap.add_argument("--panel-stream", type=int, default=0,
+                    help="stream of the LDS-panel kernels (hspmm_set_panel_stream): 0 tiles, 1 two units per wave, 2 packed tiles")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain device copy of 1 GiB (reference point for traffic counters)")
     args = ap.parse_args()
@@ -109,6 +111,7 @@ def main():
     t_gen = time.perf_counter() - t_gen
 
     hs.set_kernel_mode(args.mode)
+    hs.set_panel_stream(args.panel_stream)
     hs.configure(args.stages, args.waves_per_group, args.ranges_per_simd, 0)
     torch.zeros(1, device="cuda")                    # runtime initialised before anything is timed
     torch.cuda.synchronize()

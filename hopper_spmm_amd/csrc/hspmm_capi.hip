@@ -70,6 +70,7 @@ struct Config {
     int panel_max_windows = 0;          // 2 or 4: windows per unit of the panel stream (0: by matrix size)
     int panel_tall = 0;                 // LDS-panel waves with two units each (1: whenever the stream allows)
     int panel_packed = 0;               // ... and their tiles stored without zeros (1: whenever the stream allows)
+    int aligned_small = -1;             // small matrices: waves per unit of the one-workgroup-per-unit partition (-1: by size; 0, 4, 8)
     int xcd_split = -1;                 // gather kernels: two feature blocks dealt out by XCD half (-1: by matrix, 0 never, 1 always)
 
     void read_environment()
@@ -85,6 +86,7 @@ struct Config {
         if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) panel_chunks = std::max(1, std::atoi(e));
         if (const char *e = std::getenv("HSPMM_PANEL_MAX_WINDOWS")) panel_max_windows = std::atoi(e) >= 4 ? 4 : 2;
         if (const char *e = std::getenv("HSPMM_XCD_SPLIT")) xcd_split = std::atoi(e) != 0;
+        if (const char *e = std::getenv("HSPMM_ALIGNED_SMALL")) { const int v = std::atoi(e); aligned_small = v == 4 || v == 8 ? v : 0; }
         if (const char *e = std::getenv("HSPMM_PANEL_TALL")) panel_tall = std::atoi(e) != 0;
         if (const char *e = std::getenv("HSPMM_PANEL_PACKED")) panel_packed = std::atoi(e) != 0;
     }
@@ -1319,6 +1321,18 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
             const double four_from = p->cfg.aligned_four_from;
             const int group = ways >= 8.0 ? hspmm::kAlignedGroupWaves : ways >= four_from ? hspmm::kMaxWavesPerGroup : 0;
             if (group && shortest >= 8u * uint32_t(group) && uint64_t(p->n_units) * group <= (1u << 24)) p->aligned_group = group;
+            // A matrix too small to fill the waves of the GPU with ranges of useful length: what its launch takes
+            // is one wave walking its range step by step (4096 x 4096 at 1 %: 434 waves of 24 dependent steps).
+            // One workgroup per unit, its waves a quarter (an eighth) of the unit's steps each, shortens that walk.
+            const uint64_t wave_slots = uint64_t(p->compute_units) * 16u;
+            int small_group = 0;
+            if (p->cfg.aligned_small < 0) {
+                if (!p->aligned_group && p->parts[0].part.ranges.size() * 4u <= wave_slots && uint64_t(p->n_units) * 4u <= wave_slots)
+                    small_group = hspmm::kMaxWavesPerGroup;      // (eight waves per unit measured no faster: 7.2 against 6.8 us)
+            } else {
+                small_group = p->cfg.aligned_small;
+            }
+            if (small_group && shortest >= 2u * uint32_t(small_group)) p->aligned_group = small_group;
         }
         // (the LDS-panel stream re-tiles ascending column lists; a caller's lists in another order stay
         // with the gather and all-shapes kernels)
@@ -1591,7 +1605,8 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     // 18.9 + 6.4 us -> 19 us; random 8192 x 8192 at 2 %, N = 128: 26.8 + 7.1 -> 22.8 us).  With the default
     // knobs only: the eight-wave kernels exist for the default depths.
     const bool aligned = combine && p->aligned_group && c.narrow && p->cfg.consumer_warp_num == 0 &&
-                         p->cfg.buffer_stage == 0 && p->cfg.producer_warp_group_num == 0;
+                         (p->cfg.buffer_stage == 0 || p->aligned_group == hspmm::kMaxWavesPerGroup) &&
+                         p->cfg.producer_warp_group_num == 0;
     if (aligned) wpg = p->aligned_group;
     hspmm_plan::DevPartition &dp = p->parts[aligned ? 4 : combine ? 3 : level];
     {

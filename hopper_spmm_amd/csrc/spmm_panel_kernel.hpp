@@ -381,7 +381,7 @@ struct PanelOps<Fp32Split<G_>> {
     }
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) & 15u; }
     __device__ static __forceinline__ bool second_unit(const Idx I) { return (__builtin_amdgcn_readfirstlane(I) >> 28) & 1u; }
-    static constexpr uint32_t kPackedRing = 4;                    // steps in flight when the tiles are packed
+    static constexpr uint32_t kPackedRing = 2;                    // steps in flight when the tiles are packed (four measured slower)
     // the lane's eight values (hi half | lo half << 16) from their positions in the packed values
     // (position 0 holds a zero), rearranged to four words of hi halves and four of lo halves
     __device__ static __forceinline__ AVec gather_a(const void *vals, const uint32_t (&pos)[8])

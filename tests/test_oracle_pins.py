@@ -109,6 +109,32 @@ def test_loader_matches_scipy_on_random_files(oracle, tmp_path):
                 assert np.array_equal(m["values"], ref.data.astype(np.float16).view(np.uint16))
 
 
+def test_csr_validate_counts_every_kind_of_violation(oracle):
+    """orc_csr_validate restates the structural checks of the reference's loader (src/utils/load.h:44-73):
+    row_ptr[0] == 0, row_ptr[rows] == nnz, row_ptr never decreasing, every column index below cols.
+    Each violation is planted alone and together, and counted."""
+    rows, cols = 4, 6
+    good_ptr = np.array([0, 2, 2, 5, 6], np.uint32)
+    good_idx = np.array([0, 5, 1, 2, 4, 3], np.uint32)
+    assert oracle.csr_validate(rows, cols, good_ptr, good_idx) == 0
+    # first offset not zero (load.h:44-47); the offsets stay ascending and end at nnz
+    assert oracle.csr_validate(rows, cols, np.array([1, 2, 2, 5, 6], np.uint32), good_idx) == 1
+    # last offset differs from the number of entries (load.h:49-53)
+    assert oracle.csr_validate(rows, cols, np.array([0, 2, 2, 5, 5], np.uint32), good_idx) == 1
+    # offsets that decrease, once and twice (load.h:56-62)
+    assert oracle.csr_validate(rows, cols, np.array([0, 3, 2, 5, 6], np.uint32), good_idx) == 1
+    assert oracle.csr_validate(rows, cols, np.array([0, 3, 2, 1, 6], np.uint32), good_idx) == 2
+    # column indices outside the matrix, one and three of them (load.h:66-73); cols - 1 is the last valid one
+    bad_idx = good_idx.copy(); bad_idx[1] = cols
+    assert oracle.csr_validate(rows, cols, good_ptr, bad_idx) == 1
+    bad_idx[[0, 4]] = [cols + 7, 0xFFFFFFFF]
+    assert oracle.csr_validate(rows, cols, good_ptr, bad_idx) == 3
+    # everything at once: 1 (first offset) + 1 (last offset) + 1 (decrease) + 3 (columns)
+    assert oracle.csr_validate(rows, cols, np.array([1, 3, 2, 5, 7], np.uint32), bad_idx) == 6
+    # an empty matrix is valid
+    assert oracle.csr_validate(0, 0, np.array([0], np.uint32), np.zeros(0, np.uint32)) == 0
+
+
 def test_loader_failure_paths(oracle, tmp_path):
     with pytest.raises(OSError):
         oracle.mtx_read(str(tmp_path / "missing.mtx"), "fp16")          # load.h:176-180

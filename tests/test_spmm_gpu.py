@@ -1117,3 +1117,42 @@ def test_panel_stream_with_two_units_per_wave_and_packed_tiles(torch_cuda, hs, o
     finally:
         hs.set_panel_stream(0)
         hs.set_kernel_mode(0)
+
+
+# ------------------------------------------------------------------ staging layout of the LDS-panel kernels
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_lds_staging_hands_every_b_row_to_its_column(torch_cuda, hs, dtype):
+    """The LDS-staging kernels copy rows of B into an LDS image and read them back with the
+    transposing LDS read (the row gathered by the address, four k of one feature per lane).  Here every
+    row of A has a single entry 1 at column c, and B[k][f] encodes (k, f): row r of C must be row c of
+    B, bit for bit.  The entry visits every k-slot of a 32-column step, both windows of a pair of
+    windows, columns in several panels and both LDS images (the reference checks its staged copy the
+    same way, by coordinates: test/01.tma_copy_matrix/copy.cu:149-170)."""
+    rng = np.random.default_rng(90 + dtype)
+    rows, cols, N = 16, 700, 128 if dtype != 1 else 64
+    k_idx, f_idx = np.meshgrid(np.arange(cols), np.arange(N), indexing="ij")
+    Bm = (k_idx * 5 + f_idx * 3) % 251                                   # exact in every element type; rows differ
+    B = encode(Bm.astype(np.float32), dtype)
+    # 40 columns: a full step of 32 in panel 0, some in panel 1 (256..511) and panel 2
+    used = np.sort(np.concatenate([rng.choice(256, 32, replace=False), 256 + rng.choice(256, 5, replace=False),
+                                   512 + rng.choice(188, 3, replace=False)])).astype(np.uint32)
+    hs.set_kernel_mode(4)
+    try:
+        for shift in range(used.size):
+            # every used column appears (so that the window's column list, and the step layout, stay the same)
+            # with value 0, except the one per row that carries the 1
+            hot = used[(np.arange(rows) * 3 + shift) % used.size]
+            vals = np.zeros((rows, used.size), np.float32)
+            vals[np.arange(rows), (np.arange(rows) * 3 + shift) % used.size] = 1.0
+            rp = (np.arange(rows + 1) * used.size).astype(np.uint32)
+            A = dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=np.tile(used, rows),
+                     values=encode(vals.reshape(-1), dtype))
+            b = convert(hs, A)
+            plan = hs.Plan(b)
+            got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+            assert plan.info()["last_kernel_family"] == 3
+            plan.close()
+            want = decode(B, dtype)[hot]
+            assert np.array_equal(decode(got, dtype), want), "shift %d" % shift
+    finally:
+        hs.set_kernel_mode(0)
