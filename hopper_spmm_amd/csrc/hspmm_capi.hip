@@ -57,7 +57,8 @@ struct Config {
     int producer_warp_group_num = 0;
     int sm_num = 0;
     int kernel_mode = 0;
-    int fused_fixup = 0;                // 1: the last wave of a cut unit adds its partial sums; 0: second kernel
+    int fused_fixup = -1;               // 1: the last wave of a cut unit adds its partial sums; 0: second kernel;
+                                        // -1: the former where few units are cut (gather kernels, several feature blocks)
     int pairing = 0;                    // 0 automatic, 1 never, 2 whenever two windows share a column list
     // Tuning overrides from the environment (HSPMM_*), read once by hspmm_create: a plan's behaviour does
     // not change with the environment afterwards and the launch path reads no variable.
@@ -75,7 +76,7 @@ struct Config {
 
     void read_environment()
     {
-        if (const char *e = std::getenv("HSPMM_FUSED_FIXUP")) fused_fixup = std::atoi(e);
+        if (const char *e = std::getenv("HSPMM_FUSED_FIXUP")) fused_fixup = std::atoi(e) != 0;
         if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);
         if (const char *e = std::getenv("HSPMM_SLACK")) slack = std::atof(e);
         if (const char *e = std::getenv("HSPMM_WHOLE_WINDOW_MARGIN")) whole_window_margin = std::atof(e);
@@ -147,6 +148,7 @@ struct hspmm_plan {
         bool tall = false;                                       // two units per consumer wave: poff per pair of units,
                                                                  // their steps merged panel by panel
         bool packed = false;                                     // tiles without their zeros: masks, values, step_voff
+        double unit_lines = 0.0;                                 // 128-byte lines of tiles and ids per unit and panel (tall streams)
         uint64_t *d_masks = nullptr;
         void *d_vals = nullptr;
         uint32_t *d_step_voff = nullptr;
@@ -951,6 +953,14 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
         pl.d_tiles = dt;
     }
     pl.tall = tall; pl.packed = packed;
+    if (tall) {
+        size_t stored = 0;
+        const uint16_t *hv = reinterpret_cast<const uint16_t *>(tiles.data());
+        if (packed) for (size_t i = 0, n = tiles.size() * 2; i < n; ++i) stored += hv[i] != 0;
+        const double step_bytes = 64.0 + (packed ? 64.0 + 2.0 * double(stored) / double(std::max<uint32_t>(ps.n_steps, 1u))
+                                                 : double(tiles.size()) * 4.0 / double(std::max<uint32_t>(ps.n_steps, 1u)));
+        pl.unit_lines = step_bytes * double(ps.n_steps) / (double(U) * double(NP)) / 128.0;
+    }
     if ((rc = upload(&pl.d_unitRow, st.unitRow.data(), st.unitRow.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     pl.n_units = U; pl.G = st.G; pl.n_paired = st.n_paired; pl.n_wide = st.n_wide;
     pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.split = split; pl.density = density; pl.built = true;
@@ -1482,8 +1492,11 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         const uint64_t ppc = (pl.n_panels + ch - 1) / ch;
         ch = (pl.n_panels + ppc - 1) / ppc;
         const uint64_t rounds = (base * ch + slots - 1) / slots;
-        const double units_here = double(nc) * (pl.tall ? 2.0 : 1.0);
-        const double cost = double(rounds) * double(ppc) * (units_here + 3.0) + (ch > 1 ? 80.0 : 0.0);
+        // (streams with two units per wave: the same in 128-byte lines - per panel its copy and every unit's
+        // tiles and ids - which is what those streams were measured with)
+        const double cost = pl.tall ? double(rounds) * double(ppc) * (512.0 + 2.0 * double(nc) * pl.unit_lines) +
+                                          (ch > 1 ? 2500.0 + 300.0 * double(ch) : 0.0)
+                                    : double(rounds) * double(ppc) * (double(nc) + 3.0) + (ch > 1 ? 80.0 : 0.0);
         if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best_units = nc; chunks = ch; }
     }
     pa.units_per_group = uint32_t(best_units);
@@ -1510,7 +1523,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
             // (experiment, as in the gather kernels: the wave that brings a unit's last chunk adds the chunk sums
             // itself; the device-scope accesses cost more than the second launch: 61.7 + 8.8 -> 76.8 us on the
             // block-clustered configuration at N = 512)
-            if (p->cfg.fused_fixup && mode != RunMode::kStatic &&
+            if (p->cfg.fused_fixup > 0 && mode != RunMode::kStatic &&
                 (rc = ensure_arrive(p, size_t(pl.n_units) * pa.n_feat_blocks, &pa.arrive)))
                 return rc;
         }
@@ -1597,13 +1610,13 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     // One feature block: the waves of a workgroup walk consecutive ranges and add the partial sums of
     // one unit among themselves.
     int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
-    const bool fused = p->cfg.fused_fixup && mode != RunMode::kStatic;
-    const bool combine = level == 0 && ka.n_feat_blocks == 1 && wpg > 1 && !p->cfg.fused_fixup;
+    const bool combine = level == 0 && ka.n_feat_blocks == 1 && wpg > 1 && p->cfg.fused_fixup <= 0;
     // Units that are all long (block-clustered, pruned or dense-ish random matrices at a small N): every
     // unit is cut into the ranges of one workgroup of four or eight waves, which stores it itself - no
     // partial sums leave the chip and there is no second launch (block-clustered 4096 x 14336, N = 16:
     // 18.9 + 6.4 us -> 19 us; random 8192 x 8192 at 2 %, N = 128: 26.8 + 7.1 -> 22.8 us).  With the default
     // knobs only: the eight-wave kernels exist for the default depths.
+    bool fused = false;
     const bool aligned = combine && p->aligned_group && c.narrow && p->cfg.consumer_warp_num == 0 &&
                          (p->cfg.buffer_stage == 0 || p->aligned_group == hspmm::kMaxWavesPerGroup) &&
                          p->cfg.producer_warp_group_num == 0;
@@ -1621,6 +1634,12 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         }
         ka.n_ranges = uint32_t(dp.part.ranges.size());
         ka.n_split = uint32_t(dp.part.split.size());
+        // The wave that brings a cut unit's last partial sum adds them itself (in range order, as the second
+        // kernel would): worth it where few units are cut and the second launch is most of what they cost
+        // (power-law graph, 382 of 110 746 units: 540.6 + 9.4 -> 541.1 us); where every unit is cut the
+        // device-scope traffic costs more than the launch (block-clustered: 30 -> 129 us).
+        fused = mode != RunMode::kStatic && !combine &&
+                (p->cfg.fused_fixup > 0 || (p->cfg.fused_fixup < 0 && ka.n_split && uint64_t(ka.n_split) * 32u <= p->n_units));
         if (uint64_t(ka.n_ranges) * ka.n_feat_blocks > 0x7FFFFFFFull)
             return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many work items", N);
         const size_t need = size_t(dp.part.n_slots) * ka.n_feat_blocks * size_t(c.V) * size_t(p->G) * 64u * 16u;
