@@ -72,6 +72,7 @@ struct Config {
     int panel_tall = 0;                 // LDS-panel waves with two units each (1: whenever the stream allows)
     int panel_packed = 0;               // ... and their tiles stored without zeros (1: whenever the stream allows)
     int aligned_small = -1;             // small matrices: waves per unit of the one-workgroup-per-unit partition (-1: by size; 0, 4, 8)
+    int gather_bitmap = -1;             // gather kernels read single 16-bit windows as bitmap + stored elements (-1: by fill)
     int xcd_split = -1;                 // gather kernels: two feature blocks dealt out by XCD half (-1: by matrix, 0 never, 1 always)
 
     void read_environment()
@@ -87,6 +88,7 @@ struct Config {
         if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) panel_chunks = std::max(1, std::atoi(e));
         if (const char *e = std::getenv("HSPMM_PANEL_MAX_WINDOWS")) panel_max_windows = std::atoi(e) >= 4 ? 4 : 2;
         if (const char *e = std::getenv("HSPMM_XCD_SPLIT")) xcd_split = std::atoi(e) != 0;
+        if (const char *e = std::getenv("HSPMM_GATHER_BITMAP")) gather_bitmap = std::atoi(e) != 0;
         if (const char *e = std::getenv("HSPMM_ALIGNED_SMALL")) { const int v = std::atoi(e); aligned_small = v == 4 || v == 8 ? v : 0; }
         if (const char *e = std::getenv("HSPMM_PANEL_TALL")) panel_tall = std::atoi(e) != 0;
         if (const char *e = std::getenv("HSPMM_PANEL_PACKED")) panel_packed = std::atoi(e) != 0;
@@ -154,6 +156,15 @@ struct hspmm_plan {
         uint32_t *d_step_voff = nullptr;
         double density = 0.0;                                    // steps per unit and 128 columns of the gather stream
     } panel;
+    // Bitmap stream of the gather kernels (single 16-bit windows whose tiles are mostly zeros): per tile 8 words
+    // of header (the reference's tcBit words of the tile, bit counts, position of the first stored element) and
+    // the stored elements of all tiles in ascending bit order - nnzOffset / tcBit / data of the reference's BTCF_MTX
+    struct Bitmap {
+        bool built = false;
+        uint32_t *d_header = nullptr;
+        void *d_vals = nullptr;
+        uint64_t stored = 0;
+    } bm;
     float *d_scratch = nullptr;
     size_t scratch_bytes = 0;
     uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
@@ -706,6 +717,39 @@ void pack_steps(size_t n_steps, bool split, const std::vector<uint32_t> &tiles, 
     });
 }
 
+// The bitmap stream of the gather kernels (Fp16TileDWB in spmm_mfma_kernel.hpp) from the uncompressed 8 x 16 tiles
+// of a 16-bit matrix: per tile the bitmap of the reference's CSR2BTCF (bit 16 r + k for element (r, k), reference
+// src/utils/convert.h:83-101; an element is stored when its bit pattern is not +0) as four 32-bit words, the bit
+// counts of words 0, 0..1 and 0..2 in bytes 1..3 of word 4, and in word 5 the position of the tile's first stored
+// element in `vals` (the reference's nnzOffset), where the stored elements follow tile after tile in bit order.
+void build_gather_bitmap(uint32_t T, const void *data, std::vector<uint32_t> &header, std::vector<uint16_t> &vals)
+{
+    const uint16_t *h = static_cast<const uint16_t *>(data);
+    header.assign(size_t(T) * 8u, 0u);
+    std::vector<uint32_t> count(size_t(T) + 1, 0u);
+    hspmm_host::parallel_blocks(T, 4096, [&](size_t tb, size_t te) {
+        for (size_t t = tb; t < te; ++t) {
+            const uint16_t *tile = h + t * 128u;
+            uint32_t *hd = header.data() + t * 8u;
+            for (uint32_t b = 0; b < 128u; ++b) if (tile[b]) hd[b >> 5] |= 1u << (b & 31u);
+            const uint32_t c0 = uint32_t(__builtin_popcount(hd[0])), c1 = c0 + uint32_t(__builtin_popcount(hd[1])),
+                           c2 = c1 + uint32_t(__builtin_popcount(hd[2]));
+            hd[4] = c0 << 8 | c1 << 16 | c2 << 24;
+            count[t + 1] = c2 + uint32_t(__builtin_popcount(hd[3]));
+        }
+    });
+    uint64_t total = 0;
+    for (size_t t = 0; t < T; ++t) { header[t * 8u + 5u] = uint32_t(total); total += count[t + 1]; }
+    vals.assign(size_t(total) + 4u, 0);                            // a lane reads 8 bytes from its first element
+    hspmm_host::parallel_blocks(T, 4096, [&](size_t tb, size_t te) {
+        for (size_t t = tb; t < te; ++t) {
+            const uint16_t *tile = h + t * 128u;
+            size_t at = header[t * 8u + 5u];
+            for (uint32_t b = 0; b < 128u; ++b) if (tile[b]) vals[at++] = tile[b];
+        }
+    });
+}
+
 // Re-tiles the matrix panel by panel for the LDS-panel kernels (spmm_panel_kernel.hpp):
 // inside every window the columns of one panel of kPanelRows columns get tiles of
 // their own.  Every step carries the number of panels it lies behind the step in
@@ -999,6 +1043,7 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
         if (N % 8 == 0 && !(align & 15u) && N > 32) c.V = 4;
         else if (N % 4 == 0 && !(align & 7u) && N > 16) c.V = 2;
         else c.V = 1;
+        if (split_features && c.V == 4 && (N == 128 || N == 256 || N == 512)) c.V = 2;
         c.block_feat = 32 * c.V;
         return c;
     }
@@ -1318,6 +1363,34 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
             if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) return bail(rc);
             p->d_tiles = dt;
         }
+        // Single 16-bit windows with few stored elements per tile (graphs: 16 of 128): the gather kernels read the
+        // tiles as bitmap + stored elements, 32 + 2 x 16 bytes per tile instead of 256 (power-law graph 2^20 at
+        // N = 128, where the stream is read once per XCD half: 0.64 -> 0.19 GB per launch).
+        if (dtype != HSPMM_TF32 && st.G == 1 && p->cfg.gather_bitmap != 0 && total_tiles) {
+            size_t stored = 0;
+            if (p->cfg.gather_bitmap < 0) {
+                const uint16_t *hv = static_cast<const uint16_t *>(data);
+                const size_t n = size_t(total_tiles) * 128u, sample = std::min<size_t>(n, size_t(1) << 22);
+                for (size_t i = 0; i < sample; ++i) stored += hv[i] != 0;
+                stored = size_t(double(stored) * double(n) / double(sample));
+            }
+            // 32 + 2 e bytes against 256 per tile with e stored elements: worth it below about a third full, and
+            // where the tile stream is large enough to be traffic at all (a matrix whose tiles sit in the L2s only
+            // pays the longer dependent chain: 4096 x 4096 at 1 %, 2.7 MB of tiles: 6.8 -> 7.5 us)
+            if (p->cfg.gather_bitmap > 0 ||
+                (stored * 3u < size_t(total_tiles) * 128u && size_t(total_tiles) * 256u >= (size_t(8) << 20))) {
+                std::vector<uint32_t> header;
+                std::vector<uint16_t> vals;
+                try { build_gather_bitmap(total_tiles, data, header, vals); }
+                catch (const std::bad_alloc &) { return bail(fail(HSPMM_ERR_ALLOC, "out of host memory")); }
+                if (vals.size() < (size_t(1) << 31)) {               // positions are 32-bit
+                    uint16_t *dv = nullptr;
+                    if ((rc = upload(&p->bm.d_header, header.data(), header.size(), &p->fixed_bytes))) return bail(rc);
+                    if ((rc = upload(&dv, vals.data(), vals.size(), &p->fixed_bytes))) return bail(rc);
+                    p->bm.d_vals = dv; p->bm.stored = vals.size() - 4u; p->bm.built = true;
+                }
+            }
+        }
         p->h_unitOffset = st.unitOffset;
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
         {
@@ -1417,6 +1490,7 @@ void hspmm_destroy(hspmm_plan *p)
     (void)hipFree(p->panel.d_unitRow);
     (void)hipFree(p->panel.d_step_panel);
     (void)hipFree(p->panel.d_masks); (void)hipFree(p->panel.d_vals); (void)hipFree(p->panel.d_step_voff);
+    (void)hipFree(p->bm.d_header); (void)hipFree(p->bm.d_vals);
     (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive);
     for (void *old : p->retired) (void)hipFree(old);
     delete p;
@@ -1595,6 +1669,11 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         return HSPMM_OK;
     }
     ka.unitOffset = p->d_unitOffset; ka.unitRow = p->d_unitRow; ka.ids = p->d_ids; ka.tiles = p->d_tiles;
+    int layout = c.layout;
+    if (p->bm.built && c.layout == hspmm::kLayoutDW && (c.V == 2 || c.V == 4) && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 3)) {
+        layout = hspmm::kLayoutDWB;                   // tiles as bitmap + stored elements
+        ka.tiles = p->bm.d_vals; ka.bm_header = p->bm.d_header;
+    }
     ka.n_units = p->n_units;
     ka.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
     ka.xcd_split = (want_split && (ka.n_feat_blocks == 2u || ka.n_feat_blocks == 4u || ka.n_feat_blocks == 8u)) ? 1u : 0u;
@@ -1654,7 +1733,7 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage
                          : p->dtype == HSPMM_TF32 ? (p->G == 2 && c.V == 4 ? 3 : 4)
                          : (p->G == 2 && c.V == 4 ? 2 : 3);
-    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, c.layout, p->G, ka, c.V, prefetch, c.narrow, wpg, s, mid));
+    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, layout, p->G, ka, c.V, prefetch, c.narrow, wpg, s, mid));
     return HSPMM_OK;
 }
 
@@ -1785,6 +1864,7 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_panel_paired_units = p->panel.built ? p->panel.n_paired : 0u;
     info->n_panel_wide_units = p->panel.built ? p->panel.n_wide : 0u;
     info->last_kernel_family = p->last_family.load(std::memory_order_relaxed);
+    info->gather_bitmap = p->bm.built ? 1u : 0u;
     info->panel_stream_mode = !p->panel.built ? 0u : p->panel.packed ? 2u : p->panel.tall ? 1u : 0u;
     return HSPMM_OK;
 }

@@ -26,7 +26,9 @@ struct KernelArgs {
     const uint32_t *unitOffset;  // n_units + 1: first step of every unit
     const uint32_t *unitRow;     // n_units: first matrix row of the unit | its windows less one (1: a pair)
     const uint32_t *ids;         // per step, lane order, padding ids renamed
-    const void     *tiles;       // per step, lane order
+    const void     *tiles;       // per step, lane order; bitmap stream: the stored elements, tile after tile
+    const uint32_t *bm_header;   // bitmap stream (kLayoutDWB): per step 8 words - the tile's four bitmap words, the bit
+                                 // counts of words 0, 0..1, 0..2 (bytes 1..3), the position of its first stored element
     // partition
     const uint32_t *ranges;      // n_ranges x kRangeWords
     const uint32_t *split;       // n_split x kFixWords {unit, slot_begin, slot_count, 0}
@@ -46,7 +48,7 @@ struct KernelArgs {
 // per B row (1, 2 or 4).
 // layout (fp16 only): kLayoutX4 = wide loads, contiguous features per lane, N % (2V) == 0;
 // kLayoutDW = word loads, features strided by 32 per lane, N % (32V) == 0.
-constexpr int kLayoutX4 = 0, kLayoutDW = 1;
+constexpr int kLayoutX4 = 0, kLayoutDW = 1, kLayoutDWB = 2;   // DWB: word loads, tiles as bitmap + stored elements (16-bit, G = 1)
 // element types, numbered as HSPMM_FP16 / HSPMM_TF32 / HSPMM_BF16 of the public header
 constexpr int kDtypeF16 = 0, kDtypeF32 = 1, kDtypeBf16 = 2;
 // narrow: B < 4 GiB and cols < 2^24 (32-bit gather offsets).

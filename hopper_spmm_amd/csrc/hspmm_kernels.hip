@@ -84,9 +84,19 @@ HSPMM_DECLARE_LAUNCH(launch_mfma_bf16_g1) HSPMM_DECLARE_LAUNCH(launch_mfma_bf16_
 HSPMM_DECLARE_LAUNCH(launch_mfma_f32_g1) HSPMM_DECLARE_LAUNCH(launch_mfma_f32_g2)
 #undef HSPMM_DECLARE_LAUNCH
 
+hipError_t launch_mfma_f16_bm(const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, hipStream_t s,
+                              hipEvent_t mid);
+hipError_t launch_mfma_bf16_bm(const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, hipStream_t s,
+                               hipEvent_t mid);
+
 hipError_t launch_spmm_mfma(int dtype, int layout, int G, const KernelArgs &ka, int V, int prefetch, bool narrow,
                             int waves_per_group, hipStream_t s, hipEvent_t mid)
 {
+    if (layout == kLayoutDWB) {
+        if (G != 1 || dtype == kDtypeF32) return hipErrorInvalidValue;
+        return dtype == kDtypeBf16 ? launch_mfma_bf16_bm(ka, V, prefetch, narrow, waves_per_group, s, mid)
+                                   : launch_mfma_f16_bm(ka, V, prefetch, narrow, waves_per_group, s, mid);
+    }
     if (dtype == kDtypeF32)
         return G == 2 ? launch_mfma_f32_g2(layout, ka, V, prefetch, narrow, waves_per_group, s, mid)
                       : launch_mfma_f32_g1(layout, ka, V, prefetch, narrow, waves_per_group, s, mid);

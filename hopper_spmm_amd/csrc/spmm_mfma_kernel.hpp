@@ -171,8 +171,11 @@ struct Fp16Lane {
     uint32_t sel_lo, sel_hi;                   // byte selectors for the sparse operand
     const uint32_t *a_src;                     // lane's words inside step 0
     const uint32_t *idx_src;                   // lane's ids inside step 0
+    const void *a_base;                        // the tile array itself
+    __device__ __forceinline__ const void *a_src_base() const { return a_base; }
     __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
     {
+        a_base = tiles;
         g = lane >> 4; j = lane & 15u;
         const uint32_t r = j >> 1, parity = j & 1u;
         // v_perm_b32 selectors: bytes 0-3 come from the second source, 0x0c gives 0x00.
@@ -366,6 +369,101 @@ struct Fp16TileDW {
     }
 };
 
+// fp16 / bf16, layout "DW", single windows, tiles read as bitmap + stored values: the reference's
+// bitmap tile format (BTCF_MTX of reference src/utils/class.h:55-67, written by CSR2BTCF,
+// src/utils/convert.h:83-101, and never read by the reference's kernel) - per 8 x 16 tile
+// 128 bits, bit 16 r + k set for a stored element, and the stored elements of all tiles one
+// after the other in ascending bit order.  A lane's four elements a[j/2][4g .. 4g + 3] are four
+// consecutive bits, so its stored elements are consecutive too: it counts the tile's bits in
+// front of them, loads 8 bytes from there (2-byte aligned) and puts the element of bit i, if
+// set, where the dense form has it - the v_perm of the dense form with selectors made from the
+// four bits.  A power-law graph stores 16 of a tile's 128 elements: 48 bytes instead of 256.
+//   header per step (uniform, scalar loads): the four bitmap words, the counts of words 0, 0..1,
+//   0..2 (one byte each, from bit 8 on) and the position of the tile's first stored element.
+typedef u32x2 u32x2_unaligned __attribute__((aligned(2)));
+struct BitmapHeader { uint32_t d[4]; uint32_t counts; uint32_t first; };
+
+template <int V_, bool BF = false>
+struct Fp16TileDWB : Fp16TileDW<V_, 1, BF> {
+    typedef Fp16TileDW<V_, 1, BF> Base;
+    static constexpr int V = V_, G = 1;
+    typedef typename Base::BVec BVec;
+    struct Idx { u32x4 ids; BitmapHeader h; };
+    struct AVec { u32x2 stored; uint32_t bits; };  // the 8 bytes at the lane's first stored element; its four bits
+    struct Lane : Fp16Lane<1> {
+        const uint32_t *header;                    // 8 words per step
+        uint32_t word, low_mask, shift, sel_base, sel_step;
+        __device__ __forceinline__ void init(uint32_t lane, const void *vals, const uint32_t *ids)
+        {
+            Fp16Lane<1>::init(lane, vals, ids);
+            const uint32_t r = this->j >> 1, parity = this->j & 1u;
+            word = r >> 1;                          // bitmap word of row r: bits 16 (r & 1) + k
+            shift = 16u * (r & 1u) + 4u * this->g;  // the lane's first bit inside that word
+            low_mask = (1u << shift) - 1u;
+            // v_perm_b32 selector of stored element n (bytes 2n, 2n + 1 of the 8 loaded): into the low half
+            // for an even MFMA row, the high half for an odd one; 0x0c gives 0x00
+            sel_base = parity ? 0x01000c0cu : 0x0c0c0100u;
+            sel_step = parity ? 0x02020000u : 0x00000202u;
+        }
+        __device__ __forceinline__ void bind_bitmap(const uint32_t *h) { header = h; }
+    };
+    __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t step)
+    {
+        Idx I;
+        I.ids = L.load_idx(step);
+        const const_u32_ptr h = as_const(L.header) + size_t(step) * 8u;      // uniform: scalar loads
+#pragma unroll
+        for (int i = 0; i < 4; ++i) I.h.d[i] = h[i];
+        I.h.counts = h[4]; I.h.first = h[5];
+        return I;
+    }
+    template <class GT>
+    __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t, const Idx &I, const GT &gat,
+                                                     BVec &b0, BVec &b1, BVec &b2, BVec &b3, AVec &a)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(gat.row(I.ids[q]));
+            b0[q] = src[0];
+            if constexpr (V > 1) b1[q] = src[16];
+            if constexpr (V > 2) b2[q] = src[32];
+            if constexpr (V > 3) b3[q] = src[48];
+        }
+        const uint32_t w = L.word == 0u ? I.h.d[0] : L.word == 1u ? I.h.d[1] : L.word == 2u ? I.h.d[2] : I.h.d[3];
+        const uint32_t before = __builtin_amdgcn_ubfe(I.h.counts, 8u * L.word, 8u) + uint32_t(__builtin_popcount(w & L.low_mask));
+        a.bits = (w >> L.shift) & 15u;
+        const char *vals = reinterpret_cast<const char *>(L.a_src_base());
+        a.stored = *reinterpret_cast<const u32x2_unaligned *>(vals + 2u * size_t(I.h.first + before));
+    }
+    __device__ static __forceinline__ u32x4 sparse_operand(const Lane &L, const AVec &a)
+    {
+        // element i of the four sits at stored position (set bits below bit i), if its bit is set
+        const uint32_t n1 = a.bits & 1u, n2 = uint32_t(__builtin_popcount(a.bits & 3u)), n3 = uint32_t(__builtin_popcount(a.bits & 7u));
+        const uint32_t none = 0x0c0c0c0cu;
+        const uint32_t s0 = (a.bits & 1u) ? L.sel_base : none;
+        const uint32_t s1 = (a.bits & 2u) ? L.sel_base + n1 * L.sel_step : none;
+        const uint32_t s2 = (a.bits & 4u) ? L.sel_base + n2 * L.sel_step : none;
+        const uint32_t s3 = (a.bits & 8u) ? L.sel_base + n3 * L.sel_step : none;
+        u32x4 aw;
+        aw[0] = __builtin_amdgcn_perm(a.stored[1], a.stored[0], s0);
+        aw[1] = __builtin_amdgcn_perm(a.stored[1], a.stored[0], s1);
+        aw[2] = __builtin_amdgcn_perm(a.stored[1], a.stored[0], s2);
+        aw[3] = __builtin_amdgcn_perm(a.stored[1], a.stored[0], s3);
+        return aw;
+    }
+    __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
+                                               const BVec &b3, const AVec &a, f32x4 (&acc)[V])
+    {
+        const u32x4 av = sparse_operand(L, a);
+        acc[0] = HalfOps<BF>::mfma(av, b0, acc[0]);
+        if constexpr (V > 1) acc[1] = HalfOps<BF>::mfma(av, b1, acc[1]);
+        if constexpr (V > 2) acc[2] = HalfOps<BF>::mfma(av, b2, acc[2]);
+        if constexpr (V > 3) acc[3] = HalfOps<BF>::mfma(av, b3, acc[3]);
+    }
+};
+template <class TT> struct TileTraits { static constexpr bool kBitmap = false; };
+template <int V, bool BF> struct TileTraits<Fp16TileDWB<V, BF>> { static constexpr bool kBitmap = true; };
+
 // fp32 storage ("tf32" build of the reference): 8x8 tiles, v_mfma_f32_16x16x4_f32.
 // MFMA rows 0..7 are the window rows, rows 8..15 zero; lane (g, j) supplies k = g
 // and k = g + 4 of a tile and V contiguous features.
@@ -533,6 +631,7 @@ void spmm_mfma_kernel(const KernelArgs ka)
 
     typename TT::Lane L;
     L.init(lane, ka.tiles, ka.ids);
+    if constexpr (TileTraits<TT>::kBitmap) L.bind_bitmap(ka.bm_header);
     const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
     const bool active = feat < ka.N;
     const size_t row_bytes = size_t(ka.N) * TT::kElem;

@@ -223,6 +223,8 @@ typedef struct {
     uint32_t n_panel_wide_units;    /* of those: units of three or four windows */
     uint32_t last_kernel_family;    /* what the last hspmm_run launched: 0 nothing yet, 1 all-shapes kernel, 2 gather (MFMA) kernels,
                                        3 LDS-staging kernels, 4 clear only (matrix without entries) */
+    uint32_t gather_bitmap;         /* 1: the gather kernels read this plan's tiles as bitmap + stored elements (single 16-bit
+                                     * windows with few stored elements per tile), 0: as uncompressed tiles */
     uint32_t panel_stream_mode;     /* the LDS-staging stream as built (hspmm_set_panel_stream): 0 uncompressed tiles, 1 two units
                                      * per consumer wave, 2 also tiles without their zeros; 0 when the plan has no such stream */
 } hspmm_plan_info;

@@ -1156,3 +1156,57 @@ def test_lds_staging_hands_every_b_row_to_its_column(torch_cuda, hs, dtype):
             assert np.array_equal(decode(got, dtype), want), "shift %d" % shift
     finally:
         hs.set_kernel_mode(0)
+
+
+# ------------------------------------------------------------------ bitmap tiles in the gather kernels
+@pytest.mark.parametrize("dtype", [0, 2])
+def test_gather_kernels_read_bitmap_tiles(torch_cuda, hs, oracle, dtype):
+    """Single 16-bit windows with few stored elements per tile are kept on the device as the reference's
+    bitmap tiles (128 bits per 8 x 16 tile + the stored elements) and expanded in registers by the gather
+    kernels.  The MFMA inputs are those of the uncompressed tiles, so the results are bit-identical; stored
+    zeros, negative zeros, full tiles and tiles with one element are all in here."""
+    rng = np.random.default_rng(120 + dtype)
+    rows, cols = 530, 1500
+    A = random_csr(rng, rows, cols, 0.01, dtype, empty_row_prob=0.1, heavy_rows=(7, 300))
+    v = decode(A["values"], dtype).astype(np.float32)
+    v[::13] = 0.0                                    # stored zeros (not kept by the bitmap: +0 is "not stored")
+    v[3::31] = -0.0                                  # negative zeros are
+    A["values"] = encode(v, dtype)
+    b = convert(hs, A)
+    for N in (64, 128, 256, 512):
+        B = make_b(rng, cols, N, dtype)
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        got = {}
+        for use in ("0", "1"):
+            os.environ["HSPMM_GATHER_BITMAP"] = use
+            try:
+                plan = hs.Plan(b)
+            finally:
+                os.environ.pop("HSPMM_GATHER_BITMAP", None)
+            got[use] = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+            info = plan.info()
+            plan.close()
+            assert info["last_kernel_family"] == 2 and info["gather_bitmap"] == int(use)
+        assert_parity(got["0"], ref, mag, dtype, "tiles N=%d" % N)
+        assert np.array_equal(got["1"], got["0"]), "bitmap tiles differ at N=%d" % N
+    # dense 8 x 16 tiles (every bit set) next to empty windows, forced through the bitmap path
+    D = np.zeros((64, 96))
+    D[0:8, 0:16] = rng.integers(1, 4, (8, 16))
+    D[8:16, 5:85] = rng.integers(-3, 4, (8, 80))
+    D[40, 95] = 2
+    rr, cc = np.nonzero(D)
+    rp = np.zeros(65, np.uint32)
+    rp[1:] = np.cumsum(np.bincount(rr, minlength=64))
+    Ai = dict(rows=64, cols=96, dtype=dtype, row_ptr=rp, col_idx=cc.astype(np.uint32), values=encode(D[rr, cc].astype(np.float32), dtype))
+    Bm = rng.integers(-4, 5, (96, 128))
+    os.environ["HSPMM_GATHER_BITMAP"] = "1"
+    hs.set_kernel_mode(3)                            # (dense windows: keep the plan off the LDS-staging kernels)
+    try:
+        plan = hs.Plan(convert(hs, Ai))
+    finally:
+        hs.set_kernel_mode(0)
+        os.environ.pop("HSPMM_GATHER_BITMAP", None)
+    got = gpu_spmm(torch_cuda, hs, convert(hs, Ai), encode(Bm, dtype), 128, plan=plan)
+    assert plan.info()["gather_bitmap"] == 1 and plan.info()["last_kernel_family"] == 2
+    plan.close()
+    assert np.array_equal(decode(got, dtype), decode(encode(D @ Bm, dtype), dtype))
