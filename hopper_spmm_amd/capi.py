@@ -42,12 +42,13 @@ def build_library(force=True):
     cli = ["make", "-C", os.path.join(_HERE, "host")]
     if force:
         subprocess.check_call(cli + ["clean"], stdout=subprocess.DEVNULL)
-    subprocess.check_call(cli + ["-j3", "fp16_test", "bf16_test", "tf32_test"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(cli + ["-j4", "fp16_test", "bf16_test", "tf32_test", "fp16_transposed_test"], stdout=subprocess.DEVNULL)
     return _LIB
 
 
 def cli_path(name):
-    """Path of a built command-line driver: 'fp16_test', 'bf16_test' or 'tf32_test'."""
+    """Path of a built command-line driver: 'fp16_test', 'bf16_test', 'tf32_test', or
+    'fp16_transposed_test' (fp16_test built with -DSPARSE_A_TRANSPOSE)."""
     return os.path.join(_HERE, "host", name)
 
 
@@ -88,6 +89,9 @@ def load_library():
     u32, vp, i = C.c_uint32, C.c_void_p, C.c_int
     L.hspmm_last_error.restype = C.c_char_p
     L.hspmm_create.argtypes = [C.POINTER(vp), i, u32, u32, u32, u32, vp, vp, vp, vp]
+    L.hspmm_btcf_relayout_sizes.argtypes = [i, u32, u32, vp, vp, C.POINTER(u32)]
+    L.hspmm_btcf_relayout_fill.argtypes = [i, u32, i, u32, vp, vp, vp, vp, vp, vp]
+    L.hspmm_create_layout.argtypes = [C.POINTER(vp), i, u32, i, u32, u32, u32, u32, vp, vp, vp, vp]
     L.hspmm_run.argtypes = [vp, vp, vp, u32, vp]
     L.hspmm_run_static.argtypes = [vp, vp, vp, u32, vp]
     L.hspmm_prepare.argtypes = [vp, u32]
@@ -227,9 +231,38 @@ def csr_to_btcf(rows, cols, row_ptr, col_idx, values, dtype, transpose=False):
     rowIdx = np.empty(W, np.uint32)
     _check(L.hspmm_btcf_fill(dtype, rows, _p(row_ptr), _p(col_idx), _p(values), int(transpose),
                              _p(rowOffset), _p(tcA2B), _p(data), _p(rowIdx)))
-    return dict(rows=rows, cols=cols, nnzs=int(col_idx.size), dtype=dtype, cw=cw,
+    return dict(rows=rows, cols=cols, nnzs=int(col_idx.size), dtype=dtype, cw=cw, transposed=bool(transpose),
                 total_row_windows=(rows + ROW_WINDOW - 1) // ROW_WINDOW, eff_row_windows=W,
                 total_tiles=T, rowOffset=rowOffset, tcA2B=tcA2B, data=data, rowIdx=rowIdx)
+
+
+
+def btcf_relayout(btcf):
+    """Tiles in the layout of one of the reference's build switches (btcf["cw"] = 4 for fp32 storage:
+    -DMMA_M16N8K4, src/common.h:28-35; btcf["transposed"]: -DSPARSE_A_TRANSPOSE,
+    src/utils/convert.h:207-209) as default tiles; host only."""
+    L = load_library()
+    dtype = int(btcf["dtype"])
+    vt = _val_dtype(dtype)
+    cw_default = 8 if dtype == TF32 else 16
+    W = int(btcf["eff_row_windows"])
+    ro = np.ascontiguousarray(btcf["rowOffset"], np.uint32)
+    a2b = np.ascontiguousarray(btcf["tcA2B"], np.uint32)
+    data = np.ascontiguousarray(btcf["data"], vt)
+    cw = int(btcf.get("cw", cw_default))
+    if a2b.size != int(btcf["total_tiles"]) * cw or data.size != a2b.size * ROW_WINDOW or ro.size != W + 1:
+        raise ValueError("array sizes do not match eff_row_windows / total_tiles / cw")
+    T = C.c_uint32()
+    _check(L.hspmm_btcf_relayout_sizes(dtype, cw, W, _p(ro), _p(a2b), C.byref(T)))
+    T = T.value
+    n_ro = np.empty(W + 1, np.uint32)
+    n_a2b = np.empty(T * cw_default, np.uint32)
+    n_data = np.empty(T * ROW_WINDOW * cw_default, vt)
+    _check(L.hspmm_btcf_relayout_fill(dtype, cw, int(bool(btcf.get("transposed"))), W, _p(ro), _p(a2b), _p(data),
+                                      _p(n_ro), _p(n_a2b), _p(n_data)))
+    out = dict(btcf)
+    out.update(cw=cw_default, transposed=False, total_tiles=T, rowOffset=n_ro, tcA2B=n_a2b, data=n_data)
+    return out
 
 
 BITS_PER_TILE = 0       # HSPMM_BITS_PER_TILE: every tile owns its bitmap words
@@ -398,6 +431,14 @@ class Plan:
             _check(L.hspmm_create_bitmap(C.byref(self._h), self.dtype, self.rows, self.cols,
                                          int(btcf["eff_row_windows"]), int(btcf["total_tiles"]),
                                          _p(ro), _p(no), _p(a2b), _p(bits), _p(data), _p(ri)))
+            return
+        cw_default = 8 if self.dtype == TF32 else 16
+        if btcf.get("transposed") or int(btcf.get("cw", cw_default)) != cw_default:
+            # tiles in the order of -DSPARSE_A_TRANSPOSE and / or the 8 x 4 tiles of -DMMA_M16N8K4
+            _check(L.hspmm_create_layout(C.byref(self._h), self.dtype, int(btcf.get("cw", 0)),
+                                         int(bool(btcf.get("transposed"))), self.rows, self.cols,
+                                         int(btcf["eff_row_windows"]), int(btcf["total_tiles"]),
+                                         _p(ro), _p(a2b), _p(data), _p(ri)))
             return
         _check(L.hspmm_create(C.byref(self._h), self.dtype, self.rows, self.cols,
                               int(btcf["eff_row_windows"]), int(btcf["total_tiles"]),

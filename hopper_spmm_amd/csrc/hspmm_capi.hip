@@ -1430,6 +1430,115 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
     return HSPMM_OK;
 }
 
+namespace {
+// Widths a tile layout may have for an element type: the default one, and 4 for fp32 storage.
+int layout_widths(int dtype, uint32_t col_window, uint32_t &cw, uint32_t &cw_default, uint32_t &elem)
+{
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16)
+        return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
+    cw_default = dtype == HSPMM_TF32 ? 8u : 16u;
+    elem = dtype == HSPMM_TF32 ? 4u : 2u;
+    cw = col_window ? col_window : cw_default;
+    if (cw != cw_default && !(dtype == HSPMM_TF32 && cw == 4u))
+        return fail(HSPMM_ERR_INVALID, "col_window %u: %u, or 4 for HSPMM_TF32", col_window, cw_default);
+    return HSPMM_OK;
+}
+}  // namespace
+
+int hspmm_btcf_relayout_sizes(int dtype, uint32_t col_window, uint32_t eff_row_windows, const uint32_t *rowOffset,
+                              const uint32_t *tcA2B, uint32_t *total_tiles)
+{
+    uint32_t cw, cw_default, elem;
+    if (int rc = layout_widths(dtype, col_window, cw, cw_default, elem)) return rc;
+    if (!total_tiles) return fail(HSPMM_ERR_INVALID, "null output");
+    const uint32_t W = eff_row_windows;
+    if (W && (!rowOffset || !tcA2B)) return fail(HSPMM_ERR_INVALID, "null format array");
+    if (W && rowOffset[0] != 0) return fail(HSPMM_ERR_INVALID, "rowOffset[0] = %u, expected 0", rowOffset[0]);
+    uint64_t tiles = 0;
+    for (uint32_t w = 0; w < W; ++w) {
+        if (rowOffset[w + 1] <= rowOffset[w])
+            return fail(HSPMM_ERR_INVALID, "rowOffset not strictly increasing at window %u", w);
+        const uint32_t *ids = tcA2B + size_t(rowOffset[w]) * cw;
+        uint32_t real = 0;
+        for (size_t i = 0, n = size_t(rowOffset[w + 1] - rowOffset[w]) * cw; i < n; ++i) real += ids[i] != HSPMM_IDX_MAX;
+        if (!real) return fail(HSPMM_ERR_INVALID, "window %u has no column", w);
+        tiles += (real + cw_default - 1u) / cw_default;
+    }
+    if (tiles > 0xffffffffull) return fail(HSPMM_ERR_INVALID, "more than 2^32 - 1 tiles");
+    *total_tiles = uint32_t(tiles);
+    return HSPMM_OK;
+}
+
+int hspmm_btcf_relayout_fill(int dtype, uint32_t col_window, int transposed, uint32_t eff_row_windows,
+                             const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
+                             uint32_t *out_rowOffset, uint32_t *out_tcA2B, void *out_data)
+{
+    uint32_t cw, cw_default, elem, NT = 0;
+    if (int rc = hspmm_btcf_relayout_sizes(dtype, col_window, eff_row_windows, rowOffset, tcA2B, &NT)) return rc;
+    layout_widths(dtype, col_window, cw, cw_default, elem);
+    const uint32_t W = eff_row_windows;
+    if (!out_rowOffset || (NT && (!data || !out_tcA2B || !out_data))) return fail(HSPMM_ERR_INVALID, "null array");
+    out_rowOffset[0] = 0;
+    for (uint32_t w = 0; w < W; ++w) {
+        const uint32_t *ids = tcA2B + size_t(rowOffset[w]) * cw;
+        uint32_t real = 0;
+        for (size_t i = 0, n = size_t(rowOffset[w + 1] - rowOffset[w]) * cw; i < n; ++i) real += ids[i] != HSPMM_IDX_MAX;
+        out_rowOffset[w + 1] = out_rowOffset[w] + (real + cw_default - 1u) / cw_default;
+    }
+    std::fill(out_tcA2B, out_tcA2B + size_t(NT) * cw_default, HSPMM_IDX_MAX);
+    std::memset(out_data, 0, size_t(NT) * 8u * cw_default * elem);
+    const uint8_t *src = static_cast<const uint8_t *>(data);
+    uint8_t *dst = static_cast<uint8_t *>(out_data);
+    hspmm_host::parallel_blocks(W, 1024, [&](size_t wb, size_t we) {
+        for (size_t w = wb; w < we; ++w) {
+            size_t at = size_t(out_rowOffset[w]) * cw_default;                // next column slot of the window
+            for (uint32_t t = rowOffset[w]; t < rowOffset[w + 1]; ++t)
+                for (uint32_t k = 0; k < cw; ++k) {
+                    const uint32_t id = tcA2B[size_t(t) * cw + k];
+                    if (id == HSPMM_IDX_MAX) continue;                        // the real columns keep their order
+                    const size_t nt = at / cw_default, nk = at % cw_default;
+                    out_tcA2B[at] = id;
+                    for (uint32_t r = 0; r < 8u; ++r) {
+                        const size_t from = size_t(t) * 8u * cw + (transposed ? size_t(k) * 8u + r : size_t(r) * cw + k);
+                        std::memcpy(dst + ((nt * 8u + r) * cw_default + nk) * elem, src + from * elem, elem);
+                    }
+                    ++at;
+                }
+        }
+    });
+    return HSPMM_OK;
+}
+
+int hspmm_create_layout(hspmm_plan **out, int dtype, uint32_t col_window, int transposed, uint32_t rows, uint32_t cols,
+                        uint32_t eff_row_windows, uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *tcA2B,
+                        const void *data, const uint32_t *rowIdx)
+{
+    if (!out) return fail(HSPMM_ERR_INVALID, "null plan pointer");
+    *out = nullptr;
+    uint32_t cw, cw_default, elem;
+    if (int rc = layout_widths(dtype, col_window, cw, cw_default, elem)) return rc;
+    if (cw == cw_default && !transposed)
+        return hspmm_create(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, tcA2B, data, rowIdx);
+    const uint32_t W = eff_row_windows;
+    if (W && (!rowOffset || !tcA2B || !data || !rowIdx)) return fail(HSPMM_ERR_INVALID, "null format array");
+    for (uint32_t w = 0; w < W; ++w)
+        if (rowOffset[w + 1] > total_tiles)
+            return fail(HSPMM_ERR_INVALID, "rowOffset[%u] = %u beyond total_tiles = %u", w + 1, rowOffset[w + 1], total_tiles);
+    if (W && rowOffset[W] != total_tiles)
+        return fail(HSPMM_ERR_INVALID, "rowOffset[%u] = %u differs from total_tiles = %u", W, rowOffset[W], total_tiles);
+    // the same matrix in the layout hspmm_create reads: tiles of the default width, element (r, k) at r * width + k
+    try {
+        uint32_t NT = 0;
+        if (int rc = hspmm_btcf_relayout_sizes(dtype, col_window, W, rowOffset, tcA2B, &NT)) return rc;
+        std::vector<uint32_t> n_rowOffset(size_t(W) + 1), n_ids(size_t(NT) * cw_default);
+        std::vector<uint8_t> n_data(size_t(NT) * 8u * cw_default * elem);
+        if (int rc = hspmm_btcf_relayout_fill(dtype, col_window, transposed, W, rowOffset, tcA2B, data, n_rowOffset.data(),
+                                              n_ids.data(), n_data.data()))
+            return rc;
+        return hspmm_create(out, dtype, rows, cols, W, NT, n_rowOffset.data(), n_ids.data(), n_data.data(), rowIdx);
+    } catch (const std::bad_alloc &) { return fail(HSPMM_ERR_ALLOC, "out of host memory"); }
+}
+
 int hspmm_create_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
                         uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *nnzOffset,
                         const uint32_t *tcA2B, const uint64_t *tcBit, const void *data, const uint32_t *rowIdx)

@@ -312,9 +312,15 @@ inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX_NO_BITMAP &a, DENSE_MTX &dense_b, DEN
 {
     hspmm_cpp::check_shapes(a.rows, a.cols, dense_b, dense_c);
     hspmm_plan *plan = nullptr;
-    if (hspmm_create(&plan, HSPMM_BUILD_DTYPE, a.rows, a.cols, a.eff_row_windows, a.total_tiles, a.rowOffset.data(),
-                     a.tcA2B.data(), a.data.data(), a.rowIdx.data()) != HSPMM_OK)
-        hspmm_cpp::die("hspmm_create");
+    // (the tile order of -DSPARSE_A_TRANSPOSE, which the converters above honour, goes through the layout entry)
+#ifdef SPARSE_A_TRANSPOSE
+    constexpr int transposed = 1;
+#else
+    constexpr int transposed = 0;
+#endif
+    if (hspmm_create_layout(&plan, HSPMM_BUILD_DTYPE, COL_WINDOW, transposed, a.rows, a.cols, a.eff_row_windows, a.total_tiles,
+                            a.rowOffset.data(), a.tcA2B.data(), a.data.data(), a.rowIdx.data()) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_create_layout");
     return hspmm_cpp::run_plan(plan, dense_b, dense_c);
 }
 
@@ -325,6 +331,16 @@ inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX &a, DENSE_MTX &dense_b, DENSE_MTX &de
     hspmm_cpp::check_shapes(a.rows, a.cols, dense_b, dense_c);
     hspmm_plan *plan = nullptr;
     const uint32_t tiles = a.rowOffset.empty() ? 0u : a.rowOffset.back();
+#ifdef SPARSE_A_TRANSPOSE
+    // bit k * 8 + r, stored entries column by column (convert.h:88-90, 120-126): expanded, these are transposed tiles
+    std::vector<MAT_VAL_TYPE> dense(size_t(tiles) * ROW_WINDOW * COL_WINDOW);
+    if (hspmm_bitmap_expand(HSPMM_BUILD_DTYPE, tiles, a.nnzOffset.data(), a.tcBit.data(), a.data.data(), dense.data()) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_bitmap_expand");
+    if (hspmm_create_layout(&plan, HSPMM_BUILD_DTYPE, COL_WINDOW, 1, a.rows, a.cols, a.eff_row_windows, tiles, a.rowOffset.data(),
+                            a.tcA2B.data(), dense.data(), a.rowIdx.data()) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_create_layout");
+    return hspmm_cpp::run_plan(plan, dense_b, dense_c);
+#endif
     if (hspmm_create_bitmap(&plan, HSPMM_BUILD_DTYPE, a.rows, a.cols, a.eff_row_windows, tiles, a.rowOffset.data(),
                             a.nnzOffset.data(), a.tcA2B.data(), a.tcBit.data(), a.data.data(),
                             a.rowIdx.data()) != HSPMM_OK)
@@ -336,6 +352,10 @@ inline PERF_RESULT hspmm_cpp_spmm(GBTCF_MTX &a, DENSE_MTX &dense_b, DENSE_MTX &d
 {
     hspmm_cpp::check_shapes(a.rows, a.cols, dense_b, dense_c);
     hspmm_plan *plan = nullptr;
+#ifdef SPARSE_A_TRANSPOSE
+    std::fprintf(stderr, "hspmm: groups of transposed bitmap tiles (-DSPARSE_A_TRANSPOSE) are not accepted; use BTCF_MTX\n");
+    std::exit(1);
+#endif
     if (hspmm_create_grouped(&plan, HSPMM_BUILD_DTYPE, a.rows, a.cols, a.total_groups, a.groupOffset.data(),
                              a.nnzOffset.data(), a.tcA2B.data(), a.tcBit.data(), a.data.data(), a.rowIdx.data(),
                              a.atomic.data()) != HSPMM_OK)

@@ -285,7 +285,7 @@ void hspmm_csr_free(hspmm_csr *m);
 /* Replaces CSR2BTCFNOBITMAP (reference src/utils/convert.h:146-225) in two
  * calls so that the caller owns the arrays: first the sizes, then the fill.
  * `transpose` != 0 gives the SPARSE_A_TRANSPOSE tile order (convert.h:207-209),
- * which the device operator does not accept. */
+ * which the device operator takes through hspmm_create_layout. */
 int hspmm_btcf_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
                      uint32_t *eff_row_windows, uint32_t *total_tiles);
 int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
@@ -330,6 +330,28 @@ int hspmm_bitmap_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const u
  * nnzOffset span. */
 int hspmm_bitmap_expand(int dtype, uint32_t total_tiles, const uint32_t *nnzOffset, const uint64_t *tcBit,
                         const void *data, void *dense_tiles);
+
+/* hspmm_create for the two tile layouts behind the reference's optional build switches:
+ *   col_window 4 (HSPMM_TF32 only): 8 x 4 tiles, the format of -DMMA_M16N8K4 (reference
+ *     src/common.h:28-35: COL_WINDOW 4); 0 or the element type's default (16 / 8) otherwise;
+ *   transposed != 0: element (r, k) of a tile at k * 8 + r, as the converters write it with
+ *     -DSPARSE_A_TRANSPOSE (reference src/utils/convert.h:207-209).
+ * The plan re-lays the tiles out once on the host (the real columns of every window keep their
+ * order and are re-tiled with the default width); everything else is hspmm_create. */
+int hspmm_create_layout(hspmm_plan **plan, int dtype, uint32_t col_window, int transposed, uint32_t rows, uint32_t cols,
+                        uint32_t eff_row_windows, uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *tcA2B,
+                        const void *data, const uint32_t *rowIdx);
+/* The re-layout hspmm_create_layout does, for callers that keep the arrays (host only, no GPU):
+ * tiles of width `col_window` (0 = default), column-major inside a tile if `transposed`, to tiles of
+ * the default width in the order hspmm_create reads.  First the number of tiles, then the fill:
+ * out_rowOffset[eff_row_windows + 1], out_tcA2B[total_tiles * width], out_data[total_tiles * 8 * width];
+ * rowIdx does not change.  For tiles the reference's converter wrote (convert.h:146-225: every window's
+ * sorted columns cut into tiles), the output is what that converter writes without the switches. */
+int hspmm_btcf_relayout_sizes(int dtype, uint32_t col_window, uint32_t eff_row_windows, const uint32_t *rowOffset,
+                              const uint32_t *tcA2B, uint32_t *total_tiles);
+int hspmm_btcf_relayout_fill(int dtype, uint32_t col_window, int transposed, uint32_t eff_row_windows,
+                             const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
+                             uint32_t *out_rowOffset, uint32_t *out_tcA2B, void *out_data);
 
 /* Same as hspmm_create for a matrix held as bitmap tiles (row-major bit order,
  * HSPMM_BITS_PER_TILE).  The tiles are expanded once, here, into the plan's own

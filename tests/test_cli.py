@@ -52,7 +52,9 @@ def test_cli_end_to_end_with_verification(hs, tmp_path):
             f.write("%d %d %.6g\n" % (k // cols + 1, k % cols + 1, rng.normal()))
     for name, n, fmt in (("fp16_test", "128", "tiles"), ("fp16_test", "7", "tiles"), ("tf32_test", "64", "tiles"),
                          ("bf16_test", "128", "tiles"), ("bf16_test", "5", "tiles"), ("fp16_test", "64", "bitmap"),
-                         ("tf32_test", "32", "grouped"), ("bf16_test", "64", "grouped")):
+                         ("tf32_test", "32", "grouped"), ("bf16_test", "64", "grouped"),
+                         # tiles written column by column (-DSPARSE_A_TRANSPOSE)
+                         ("fp16_transposed_test", "128", "tiles"), ("fp16_transposed_test", "40", "bitmap")):
         r = run(hs, name, str(p), n, "--seed", "42", "--verify", "--format", fmt)
         assert r.returncode == 0, r.stdout + r.stderr
         assert "verification passed" in r.stdout

@@ -176,6 +176,45 @@ def test_converter_equals_oracle(hs, oracle, dtype):
             _same_btcf(a, o)
 
 
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_relayout_of_the_build_switch_formats_gives_the_default_tiles(hs, oracle, dtype):
+    """Tiles written with -DSPARSE_A_TRANSPOSE (convert.h:207-209) and, for fp32 storage, the
+    8 x 4 tiles of -DMMA_M16N8K4 (common.h:28-35), both from the oracle's converter, re-laid
+    out by the library: exactly the arrays the oracle's converter writes without the switches
+    (every window's sorted columns, cut into tiles of the default width)."""
+    rng = np.random.default_rng(260 + dtype)
+    shapes = [(1, 1, 1.0, 0.0), (8, 16, 0.5, 0.0), (9, 17, 0.5, 0.0), (27, 12, 0.1, 0.7), (64, 500, 0.05, 0.3),
+              (203, 77, 0.3, 0.1), (1000, 1000, 0.004, 0.5), (16, 4000, 0.6, 0.0)]
+    for rows, cols, dens, erp in shapes:
+        A = random_csr(rng, rows, cols, dens, dtype, erp)
+        csr = (rows, cols, A["row_ptr"], A["col_idx"], A["values"], DT[dtype])
+        want = oracle.csr_to_btcf(*csr)
+        for cw in ((None, 4) if dtype == 1 else (None,)):
+            for tr in (False, True):
+                src = dict(oracle.csr_to_btcf(*csr, transpose=tr, cw=cw))
+                if cw == 4:
+                    assert src["tcA2B"].size == 4 * src["total_tiles"]
+                src.update(dtype=dtype, transposed=tr)
+                _same_btcf(hs.btcf_relayout(src), want)
+    # padding columns between real ones (not what the converter writes, but a valid tile list) are dropped,
+    # a window of padding only is refused, and so is a width the element type does not have
+    src = dict(rows=8, cols=40, dtype=1, cw=4, transposed=True, eff_row_windows=1, total_tiles=3,
+               rowOffset=np.array([0, 3], np.uint32), rowIdx=np.array([0], np.uint32),
+               tcA2B=np.array([7, hs.IDX_MAX, 9, hs.IDX_MAX] + [hs.IDX_MAX] * 4 + [30, 31, 32, 33], np.uint32),
+               data=np.arange(96, dtype=np.float32))
+    out = hs.btcf_relayout(src)
+    assert out["total_tiles"] == 1 and out["tcA2B"].tolist() == [7, 9, 30, 31, 32, 33, hs.IDX_MAX, hs.IDX_MAX]
+    tile = out["data"].reshape(8, 8)
+    for k, (t, kk) in enumerate([(0, 0), (0, 2), (2, 0), (2, 1), (2, 2), (2, 3)]):
+        assert tile[:, k].tolist() == [32 * t + 8 * kk + r for r in range(8)]
+    assert not tile[:, 6:].any()
+    src["tcA2B"][:] = hs.IDX_MAX
+    with pytest.raises(hs.HspmmError):
+        hs.btcf_relayout(src)
+    with pytest.raises(hs.HspmmError):
+        hs.btcf_relayout(dict(src, dtype=0, data=np.zeros(96, np.uint16)))
+
+
 def test_converter_large_multithreaded_equals_oracle(hs, oracle):
     # big enough that the library's window loop runs on several threads
     from hopper_spmm_amd import generators as G

@@ -299,6 +299,45 @@ def test_plans_from_bitmap_and_grouped_formats(torch_cuda, hs, oracle, dtype):
     assert_parity(gpu_spmm(torch_cuda, hs, bitmap, B, 32), ref, mag, dtype, "tiny.mtx bitmap")
 
 
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_plans_from_transposed_tiles_and_from_tiles_four_columns_wide(torch_cuda, hs, oracle, dtype):
+    """The tile layouts of the reference's two optional build switches describe the same matrix:
+    tiles written column by column (-DSPARSE_A_TRANSPOSE, src/utils/convert.h:207-209), by the
+    library's converter and by the oracle's, and for fp32 storage the 8 x 4 tiles of -DMMA_M16N8K4
+    (src/common.h:28-35), which only the oracle's converter writes.  Their plans give bit for bit
+    what the plan of the default layout gives, and that agrees with the oracle."""
+    rng = np.random.default_rng(190 + dtype)
+    for rows, cols, dens, erp, heavy in [(27, 100, 0.1, 0.5, ()), (300, 3000, 0.004, 0.2, (5, 100, 101, 299)),
+                                         (1000, 700, 0.01, 0.6, (512,)), (64, 64, 1.0, 0.0, ())]:
+        A = random_csr(rng, rows, cols, dens, dtype, erp, heavy)
+        plain = convert(hs, A)
+        csr = (rows, cols, A["row_ptr"], A["col_idx"], A["values"])
+        layouts = [("transposed", hs.csr_to_btcf(*csr, dtype, transpose=True))]
+        assert layouts[0][1]["transposed"] and not np.array_equal(layouts[0][1]["data"], plain["data"])
+        for name, kw in (("oracle transposed", dict(transpose=True)), ("8x4", dict(cw=4)),
+                         ("8x4 transposed", dict(cw=4, transpose=True))):
+            if "cw" in kw and dtype != 1:
+                continue
+            o = dict(oracle.csr_to_btcf(*csr, DT[dtype], **kw))
+            o.update(dtype=dtype, transposed=bool(kw.get("transpose")))
+            if "cw" in kw:
+                assert o["cw"] == 4 and o["total_tiles"] >= plain["total_tiles"]
+            layouts.append((name, o))
+        for N in (8, 64, 136):
+            B = make_b(rng, cols, N, dtype)
+            want = gpu_spmm(torch_cuda, hs, plain, B, N)
+            ref, mag = oracle_spmm(oracle, A, B, N)
+            assert_parity(want, ref, mag, dtype, "plain %dx%d N=%d" % (rows, cols, N))
+            for name, fmt in layouts:
+                got = gpu_spmm(torch_cuda, hs, fmt, B, N)
+                assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "%s %dx%d N=%d" % (name, rows, cols, N)
+    # what the entry point refuses
+    bad = dict(plain, cw=4)
+    if dtype != 1:
+        with pytest.raises(hs.HspmmError):
+            hs.Plan(bad)
+
+
 PANEL_SHAPES = [
     # rows, cols, density, empty-row probability, heavy rows
     (8, 16, 1.0, 0.0, ()),                      # one window, one panel
