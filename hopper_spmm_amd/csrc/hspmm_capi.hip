@@ -1758,7 +1758,9 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         // (a 16-bit matrix near the break-even is served as fast or faster by the gather kernels while
         // one wave of theirs covers all of N)
         const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
-        if (pays && N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
+        // (the producers address a panel of B - up to 256 rows - with 32-bit offsets)
+        const bool offsets_fit = uint64_t(N) * p->elem < (uint64_t(1) << 24);
+        if (pays && offsets_fit && N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
     }
     // Feature blocks with XCDs of their own (see spmm_mfma_kernel): pays when B is far larger than an
     // XCD's 4 MB L2, so that what an L2 can keep of it decides the hit rate of the gathers (power-law

@@ -26,6 +26,7 @@
 //   * With more than one chunk of panels per unit, every chunk leaves fp32 partial
 //     sums in scratch slots that spmm_fixup_kernel adds in chunk order.
 #pragma once
+#include <type_traits>
 #include "spmm_mfma_kernel.hpp"
 
 namespace hspmm {
@@ -113,14 +114,28 @@ struct PanelOps {
         return *reinterpret_cast<const AVec *>(L.a_src + size_t(step) * (64u * TT::G));
     }
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I) >> 28; }
-    // img: LDS byte offset of the lane's 16 bytes of row 0 of the current panel image
-    __device__ static __forceinline__ void step(const typename TT::Lane &L, const char *smem, uint32_t img, const Idx I,
-                                                const AVec &A, f32x4 (&acc)[kLive])
+    // A step in two halves (see the consumer loop of spmm_panel_kernel): read_half<H> requests the
+    // second operands of half H from LDS, mma_half<H> multiplies them.  Here the first half is the
+    // whole step.  img: LDS byte offset of the lane's 16 bytes of row 0 of the current panel image.
+    template <int H> struct Half { typename TT::BVec b0, b1; };
+    template <int H>
+    __device__ static __forceinline__ Half<H> read_half(const typename TT::Lane &, const char *smem, uint32_t img, const Idx I)
     {
-        typename TT::BVec b0, b1, b2 = {}, b3 = {};
-        b0 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 0, 7) << 8));
-        b1 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 7, 7) << 8));
-        TT::mma(L, b0, b1, b2, b3, A, acc);
+        Half<H> B = {};
+        if constexpr (H == 0) {
+            B.b0 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 0, 7) << 8));
+            B.b1 = *reinterpret_cast<const u32x4 *>(smem + img + (__builtin_amdgcn_ubfe(I, 7, 7) << 8));
+        }
+        return B;
+    }
+    template <int H>
+    __device__ static __forceinline__ void mma_half(const typename TT::Lane &L, const AVec &A, const Half<H> &B,
+                                                    f32x4 (&acc)[kLive])
+    {
+        if constexpr (H == 0) {
+            typename TT::BVec b2 = {}, b3 = {};
+            TT::mma(L, B.b0, B.b1, b2, b3, A, acc);
+        }
     }
     __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return L.j * 16u; }
 };
@@ -215,7 +230,7 @@ struct PanelOps<Fp16Tr<G_, BF>> {
     }
     static constexpr bool kFour = G_ == 4;                        // units of up to four windows
     static constexpr int kConsumers = kFour ? 8 : 12;             // twice the accumulators: fewer, larger waves
-    static constexpr uint32_t kRing = kFour ? 4 : 6;
+    static constexpr uint32_t kRing = kFour ? 3 : 4;              // (registers: a step's second operands are held twice)
     static constexpr int kLive = TT::G * TT::V;
     __device__ static __forceinline__ void fold(f32x4 (&)[kLive]) {}
     typedef uint32_t Idx;
@@ -247,22 +262,34 @@ struct PanelOps<Fp16Tr<G_, BF>> {
         return a;
     }
     typedef tr16x4 __attribute__((address_space(3))) *lds_tr_ptr;
-    __device__ static __forceinline__ void step(const typename TT::Lane &, const char *smem, uint32_t img, const Idx I,
-                                                const AVec &A, f32x4 (&acc)[kLive])
+    // A step in two halves of four accumulators (64 features) each: read_half<H> requests the second
+    // operands of half H from LDS, mma_half<H> multiplies them.
+    template <int H> struct Half { u32x4 b[4]; };
+    template <int H>
+    __device__ static __forceinline__ Half<H> read_half(const typename TT::Lane &, const char *smem, uint32_t img, const Idx I)
     {
         typedef __attribute__((address_space(3))) char *lds_char_ptr;
         const lds_char_ptr base = (lds_char_ptr)smem + img;
         const lds_char_ptr a0 = base + (__builtin_amdgcn_ubfe(I, 4, 12) << 5);
         const lds_char_ptr a1 = base + (__builtin_amdgcn_ubfe(I, 16, 12) << 5);
+        Half<H> B;
 #pragma unroll
-        for (int p = 0; p < 8; ++p) {
-            const tr16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a0 + 32 * p));
-            const tr16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a1 + 32 * p));
-            u32x4 b;
+        for (int p = 0; p < 4; ++p) {
+            const tr16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a0 + 32 * (4 * H + p)));
+            const tr16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a1 + 32 * (4 * H + p)));
             const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-            b[0] = l2[0]; b[1] = l2[1]; b[2] = h2[0]; b[3] = h2[1];
-            acc[p] = HalfOps<BF>::mfma(A.r[0], b, acc[p]);
-            if constexpr (kFour) acc[8 + p] = HalfOps<BF>::mfma(A.r[1], b, acc[8 + p]);
+            B.b[p][0] = l2[0]; B.b[p][1] = l2[1]; B.b[p][2] = h2[0]; B.b[p][3] = h2[1];
+        }
+        return B;
+    }
+    template <int H>
+    __device__ static __forceinline__ void mma_half(const typename TT::Lane &, const AVec &A, const Half<H> &B,
+                                                    f32x4 (&acc)[kLive])
+    {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            acc[4 * H + p] = HalfOps<BF>::mfma(A.r[0], B.b[p], acc[4 * H + p]);
+            if constexpr (kFour) acc[8 + 4 * H + p] = HalfOps<BF>::mfma(A.r[1], B.b[p], acc[8 + 4 * H + p]);
         }
     }
     __device__ static __forceinline__ uint32_t lane_bytes(const typename TT::Lane &L) { return (L.j & 3u) * 8u; }
@@ -407,29 +434,42 @@ struct PanelOps<Fp32Split<G_>> {
         b[0] = l2[0]; b[1] = l2[1]; b[2] = h2[0]; b[3] = h2[1];
         return b;
     }
-    __device__ static __forceinline__ void step(const typename TT::Lane &, const char *smem, uint32_t img, const Idx I,
-                                                const AVec &A, f32x4 (&acc)[kLive])
+    // A step in two halves of two accumulators (32 features) each, as for the 16-bit types.
+    template <int H> struct Half { u32x4 hi[2], lo[2]; };
+    template <int H>
+    __device__ static __forceinline__ Half<H> read_half(const typename TT::Lane &, const char *smem, uint32_t img, const Idx I)
     {
         typedef __attribute__((address_space(3))) char *lds_char_ptr;
         const lds_char_ptr base = (lds_char_ptr)smem + img;
         const lds_char_ptr a0 = base + (__builtin_amdgcn_ubfe(I, 4, 12) << 5);
         const lds_char_ptr a1 = base + (__builtin_amdgcn_ubfe(I, 16, 12) << 5);
-        constexpr int kHalves = kFour ? 2 : 1;
-        u32x4 a_hi[kHalves], a_lo[kHalves];
+        Half<H> B;
 #pragma unroll
-        for (int h = 0; h < kHalves; ++h)
+        for (int p = 0; p < 2; ++p) {
+            B.hi[p] = operand(a0, a1, 32 * (2 * H + p));
+            B.lo[p] = operand(a0, a1, 128 + 32 * (2 * H + p));
+        }
+        return B;
+    }
+    template <int H>
+    __device__ static __forceinline__ void mma_half(const typename TT::Lane &, const AVec &A, const Half<H> &B,
+                                                    f32x4 (&acc)[kLive])
+    {
+        constexpr int kRowSets = kFour ? 2 : 1;
+        u32x4 a_hi[kRowSets], a_lo[kRowSets];
+#pragma unroll
+        for (int h = 0; h < kRowSets; ++h)
 #pragma unroll
             for (int i = 0; i < 4; ++i) { a_hi[h][i] = A.r[h][i]; a_lo[h][i] = A.r[h][4 + i]; }
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const u32x4 b_hi = operand(a0, a1, 32 * p);
-            const u32x4 b_lo = operand(a0, a1, 128 + 32 * p);
+        for (int p = 0; p < 2; ++p) {
 #pragma unroll
-            for (int h = 0; h < kHalves; ++h) {
+            for (int h = 0; h < kRowSets; ++h) {
                 // small terms first; a_lo * b_lo (below 2^-14 |a||b|, 2^-16 on average) is left out
-                f32x4 c = HalfOps<true>::mfma(a_lo[h], b_hi, acc[4 * h + p]);
-                c = HalfOps<true>::mfma(a_hi[h], b_lo, c);
-                acc[4 * h + p] = HalfOps<true>::mfma(a_hi[h], b_hi, c);
+                const int q = 4 * h + 2 * H + p;
+                f32x4 c = HalfOps<true>::mfma(a_lo[h], B.hi[p], acc[q]);
+                c = HalfOps<true>::mfma(a_hi[h], B.lo[p], c);
+                acc[q] = HalfOps<true>::mfma(a_hi[h], B.hi[p], c);
             }
         }
     }
@@ -461,27 +501,38 @@ struct PanelOps<Fp32Quad> {
         return *reinterpret_cast<const u32x8 *>(L.a_src + size_t(step) * 64u);
     }
     __device__ static __forceinline__ uint32_t jump(const Idx I) { return __builtin_amdgcn_readfirstlane(I[0]) & 15u; }
-    __device__ static __forceinline__ void step(const Fp32Quad::Lane &, const char *smem, uint32_t img, const Idx I,
-                                                const AVec &A, f32x4 (&acc)[4])
+    // The first "half" is the whole step (see the consumer loop of spmm_panel_kernel).
+    template <int H> struct Half { float lo[8], hi[8]; };
+    template <int H>
+    __device__ static __forceinline__ Half<H> read_half(const Fp32Quad::Lane &, const char *smem, uint32_t img, const Idx I)
     {
-        // word w holds the offsets of the rows whose tile values are A[2w] and A[2w + 1]
-        float lo[8], hi[8];
+        Half<H> B = {};
+        if constexpr (H == 0) {
+            // word w holds the offsets of the rows whose tile values are A[2w] and A[2w + 1]
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const uint32_t word = I[w];
-            const uint32_t sw = __builtin_amdgcn_readfirstlane(word);
-            const uint32_t off0 = sw & 0xFF00u, off1 = sw >> 16;
-            const float *r0 = reinterpret_cast<const float *>(smem + (img + off0));
-            const float *r1 = reinterpret_cast<const float *>(smem + (img + off1));
-            lo[2 * w] = r0[0]; hi[2 * w] = r0[32];
-            lo[2 * w + 1] = r1[0]; hi[2 * w + 1] = r1[32];
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t word = I[w];
+                const uint32_t sw = __builtin_amdgcn_readfirstlane(word);
+                const uint32_t off0 = sw & 0xFF00u, off1 = sw >> 16;
+                const float *r0 = reinterpret_cast<const float *>(smem + (img + off0));
+                const float *r1 = reinterpret_cast<const float *>(smem + (img + off1));
+                B.lo[2 * w] = r0[0]; B.hi[2 * w] = r0[32];
+                B.lo[2 * w + 1] = r1[0]; B.hi[2 * w + 1] = r1[32];
+            }
         }
+        return B;
+    }
+    template <int H>
+    __device__ static __forceinline__ void mma_half(const Fp32Quad::Lane &, const AVec &A, const Half<H> &B, f32x4 (&acc)[4])
+    {
+        if constexpr (H == 0) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t aw = A[i];
-            const float a = __builtin_bit_cast(float, aw);
-            acc[2 * (i & 1)] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, lo[i], acc[2 * (i & 1)], 0, 0, 0);
-            acc[2 * (i & 1) + 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, hi[i], acc[2 * (i & 1) + 1], 0, 0, 0);
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t aw = A[i];
+                const float a = __builtin_bit_cast(float, aw);
+                acc[2 * (i & 1)] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, B.lo[i], acc[2 * (i & 1)], 0, 0, 0);
+                acc[2 * (i & 1) + 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, B.hi[i], acc[2 * (i & 1) + 1], 0, 0, 0);
+            }
         }
     }
     __device__ static __forceinline__ uint32_t lane_bytes(const Fp32Quad::Lane &L) { return L.j * 4u; }
@@ -502,9 +553,10 @@ __device__ __forceinline__ PackedHeader load_packed_header(const uint64_t *masks
 // One barrier of the workgroup with the LDS writes in front of it visible behind it.
 __device__ __forceinline__ void panel_barrier()
 {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    // (fences for LDS alone: they must not wait for the global loads a wave has in flight)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 // NC consumer waves (one unit each) and NPW producer waves that do nothing but copy
@@ -550,26 +602,53 @@ void spmm_panel_kernel(const PanelArgs pa)
         // the barrier of panel q - 1.
         const uint32_t pt = threadIdx.x - uint32_t(NC) * 64u;       // 0 .. NPW*64-1
         // piece c = pt + i * NPW*64 is bytes [16c, 16c + 16) of the image: row c / 16, 16-byte column c % 16
-        const char *b_col = reinterpret_cast<const char *>(pa.B) + size_t(fb) * kPanelRowBytes + (pt & 15u) * 16u;
-        const uint32_t piece_row0 = pt >> 4;
-        // The loads of panel q + 1 are in flight (in registers) while the consumers multiply
-        // panel q: a panel has a whole barrier period to arrive.  (Three panels in flight, with
-        // four producer waves, measured no faster.)
+        const char *b_block = reinterpret_cast<const char *>(pa.B) + size_t(fb) * kPanelRowBytes;
+        const uint32_t piece_row0 = pt >> 4, col_bytes = (pt & 15u) * 16u;
+        // Addresses: the panel's first row (the same in all lanes) plus 32-bit offsets inside the panel
+        // (the host checks that a panel of B spans less than 4 GB).  Rows past the matrix are never
+        // referenced: their loads are bent to the matrix's last row.
+        const uint32_t row_bytes32 = uint32_t(row_bytes);
+        const uint32_t row_off0 = piece_row0 * row_bytes32, row_stride = uint32_t(NPW * 4) * row_bytes32;
+        auto panel_base = [&](uint32_t q) __attribute__((always_inline)) -> const char * {
+            return b_block + size_t(q) * kPanelRows * row_bytes;
+        };
+        auto last_row_off = [&](uint32_t q) __attribute__((always_inline)) -> uint32_t {
+            return (umin32(pa.cols - q * kPanelRows, kPanelRows) - 1u) * row_bytes32;
+        };
+        auto load_piece = [&](const char *panel, uint32_t last_off, int i) __attribute__((always_inline)) -> u32x4 {
+            const uint32_t off = umin32(row_off0 + uint32_t(i) * row_stride, last_off) + col_bytes;
+            return *reinterpret_cast<const u32x4 *>(panel + off);
+        };
+        // The loads of panel q + 1 are in flight (in registers) while the consumers multiply panel q.
+        // A piece's register is reloaded as soon as the piece is written, so that the copy to LDS and
+        // the requests for the next panel overlap: one after the other they are most of a barrier
+        // period, and the consumers wait for them.  (Three panels in flight, with four producer waves,
+        // measured no faster.)
         u32x4 X[kPieces];
-        auto issue = [&](uint32_t q) __attribute__((always_inline)) {
+        {
+            const char *panel = panel_base(p_begin);
+            const uint32_t last_off = last_row_off(p_begin);
 #pragma unroll
             for (int i = 0; i < kPieces; ++i) {
-                uint32_t row = q * kPanelRows + piece_row0 + uint32_t(i) * (NPW * 4);
-                row = umin32(row, pa.cols - 1u);                   // rows past the matrix are never referenced
-                X[i] = *reinterpret_cast<const u32x4 *>(b_col + size_t(row) * row_bytes);
+                X[i] = load_piece(panel, last_off, i);
+                __builtin_amdgcn_sched_barrier(0);                  // in the order they are used
             }
-        };
-        issue(p_begin);
+        }
         for (uint32_t q = p_begin; q < p_end; ++q) {
             char *img = smem + (q & 1u) * kImage + piece_row0 * kPitch;
+            if (q + 1u < p_end) {
+                const char *panel = panel_base(q + 1u);
+                const uint32_t last_off = last_row_off(q + 1u);
 #pragma unroll
-            for (int i = 0; i < kPieces; ++i) Ops::write_piece(img + uint32_t(i) * (NPW * 4) * kPitch, pt & 15u, X[i]);
-            if (q + 1u < p_end) issue(q + 1u);
+                for (int i = 0; i < kPieces; ++i) {
+                    Ops::write_piece(img + uint32_t(i) * (NPW * 4) * kPitch, pt & 15u, X[i]);
+                    X[i] = load_piece(panel, last_off, i);
+                    __builtin_amdgcn_sched_barrier(0);              // in the order the loads return
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < kPieces; ++i) Ops::write_piece(img + uint32_t(i) * (NPW * 4) * kPitch, pt & 15u, X[i]);
+            }
             panel_barrier();
         }
         return;
@@ -640,15 +719,16 @@ void spmm_panel_kernel(const PanelArgs pa)
     };
     // register ring of kRing steps (separate variables: an array would go to scratch)
 #define HSPMM_RING(X) X(0) X(1) X(2) X(3) X(4) X(5)
+#define HSPMM_RING2(X) X(0, 1) X(1, 2) X(2, 3) X(3, 4) X(4, 5) X(5, 6)
 #define HSPMM_HEADER(k) ((k##u & 1u) ? H1 : H0)
 #define HSPMM_OTHER_HEADER(k) ((k##u & 1u) ? H0 : H1)
-    // (two sets of accumulators leave registers for four steps in flight; packed tiles: see Ops::kPackedRing)
+    // (two sets of accumulators leave registers for fewer steps in flight; packed tiles: see Ops::kPackedRing)
 #ifdef HSPMM_PANEL_RING
     constexpr uint32_t kRing = HSPMM_PANEL_RING;                    // (measurement builds)
 #else
     constexpr uint32_t kRing = [] {
         if constexpr (PACKED) return Ops::kPackedRing;
-        else return (TALL && Ops::kRing > 4u) ? 4u : Ops::kRing;
+        else return (TALL && TT::kElem == 2) ? 2u : Ops::kRing;
     }();
 #endif
     static_assert(kRing >= 1 && kRing <= 6, "ring slots are named variables");
@@ -660,52 +740,82 @@ void spmm_panel_kernel(const PanelArgs pa)
                                I##k = ring_idx(t0 + k##u); A##k = ring_a(HSPMM_HEADER(k), t0 + k##u); }
     HSPMM_RING(HSPMM_RING_DECL)
 #undef HSPMM_RING_DECL
+    const Idx I6 = {};                                              // (a name for "the slot behind the last"; never read)
     panel_barrier();                                                // panel p_begin is in its buffer
     --owed;
     // the lane's bytes of a row, in the buffer of the current panel
     uint32_t img = (p_begin & 1u) * kImage + Ops::lane_bytes(L);
     const uint32_t img_both = kImage + 2u * Ops::lane_bytes(L);     // img of one buffer + img of the other
 
-    // One step: first the barriers that lie between it and the step in front of it.
-    auto step = [&](const Idx &I, const AVec &A, const uint32_t jump) __attribute__((always_inline)) {
+    // The barriers between a step and the step in front of it.
+    auto enter = [&](const uint32_t jump) __attribute__((always_inline)) {
         for (uint32_t n = jump; n && owed; --n) {                   // never more barriers than the producers pass
             panel_barrier();
             img = img_both - img;
             --owed;
         }
+    };
+    // A step runs in two halves, and the LDS reads of a half are requested before the MFMAs of the half
+    // in front of it are issued: a wave that reads, waits and then multiplies leaves both the LDS and the
+    // matrix cores idle for most of a step (the waves of a workgroup leave every barrier in phase).
+    // Bq: the second operands of the first half of the step about to run, requested by the step in front
+    // of it between its two halves.  Where the next step lies in another panel, the barriers come first:
+    // the wave then arrives with its second half still to multiply, which is safe - the operands of that
+    // half are in registers (the barrier waits for the wave's LDS reads).
+    typename Ops::template Half<0> Bq = {};
+    auto mma = [&](auto half, const Idx &I, const AVec &A, const auto &B) __attribute__((always_inline)) {
+        constexpr int H = decltype(half)::value;
         if constexpr (TALL) {
-            if (Ops::second_unit(I)) Ops::step(L, smem, img, I, A, live2);
-            else Ops::step(L, smem, img, I, A, live);
+            if (Ops::second_unit(I)) Ops::template mma_half<H>(L, A, B, live2);
+            else Ops::template mma_half<H>(L, A, B, live);
         } else {
-            Ops::step(L, smem, img, I, A, live);
+            Ops::template mma_half<H>(L, A, B, live);
         }
     };
-    auto jump_of = [&](const Idx &I, const uint32_t t) __attribute__((always_inline)) -> uint32_t {
-        const uint32_t stored = Ops::jump(I);
-        return t == t0 ? first_jump : stored;
+    // In: the ids of the next step, jump_next: the barriers in front of it (0 when there is no next step:
+    // In then repeats the last step's ids, and what is read for it is not used)
+    auto step = [&](const Idx &I, const AVec &A, const Idx &In, const uint32_t jump_next) __attribute__((always_inline)) {
+        // (the scheduling barriers keep the compiler from moving the reads behind the MFMAs again)
+        const typename Ops::template Half<1> B1 = Ops::template read_half<1>(L, smem, img, I);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(std::integral_constant<int, 0>{}, I, A, Bq);
+        __builtin_amdgcn_sched_barrier(0);
+        enter(jump_next);
+        Bq = Ops::template read_half<0>(L, smem, img, In);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(std::integral_constant<int, 1>{}, I, A, B1);
+        __builtin_amdgcn_sched_barrier(0);
     };
 
     uint32_t t = t0;
+    if (t0 < t1) {
+        enter(first_jump);
+        Bq = Ops::template read_half<0>(L, smem, img, I0);
+    }
     // Steady state: every slot runs its step and reloads its registers with the step kRing
     // further on, without conditions on the loads.  (After the prologue the header of step
     // t0 + kRing is in H0 / H1 by the parity of kRing, i.e. in slot 0's header.)
+    // The step behind slot k's is in slot k + 1, behind the last slot's in slot 0 (just reloaded).
+#define HSPMM_NEXT_IDX(k, kn) ((k##u + 1u == kRing) ? I0 : I##kn)
     for (; t + 2u * kRing <= t1; t += kRing) {
-#define HSPMM_PANEL_STEADY(k) if constexpr (kRing > k) { \
-        step(I##k, A##k, jump_of(I##k, t + k##u)); \
+#define HSPMM_PANEL_STEADY(k, kn) if constexpr (kRing > k) { \
+        step(I##k, A##k, HSPMM_NEXT_IDX(k, kn), Ops::jump(HSPMM_NEXT_IDX(k, kn))); \
         request(HSPMM_OTHER_HEADER(k), t + k##u + kRing + 1u); \
         I##k = ring_idx(t + k##u + kRing); A##k = ring_a(HSPMM_HEADER(k), t + k##u + kRing); }
-        HSPMM_RING(HSPMM_PANEL_STEADY)
+        HSPMM_RING2(HSPMM_PANEL_STEADY)
 #undef HSPMM_PANEL_STEADY
     }
     for (; t < t1; t += kRing) {
-#define HSPMM_PANEL_DRAIN(k) if constexpr (kRing > k) { \
-        if (t + k##u < t1) step(I##k, A##k, jump_of(I##k, t + k##u)); \
+#define HSPMM_PANEL_DRAIN(k, kn) if constexpr (kRing > k) { \
+        if (t + k##u < t1) step(I##k, A##k, HSPMM_NEXT_IDX(k, kn), t + k##u + 1u < t1 ? Ops::jump(HSPMM_NEXT_IDX(k, kn)) : 0u); \
         request(HSPMM_OTHER_HEADER(k), t + k##u + kRing + 1u); \
         if (t + k##u + kRing < t1) { I##k = ring_idx(t + k##u + kRing); A##k = ring_a(HSPMM_HEADER(k), t + k##u + kRing); } }
-        HSPMM_RING(HSPMM_PANEL_DRAIN)
+        HSPMM_RING2(HSPMM_PANEL_DRAIN)
 #undef HSPMM_PANEL_DRAIN
     }
+#undef HSPMM_NEXT_IDX
 #undef HSPMM_RING
+#undef HSPMM_RING2
 #undef HSPMM_HEADER
 #undef HSPMM_OTHER_HEADER
     // the panels behind the unit's last step
