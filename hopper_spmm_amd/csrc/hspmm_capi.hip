@@ -58,7 +58,7 @@ struct Config {
     int sm_num = 0;
     int kernel_mode = 0;
     int fused_fixup = -1;               // 1: the last wave of a cut unit adds its partial sums; 0: second kernel;
-                                        // -1: the former where few units are cut (gather kernels, several feature blocks)
+                                        // -1: the former in the LDS-panel kernels, and in the gather kernels where few units are cut
     int pairing = 0;                    // 0 automatic, 1 never, 2 whenever two windows share a column list
     // Tuning overrides from the environment (HSPMM_*), read once by hspmm_create: a plan's behaviour does
     // not change with the environment afterwards and the launch path reads no variable.
@@ -1703,10 +1703,10 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
             std::lock_guard<std::mutex> lk(p->mu);
             int rc = scratch_for(p, need, mode, &pa.scratch);
             if (rc) return rc;
-            // (experiment, as in the gather kernels: the wave that brings a unit's last chunk adds the chunk sums
-            // itself; the device-scope accesses cost more than the second launch: 61.7 + 8.8 -> 76.8 us on the
-            // block-clustered configuration at N = 512)
-            if (p->cfg.fused_fixup > 0 && mode != RunMode::kStatic &&
+            // As in the gather kernels, the wave that brings a unit's last chunk adds the chunk sums itself
+            // (16-byte device-scope accesses; block-clustered configuration at N = 512: 56.0 + 8.1 us in two
+            // launches, 60.3 us in one).  It addresses a unit's chunk sums with 32-bit offsets.
+            if (p->cfg.fused_fixup != 0 && mode != RunMode::kStatic && uint64_t(pa.n_chunks) * pa.n_feat_blocks * nacc * 1024u < (1ull << 31) &&
                 (rc = ensure_arrive(p, size_t(pl.n_units) * pa.n_feat_blocks, &pa.arrive)))
                 return rc;
         }

@@ -109,21 +109,23 @@ template <> struct HalfOps<true> {
     }
 };
 
-// Device-scope ("agent") relaxed accesses, word by word: visible to every XCD.
-__device__ __forceinline__ void store_device_scope(f32x4 *p, const f32x4 v)
+// Device-scope ("agent") accesses of 16 bytes, visible to every XCD: buffer instructions with the sc1
+// policy (stores are written through to memory, loads go past the L2 of the XCD).  base is the same in
+// every lane, off the lane's byte offset from it (below 2 GB).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t device_scope_buffer(const void *base)
 {
-    float *q = reinterpret_cast<float *>(p);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { const float f = v[i]; __hip_atomic_store(q + i, f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7FFFFFFF, 0x00020000);
 }
-__device__ __forceinline__ f32x4 load_device_scope(const f32x4 *p)
+__device__ __forceinline__ void store_device_scope(const __amdgpu_buffer_rsrc_t r, const uint32_t off, const f32x4 v)
 {
-    const float *q = reinterpret_cast<const float *>(p);
-    f32x4 v;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = __hip_atomic_load(q + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return v;
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, off, 0, 16);
 }
+__device__ __forceinline__ f32x4 load_device_scope(const __amdgpu_buffer_rsrc_t r, const uint32_t off)
+{
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 16));
+}
+// The stores in front of it are acknowledged (vmcnt(0)); the compiler moves no memory access across it.
+__device__ __forceinline__ void wait_stores_acknowledged() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Uniform (per-wave) reads of the small index arrays go through the constant
 // address space so that they become scalar loads, which do not share the
@@ -694,9 +696,9 @@ void spmm_mfma_kernel(const KernelArgs ka)
                 const bool head = ww.seg_start == t0;
                 const uint32_t slot = head ? head_slot : tail_slot;
                 if (slot != kIdxMax && !combine) {
-                    f32x4 *dst = reinterpret_cast<f32x4 *>(ka.scratch) +
-                                 (size_t(slot) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
+                    f32x4 *slot_sums = reinterpret_cast<f32x4 *>(ka.scratch) + (size_t(slot) * ka.n_feat_blocks + fb) * (NACC * 64u);
                     if (!ka.arrive) {
+                        f32x4 *dst = slot_sums + lane;
 #pragma unroll
                         for (int p = 0; p < NACC; ++p) dst[p * 64] = acc[p];
                     } else {
@@ -706,9 +708,10 @@ void spmm_mfma_kernel(const KernelArgs ka)
                         // XCDs: they are written and read with device-scope accesses (which go
                         // past the L2 of the XCD), the writes are waited for before the arrival
                         // is counted, and no whole-cache write-back or invalidate is needed.
+                        const __amdgpu_buffer_rsrc_t out = device_scope_buffer(slot_sums);
 #pragma unroll
-                        for (int p = 0; p < NACC; ++p) store_device_scope(dst + p * 64, acc[p]);
-                        __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): the stores are acknowledged
+                        for (int p = 0; p < NACC; ++p) store_device_scope(out, lane * 16u + uint32_t(p) * 1024u, acc[p]);
+                        wait_stores_acknowledged();
                         const uint32_t entry = head ? head_split : tail_split;
                         const uint32_t *fx = ka.split + size_t(entry) * kFixWords;
                         uint32_t *ctr = ka.arrive + size_t(entry) * ka.n_feat_blocks + fb;
@@ -722,10 +725,10 @@ void spmm_mfma_kernel(const KernelArgs ka)
                             for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
                             for (uint32_t i = 0; i < sc; ++i) {
                                 const uint32_t sl = ka.fix_slots[sb + i];
-                                const f32x4 *src = reinterpret_cast<const f32x4 *>(ka.scratch) +
-                                                   (size_t(sl) * ka.n_feat_blocks + fb) * (NACC * 64u) + lane;
+                                const __amdgpu_buffer_rsrc_t in = device_scope_buffer(
+                                    reinterpret_cast<const f32x4 *>(ka.scratch) + (size_t(sl) * ka.n_feat_blocks + fb) * (NACC * 64u));
 #pragma unroll
-                                for (int p = 0; p < NACC; ++p) acc[p] += load_device_scope(src + p * 64);
+                                for (int p = 0; p < NACC; ++p) acc[p] += load_device_scope(in, lane * 16u + uint32_t(p) * 1024u);
                             }
                             TT::template store_window<0>(L, acc, c_lane, row_bytes, row0, rows, active);
                             if constexpr (G > 1) {

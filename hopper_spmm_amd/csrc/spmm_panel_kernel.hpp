@@ -579,19 +579,24 @@ void spmm_panel_kernel(const PanelArgs pa)
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // The hardware hands consecutive workgroups to the eight XCDs in turn, and every XCD has an L2 of
-    // its own.  The workgroups of one row block and chunk - one per feature block - read the same
-    // tiles and ids: they get numbers that are equal mod 8 and adjacent in the launch order, so that
-    // one of them fetches the tile stream into its XCD's L2 and the others hit it.
+    // its own, filled over a path that delivers about 0.7 TB/s per XCD: what the L2s miss sets the pace
+    // of this kernel, so every line should be fetched by as few XCDs as possible.
+    //   * The workgroups of one row block and chunk - one per feature block - read the same tiles and
+    //     ids: they run on one XCD, adjacent in its launch order, so that one of them fetches the
+    //     tile stream and the others hit it.
+    //   * A chunk of panels is a range of rows of B: with the chunk as the slowest index an XCD works on
+    //     one chunk (or two), and only the XCDs of a chunk fetch its rows of B (every XCD reading all of
+    //     B costs 8 x B; the block-clustered matrix at N = 512: 118 of 197 MB per launch).
     //   position in launch order: XCD x = blockIdx % 8 runs blocks x, x + 8, ...; the work items
-    //   (row block, chunk, feature block), feature block fastest, are dealt out XCD by XCD.
+    //   (chunk, row block, feature block), feature block fastest, are dealt out XCD by XCD.
     constexpr uint32_t kXcds = 8;
     const uint32_t n_blocks = gridDim.x, xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
     const uint32_t item = xcd * (n_blocks / kXcds) + umin32(xcd, n_blocks % kXcds) + slot;
-    const uint32_t per_rb = pa.n_feat_blocks * pa.n_chunks;
-    const uint32_t rb = item / per_rb;
-    const uint32_t rest = item - rb * per_rb;
-    const uint32_t chunk = rest / pa.n_feat_blocks;
-    const uint32_t fb = rest - chunk * pa.n_feat_blocks;
+    const uint32_t per_chunk = n_blocks / pa.n_chunks;              // row blocks x feature blocks
+    const uint32_t chunk = item / per_chunk;
+    const uint32_t rest = item - chunk * per_chunk;
+    const uint32_t rb = rest / pa.n_feat_blocks;
+    const uint32_t fb = rest - rb * pa.n_feat_blocks;
     const uint32_t p_begin = chunk * pa.panels_per_chunk;
     const uint32_t p_end = umin32(p_begin + pa.panels_per_chunk, pa.n_panels);
     const size_t row_bytes = size_t(pa.N) * TT::kElem;
@@ -843,13 +848,12 @@ void spmm_panel_kernel(const PanelArgs pa)
             // result does not depend on who is last), and stores the unit.  The sums cross the L2s of
             // different XCDs: they are written and read with device-scope accesses, and the writes are
             // waited for before the arrival is counted.
-            f32x4 *slot0 = reinterpret_cast<f32x4 *>(pa.scratch) +
-                           (size_t(unit) * pa.n_chunks * pa.n_feat_blocks + fb) * (NACC * 64u) + lane;
-            const size_t chunk_stride = size_t(pa.n_feat_blocks) * (NACC * 64u);
-            f32x4 *dst = slot0 + chunk * chunk_stride;
+            const __amdgpu_buffer_rsrc_t sums = device_scope_buffer(
+                reinterpret_cast<f32x4 *>(pa.scratch) + (size_t(unit) * pa.n_chunks * pa.n_feat_blocks + fb) * (NACC * 64u));
+            const uint32_t chunk_stride = pa.n_feat_blocks * (NACC * 1024u);   // bytes from one chunk's sums to the next
 #pragma unroll
-            for (int i = 0; i < NACC; ++i) store_device_scope(dst + i * 64, acc[i]);
-            __builtin_amdgcn_s_waitcnt(0x0F70);                        // vmcnt(0): the stores are acknowledged
+            for (int i = 0; i < NACC; ++i) store_device_scope(sums, chunk * chunk_stride + uint32_t(i) * 1024u + lane * 16u, acc[i]);
+            wait_stores_acknowledged();
             uint32_t *ctr = pa.arrive + size_t(unit) * pa.n_feat_blocks + fb;
             uint32_t old = 0;
             if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -859,7 +863,7 @@ void spmm_panel_kernel(const PanelArgs pa)
                 for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
                 for (uint32_t c = 0; c < pa.n_chunks; ++c) {
 #pragma unroll
-                    for (int i = 0; i < NACC; ++i) acc[i] += load_device_scope(slot0 + c * chunk_stride + i * 64);
+                    for (int i = 0; i < NACC; ++i) acc[i] += load_device_scope(sums, c * chunk_stride + uint32_t(i) * 1024u + lane * 16u);
                 }
                 store_unit<TT>(L, acc, c_lane, row_bytes, row0, nwin, pa.rows, true);
                 if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
