@@ -17,7 +17,8 @@ IDX_MAX = 0xFFFFFFFF
 ROW_WINDOW = 8
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB = os.path.join(_HERE, "libhspmm.so")
+# HSPMM_LIBRARY: another build of the library to load instead (the measurement builds of `make measure`)
+_LIB = os.environ.get("HSPMM_LIBRARY") or os.path.join(_HERE, "libhspmm.so")
 _lib = None
 
 

@@ -1657,7 +1657,8 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     if (p->cfg.panel_units_per_group)          // fewer units than the shape has consumer waves
         forced_units = std::min(p->cfg.panel_units_per_group, units == 13 ? 12 : units);
     // (units of up to four windows: eight consumer waves with twice the accumulators)
-    const int max_units = pl.G == 4 ? 8 : units == 13 ? 12 : units;
+    // (two 16-bit units per wave: eight larger consumer waves as well)
+    const int max_units = (pl.G == 4 || (pl.tall && p->dtype != HSPMM_TF32)) ? 8 : units == 13 ? 12 : units;
     // what one consumer wave takes: a unit, or (tall streams) two
     const uint32_t wave_units = pl.tall ? (pl.n_units + 1u) / 2u : pl.n_units;
     if (forced_units) forced_units = std::min(forced_units, max_units);

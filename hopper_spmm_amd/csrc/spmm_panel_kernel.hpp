@@ -29,7 +29,18 @@
 #include <type_traits>
 #include "spmm_mfma_kernel.hpp"
 
+// Measurement builds (make measure): HSPMM_MEASURE_SKIP is a mask of work that the kernels built on the
+// 16-bit MFMA leave out, to see what the rest of a launch costs.  The results of such a build are wrong.
+//   1: the consumers' MFMAs            2: the consumers' LDS reads
+//   4: the producers' copy to LDS      8: the producers' loads of B
+//  16: the consumers' loads of tiles and ids behind the first ring
+#ifndef HSPMM_MEASURE_SKIP
+#define HSPMM_MEASURE_SKIP 0
+#endif
+
 namespace hspmm {
+
+constexpr int kMeasureSkip = HSPMM_MEASURE_SKIP;
 
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
 
@@ -275,6 +286,10 @@ struct PanelOps<Fp16Tr<G_, BF>> {
         Half<H> B;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
+            if constexpr (kMeasureSkip & 2) {
+                B.b[p] = u32x4{I, uint32_t(p), I, 0u};
+                continue;
+            }
             const tr16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a0 + 32 * (4 * H + p)));
             const tr16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a1 + 32 * (4 * H + p)));
             const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
@@ -288,6 +303,10 @@ struct PanelOps<Fp16Tr<G_, BF>> {
     {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
+            if constexpr (kMeasureSkip & 1) {
+                asm volatile("" :: "v"(B.b[p]), "v"(A.r[0]));
+                continue;
+            }
             acc[4 * H + p] = HalfOps<BF>::mfma(A.r[0], B.b[p], acc[4 * H + p]);
             if constexpr (kFour) acc[8 + 4 * H + p] = HalfOps<BF>::mfma(A.r[1], B.b[p], acc[8 + 4 * H + p]);
         }
@@ -446,6 +465,10 @@ struct PanelOps<Fp32Split<G_>> {
         Half<H> B;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
+            if constexpr (kMeasureSkip & 2) {
+                B.hi[p] = u32x4{I, uint32_t(p), I, 0u}; B.lo[p] = u32x4{I, 1u, I, uint32_t(p)};
+                continue;
+            }
             B.hi[p] = operand(a0, a1, 32 * (2 * H + p));
             B.lo[p] = operand(a0, a1, 128 + 32 * (2 * H + p));
         }
@@ -465,6 +488,10 @@ struct PanelOps<Fp32Split<G_>> {
         for (int p = 0; p < 2; ++p) {
 #pragma unroll
             for (int h = 0; h < kRowSets; ++h) {
+                if constexpr (kMeasureSkip & 1) {
+                    asm volatile("" :: "v"(B.hi[p]), "v"(B.lo[p]), "v"(a_hi[h]), "v"(a_lo[h]));
+                    continue;
+                }
                 // small terms first; a_lo * b_lo (below 2^-14 |a||b|, 2^-16 on average) is left out
                 const int q = 4 * h + 2 * H + p;
                 f32x4 c = HalfOps<true>::mfma(a_lo[h], B.hi[p], acc[q]);
@@ -630,6 +657,10 @@ void spmm_panel_kernel(const PanelArgs pa)
         // period, and the consumers wait for them.  (Three panels in flight, with four producer waves,
         // measured no faster.)
         u32x4 X[kPieces];
+        auto copy_piece = [&](char *row, const u32x4 &x) __attribute__((always_inline)) {
+            if constexpr (kMeasureSkip & 4) asm volatile("" :: "v"(x));
+            else Ops::write_piece(row, pt & 15u, x);
+        };
         {
             const char *panel = panel_base(p_begin);
             const uint32_t last_off = last_row_off(p_begin);
@@ -646,13 +677,13 @@ void spmm_panel_kernel(const PanelArgs pa)
                 const uint32_t last_off = last_row_off(q + 1u);
 #pragma unroll
                 for (int i = 0; i < kPieces; ++i) {
-                    Ops::write_piece(img + uint32_t(i) * (NPW * 4) * kPitch, pt & 15u, X[i]);
-                    X[i] = load_piece(panel, last_off, i);
+                    copy_piece(img + uint32_t(i) * (NPW * 4) * kPitch, X[i]);
+                    if constexpr (!(kMeasureSkip & 8)) X[i] = load_piece(panel, last_off, i);
                     __builtin_amdgcn_sched_barrier(0);              // in the order the loads return
                 }
             } else {
 #pragma unroll
-                for (int i = 0; i < kPieces; ++i) Ops::write_piece(img + uint32_t(i) * (NPW * 4) * kPitch, pt & 15u, X[i]);
+                for (int i = 0; i < kPieces; ++i) copy_piece(img + uint32_t(i) * (NPW * 4) * kPitch, X[i]);
             }
             panel_barrier();
         }
@@ -733,7 +764,7 @@ void spmm_panel_kernel(const PanelArgs pa)
 #else
     constexpr uint32_t kRing = [] {
         if constexpr (PACKED) return Ops::kPackedRing;
-        else return (TALL && TT::kElem == 2) ? 2u : Ops::kRing;
+        else return Ops::kRing;
     }();
 #endif
     static_assert(kRing >= 1 && kRing <= 6, "ring slots are named variables");
@@ -806,7 +837,7 @@ void spmm_panel_kernel(const PanelArgs pa)
 #define HSPMM_PANEL_STEADY(k, kn) if constexpr (kRing > k) { \
         step(I##k, A##k, HSPMM_NEXT_IDX(k, kn), Ops::jump(HSPMM_NEXT_IDX(k, kn))); \
         request(HSPMM_OTHER_HEADER(k), t + k##u + kRing + 1u); \
-        I##k = ring_idx(t + k##u + kRing); A##k = ring_a(HSPMM_HEADER(k), t + k##u + kRing); }
+        if constexpr (!(kMeasureSkip & 16)) { I##k = ring_idx(t + k##u + kRing); A##k = ring_a(HSPMM_HEADER(k), t + k##u + kRing); } }
         HSPMM_RING2(HSPMM_PANEL_STEADY)
 #undef HSPMM_PANEL_STEADY
     }
@@ -924,8 +955,11 @@ template <class TT>
 static hipError_t launch_panel_tall(const PanelArgs &pa, const KernelArgs &ka, bool packed, hipStream_t s, hipEvent_t mid)
 {
     static_assert(PanelOps<TT>::kRows > 128u && TT::G <= 2, "two units per wave: 16 rows each");
-    return packed ? launch_panel_tt<TT, PanelOps<TT>::kConsumers, 4, true, true>(pa, ka, s, mid)
-                  : launch_panel_tt<TT, PanelOps<TT>::kConsumers, 4, true, false>(pa, ka, s, mid);
+    // (16-bit types: two sets of eight accumulators and two sets of second operands - eight consumer waves,
+    // so that a wave may hold 168 registers)
+    constexpr int kTallConsumers = TT::kElem == 2 ? 8 : PanelOps<TT>::kConsumers;
+    return packed ? launch_panel_tt<TT, kTallConsumers, 4, true, true>(pa, ka, s, mid)
+                  : launch_panel_tt<TT, kTallConsumers, 4, true, false>(pa, ka, s, mid);
 }
 
 }  // namespace hspmm
