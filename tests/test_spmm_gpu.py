@@ -483,9 +483,10 @@ def test_long_units_are_walked_by_one_workgroup_each(torch_cuda, hs, oracle, dty
 
 @pytest.mark.parametrize("dtype", [0, 1])
 def test_partial_sums_added_inside_the_main_kernel(torch_cuda, hs, oracle, dtype):
-    """HSPMM_FUSED_FIXUP=1 (an experiment switch, slower than the second launch): the wave that brings
-    the last partial sum of a cut unit, or of a unit's chunks of panels, adds them in the fixed order and
-    stores the unit: the same bits launch after launch, whoever arrives last."""
+    """The wave that brings the last partial sum of a cut unit, or of a unit's chunks of panels, adds them
+    in the fixed order and stores the unit (the default of the LDS-staging kernels, and of the gather kernels
+    where few units are cut; HSPMM_FUSED_FIXUP = 1 / 0 forces it / the second launch): the same bits launch
+    after launch, whoever arrives last, and for chunks of panels the bits of the two-launch path."""
     torch = torch_cuda
     rng = np.random.default_rng(33 + dtype)
     block = 64 if dtype == 1 else 128
@@ -497,8 +498,17 @@ def test_partial_sums_added_inside_the_main_kernel(torch_cuda, hs, oracle, dtype
         hs.configure(producer_warp_group_num=16)
         os.environ["HSPMM_PANEL_CHUNKS"] = "3"
         try:
-            two = hs.Plan(b)
+            os.environ["HSPMM_FUSED_FIXUP"] = "0"
+            try:
+                two = hs.Plan(b)
+            finally:
+                os.environ.pop("HSPMM_FUSED_FIXUP", None)
             want = gpu_spmm(torch, hs, b, B, N, plan=two)
+            tt = torch.float32 if dtype == 1 else torch.int16
+            dB = torch.zeros((3000, N), dtype=tt, device="cuda")
+            dC = torch.empty((300, N), dtype=tt, device="cuda")
+            main_ms, sum_ms = two.profile(dB.data_ptr(), dC.data_ptr(), N, runs=2)
+            assert main_ms > 0 and sum_ms > 0                  # two launches
             two.close()
             os.environ["HSPMM_FUSED_FIXUP"] = "1"
             try:
@@ -813,7 +823,7 @@ def test_run_captured_in_a_hip_graph_replays_correctly(torch_cuda, hs, oracle):
     rng = np.random.default_rng(15)
     for dtype, panels in ((0, False), (1, False), (0, True), (1, True)):
         if panels:
-            # dense windows: the LDS-panel kernel and the kernel that adds its chunk sums
+            # dense windows: the LDS-panel kernel, whose waves add the chunk sums of their units
             A = random_csr(rng, 400, 4000, 0.1, dtype, 0.1)
             b = convert(hs, A)
             plan = hs.Plan(b)
