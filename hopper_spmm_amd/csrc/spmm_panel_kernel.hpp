@@ -34,6 +34,7 @@
 //   1: the consumers' MFMAs            2: the consumers' LDS reads
 //   4: the producers' copy to LDS      8: the producers' loads of B
 //  16: the consumers' loads of tiles and ids behind the first ring
+//  32: the producers' split of fp32 rows of B into bf16 parts (the words are copied as they are)
 #ifndef HSPMM_MEASURE_SKIP
 #define HSPMM_MEASURE_SKIP 0
 #endif
@@ -398,6 +399,12 @@ struct PanelOps<Fp32Split<G_>> {
     __device__ static __forceinline__ void write_piece(char *row, uint32_t c, const u32x4 x)
     {
         u32x2 hi, lo;
+        if constexpr (kMeasureSkip & 32) {
+            hi[0] = x[0]; hi[1] = x[1]; lo[0] = x[2]; lo[1] = x[3];
+            *reinterpret_cast<u32x2 *>(row + c * 8u) = hi;
+            *reinterpret_cast<u32x2 *>(row + 128u + c * 8u) = lo;
+            return;
+        }
         hi[0] = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);       // the upper halves
         hi[1] = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
         lo[0] = pack_bf16_rn(split_rest(x[0]), split_rest(x[1]));
