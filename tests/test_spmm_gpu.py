@@ -536,6 +536,45 @@ def test_partial_sums_added_inside_the_main_kernel(torch_cuda, hs, oracle, dtype
         assert_parity(want, ref, mag, dtype, "two-kernel path")
 
 
+def test_error_of_the_three_product_fp32_arithmetic_against_fp64(torch_cuda, hs):
+    """The LDS-staging kernels multiply fp32 storage as bf16 parts in three products (a_lo b_lo left out):
+    against an fp64 product the error stays below 2^-16 sum |a||b| on normal entries and below the hard bound
+    2^-14 sum |a||b| on the adversarial input - every factor positive with all low mantissa bits set, so that
+    nothing cancels and every left-out product is as large as it can be; with fp32 products (kernel mode 5)
+    it is rounding of the fp32 sums only."""
+    rng = np.random.default_rng(404)
+    rows, cols, N = 512, 2048, 64
+    mask = rng.random((rows, cols)) < 0.1
+    rp = np.concatenate([[0], np.cumsum(mask.sum(axis=1))]).astype(np.uint32)
+    ci = np.nonzero(mask)[1].astype(np.uint32)
+    all_ones = np.float32(np.frombuffer(np.uint32(0x3FFFFFFF).tobytes(), np.float32)[0])      # 1.9999999
+    cases = {
+        "normal": (rng.normal(size=ci.size).astype(np.float32), rng.normal(size=(cols, N)).astype(np.float32), 2.0 ** -16),
+        "adversarial": ((all_ones * np.exp2(rng.integers(-3, 4, ci.size))).astype(np.float32),
+                        (all_ones * np.exp2(rng.integers(-3, 4, (cols, N)))).astype(np.float32), 2.0 ** -14),
+    }
+    for name, (vals, B, bound) in cases.items():
+        D = np.zeros((rows, cols), np.float64)
+        D[mask] = vals
+        ref = D @ B.astype(np.float64)
+        mag = np.abs(D) @ np.abs(B).astype(np.float64)
+        A = dict(rows=rows, cols=cols, row_ptr=rp, col_idx=ci, values=vals, dtype=1)
+        b = convert(hs, A)
+        for mode, limit in ((0, bound), (5, 2.0 ** -20)):
+            hs.set_kernel_mode(mode)
+            try:
+                plan = hs.Plan(b)
+                got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+                assert plan.info()["last_kernel_family"] == 3, (name, mode)
+                plan.close()
+            finally:
+                hs.set_kernel_mode(0)
+            worst = float((np.abs(got.astype(np.float64) - ref) / mag).max())
+            assert worst <= limit, "%s, kernel mode %d: %.3g sum |a||b| (2^%.1f)" % (name, mode, worst, np.log2(worst))
+            if mode == 0 and name == "adversarial":
+                assert worst > 2.0 ** -17        # the left-out product is there: this input does exercise the bound
+
+
 def test_lds_panel_kernels_are_chosen_for_dense_windows_only(torch_cuda, hs):
     from hopper_spmm_amd import generators as G
     dense = G.make_config(4, 8)["A"]            # block-clustered: every window meets half of all columns
