@@ -3,6 +3,8 @@
 #pragma once
 #include <algorithm>
 #include <cstddef>
+#include <cstdlib>
+#include <new>
 #include <exception>
 #include <thread>
 #include <vector>
@@ -38,5 +40,35 @@ void parallel_blocks(size_t n, size_t min_per_worker, F &&fn)
     for (auto &t : th) t.join();
     for (auto &e : err) if (e) std::rethrow_exception(e);
 }
+
+// n elements that read as zero, without the single-threaded pass a std::vector spends on clearing them
+// (a fifth of a second for the arrays of a large plan): the memory comes from calloc, whose fresh pages are
+// zero already, and is first touched by whichever worker fills it.  Trivial element types only.
+template <class T>
+class ZeroedBuffer {
+    T *p_ = nullptr;
+    size_t n_ = 0;
+public:
+    ZeroedBuffer() = default;
+    explicit ZeroedBuffer(size_t n) : p_(static_cast<T *>(std::calloc(n ? n : 1, sizeof(T)))), n_(n)
+    {
+        if (!p_) throw std::bad_alloc();
+    }
+    ZeroedBuffer(const ZeroedBuffer &) = delete;
+    ZeroedBuffer &operator=(const ZeroedBuffer &) = delete;
+    ZeroedBuffer(ZeroedBuffer &&o) noexcept : p_(o.p_), n_(o.n_) { o.p_ = nullptr; o.n_ = 0; }
+    ZeroedBuffer &operator=(ZeroedBuffer &&o) noexcept
+    {
+        if (this != &o) { std::free(p_); p_ = o.p_; n_ = o.n_; o.p_ = nullptr; o.n_ = 0; }
+        return *this;
+    }
+    ~ZeroedBuffer() { std::free(p_); }
+    T *data() { return p_; }
+    const T *data() const { return p_; }
+    size_t size() const { return n_; }
+    T &operator[](size_t i) { return p_[i]; }
+    const T &operator[](size_t i) const { return p_[i]; }
+    void swap(ZeroedBuffer &o) noexcept { std::swap(p_, o.p_); std::swap(n_, o.n_); }
+};
 
 }  // namespace hspmm_host

@@ -13,6 +13,7 @@
 #include <vector>
 #include <mutex>
 #include <atomic>
+#include <chrono>
 #include <new>
 #include <algorithm>
 
@@ -185,6 +186,19 @@ struct hspmm_plan {
 
 namespace {
 
+// HSPMM_TIMING=1 in the environment: hspmm_create prints what each of its phases took (stderr).
+struct PhaseTimer {
+    bool on = std::getenv("HSPMM_TIMING") != nullptr;
+    std::chrono::steady_clock::time_point last = std::chrono::steady_clock::now();
+    void mark(const char *what)
+    {
+        if (!on) return;
+        const auto now = std::chrono::steady_clock::now();
+        std::fprintf(stderr, "hspmm_create: %-28s %8.2f ms\n", what, std::chrono::duration<double, std::milli>(now - last).count());
+        last = now;
+    }
+};
+
 template <typename T>
 int upload(T **dst, const T *src, size_t n, size_t *acc_bytes)
 {
@@ -302,7 +316,7 @@ struct StepStream {
 };
 
 StepStream build_units(uint32_t W, uint32_t cw, const uint32_t *rowOffset, const uint32_t *rowIdx,
-                       const std::vector<uint32_t> &ids_clean, int pairing)
+                       const uint32_t *ids_clean, int pairing)
 {
     StepStream st;
     // which windows could pair with their successor
@@ -312,8 +326,8 @@ StepStream build_units(uint32_t W, uint32_t cw, const uint32_t *rowOffset, const
         for (uint32_t w = 0; w + 1 < W; ++w) {
             const uint32_t n = rowOffset[w + 1] - rowOffset[w];
             if (rowIdx[w + 1] != rowIdx[w] + HSPMM_ROW_WINDOW || rowOffset[w + 2] - rowOffset[w + 1] != n) continue;
-            const uint32_t *a = ids_clean.data() + size_t(rowOffset[w]) * cw;
-            const uint32_t *b = ids_clean.data() + size_t(rowOffset[w + 1]) * cw;
+            const uint32_t *a = ids_clean + size_t(rowOffset[w]) * cw;
+            const uint32_t *b = ids_clean + size_t(rowOffset[w + 1]) * cw;
             if (std::memcmp(a, b, size_t(n) * cw * 4) == 0) can[w] = 1;
         }
         for (uint32_t w = 0; w + 1 < W;) {
@@ -339,60 +353,62 @@ StepStream build_units(uint32_t W, uint32_t cw, const uint32_t *rowOffset, const
 }
 
 // ids per step in lane order.  fp16: the 16 ids of the step's tile.  fp32: [g][2] = (id g, id g + 4).
-std::vector<uint32_t> lane_order_ids(const StepStream &st, int dtype, const uint32_t *rowOffset,
-                                     const std::vector<uint32_t> &ids_clean)
+hspmm_host::ZeroedBuffer<uint32_t> lane_order_ids(const StepStream &st, int dtype, const uint32_t *rowOffset, const uint32_t *ids_clean)
 {
     const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
-    std::vector<uint32_t> out(size_t(st.n_steps) * cw);
-    for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
-        const uint32_t t0 = rowOffset[st.unitWindow[u]];
-        for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
-            const uint32_t *src = ids_clean.data() + size_t(t0 + i) * cw;
-            uint32_t *dst = out.data() + size_t(st.unitOffset[u] + i) * cw;
-            if (dtype != HSPMM_TF32) std::memcpy(dst, src, 64);
-            else for (uint32_t g = 0; g < 4; ++g) { dst[2 * g] = src[g]; dst[2 * g + 1] = src[g + 4]; }
+    hspmm_host::ZeroedBuffer<uint32_t> out(size_t(st.n_steps) * cw);
+    hspmm_host::parallel_blocks(st.unitRow.size(), 256, [&](size_t ub, size_t ue) {
+        for (size_t u = ub; u < ue; ++u) {
+            const uint32_t t0 = rowOffset[st.unitWindow[u]];
+            for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
+                const uint32_t *src = ids_clean + size_t(t0 + i) * cw;
+                uint32_t *dst = out.data() + size_t(st.unitOffset[u] + i) * cw;
+                if (dtype != HSPMM_TF32) std::memcpy(dst, src, 64);
+                else for (uint32_t g = 0; g < 4; ++g) { dst[2 * g] = src[g]; dst[2 * g + 1] = src[g + 4]; }
+            }
         }
-    }
+    });
     return out;
 }
 
 // tiles per step in lane order, as 32-bit words.
 //   fp16: [row r][g][window][2 words = halves 4g..4g+3 of row r]
 //   fp32: [row r][g][window][2 words = a[r][g], a[r][g+4]]
-std::vector<uint32_t> lane_order_tiles(const StepStream &st, int dtype, const uint32_t *rowOffset, const void *data)
+hspmm_host::ZeroedBuffer<uint32_t> lane_order_tiles(const StepStream &st, int dtype, const uint32_t *rowOffset, const void *data)
 {
     const int G = st.G;
     const uint32_t *words = static_cast<const uint32_t *>(data);     // a tile is 64 words in both formats
-    std::vector<uint32_t> out(size_t(st.n_steps) * 64u * G, 0u);
-    for (size_t u = 0; u + 1 < st.unitOffset.size(); ++u) {
-        const uint32_t w0 = st.unitWindow[u];
-        const int nwin = (st.unitRow[u] & 1u) ? 2 : 1;
-        for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
-            uint32_t *dst = out.data() + size_t(st.unitOffset[u] + i) * 64u * G;
-            for (int w = 0; w < nwin; ++w) {
-                const uint32_t *src = words + size_t(rowOffset[w0 + w] + i) * 64u;
-                for (uint32_t r = 0; r < 8; ++r)
-                    for (uint32_t g = 0; g < 4; ++g) {
-                        uint32_t *d = dst + ((r * 4 + g) * G + w) * 2;
-                        if (dtype != HSPMM_TF32) { d[0] = src[r * 8 + 2 * g]; d[1] = src[r * 8 + 2 * g + 1]; }
-                        else { d[0] = src[r * 8 + g]; d[1] = src[r * 8 + g + 4]; }
-                    }
+    hspmm_host::ZeroedBuffer<uint32_t> out(size_t(st.n_steps) * 64u * G);
+    hspmm_host::parallel_blocks(st.unitRow.size(), 64, [&](size_t ub, size_t ue) {
+        for (size_t u = ub; u < ue; ++u) {
+            const uint32_t w0 = st.unitWindow[u];
+            const int nwin = (st.unitRow[u] & 1u) ? 2 : 1;
+            for (uint32_t i = 0, n = st.unitOffset[u + 1] - st.unitOffset[u]; i < n; ++i) {
+                uint32_t *dst = out.data() + size_t(st.unitOffset[u] + i) * 64u * G;
+                for (int w = 0; w < nwin; ++w) {
+                    const uint32_t *src = words + size_t(rowOffset[w0 + w] + i) * 64u;
+                    for (uint32_t r = 0; r < 8; ++r)
+                        for (uint32_t g = 0; g < 4; ++g) {
+                            uint32_t *d = dst + ((r * 4 + g) * G + w) * 2;
+                            if (dtype != HSPMM_TF32) { d[0] = src[r * 8 + 2 * g]; d[1] = src[r * 8 + 2 * g + 1]; }
+                            else { d[0] = src[r * 8 + g]; d[1] = src[r * 8 + g + 4]; }
+                        }
+                }
             }
         }
-    }
+    });
     return out;
 }
-
 
 // 16-bit steps of 32 columns for the LDS-panel kernels (Fp16Tr in spmm_panel_kernel.hpp): a re-tiled
 // step of a window is [row r][32 halves]; lane l = (g, m) of the step's 1 KB gets the 16 bytes
 // a[m][8g .. 8g + 7], m = row of the unit's 16 rows (rows 8..15: the second window of a pair, else zero).
 // A stream with units of up to four windows (G = 4) has a second KB per step for windows 2 and 3.
-std::vector<uint32_t> lane_order_wide_steps(const StepStream &st, const uint32_t *rowOffset, const void *data)
+hspmm_host::ZeroedBuffer<uint32_t> lane_order_wide_steps(const StepStream &st, const uint32_t *rowOffset, const void *data)
 {
     const uint16_t *halves = static_cast<const uint16_t *>(data);   // a step of a window is 8 x 32 halves
     const size_t step_words = st.G == 4 ? 512u : 256u;
-    std::vector<uint32_t> out(size_t(st.n_steps) * step_words, 0u);
+    hspmm_host::ZeroedBuffer<uint32_t> out(size_t(st.n_steps) * step_words);
     hspmm_host::parallel_blocks(st.unitRow.size(), 16, [&](size_t ub, size_t ue) {
         for (size_t u = ub; u < ue; ++u) {
             const uint32_t w0 = st.unitWindow[u];
@@ -432,11 +448,11 @@ uint32_t split_bf16_host(float v)
 // fp32 steps of 32 columns in the split form (Fp32Split): a re-tiled step of a window is [row r][32 floats];
 // lane l = (g, m) gets 32 bytes: the 8 hi halves, then the 8 lo halves of a[m][8g .. 8g + 7].  A stream with
 // units of up to four windows (G = 4) has a second 2 KB per step for windows 2 and 3.
-std::vector<uint32_t> lane_order_split_steps(const StepStream &st, const uint32_t *rowOffset, const void *data)
+hspmm_host::ZeroedBuffer<uint32_t> lane_order_split_steps(const StepStream &st, const uint32_t *rowOffset, const void *data)
 {
     const float *vals = static_cast<const float *>(data);            // a step of a window is 8 x 32 floats
     const size_t step_words = st.G == 4 ? 1024u : 512u;
-    std::vector<uint32_t> out(size_t(st.n_steps) * step_words, 0u);
+    hspmm_host::ZeroedBuffer<uint32_t> out(size_t(st.n_steps) * step_words);
     hspmm_host::parallel_blocks(st.unitRow.size(), 16, [&](size_t ub, size_t ue) {
         for (size_t u = ub; u < ue; ++u) {
             const uint32_t w0 = st.unitWindow[u];
@@ -474,7 +490,7 @@ std::vector<uint32_t> lane_order_split_steps(const StepStream &st, const uint32_
 // panel.  Returns false (outputs unused) when no two groups merge.
 struct Unioned {
     std::vector<uint32_t> rowOffset, tcA2B;
-    std::vector<uint8_t> data;
+    hspmm_host::ZeroedBuffer<uint8_t> data;
     uint32_t T = 0;
 };
 
@@ -519,7 +535,9 @@ bool merge_groups(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, u
     const size_t NG = first.size();
     std::vector<uint8_t> can(NG, 0), join(NG, 0);
     std::vector<uint32_t> union_tiles(NG, 0u), tiles(W);
-    hspmm_host::parallel_blocks(NG - 1, 256, [&](size_t gb, size_t ge) {
+    // (as many groups per worker as make a few thousand tiles)
+    const size_t groups_per_worker = std::max<size_t>(1, (size_t(1) << 12) / std::max<uint32_t>(1u, rowOffset[W] / W));
+    hspmm_host::parallel_blocks(NG - 1, groups_per_worker, [&](size_t gb, size_t ge) {
         std::vector<uint32_t> merged;
         for (size_t g = gb; g < ge; ++g) {
             const uint32_t wa = first[g], wb = first[g + 1], nw = count[g] + count[g + 1];
@@ -550,7 +568,7 @@ bool merge_groups(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, u
     for (uint32_t w = 0; w < W; ++w) out.rowOffset[w + 1] = out.rowOffset[w] + tiles[w];
     out.T = out.rowOffset[W];
     out.tcA2B.assign(size_t(out.T) * cw, HSPMM_IDX_MAX);
-    out.data.assign(size_t(out.T) * tile_bytes, 0);
+    out.data = hspmm_host::ZeroedBuffer<uint8_t>(size_t(out.T) * tile_bytes);
     // second pass: copy, or spread a window's tile columns over the merged list's columns
     auto spread = [&](uint32_t w, const uint32_t *ids, uint32_t n_ids) {
         const uint32_t *c = tcA2B + size_t(rowOffset[w]) * cw;
@@ -574,7 +592,7 @@ bool merge_groups(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, u
         second.push_back(join[g] ? first[g + 1] : HSPMM_IDX_MAX);
         if (join[g]) ++g;
     }
-    hspmm_host::parallel_blocks(out_first.size(), 64, [&](size_t gb, size_t ge) {
+    hspmm_host::parallel_blocks(out_first.size(), groups_per_worker, [&](size_t gb, size_t ge) {
         std::vector<uint32_t> merged;
         for (size_t g = gb; g < ge; ++g) {
             const uint32_t wa = out_first[g], nw = out_count[g];
@@ -628,11 +646,12 @@ void group_windows(uint32_t W, uint32_t cw, uint32_t elem, uint32_t panel_cols, 
 // LDS then serves twice as many rows.  ids: 16 words per step; tiles: tile_words per step.
 void merge_unit_pairs(uint32_t U, uint32_t NP, size_t tile_words, const std::vector<uint32_t> &unitOffset,
                       std::vector<uint32_t> &poff, std::vector<uint32_t> &step_panel, std::vector<uint32_t> &ids,
-                      std::vector<uint32_t> &tiles)
+                      hspmm_host::ZeroedBuffer<uint32_t> &tiles)
 {
     const uint32_t Q = (U + 1u) / 2u;
     const size_t n_steps = step_panel.size();
-    std::vector<uint32_t> n_poff(size_t(Q) * (NP + 1)), n_panel(n_steps), n_ids(ids.size()), n_tiles(tiles.size());
+    std::vector<uint32_t> n_poff(size_t(Q) * (NP + 1)), n_panel(n_steps), n_ids(ids.size());
+    hspmm_host::ZeroedBuffer<uint32_t> n_tiles(tiles.size());
     hspmm_host::parallel_blocks(Q, 8, [&](size_t qb, size_t qe) {
         for (size_t q = qb; q < qe; ++q) {
             const uint32_t a = uint32_t(2 * q), b = a + 1u;
@@ -672,7 +691,7 @@ void merge_unit_pairs(uint32_t U, uint32_t NP, size_t tile_words, const std::vec
 // 0 holds a zero, and a step's worth of zeros follows the last value.  This is the bitmap layout of the
 // reference's BTCF_MTX (nnzOffset / tcBit / packed data, reference src/utils/class.h:55-67 and
 // src/utils/convert.h:83-101) with one bitmap per step and the bits in the order the lanes need them.
-void pack_steps(size_t n_steps, bool split, const std::vector<uint32_t> &tiles, std::vector<uint64_t> &masks,
+void pack_steps(size_t n_steps, bool split, const hspmm_host::ZeroedBuffer<uint32_t> &tiles, std::vector<uint64_t> &masks,
                 std::vector<uint8_t> &vals, std::vector<uint32_t> &step_voff)
 {
     const size_t lane_halves = split ? 16 : 8, es = split ? 4 : 2;
@@ -722,10 +741,10 @@ void pack_steps(size_t n_steps, bool split, const std::vector<uint32_t> &tiles, 
 // src/utils/convert.h:83-101; an element is stored when its bit pattern is not +0) as four 32-bit words, the bit
 // counts of words 0, 0..1 and 0..2 in bytes 1..3 of word 4, and in word 5 the position of the tile's first stored
 // element in `vals` (the reference's nnzOffset), where the stored elements follow tile after tile in bit order.
-void build_gather_bitmap(uint32_t T, const void *data, std::vector<uint32_t> &header, std::vector<uint16_t> &vals)
+void build_gather_bitmap(uint32_t T, const void *data, hspmm_host::ZeroedBuffer<uint32_t> &header, hspmm_host::ZeroedBuffer<uint16_t> &vals)
 {
     const uint16_t *h = static_cast<const uint16_t *>(data);
-    header.assign(size_t(T) * 8u, 0u);
+    header = hspmm_host::ZeroedBuffer<uint32_t>(size_t(T) * 8u);
     std::vector<uint32_t> count(size_t(T) + 1, 0u);
     hspmm_host::parallel_blocks(T, 4096, [&](size_t tb, size_t te) {
         for (size_t t = tb; t < te; ++t) {
@@ -740,7 +759,7 @@ void build_gather_bitmap(uint32_t T, const void *data, std::vector<uint32_t> &he
     });
     uint64_t total = 0;
     for (size_t t = 0; t < T; ++t) { header[t * 8u + 5u] = uint32_t(total); total += count[t + 1]; }
-    vals.assign(size_t(total) + 4u, 0);                            // a lane reads 8 bytes from its first element
+    vals = hspmm_host::ZeroedBuffer<uint16_t>(size_t(total) + 4u);                // a lane reads 8 bytes from its first element
     hspmm_host::parallel_blocks(T, 4096, [&](size_t tb, size_t te) {
         for (size_t t = tb; t < te; ++t) {
             const uint16_t *tile = h + t * 128u;
@@ -759,6 +778,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
                         const void *data, const uint32_t *rowIdx, bool forced, int *rc_out)
 {
     *rc_out = HSPMM_OK;
+    PhaseTimer timer;
     const uint32_t cw = p->cw, W = p->W;
     // fp32: products of bf16 hi / lo parts (Fp32Split) unless the caller asked for fp32 products
     const bool split = p->dtype == HSPMM_TF32 && p->cfg.kernel_mode != 5;
@@ -814,12 +834,12 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
         st.n_steps = st.unitOffset.back();
         st.G = widest >= 3u ? 4 : int(widest);
     }
+    timer.mark("  panel: units of windows");
     const uint32_t U = uint32_t(st.unitRow.size());
     const uint32_t T = rowOffset[W];
     const size_t es = p->elem, src_tile_bytes = size_t(8) * cw * es, tile_bytes = size_t(8) * rw * es;
     // Two passes over the windows, both on all cores: the steps every window gets, then the steps.
-    std::vector<uint32_t> rt_rowOffset(size_t(W) + 1, 0u), rt_ids, rt_panel;
-    std::vector<uint8_t> rt_data;
+    std::vector<uint32_t> rt_rowOffset(size_t(W) + 1, 0u), rt_panel;
     const uint8_t *src_data = static_cast<const uint8_t *>(data);
     auto real_columns = [&](uint32_t w) {
         const uint32_t *col = tcA2B + size_t(rowOffset[w]) * cw;
@@ -845,9 +865,9 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     });
     for (uint32_t w = 0; w < W; ++w) rt_rowOffset[w + 1] += rt_rowOffset[w];
     const size_t RT = rt_rowOffset[W];
-    rt_ids.assign(RT * rw, 0u);
+    hspmm_host::ZeroedBuffer<uint32_t> rt_ids(RT * rw);
     rt_panel.assign(RT, 0u);
-    rt_data.assign(RT * tile_bytes, 0);
+    hspmm_host::ZeroedBuffer<uint8_t> rt_data(RT * tile_bytes);
     hspmm_host::parallel_blocks(W, windows_per_worker, [&](size_t wb, size_t we) {
         for (size_t w = wb; w < we; ++w) {
             const uint32_t t0 = rowOffset[w];
@@ -904,6 +924,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
             }
         }
     });
+    timer.mark("  panel: steps per panel");
     // the units with the re-tiled step counts
     StepStream ps;
     ps.G = st.G; ps.unitRow = st.unitRow; ps.unitWindow = st.unitWindow; ps.n_paired = st.n_paired; ps.n_wide = st.n_wide;
@@ -956,9 +977,10 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
             }
         }
     });
+    timer.mark("  panel: ids, offsets");
     hspmm_plan::Panel &pl = p->panel;
     int rc;
-    std::vector<uint32_t> tiles = split      ? lane_order_split_steps(ps, rt_rowOffset.data(), rt_data.data())
+    hspmm_host::ZeroedBuffer<uint32_t> tiles = split      ? lane_order_split_steps(ps, rt_rowOffset.data(), rt_data.data())
                                   : cw == 16 ? lane_order_wide_steps(ps, rt_rowOffset.data(), rt_data.data())
                                              : lane_order_tiles(ps, p->dtype, rt_rowOffset.data(), rt_data.data());
     // Two units per consumer wave, and tiles without their zeros (kernels built on the 16-bit MFMA, units of one
@@ -967,6 +989,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     // by a third and by 60 % and the time does not: what binds these kernels is the LDS reads and MFMAs of a
     // step, which a SIMD runs one after the other.  Both are therefore taken on request only
     // (hspmm_set_panel_stream, HSPMM_PANEL_TALL / HSPMM_PANEL_PACKED).
+    timer.mark("  panel: tiles in lane order");
     bool tall = false, packed = false;
     if (rw == 32 && ps.G <= 2 && U >= 2 && (p->cfg.panel_tall > 0 || p->cfg.panel_packed > 0)) {
         tall = true;
@@ -1008,6 +1031,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     if ((rc = upload(&pl.d_unitRow, st.unitRow.data(), st.unitRow.size(), &p->fixed_bytes))) { *rc_out = rc; return false; }
     pl.n_units = U; pl.G = st.G; pl.n_paired = st.n_paired; pl.n_wide = st.n_wide;
     pl.n_panels = NP; pl.n_steps = ps.n_steps; pl.quad = quad; pl.split = split; pl.density = density; pl.built = true;
+    timer.mark("  panel: upload");
     return true;
 }
 
@@ -1301,9 +1325,11 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
     const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
     const uint32_t elem = dtype == HSPMM_TF32 ? 4u : 2u;
+    PhaseTimer timer;
     bool canonical = true;
     int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx, &canonical);
     if (rc) return rc;
+    timer.mark("validate");
 
     hspmm_plan *p = new (std::nothrow) hspmm_plan;
     if (!p) return fail(HSPMM_ERR_ALLOC, "out of host memory");
@@ -1328,7 +1354,8 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         if ((rc = static_scratch_address(p->device, &unused))) return bail(rc);
     }
 
-    if (p->W) {
+    // (a host allocation that fails anywhere below ends the call with HSPMM_ERR_ALLOC)
+    if (p->W) try {
         const size_t n_ids = size_t(total_tiles) * cw;
         if ((rc = upload(&p->d_rowOffset, rowOffset, size_t(p->W) + 1, &p->fixed_bytes))) return bail(rc);
         if ((rc = upload(&p->d_rowIdx, rowIdx, size_t(p->W), &p->fixed_bytes))) return bail(rc);
@@ -1340,11 +1367,20 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
                 return bail(rc);
             p->d_data = dd;
         }
+        timer.mark("upload format arrays");
         // padding ids -> the real id in front of them (the tile column is all zero)
-        std::vector<uint32_t> clean(tcA2B, tcA2B + n_ids);
-        for (size_t i = 1; i < n_ids; ++i)
-            if (clean[i] == HSPMM_IDX_MAX) clean[i] = clean[i - 1];
+        // (padding trails a window's real ids, of which every window has one at least)
+        hspmm_host::ZeroedBuffer<uint32_t> clean_ids;
+        try { clean_ids = hspmm_host::ZeroedBuffer<uint32_t>(n_ids); }
+        catch (const std::bad_alloc &) { return bail(fail(HSPMM_ERR_ALLOC, "out of host memory")); }
+        uint32_t *clean = clean_ids.data();
+        hspmm_host::parallel_blocks(p->W, 1024, [&](size_t wb, size_t we) {
+            for (size_t i = size_t(rowOffset[wb]) * cw, e = size_t(rowOffset[we]) * cw; i < e; ++i)
+                clean[i] = (tcA2B[i] == HSPMM_IDX_MAX && i) ? clean[i - 1] : tcA2B[i];
+        });
+        timer.mark("ids without padding");
         const StepStream st = build_units(p->W, cw, rowOffset, rowIdx, clean, p->cfg.pairing);
+        timer.mark("units");
         p->G = st.G;
         p->n_units = uint32_t(st.unitRow.size());
         p->n_paired = st.n_paired;
@@ -1352,17 +1388,18 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         if ((rc = upload(&p->d_unitOffset, st.unitOffset.data(), st.unitOffset.size(), &p->fixed_bytes))) return bail(rc);
         if ((rc = upload(&p->d_unitRow, st.unitRow.data(), st.unitRow.size(), &p->fixed_bytes))) return bail(rc);
         {
-            const std::vector<uint32_t> ids = lane_order_ids(st, dtype, rowOffset, clean);
+            const hspmm_host::ZeroedBuffer<uint32_t> ids = lane_order_ids(st, dtype, rowOffset, clean);
             if ((rc = upload(&p->d_ids, ids.data(), ids.size(), &p->fixed_bytes))) return bail(rc);
         }
         if (dtype != HSPMM_TF32 && st.G == 1) {
             p->d_tiles = p->d_data;                 // the caller's tile layout already is the lane order
         } else {
-            const std::vector<uint32_t> tiles = lane_order_tiles(st, dtype, rowOffset, data);
+            const hspmm_host::ZeroedBuffer<uint32_t> tiles = lane_order_tiles(st, dtype, rowOffset, data);
             uint32_t *dt = nullptr;
             if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) return bail(rc);
             p->d_tiles = dt;
         }
+        timer.mark("step stream (ids, tiles)");
         // Single 16-bit windows with few stored elements per tile (graphs: 16 of 128): the gather kernels read the
         // tiles as bitmap + stored elements, 32 + 2 x 16 bytes per tile instead of 256 (power-law graph 2^20 at
         // N = 128, where the stream is read once per XCD half: 0.64 -> 0.19 GB per launch).
@@ -1379,8 +1416,8 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
             // pays the longer dependent chain: 4096 x 4096 at 1 %, 2.7 MB of tiles: 6.8 -> 7.5 us)
             if (p->cfg.gather_bitmap > 0 ||
                 (stored * 3u < size_t(total_tiles) * 128u && size_t(total_tiles) * 256u >= (size_t(8) << 20))) {
-                std::vector<uint32_t> header;
-                std::vector<uint16_t> vals;
+                hspmm_host::ZeroedBuffer<uint32_t> header;
+                hspmm_host::ZeroedBuffer<uint16_t> vals;
                 try { build_gather_bitmap(total_tiles, data, header, vals); }
                 catch (const std::bad_alloc &) { return bail(fail(HSPMM_ERR_ALLOC, "out of host memory")); }
                 if (vals.size() < (size_t(1) << 31)) {               // positions are 32-bit
@@ -1391,8 +1428,10 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
                 }
             }
         }
+        timer.mark("bitmap tiles");
         p->h_unitOffset = st.unitOffset;
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
+        timer.mark("partition");
         {
             // all units long, and so long that the balanced partition cuts each of them several ways:
             // eight ranges per unit where it would cut eight ways or more, four from `four_from` ways on
@@ -1424,7 +1463,10 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
             try { (void)build_panel_stream(p, st, rowOffset, tcA2B, data, rowIdx, p->cfg.kernel_mode >= 4, &prc); }
             catch (const std::bad_alloc &) { return bail(fail(HSPMM_ERR_ALLOC, "out of host memory")); }
             if (prc) return bail(prc);
+            timer.mark("LDS-panel stream");
         }
+    } catch (const std::bad_alloc &) {
+        return bail(fail(HSPMM_ERR_ALLOC, "out of host memory"));
     }
     *out = p;
     return HSPMM_OK;
