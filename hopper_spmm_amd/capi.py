@@ -67,7 +67,7 @@ class PlanInfo(C.Structure):
                 ("device_bytes", C.c_uint64), ("n_panels", C.c_uint32), ("n_panel_steps", C.c_uint32),
                 ("n_panel_units", C.c_uint32), ("n_panel_paired_units", C.c_uint32),
                 ("n_panel_wide_units", C.c_uint32), ("last_kernel_family", C.c_uint32),
-                ("gather_bitmap", C.c_uint32), ("panel_stream_mode", C.c_uint32)]
+                ("gather_bitmap", C.c_uint32), ("bitmap_from_caller", C.c_uint32), ("panel_stream_mode", C.c_uint32)]
 
 
 def load_library():

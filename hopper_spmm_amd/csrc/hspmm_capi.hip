@@ -50,6 +50,15 @@ int fail(int code, const char *fmt, ...)
                         __FILE__, __LINE__);                                                 \
     } while (0)
 
+// the same where a failure has to release something first: cleanup(code) is called with the error code and its result returned
+#define HSPMM_HIP_OR(call, cleanup)                                                          \
+    do {                                                                                     \
+        hipError_t e_ = (call);                                                              \
+        if (e_ != hipSuccess)                                                                \
+            return cleanup(fail(HSPMM_ERR_DEVICE, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), \
+                                __FILE__, __LINE__));                                        \
+    } while (0)
+
 // The knobs of the reference's Scheduler singleton (reference src/scheduler.h:7-10),
 // re-read as: prefetch depth, waves per workgroup, waves per SIMD, compute units.
 struct Config {
@@ -165,6 +174,7 @@ struct hspmm_plan {
         uint32_t *d_header = nullptr;
         void *d_vals = nullptr;
         uint64_t stored = 0;
+        bool from_caller = false;     // header and elements are the caller's tcBit / nnzOffset / data, uploaded as they came
     } bm;
     float *d_scratch = nullptr;
     size_t scratch_bytes = 0;
@@ -1315,9 +1325,43 @@ int hspmm_panel_units_preview(int dtype, uint32_t rows, uint32_t cols, uint32_t 
     return HSPMM_OK;
 }
 
-int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
-                 uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
-                 const uint32_t *rowIdx)
+namespace {
+
+// The caller's bitmap tiles (16-bit element types, HSPMM_BITS_PER_TILE words): reference BTCF_MTX, src/utils/class.h:55-67.
+struct BitmapSource { const uint32_t *nnzOffset; const uint64_t *tcBit; const void *data; };
+constexpr int kNeedsPlainTiles = -1000;     // create_plan with a BitmapSource: this matrix needs the tiles on the host
+
+// Header of the gather kernels' bitmap stream straight from the caller's arrays; returns the first tile whose bit
+// count differs from its nnzOffset span (HSPMM_IDX_MAX: none).
+uint32_t bitmap_header_from_caller(uint32_t T, const BitmapSource &src, hspmm_host::ZeroedBuffer<uint32_t> &header)
+{
+    header = hspmm_host::ZeroedBuffer<uint32_t>(size_t(T) * 8u);
+    std::atomic<uint32_t> first_bad{HSPMM_IDX_MAX};
+    hspmm_host::parallel_blocks(T, 4096, [&](size_t tb, size_t te) {
+        for (size_t t = tb; t < te; ++t) {
+            uint32_t *hd = header.data() + t * 8u;
+            hd[0] = uint32_t(src.tcBit[2 * t]); hd[1] = uint32_t(src.tcBit[2 * t] >> 32);
+            hd[2] = uint32_t(src.tcBit[2 * t + 1]); hd[3] = uint32_t(src.tcBit[2 * t + 1] >> 32);
+            const uint32_t c0 = uint32_t(__builtin_popcount(hd[0])), c1 = c0 + uint32_t(__builtin_popcount(hd[1])),
+                           c2 = c1 + uint32_t(__builtin_popcount(hd[2])), c3 = c2 + uint32_t(__builtin_popcount(hd[3]));
+            hd[4] = c0 << 8 | c1 << 16 | c2 << 24;
+            hd[5] = src.nnzOffset[t];
+            if (src.nnzOffset[t + 1] < src.nnzOffset[t] || src.nnzOffset[t + 1] - src.nnzOffset[t] != c3) {
+                uint32_t seen = first_bad.load();
+                while (uint32_t(t) < seen && !first_bad.compare_exchange_weak(seen, uint32_t(t))) {}
+            }
+        }
+    });
+    return first_bad.load();
+}
+
+// hspmm_create; with `bitmap` (16-bit element types, data == nullptr) the tiles come as the caller's bitmap arrays,
+// which are uploaded as they are, kept as the gather kernels' bitmap stream and expanded on the device for the
+// kernels that read plain tiles.  Returns kNeedsPlainTiles when the plan would need the tiles on the host
+// (windows paired through equal column lists; the caller then expands them).
+int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
+                uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
+                const uint32_t *rowIdx, const BitmapSource *bitmap)
 {
     if (!out) return fail(HSPMM_ERR_INVALID, "null plan pointer");
     *out = nullptr;
@@ -1327,7 +1371,8 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
     const uint32_t elem = dtype == HSPMM_TF32 ? 4u : 2u;
     PhaseTimer timer;
     bool canonical = true;
-    int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, data, rowIdx, &canonical);
+    int rc = validate_format(rows, cols, eff_row_windows, total_tiles, cw, rowOffset, tcA2B, bitmap ? bitmap->data : data, rowIdx,
+                             &canonical);
     if (rc) return rc;
     timer.mark("validate");
 
@@ -1360,12 +1405,33 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         if ((rc = upload(&p->d_rowOffset, rowOffset, size_t(p->W) + 1, &p->fixed_bytes))) return bail(rc);
         if ((rc = upload(&p->d_rowIdx, rowIdx, size_t(p->W), &p->fixed_bytes))) return bail(rc);
         if ((rc = upload(&p->d_a2b_raw, tcA2B, n_ids, &p->fixed_bytes))) return bail(rc);
-        {
+        if (!bitmap) {
             uint8_t *dd = nullptr;
             if ((rc = upload(&dd, static_cast<const uint8_t *>(data), size_t(total_tiles) * 8u * cw * elem,
                              &p->fixed_bytes)))
                 return bail(rc);
             p->d_data = dd;
+        } else {
+            // the caller's bitmap tiles: header from tcBit / nnzOffset, the stored elements as they are (and four
+            // more: a lane of the gather kernels reads 8 bytes from its first element), plain tiles by a kernel
+            hspmm_host::ZeroedBuffer<uint32_t> header;
+            const uint32_t bad = bitmap_header_from_caller(total_tiles, *bitmap, header);
+            if (bad != HSPMM_IDX_MAX)
+                return bail(fail(HSPMM_ERR_INVALID, "tile %u: %s", bad, "the bit count of tcBit differs from the nnzOffset span"));
+            const size_t stored = bitmap->nnzOffset[total_tiles];
+            if (stored + 4u >= (size_t(1) << 31)) return bail(kNeedsPlainTiles);      // positions are 32-bit
+            if ((rc = upload(&p->bm.d_header, header.data(), header.size(), &p->fixed_bytes))) return bail(rc);
+            uint16_t *dv = nullptr;
+            HSPMM_HIP_OR(hipMalloc(reinterpret_cast<void **>(&dv), (stored + 4u) * 2u), bail);
+            p->bm.d_vals = dv; p->bm.stored = stored; p->fixed_bytes += (stored + 4u) * 2u;
+            if (stored) HSPMM_HIP_OR(hipMemcpy(dv, bitmap->data, stored * 2u, hipMemcpyHostToDevice), bail);
+            HSPMM_HIP_OR(hipMemset(dv + stored, 0, 8), bail);
+            uint8_t *dd = nullptr;
+            HSPMM_HIP_OR(hipMalloc(reinterpret_cast<void **>(&dd), size_t(total_tiles) * 256u), bail);
+            p->d_data = dd; p->fixed_bytes += size_t(total_tiles) * 256u;
+            HSPMM_HIP_OR(hspmm::launch_expand_bitmap(p->bm.d_header, dv, dd, total_tiles, nullptr), bail);
+            HSPMM_HIP_OR(hipStreamSynchronize(nullptr), bail);
+            p->bm.from_caller = true;
         }
         timer.mark("upload format arrays");
         // padding ids -> the real id in front of them (the tile column is all zero)
@@ -1381,6 +1447,7 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         timer.mark("ids without padding");
         const StepStream st = build_units(p->W, cw, rowOffset, rowIdx, clean, p->cfg.pairing);
         timer.mark("units");
+        if (bitmap && st.G != 1) return bail(kNeedsPlainTiles);         // paired windows: their tiles are re-laid out on the host
         p->G = st.G;
         p->n_units = uint32_t(st.unitRow.size());
         p->n_paired = st.n_paired;
@@ -1403,7 +1470,17 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         // Single 16-bit windows with few stored elements per tile (graphs: 16 of 128): the gather kernels read the
         // tiles as bitmap + stored elements, 32 + 2 x 16 bytes per tile instead of 256 (power-law graph 2^20 at
         // N = 128, where the stream is read once per XCD half: 0.64 -> 0.19 GB per launch).
-        if (dtype != HSPMM_TF32 && st.G == 1 && p->cfg.gather_bitmap != 0 && total_tiles) {
+        if (bitmap) {
+            // (same rule as below, with the exact number of stored elements)
+            const size_t stored = size_t(p->bm.stored);
+            p->bm.built = total_tiles && p->cfg.gather_bitmap != 0 &&
+                          (p->cfg.gather_bitmap > 0 ||
+                           (stored * 3u < size_t(total_tiles) * 128u && size_t(total_tiles) * 256u >= (size_t(8) << 20)));
+            if (!p->bm.built) {
+                (void)hipFree(p->bm.d_header); (void)hipFree(p->bm.d_vals);
+                p->bm.d_header = nullptr; p->bm.d_vals = nullptr;
+            }
+        } else if (dtype != HSPMM_TF32 && st.G == 1 && p->cfg.gather_bitmap != 0 && total_tiles) {
             size_t stored = 0;
             if (p->cfg.gather_bitmap < 0) {
                 const uint16_t *hv = static_cast<const uint16_t *>(data);
@@ -1458,7 +1535,7 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
         }
         // (the LDS-panel stream re-tiles ascending column lists; a caller's lists in another order stay
         // with the gather and all-shapes kernels)
-        if ((p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4) && p->canonical) {
+        if (!bitmap && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4) && p->canonical) {
             int prc = HSPMM_OK;
             try { (void)build_panel_stream(p, st, rowOffset, tcA2B, data, rowIdx, p->cfg.kernel_mode >= 4, &prc); }
             catch (const std::bad_alloc &) { return bail(fail(HSPMM_ERR_ALLOC, "out of host memory")); }
@@ -1470,6 +1547,15 @@ int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint
     }
     *out = p;
     return HSPMM_OK;
+}
+
+}  // namespace
+
+int hspmm_create(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
+                 uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
+                 const uint32_t *rowIdx)
+{
+    return create_plan(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, tcA2B, data, rowIdx, nullptr);
 }
 
 namespace {
@@ -1590,6 +1676,21 @@ int hspmm_create_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32_t col
     if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16)
         return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
     if (total_tiles && (!nnzOffset || !tcBit)) return fail(HSPMM_ERR_INVALID, "null nnzOffset or tcBit");
+    // Sparse windows of 16-bit elements (graphs) never need their tiles on the host: the bitmap arrays go to the
+    // device as they are - the gather kernels read them (spmm_mfma_kernel.hpp, Fp16TileDWB) - and a kernel
+    // expands them for the kernels that read plain tiles.  Dense windows (the LDS-panel stream re-tiles them on
+    // the host), paired windows and fp32 storage are expanded here first.
+    if (dtype != HSPMM_TF32 && eff_row_windows && total_tiles && rowOffset && nnzOffset[0] == 0 &&
+        (!nnzOffset[total_tiles] || data)) {
+        int mode;
+        { std::lock_guard<std::mutex> lk(g_cfg_mutex); mode = g_cfg.kernel_mode; }
+        const double density = double(total_tiles) / (double(eff_row_windows) * double((uint64_t(cols) + 127u) / 128u));
+        if (mode < 4 && density < 1.2) {
+            const BitmapSource src{nnzOffset, tcBit, data};
+            const int rc = create_plan(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, tcA2B, nullptr, rowIdx, &src);
+            if (rc != kNeedsPlainTiles) return rc;
+        }
+    }
     const size_t tile_bytes = size_t(HSPMM_ROW_WINDOW) * (dtype == HSPMM_TF32 ? 8u * 4u : 16u * 2u);
     std::vector<uint8_t> dense;
     try { dense.resize(size_t(total_tiles) * tile_bytes); }
@@ -2019,6 +2120,7 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_panel_wide_units = p->panel.built ? p->panel.n_wide : 0u;
     info->last_kernel_family = p->last_family.load(std::memory_order_relaxed);
     info->gather_bitmap = p->bm.built ? 1u : 0u;
+    info->bitmap_from_caller = p->bm.from_caller ? 1u : 0u;
     info->panel_stream_mode = !p->panel.built ? 0u : p->panel.packed ? 2u : p->panel.tall ? 1u : 0u;
     return HSPMM_OK;
 }

@@ -96,6 +96,8 @@ struct PanelArgs {
 hipError_t launch_spmm_panel(int dtype, int G, bool split, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka,
                              int units, hipStream_t s, hipEvent_t mid);
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
+// bitmap tiles (header, stored elements: see KernelArgs::bm_header) -> plain 8 x 16 tiles of 16-bit elements
+hipError_t launch_expand_bitmap(const uint32_t *header, const void *vals, void *tiles, uint32_t n_tiles, hipStream_t s);
 // Measurement only (gather_rate_kernel in hspmm_kernels.hip): loads part_bytes (128 or 256) of row ids[i] of B for
 // every i < n_ids; parts > 1: `parts` parts of part_bytes each, dealt out by XCD, every part walking all ids.
 hipError_t launch_gather_rate(const uint32_t *ids, uint64_t n_ids, const void *B, uint32_t row_bytes, uint32_t part_bytes,

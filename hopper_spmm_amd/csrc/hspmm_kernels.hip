@@ -76,6 +76,29 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint16_t *dst, size_t n_
     }
 }
 
+// Bitmap tiles -> plain 8 x 16 tiles of 16-bit elements (plans made from the reference's BTCF_MTX arrays, reference
+// src/utils/class.h:55-67): one thread per tile element; header and stored elements as the gather kernels read
+// them (hspmm_device.h: bm_header).  The kernels that take plain tiles then run on what this wrote.
+__global__ __launch_bounds__(256) void expand_bitmap_kernel(const uint32_t *__restrict__ header,
+                                                            const uint16_t *__restrict__ vals,
+                                                            uint16_t *__restrict__ tiles, uint32_t n_tiles)
+{
+    const uint32_t t = blockIdx.x * 2u + (threadIdx.x >> 7), b = threadIdx.x & 127u;
+    if (t >= n_tiles) return;
+    const uint32_t *h = header + size_t(t) * 8u;
+    const uint32_t word = b >> 5, w = h[word], bit = b & 31u;
+    const uint32_t before = ((h[4] >> (8u * word)) & 0xFFu) + uint32_t(__builtin_popcount(w & ((1u << bit) - 1u)));
+    tiles[size_t(t) * 128u + b] = ((w >> bit) & 1u) ? vals[size_t(h[5]) + before] : uint16_t(0);
+}
+
+hipError_t launch_expand_bitmap(const uint32_t *header, const void *vals, void *tiles, uint32_t n_tiles, hipStream_t s)
+{
+    if (!n_tiles) return hipSuccess;
+    expand_bitmap_kernel<<<dim3((n_tiles + 1u) / 2u), 256, 0, s>>>(header, static_cast<const uint16_t *>(vals),
+                                                                  static_cast<uint16_t *>(tiles), n_tiles);
+    return hipGetLastError();
+}
+
 #define HSPMM_DECLARE_LAUNCH(name) \
     hipError_t name(int layout, const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, \
                     hipStream_t s, hipEvent_t mid);

@@ -225,6 +225,9 @@ typedef struct {
                                        3 LDS-staging kernels, 4 clear only (matrix without entries) */
     uint32_t gather_bitmap;         /* 1: the gather kernels read this plan's tiles as bitmap + stored elements (single 16-bit
                                      * windows with few stored elements per tile), 0: as uncompressed tiles */
+    uint32_t bitmap_from_caller;    /* 1: the plan was made from bitmap tiles (hspmm_create_bitmap / _grouped) and uploaded them as they
+                                     * came - header words from tcBit and nnzOffset, the stored elements untouched; the plain tiles
+                                     * that some kernels read were written by a kernel on the device */
     uint32_t panel_stream_mode;     /* the LDS-staging stream as built (hspmm_set_panel_stream): 0 uncompressed tiles, 1 two units
                                      * per consumer wave, 2 also tiles without their zeros; 0 when the plan has no such stream */
 } hspmm_plan_info;
@@ -354,9 +357,11 @@ int hspmm_btcf_relayout_fill(int dtype, uint32_t col_window, int transposed, uin
                              uint32_t *out_rowOffset, uint32_t *out_tcA2B, void *out_data);
 
 /* Same as hspmm_create for a matrix held as bitmap tiles (row-major bit order,
- * HSPMM_BITS_PER_TILE).  The tiles are expanded once, here, into the plan's own
- * device layout; the kernels and their results are those of hspmm_create on
- * the expanded arrays. */
+ * HSPMM_BITS_PER_TILE).  Results are those of hspmm_create on the expanded arrays, bit for bit.
+ * Sparse windows of 16-bit elements go to the device as they are: the gather kernels read the
+ * caller's tcBit words and stored elements, and a kernel writes the plain tiles other kernels read
+ * (hspmm_plan_info.bitmap_from_caller = 1).  Dense windows, windows paired through equal column
+ * lists and fp32 storage are expanded on the host first. */
 int hspmm_create_bitmap(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
                         uint32_t eff_row_windows, uint32_t total_tiles,
                         const uint32_t *rowOffset, const uint32_t *nnzOffset, const uint32_t *tcA2B,

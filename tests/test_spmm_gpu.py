@@ -290,6 +290,33 @@ def test_plans_from_bitmap_and_grouped_formats(torch_cuda, hs, oracle, dtype):
             for name, fmt in (("bitmap", bitmap), ("grouped", grouped), ("grouped-32", hs.bitmap_to_grouped(bitmap))):
                 got = gpu_spmm(torch_cuda, hs, fmt, B, N)
                 assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "%s %dx%d N=%d" % (name, rows, cols, N)
+        # Sparse windows of 16-bit elements: the bitmap arrays go to the device as they are (no expansion on the
+        # host); the kernels that read plain tiles (N = 8: the all-shapes kernel) run on what a kernel expanded
+        # there, and with the bitmap stream forced the gather kernels read the caller's own words and elements.
+        sparse = plain["total_tiles"] < 1.2 * plain["eff_row_windows"] * ((cols + 127) // 128)     # (else: LDS-staging stream, built on the host)
+        plan = hs.Plan(bitmap)
+        assert plan.info()["bitmap_from_caller"] == (1 if dtype != 1 and sparse else 0), (rows, cols)
+        plan.close()
+        if dtype != 1 and sparse:
+            os.environ["HSPMM_GATHER_BITMAP"] = "1"
+            try:
+                forced = hs.Plan(bitmap)
+            finally:
+                os.environ.pop("HSPMM_GATHER_BITMAP", None)
+            info = forced.info()
+            assert info["bitmap_from_caller"] == 1 and info["gather_bitmap"] == 1
+            for N in (64, 128):
+                B = make_b(rng, cols, N, dtype)
+                got = gpu_spmm(torch_cuda, hs, bitmap, B, N, plan=forced)
+                assert forced.info()["last_kernel_family"] == 2
+                assert np.array_equal(got.view(np.uint8), gpu_spmm(torch_cuda, hs, plain, B, N).view(np.uint8))
+            forced.close()
+            # a tile whose bits and nnzOffset span disagree is refused on this path as on the other
+            broken = dict(bitmap)
+            broken["tcBit"] = bitmap["tcBit"].copy()
+            broken["tcBit"][0] ^= np.uint64(1) << np.uint64(63)
+            with pytest.raises(hs.HspmmError):
+                hs.Plan(broken)
     # golden file through the compressed format
     A = hs.mtx_load(os.path.join(GOLD, "tiny.mtx"), dtype)
     A["dtype"] = dtype
@@ -1030,6 +1057,16 @@ def test_benchmark_configurations_full_size(torch_cuda, hs, oracle, index, which
     if index == 4:
         # N = 16 and 64: gather kernels, one workgroup per unit; N = 512: LDS-panel kernel
         assert plan.info()["last_kernel_family"] == (3 if N == 512 else 2)
+    if index == 2:
+        # the same matrix handed over as bitmap tiles: they go to the device as they are (no plain tiles on the
+        # host, an eighth of the upload) and the gather kernels read the caller's words and elements - same bits
+        bm = hs.csr_to_bitmap(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], dt)
+        from_bitmap = hs.Plan(bm)
+        info = from_bitmap.info()
+        assert info["bitmap_from_caller"] == 1 and info["gather_bitmap"] == 1
+        assert np.array_equal(gpu_spmm(torch_cuda, hs, bm, B, N, plan=from_bitmap), got)
+        from_bitmap.close()
+        del bm
     rng = np.random.default_rng(index)
     lens = np.diff(A["row_ptr"].astype(np.int64))
     sel = np.unique(np.concatenate([np.argsort(lens)[-40:], rng.choice(A["rows"], 3000, replace=False)]))
