@@ -92,6 +92,7 @@ def load_library():
     L.hspmm_create.argtypes = [C.POINTER(vp), i, u32, u32, u32, u32, vp, vp, vp, vp]
     L.hspmm_btcf_relayout_sizes.argtypes = [i, u32, u32, vp, vp, C.POINTER(u32)]
     L.hspmm_btcf_relayout_fill.argtypes = [i, u32, i, u32, vp, vp, vp, vp, vp, vp]
+    L.hspmm_partition_as_groups.argtypes = [vp, u32, C.POINTER(u32), vp, vp, vp]
     L.hspmm_create_layout.argtypes = [C.POINTER(vp), i, u32, i, u32, u32, u32, u32, vp, vp, vp, vp]
     L.hspmm_run.argtypes = [vp, vp, vp, u32, vp]
     L.hspmm_run_static.argtypes = [vp, vp, vp, u32, vp]
@@ -479,6 +480,19 @@ class Plan:
         _check(load_library().hspmm_measure_gather(self._h, C.c_void_p(dB_ptr), N, runs, C.c_void_p(stream),
                                                    C.byref(ms), C.byref(nbytes)))
         return ms.value, nbytes.value
+
+    def partition_as_groups(self):
+        """hspmm_partition_as_groups: the plan's balanced partition as the group arrays of a GBTCF_MTX
+        (groupOffset, rowIdx per group, atomic) over the tile arrays the plan was made from."""
+        L = load_library()
+        n = C.c_uint32()
+        _check(L.hspmm_partition_as_groups(self._h, 0, C.byref(n), None, None, None))
+        n = n.value
+        groupOffset = np.zeros(n + 1, np.uint32)
+        rowIdx = np.zeros(n, np.uint32)
+        atomic = np.zeros(n, np.uint8)
+        _check(L.hspmm_partition_as_groups(self._h, n, C.byref(C.c_uint32()), _p(groupOffset), _p(rowIdx), _p(atomic)))
+        return dict(total_groups=n, groupOffset=groupOffset, rowIdx=rowIdx, atomic=atomic)
 
     def info(self):
         inf = PlanInfo()

@@ -145,6 +145,7 @@ struct hspmm_plan {
                                         // [4]: every unit cut into the ranges of one workgroup (aligned)
     int aligned_group = 0;              // waves of the workgroup that walks one unit in [4]; 0: units too short for it
     std::vector<uint32_t> h_unitOffset;
+    std::vector<uint32_t> h_unitRow;       // first row of every unit | its windows less one (for hspmm_partition_as_groups)
     // LDS-panel kernels (matrices whose windows touch a large share of the columns):
     // the unit stream re-tiled panel by panel, built by hspmm_create when it pays
     struct Panel {
@@ -1507,6 +1508,7 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
         }
         timer.mark("bitmap tiles");
         p->h_unitOffset = st.unitOffset;
+        p->h_unitRow = st.unitRow;
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
         timer.mark("partition");
         {
@@ -2134,6 +2136,35 @@ int hspmm_get_partition(const hspmm_plan *p, uint32_t *ranges, uint32_t capacity
         ranges[5 * i + 2] = p->parts[0].part.ranges[i].first_window;
         ranges[5 * i + 3] = p->parts[0].part.ranges[i].head_slot; ranges[5 * i + 4] = p->parts[0].part.ranges[i].tail_slot;
     }
+    return HSPMM_OK;
+}
+
+int hspmm_partition_as_groups(const hspmm_plan *p, uint32_t capacity_groups, uint32_t *total_groups, uint32_t *groupOffset,
+                              uint32_t *groupRowIdx, uint8_t *atomic)
+{
+    if (!p || !total_groups) return fail(HSPMM_ERR_INVALID, "null argument");
+    if (p->W && p->G != 1)
+        return fail(HSPMM_ERR_UNSUPPORTED, "the plan walks pairs of windows: its ranges are not groups of the caller's tiles");
+    const std::vector<hspmm::Range> &ranges = p->parts[0].part.ranges;
+    const std::vector<uint32_t> &first_tile = p->h_unitOffset;       // single windows: a step is a tile
+    const bool write = groupOffset && groupRowIdx && atomic;
+    uint32_t n = 0;
+    for (const hspmm::Range &r : ranges) {
+        uint32_t w = r.first_window;
+        for (uint32_t t = r.tile_begin; t < r.tile_end; ++w) {
+            const uint32_t end = std::min(r.tile_end, first_tile[w + 1]);
+            if (write && n < capacity_groups) {
+                groupOffset[n] = t;
+                groupRowIdx[n] = p->h_unitRow[w] & ~7u;
+                atomic[n] = (t > first_tile[w] || end < first_tile[w + 1]) ? 1 : 0;     // the window continues in another group
+            }
+            ++n;
+            t = end;
+        }
+    }
+    if (write && n <= capacity_groups) groupOffset[n] = p->T;
+    *total_groups = n;
+    if (write && n > capacity_groups) return fail(HSPMM_ERR_INVALID, "%u groups, room for %u", n, capacity_groups);
     return HSPMM_OK;
 }
 

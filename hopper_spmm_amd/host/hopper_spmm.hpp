@@ -233,6 +233,40 @@ inline void BTCF2GBTCF(BTCF_MTX &btcf, GBTCF_MTX &gbtcf)
     gbtcf.nnzOffset = btcf.nnzOffset; gbtcf.tcA2B = btcf.tcA2B; gbtcf.tcBit = btcf.tcBit; gbtcf.data = btcf.data;
 }
 
+// The groups of the library's own balanced partition instead of the reference's
+// fixed group length (src/utils/convert.h:242-258): a plan is made from the bitmap
+// tiles, every piece of a window that one wave of its kernels walks becomes a group
+// (GBTCF_MTX, src/utils/class.h:93-108), windows cut across waves are marked atomic.
+// Needs the GPU the plan is made for; the result is a matrix like BTCF2GBTCF's.
+inline void BTCF2GBTCF_balanced(BTCF_MTX &btcf, GBTCF_MTX &gbtcf)
+{
+#ifdef SPARSE_A_TRANSPOSE
+    hspmm_cpp::die("BTCF2GBTCF_balanced with -DSPARSE_A_TRANSPOSE");
+#endif
+    const uint32_t tiles = btcf.rowOffset.empty() ? 0u : btcf.rowOffset.back();
+    hspmm_plan *plan = nullptr;
+    if (hspmm_create_bitmap(&plan, HSPMM_BUILD_DTYPE, btcf.rows, btcf.cols, btcf.eff_row_windows, tiles, btcf.rowOffset.data(),
+                            btcf.nnzOffset.data(), btcf.tcA2B.data(), btcf.tcBit.data(), btcf.data.data(),
+                            btcf.rowIdx.data()) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_create_bitmap");
+    uint32_t groups = 0;
+    if (hspmm_partition_as_groups(plan, 0, &groups, nullptr, nullptr, nullptr) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_partition_as_groups");
+    gbtcf.groupOffset.assign(size_t(groups) + 1, 0);
+    gbtcf.rowIdx.assign(groups, 0);
+    gbtcf.atomic.assign(groups, 0);
+    if (hspmm_partition_as_groups(plan, groups, &groups, gbtcf.groupOffset.data(), gbtcf.rowIdx.data(),
+                                  gbtcf.atomic.data()) != HSPMM_OK)
+        hspmm_cpp::die("hspmm_partition_as_groups");
+    hspmm_destroy(plan);
+    std::printf("total groups : %u\n", groups);
+    gbtcf.total_groups = groups;
+    gbtcf.rows = btcf.rows; gbtcf.cols = btcf.cols; gbtcf.nnzs = btcf.nnzs;
+    gbtcf.total_row_windows = groups + 1;
+    gbtcf.eff_row_windows = groups + 1;
+    gbtcf.nnzOffset = btcf.nnzOffset; gbtcf.tcA2B = btcf.tcA2B; gbtcf.tcBit = btcf.tcBit; gbtcf.data = btcf.data;
+}
+
 // The checks of the reference's validateBTCF2GBTCFConversion (src/utils/convert.h:283-402)
 // with the group count of every window derived from the converter's own group
 // length; the reference's check still assumes a fixed length of 4 tiles

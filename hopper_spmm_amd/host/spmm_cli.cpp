@@ -1,5 +1,5 @@
 // Command-line driver with the reference's arguments (reference src/fp16.cu:283-319):
-//   fp16_test <matrix_file> <feature_dim> [--seed S] [--verify] [--format tiles|bitmap|grouped]
+//   fp16_test <matrix_file> <feature_dim> [--seed S] [--verify] [--format tiles|bitmap|grouped|balanced]
 // built with -DUSE_FP16; the same source with -DUSE_TF32 / -DUSE_BF16 gives
 // tf32_test / bf16_test.
 // B is filled with rand() / RAND_MAX as in the reference (src/fp16.cu:303-309);
@@ -8,7 +8,8 @@
 // implementation on the GPU, and compares the two results element by element
 // (1e-2 relative, 1e-3 for tf32_test, plus a term in sum |a||b| for sums that cancel).
 // --format hands the matrix to the operator as uncompressed tiles (the reference's
-// only path, the default), as bitmap tiles (CSR2BTCF) or as groups (BTCF2GBTCF).
+// only path, the default), as bitmap tiles (CSR2BTCF), as groups of the reference's
+// fixed length (BTCF2GBTCF) or as the groups of the library's balanced partition.
 #include <cstring>
 #include <string>
 
@@ -17,7 +18,7 @@
 int main(int argc, char *argv[])
 {
     if (argc < 3) {
-        std::printf("Usage: %s <matrix_file> <feature_dim> [--seed S] [--verify] [--format tiles|bitmap|grouped]\n",
+        std::printf("Usage: %s <matrix_file> <feature_dim> [--seed S] [--verify] [--format tiles|bitmap|grouped|balanced]\n",
                     argv[0]);
         return 1;
     }
@@ -32,7 +33,7 @@ int main(int argc, char *argv[])
         else { std::printf("unknown argument %s\n", argv[i]); return 1; }
     }
     if (fd <= 0) { std::printf("feature_dim must be positive\n"); return 1; }
-    if (format != "tiles" && format != "bitmap" && format != "grouped") {
+    if (format != "tiles" && format != "bitmap" && format != "grouped" && format != "balanced") {
         std::printf("unknown format %s\n", format.c_str());
         return 1;
     }
@@ -67,8 +68,11 @@ int main(int argc, char *argv[])
         if (format == "bitmap") perf = SPMM(bitmap, dense_b, dense_c);
         else {
             GBTCF_MTX grouped;
-            BTCF2GBTCF(bitmap, grouped);
-            if (!validateBTCF2GBTCFConversion(bitmap, grouped)) { std::printf("grouping failed its checks\n"); return 2; }
+            if (format == "balanced") BTCF2GBTCF_balanced(bitmap, grouped);
+            else {
+                BTCF2GBTCF(bitmap, grouped);
+                if (!validateBTCF2GBTCFConversion(bitmap, grouped)) { std::printf("grouping failed its checks\n"); return 2; }
+            }
             perf = SPMM(grouped, dense_b, dense_c);
         }
     }

@@ -241,6 +241,16 @@ int hspmm_get_plan_info(const hspmm_plan *plan, hspmm_plan_info *info);
  * tail_slot} (slot 0xFFFFFFFF = none). */
 int hspmm_get_partition(const hspmm_plan *plan, uint32_t *ranges, uint32_t capacity_ranges);
 
+/* The plan's own balanced partition in the form of the reference's grouped format (GBTCF_MTX, reference
+ * src/utils/class.h:93-108; BTCF2GBTCF, src/utils/convert.h:232-276, cuts every window into groups of a fixed
+ * length instead): one group per piece of a window that one wave walks, groupOffset[g] its first tile in the
+ * caller's tile arrays (groupOffset[total] = total_tiles), groupRowIdx[g] the window's first row, atomic[g] = 1
+ * where the window continues in another group.  Together with the tile arrays the plan was made from this is a
+ * GBTCF_MTX that hspmm_create_grouped takes back.  First call with the arrays NULL for *total_groups.  Plans
+ * that walk pairs of windows have no such form (HSPMM_ERR_UNSUPPORTED).  Host only. */
+int hspmm_partition_as_groups(const hspmm_plan *plan, uint32_t capacity_groups, uint32_t *total_groups,
+                              uint32_t *groupOffset, uint32_t *groupRowIdx, uint8_t *atomic);
+
 /* No reference counterpart: the partition hspmm_create would build for a
  * rowOffset array and a wanted number of ranges, computed on the host alone
  * (no device needed).  ranges as in hspmm_get_partition; any output may be NULL. */

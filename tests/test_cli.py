@@ -32,7 +32,8 @@ def test_cli_fails_loudly_without_a_device(hs):
     r = run(hs, "fp16_test", os.path.join(GOLD, "tiny.mtx"), "64")
     assert r.returncode == 1 and "hspmm_create" in r.stderr
     assert "tiles (8 x 16): 2" in r.stdout                           # the format statistics of src/fp16.cu:295-301
-    for fmt, entry in (("bitmap", "hspmm_create_bitmap"), ("grouped", "hspmm_create_grouped")):
+    for fmt, entry in (("bitmap", "hspmm_create_bitmap"), ("grouped", "hspmm_create_grouped"),
+                       ("balanced", "hspmm_create_bitmap")):
         r = run(hs, "fp16_test", os.path.join(GOLD, "tiny.mtx"), "64", "--format", fmt)
         assert r.returncode == 1 and entry in r.stderr
         assert "2 tiles, 9 stored entries" in r.stdout
@@ -53,6 +54,7 @@ def test_cli_end_to_end_with_verification(hs, tmp_path):
     for name, n, fmt in (("fp16_test", "128", "tiles"), ("fp16_test", "7", "tiles"), ("tf32_test", "64", "tiles"),
                          ("bf16_test", "128", "tiles"), ("bf16_test", "5", "tiles"), ("fp16_test", "64", "bitmap"),
                          ("tf32_test", "32", "grouped"), ("bf16_test", "64", "grouped"),
+                         ("fp16_test", "64", "balanced"), ("tf32_test", "16", "balanced"),
                          # tiles written column by column (-DSPARSE_A_TRANSPOSE)
                          ("fp16_transposed_test", "128", "tiles"), ("fp16_transposed_test", "40", "bitmap")):
         r = run(hs, name, str(p), n, "--seed", "42", "--verify", "--format", fmt)

@@ -365,6 +365,48 @@ def test_plans_from_transposed_tiles_and_from_tiles_four_columns_wide(torch_cuda
             hs.Plan(bad)
 
 
+def test_partition_exported_as_groups_round_trips(torch_cuda, hs, oracle):
+    """hspmm_partition_as_groups writes the plan's balanced partition in the reference's grouped form
+    (GBTCF_MTX, src/utils/class.h:93-108): every group is the piece of one window that one wave walks, windows
+    cut across waves are marked atomic, and the groups together with the tile arrays are a matrix that
+    hspmm_create_grouped takes back - same product, bit for bit."""
+    rng = np.random.default_rng(77)
+    A = random_csr(rng, 300, 3000, 0.004, 0, 0.2, (5, 100, 101, 299))
+    plain = convert(hs, A)
+    bitmap = hs.csr_to_bitmap(300, 3000, A["row_ptr"], A["col_idx"], A["values"], 0)
+    hs.configure(producer_warp_group_num=16)            # many short ranges: the heavy windows are cut
+    try:
+        plan = hs.Plan(plain)
+    finally:
+        hs.configure()
+    assert plan.info()["n_split_windows"] > 0
+    g = plan.partition_as_groups()
+    ranges = plan.partition()
+    go, T = g["groupOffset"].astype(np.int64), plain["total_tiles"]
+    assert go[0] == 0 and go[-1] == T and (np.diff(go) > 0).all()
+    assert set(plain["rowOffset"].tolist()) <= set(go.tolist())                     # no group straddles a window
+    assert set(ranges[:, 0].tolist()) <= set(go.tolist())                           # nor a range
+    window_of_group = np.searchsorted(plain["rowOffset"], go[:-1], side="right") - 1
+    assert np.array_equal(g["rowIdx"], plain["rowIdx"][window_of_group])
+    groups_per_window = np.bincount(window_of_group, minlength=plain["eff_row_windows"])
+    assert np.array_equal(g["atomic"].astype(bool), groups_per_window[window_of_group] > 1)
+    assert g["atomic"].sum() >= 2 * plan.info()["n_split_windows"]
+    plan.close()
+    grouped = {k: bitmap[k] for k in ("rows", "cols", "nnzs", "dtype", "cw", "nnzOffset", "tcA2B", "tcBit", "data")}
+    grouped.update(g, tgl=0, total_row_windows=g["total_groups"] + 1, eff_row_windows=g["total_groups"] + 1)
+    for N in (8, 64):
+        B = make_b(rng, 3000, N, 0)
+        want = gpu_spmm(torch_cuda, hs, plain, B, N)
+        assert np.array_equal(gpu_spmm(torch_cuda, hs, grouped, B, N), want)
+    # plans that walk pairs of windows have no such form
+    P = random_csr(rng, 64, 64, 1.0, 0)                                                 # every window has the same columns
+    pairs = hs.Plan(convert(hs, P))
+    if pairs.info()["n_paired_units"]:
+        with pytest.raises(hs.HspmmError):
+            pairs.partition_as_groups()
+    pairs.close()
+
+
 PANEL_SHAPES = [
     # rows, cols, density, empty-row probability, heavy rows
     (8, 16, 1.0, 0.0, ()),                      # one window, one panel
