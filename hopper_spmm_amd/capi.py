@@ -67,7 +67,8 @@ class PlanInfo(C.Structure):
                 ("device_bytes", C.c_uint64), ("n_panels", C.c_uint32), ("n_panel_steps", C.c_uint32),
                 ("n_panel_units", C.c_uint32), ("n_panel_paired_units", C.c_uint32),
                 ("n_panel_wide_units", C.c_uint32), ("last_kernel_family", C.c_uint32),
-                ("gather_bitmap", C.c_uint32), ("bitmap_from_caller", C.c_uint32), ("panel_stream_mode", C.c_uint32)]
+                ("gather_bitmap", C.c_uint32), ("bitmap_from_caller", C.c_uint32), ("panel_stream_mode", C.c_uint32),
+                ("group_cuts_kept", C.c_uint32)]
 
 
 def load_library():
@@ -108,12 +109,15 @@ def load_library():
     L.hspmm_set_kernel_mode.argtypes = [i]
     L.hspmm_set_window_pairing.argtypes = [i]
     L.hspmm_set_panel_stream.argtypes = [i]
+    L.hspmm_set_group_cuts.argtypes = [i]
     L.hspmm_get_plan_info.argtypes = [vp, C.POINTER(PlanInfo)]
     L.hspmm_get_partition.argtypes = [vp, vp, u32]
     L.hspmm_partition_preview.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
     L.hspmm_partition_preview_grouped.argtypes = [u32, vp, u32, u32, vp, u32, C.POINTER(u32), C.POINTER(u32),
                                                   C.POINTER(u32)]
     L.hspmm_partition_preview_aligned.argtypes = [u32, vp, u32, vp, u32, C.POINTER(u32)]
+    L.hspmm_partition_preview_group_cuts.argtypes = [u32, vp, u32, u32, vp, vp, u32, C.POINTER(u32), C.POINTER(u32),
+                                                     C.POINTER(u32)]
     L.hspmm_panel_units_preview.argtypes = [i, u32, u32, u32, u32, vp, vp, vp, vp, u32, C.POINTER(u32), vp, vp, vp,
                                             C.POINTER(u32), u32, vp, vp]
     L.hspmm_mtx_load.argtypes = [C.c_char_p, i, C.POINTER(_Csr)]
@@ -188,6 +192,12 @@ def get_kernel_mode():
 def set_window_pairing(mode):
     """0 = automatic, 1 = never, 2 = whenever two adjacent windows share a column list."""
     _check(load_library().hspmm_set_window_pairing(mode))
+
+
+def set_group_cuts(mode):
+    """1: plans made from groups (GBTCF_MTX) cut a window only where the caller's groups end; 0 (default): where
+    the plan's cost model puts the cuts.  Read by the next plan creation."""
+    _check(load_library().hspmm_set_group_cuts(mode))
 
 
 def set_panel_stream(mode):
@@ -355,15 +365,23 @@ def partition_preview_aligned(rowOffset, group):
     return ranges
 
 
-def partition_preview(rowOffset, target_ranges, group=1):
+def partition_preview(rowOffset, target_ranges, group=1, group_offset=None):
     """The work partition hspmm_create would build (host only).  group > 1: the partition
     for workgroups whose waves add the partial sums of one window among themselves
-    (ranges then have a sixth word, "combine")."""
+    (ranges then have a sixth word, "combine").  group_offset: the ends of the caller's groups
+    (GBTCF_MTX.groupOffset); windows are then cut only there (set_group_cuts(1))."""
     L = load_library()
     rowOffset = np.ascontiguousarray(rowOffset, np.uint32)
     W = rowOffset.size - 1
     n, ns, nslots = C.c_uint32(), C.c_uint32(), C.c_uint32()
-    if group == 1:
+    if group_offset is not None:
+        go = np.ascontiguousarray(group_offset, np.uint32)
+        _check(L.hspmm_partition_preview_group_cuts(W, _p(rowOffset), target_ranges, go.size - 1, _p(go), None, 0,
+                                                    C.byref(n), C.byref(ns), C.byref(nslots)))
+        ranges = np.zeros((n.value, 5), np.uint32)
+        _check(L.hspmm_partition_preview_group_cuts(W, _p(rowOffset), target_ranges, go.size - 1, _p(go), _p(ranges),
+                                                    n.value, None, None, None))
+    elif group == 1:
         _check(L.hspmm_partition_preview(W, _p(rowOffset), target_ranges, None, 0, C.byref(n), C.byref(ns),
                                          C.byref(nslots)))
         ranges = np.zeros((n.value, 5), np.uint32)

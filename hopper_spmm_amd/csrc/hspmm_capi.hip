@@ -70,6 +70,7 @@ struct Config {
     int fused_fixup = -1;               // 1: the last wave of a cut unit adds its partial sums; 0: second kernel;
                                         // -1: the former in the LDS-panel kernels, and in the gather kernels where few units are cut
     int pairing = 0;                    // 0 automatic, 1 never, 2 whenever two windows share a column list
+    int group_cuts = 0;                 // 1: plans of hspmm_create_grouped cut a window only where the caller's groups end
     // Tuning overrides from the environment (HSPMM_*), read once by hspmm_create: a plan's behaviour does
     // not change with the environment afterwards and the launch path reads no variable.
     double window_cost = 1.5, slack = 0.35, whole_window_margin = 32.0;     // cost model of partition.hpp
@@ -146,6 +147,8 @@ struct hspmm_plan {
     int aligned_group = 0;              // waves of the workgroup that walks one unit in [4]; 0: units too short for it
     std::vector<uint32_t> h_unitOffset;
     std::vector<uint32_t> h_unitRow;       // first row of every unit | its windows less one (for hspmm_partition_as_groups)
+    std::vector<uint32_t> caller_cuts;     // hspmm_create_grouped with hspmm_set_group_cuts(1): the ends of the caller's groups,
+                                           // the only places where the gather kernels' partition cuts a window
     // LDS-panel kernels (matrices whose windows touch a large share of the columns):
     // the unit stream re-tiled panel by panel, built by hspmm_create when it pays
     struct Panel {
@@ -293,7 +296,8 @@ int build_and_upload_partition(hspmm_plan *p, int level, uint32_t group = 1, boo
     const uint32_t floor_ranges = uint32_t(p->compute_units) * 4u;       // at least one range per SIMD
     if (target < floor_ranges) target = std::min<uint32_t>(floor_ranges, uint32_t(choose_ranges(p)));
     dp.part = aligned ? hspmm::build_aligned_partition(p->n_units, p->h_unitOffset.data(), group)
-                      : hspmm::build_partition(p->n_units, p->h_unitOffset.data(), target, window_cost, slack, margin, group);
+                      : hspmm::build_partition(p->n_units, p->h_unitOffset.data(), target, window_cost, slack, margin, group,
+                                               p->caller_cuts.empty() ? nullptr : &p->caller_cuts);
     const auto &part = dp.part;
     std::vector<uint32_t> rw(part.ranges.size() * hspmm::kRangeWords, 0u);
     for (size_t i = 0; i < part.ranges.size(); ++i) {
@@ -1212,6 +1216,14 @@ int hspmm_set_window_pairing(int mode)
     return HSPMM_OK;
 }
 
+int hspmm_set_group_cuts(int mode)
+{
+    if (mode < 0 || mode > 1) return fail(HSPMM_ERR_INVALID, "group cuts mode %d outside 0..1", mode);
+    std::lock_guard<std::mutex> lk(g_cfg_mutex);
+    g_cfg.group_cuts = mode;
+    return HSPMM_OK;
+}
+
 int hspmm_set_panel_stream(int mode)
 {
     if (mode < 0 || mode > 2) return fail(HSPMM_ERR_INVALID, "panel stream mode %d outside 0..2", mode);
@@ -1223,7 +1235,8 @@ int hspmm_set_panel_stream(int mode)
 
 static int partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
                              uint32_t group, uint32_t words, uint32_t *ranges, uint32_t capacity_ranges,
-                             uint32_t *n_ranges, uint32_t *n_split_windows, uint32_t *n_partial_slots)
+                             uint32_t *n_ranges, uint32_t *n_split_windows, uint32_t *n_partial_slots,
+                             const std::vector<uint32_t> *allowed_cuts = nullptr)
 {
     if (eff_row_windows && !rowOffset) return fail(HSPMM_ERR_INVALID, "null rowOffset");
     if (group < 1 || group > uint32_t(hspmm::kMaxWavesPerGroup))
@@ -1231,7 +1244,8 @@ static int partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset
     for (uint32_t w = 0; w < eff_row_windows; ++w)
         if (rowOffset[w + 1] <= rowOffset[w] || rowOffset[0] != 0)
             return fail(HSPMM_ERR_INVALID, "rowOffset must start at 0 and increase strictly");
-    const hspmm::Partition part = hspmm::build_partition(eff_row_windows, rowOffset, target_ranges, 1.5, 0.35, 32.0, group);
+    const hspmm::Partition part =
+        hspmm::build_partition(eff_row_windows, rowOffset, target_ranges, 1.5, 0.35, 32.0, group, allowed_cuts);
     if (n_ranges) *n_ranges = uint32_t(part.ranges.size());
     if (n_split_windows) *n_split_windows = uint32_t(part.split.size());
     if (n_partial_slots) *n_partial_slots = part.n_slots;
@@ -1262,6 +1276,28 @@ int hspmm_partition_preview_grouped(uint32_t eff_row_windows, const uint32_t *ro
 {
     return partition_preview(eff_row_windows, rowOffset, target_ranges, group, 6, ranges, capacity_ranges, n_ranges,
                              n_split_windows, n_partial_slots);
+}
+
+int hspmm_partition_preview_group_cuts(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
+                                       uint32_t total_groups, const uint32_t *groupOffset, uint32_t *ranges,
+                                       uint32_t capacity_ranges, uint32_t *n_ranges, uint32_t *n_split_windows,
+                                       uint32_t *n_partial_slots)
+{
+    if (!groupOffset) return fail(HSPMM_ERR_INVALID, "null groupOffset");
+    if (eff_row_windows && !rowOffset) return fail(HSPMM_ERR_INVALID, "null rowOffset");
+    // every window boundary must be the end of a group
+    uint32_t g = 0;
+    for (uint32_t w = 0; w <= eff_row_windows; ++w) {
+        while (g < total_groups && groupOffset[g] < rowOffset[w]) {
+            if (groupOffset[g + 1] <= groupOffset[g]) return fail(HSPMM_ERR_INVALID, "groupOffset does not increase at group %u", g);
+            ++g;
+        }
+        if (g > total_groups || groupOffset[g] != rowOffset[w])
+            return fail(HSPMM_ERR_INVALID, "window boundary %u (tile %u) is not the end of a group", w, rowOffset[w]);
+    }
+    const std::vector<uint32_t> cuts(groupOffset, groupOffset + size_t(total_groups) + 1u);
+    return partition_preview(eff_row_windows, rowOffset, target_ranges, 1, 5, ranges, capacity_ranges, n_ranges,
+                             n_split_windows, n_partial_slots, &cuts);
 }
 
 int hspmm_partition_preview_aligned(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t group,
@@ -1330,6 +1366,8 @@ namespace {
 
 // The caller's bitmap tiles (16-bit element types, HSPMM_BITS_PER_TILE words): reference BTCF_MTX, src/utils/class.h:55-67.
 struct BitmapSource { const uint32_t *nnzOffset; const uint64_t *tcBit; const void *data; };
+// The ends of the caller's groups (groupOffset of the reference's GBTCF_MTX, src/utils/class.h:93-108), n + 1 of them.
+struct GroupCuts { const uint32_t *offsets; uint32_t n_groups; };
 constexpr int kNeedsPlainTiles = -1000;     // create_plan with a BitmapSource: this matrix needs the tiles on the host
 
 // Header of the gather kernels' bitmap stream straight from the caller's arrays; returns the first tile whose bit
@@ -1362,7 +1400,7 @@ uint32_t bitmap_header_from_caller(uint32_t T, const BitmapSource &src, hspmm_ho
 // (windows paired through equal column lists; the caller then expands them).
 int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
                 uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *tcA2B, const void *data,
-                const uint32_t *rowIdx, const BitmapSource *bitmap)
+                const uint32_t *rowIdx, const BitmapSource *bitmap, const GroupCuts *cuts = nullptr)
 {
     if (!out) return fail(HSPMM_ERR_INVALID, "null plan pointer");
     *out = nullptr;
@@ -1509,6 +1547,8 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
         timer.mark("bitmap tiles");
         p->h_unitOffset = st.unitOffset;
         p->h_unitRow = st.unitRow;
+        // single windows walked tile by tile: the caller's tile numbers are the stream's, its cuts can be kept
+        if (cuts && p->cfg.group_cuts && st.G == 1) p->caller_cuts.assign(cuts->offsets, cuts->offsets + size_t(cuts->n_groups) + 1u);
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
         timer.mark("partition");
         {
@@ -1534,6 +1574,7 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
                 small_group = p->cfg.aligned_small;
             }
             if (small_group && shortest >= 2u * uint32_t(small_group)) p->aligned_group = small_group;
+            if (!p->caller_cuts.empty()) p->aligned_group = 0;       // (those partitions cut every unit into equal parts)
         }
         // (the LDS-panel stream re-tiles ascending column lists; a caller's lists in another order stay
         // with the gather and all-shapes kernels)
@@ -1669,9 +1710,10 @@ int hspmm_create_layout(hspmm_plan **out, int dtype, uint32_t col_window, int tr
     } catch (const std::bad_alloc &) { return fail(HSPMM_ERR_ALLOC, "out of host memory"); }
 }
 
-int hspmm_create_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
-                        uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *nnzOffset,
-                        const uint32_t *tcA2B, const uint64_t *tcBit, const void *data, const uint32_t *rowIdx)
+static int create_from_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
+                              uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *nnzOffset,
+                              const uint32_t *tcA2B, const uint64_t *tcBit, const void *data, const uint32_t *rowIdx,
+                              const GroupCuts *cuts)
 {
     if (!out) return fail(HSPMM_ERR_INVALID, "null plan pointer");
     *out = nullptr;
@@ -1689,7 +1731,8 @@ int hspmm_create_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32_t col
         const double density = double(total_tiles) / (double(eff_row_windows) * double((uint64_t(cols) + 127u) / 128u));
         if (mode < 4 && density < 1.2) {
             const BitmapSource src{nnzOffset, tcBit, data};
-            const int rc = create_plan(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, tcA2B, nullptr, rowIdx, &src);
+            const int rc = create_plan(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, tcA2B, nullptr, rowIdx, &src,
+                                       cuts);
             if (rc != kNeedsPlainTiles) return rc;
         }
     }
@@ -1700,7 +1743,15 @@ int hspmm_create_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32_t col
     // hspmm_bitmap_expand leaves its own message behind on failure
     const int rc = hspmm_bitmap_expand(dtype, total_tiles, nnzOffset, tcBit, data, dense.data());
     if (rc) return rc;
-    return hspmm_create(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, tcA2B, dense.data(), rowIdx);
+    return create_plan(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, tcA2B, dense.data(), rowIdx, nullptr, cuts);
+}
+
+int hspmm_create_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t eff_row_windows,
+                        uint32_t total_tiles, const uint32_t *rowOffset, const uint32_t *nnzOffset,
+                        const uint32_t *tcA2B, const uint64_t *tcBit, const void *data, const uint32_t *rowIdx)
+{
+    return create_from_bitmap(out, dtype, rows, cols, eff_row_windows, total_tiles, rowOffset, nnzOffset, tcA2B, tcBit, data,
+                              rowIdx, nullptr);
 }
 
 int hspmm_create_grouped(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint32_t total_groups,
@@ -1729,8 +1780,9 @@ int hspmm_create_grouped(hspmm_plan **out, int dtype, uint32_t rows, uint32_t co
     // groups of one window that are not adjacent show up as a row index that does
     // not increase, which the checks of hspmm_create reject
     const uint32_t W = uint32_t(rowIdx.size());
-    return hspmm_create_bitmap(out, dtype, rows, cols, W, rowOffset.back(), rowOffset.data(), nnzOffset, tcA2B, tcBit,
-                               data, rowIdx.data());
+    const GroupCuts cuts{groupOffset, total_groups};
+    return create_from_bitmap(out, dtype, rows, cols, W, rowOffset.back(), rowOffset.data(), nnzOffset, tcA2B, tcBit, data,
+                              rowIdx.data(), total_groups && groupOffset[0] == 0 ? &cuts : nullptr);
 }
 
 void hspmm_destroy(hspmm_plan *p)
@@ -2123,6 +2175,7 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->last_kernel_family = p->last_family.load(std::memory_order_relaxed);
     info->gather_bitmap = p->bm.built ? 1u : 0u;
     info->bitmap_from_caller = p->bm.from_caller ? 1u : 0u;
+    info->group_cuts_kept = p->caller_cuts.empty() ? 0u : 1u;
     info->panel_stream_mode = !p->panel.built ? 0u : p->panel.packed ? 2u : p->panel.tall ? 1u : 0u;
     return HSPMM_OK;
 }

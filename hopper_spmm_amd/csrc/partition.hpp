@@ -52,9 +52,12 @@ struct Partition {
 // group: ranges group * k .. group * k + group - 1 are walked by the waves of one workgroup.  Where all
 // of them lie inside one window, the workgroup adds their partial sums itself (in range order) and
 // the group takes one slot, that of its first range, instead of one per range.
+// allowed_cuts (optional; ascending, holds every window boundary): a cut inside a window moves to the
+// nearest of these positions - the ends of the caller's groups (reference GBTCF_MTX,
+// src/utils/class.h:93-108), so that a window is cut only where the caller cut it.
 inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t target_ranges,
                                  double window_cost = 1.5, double slack = 0.35, double whole_window_margin = 32.0,
-                                 uint32_t group = 1)
+                                 uint32_t group = 1, const std::vector<uint32_t> *allowed_cuts = nullptr)
 {
     Partition P;
     if (W == 0) return P;
@@ -87,6 +90,14 @@ inline Partition build_partition(uint32_t W, const uint32_t *rowOffset, uint32_t
         if (tau > we) tau = we;
         if (double(tau - ws) <= snap) tau = ws;
         else if (double(we - tau) <= snap) tau = we;
+        if (allowed_cuts && tau > ws && tau < we) {
+            auto hi = std::lower_bound(allowed_cuts->begin(), allowed_cuts->end(), tau);     // <= we: boundaries are in the list
+            const uint32_t above = hi == allowed_cuts->end() ? we : *hi;
+            const uint32_t below = hi == allowed_cuts->begin() ? ws : *(hi - 1);
+            tau = above - tau < tau - below ? above : below;
+            if (tau < ws) tau = ws;
+            if (tau > we) tau = we;
+        }
         if (tau > cuts.back() && tau < T) cuts.push_back(tau);
     }
     cuts.push_back(T);

@@ -188,6 +188,20 @@ int hspmm_set_window_pairing(int mode);
  * MFMAs of a step, not by their traffic; hence the default. */
 int hspmm_set_panel_stream(int mode);
 
+/* No reference counterpart (the reference defines the grouped format, src/utils/class.h:93-108
+ * and src/utils/convert.h:232-276, but no kernel that walks it): process-wide like
+ * hspmm_configure, read by the next hspmm_create_grouped.  mode 0 (default): consecutive groups
+ * with one row index are one window again and the plan cuts heavy windows where its own cost
+ * model puts the cuts.  mode 1: the plan's waves walk whole groups - a window given as several
+ * groups (atomic = 1) is cut only where one of its groups ends, a window given as one group is
+ * never cut; partial sums of a cut window are added in group order, not with atomics.  Kept by
+ * plans whose units are the caller's single windows walked by the gather kernels
+ * (hspmm_plan_info.group_cuts_kept = 1); plans that merge windows with one column list, the
+ * LDS-staging kernels (they walk a re-tiled stream) and the all-shapes kernel (one wave per
+ * window, nothing cut) have no use for the cuts.  The product is the same up to the order of the
+ * fp32 additions of a cut window. */
+int hspmm_set_group_cuts(int mode);
+
 /* No reference counterpart; host only (no device needed).  The grouping that the
  * LDS-staging kernels built on the 16-bit MFMA apply to their copy of the
  * matrix, for tests and for sizing: adjacent windows are merged into units of up
@@ -230,6 +244,7 @@ typedef struct {
                                      * that some kernels read were written by a kernel on the device */
     uint32_t panel_stream_mode;     /* the LDS-staging stream as built (hspmm_set_panel_stream): 0 uncompressed tiles, 1 two units
                                      * per consumer wave, 2 also tiles without their zeros; 0 when the plan has no such stream */
+    uint32_t group_cuts_kept;       /* 1: the plan cuts a window only where the caller's groups end (hspmm_set_group_cuts) */
 } hspmm_plan_info;
 
 /* No reference counterpart (the reference prints its statistics from main,
@@ -267,6 +282,16 @@ int hspmm_partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset,
 int hspmm_partition_preview_grouped(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
                                     uint32_t group, uint32_t *ranges, uint32_t capacity_ranges,
                                     uint32_t *n_ranges, uint32_t *n_split_windows, uint32_t *n_partial_slots);
+
+/* No reference counterpart; host only.  The partition of a plan that keeps the caller's
+ * group cuts (hspmm_set_group_cuts(1), hspmm_create_grouped): as hspmm_partition_preview,
+ * but a cut inside a window moves to the nearest end of one of the caller's groups
+ * (groupOffset of the reference's GBTCF_MTX, src/utils/class.h:93-108; total_groups + 1
+ * entries, every window boundary among them). */
+int hspmm_partition_preview_group_cuts(uint32_t eff_row_windows, const uint32_t *rowOffset, uint32_t target_ranges,
+                                       uint32_t total_groups, const uint32_t *groupOffset, uint32_t *ranges,
+                                       uint32_t capacity_ranges, uint32_t *n_ranges, uint32_t *n_split_windows,
+                                       uint32_t *n_partial_slots);
 
 /* No reference counterpart; host only.  The partition used where every unit is
  * long (the balanced partition would cut each of them 2.5 ways or more, and one

@@ -29,9 +29,9 @@ def simulate(ranges, ro):
     return partial, direct
 
 
-def check(hs, ro, target):
+def check(hs, ro, target, group_offset=None):
     ro = np.asarray(ro, np.uint32)
-    p = hs.partition_preview(ro, target)
+    p = hs.partition_preview(ro, target, group_offset=group_offset)
     r = p["ranges"]
     W, T = ro.size - 1, int(ro[-1])
     assert r[0, 0] == 0 and r[-1, 1] == T
@@ -66,6 +66,37 @@ def test_partition_random(hs):
         tiles = np.maximum(1, rng.pareto(1.2, W) * rng.integers(1, 8)).astype(np.int64)
         ro = np.concatenate([[0], np.cumsum(tiles)])
         check(hs, ro, int(rng.integers(1, 300)))
+
+
+def test_partition_that_keeps_the_cuts_of_the_callers_groups(hs):
+    """hspmm_set_group_cuts(1): a window is cut only where one of the caller's groups ends (groupOffset of
+    GBTCF_MTX, reference src/utils/convert.h:245-259); windows given as one group are never cut."""
+    rng = np.random.default_rng(3)
+    for trial in range(40):
+        W = int(rng.integers(1, 200))
+        tiles = np.maximum(1, rng.pareto(1.0, W) * rng.integers(1, 30)).astype(np.int64)
+        ro = np.concatenate([[0], np.cumsum(tiles)]).astype(np.uint32)
+        tgl = int(rng.integers(1, 40))
+        # the reference's grouping: every window in pieces of tgl tiles
+        go = np.unique(np.concatenate([np.arange(a, b, tgl) for a, b in zip(ro[:-1], ro[1:])] + [ro[-1:]]))
+        target = int(rng.integers(1, 300))
+        p = check(hs, ro, target, group_offset=go)
+        starts = p["ranges"][:, 0]
+        assert np.isin(starts, go).all()
+        # no further from the balanced cut than half a group: ranges stay balanced to within one group
+        free = hs.partition_preview(ro, target)["ranges"]
+        ln = (p["ranges"][:, 1] - p["ranges"][:, 0]).astype(np.int64)
+        assert ln.max() <= (free[:, 1] - free[:, 0]).max() + tgl
+    # groups = windows: nothing is cut, however heavy the window
+    ro = np.array([0, 1000, 1001, 1002], np.uint32)
+    p = check(hs, ro, 64, group_offset=ro)
+    assert p["n_split_windows"] == 0 and len(p["ranges"]) <= 3
+    assert check(hs, ro, 64)["n_split_windows"] == 1
+    # a window boundary that is not the end of a group is refused
+    with pytest.raises(hs.HspmmError):
+        hs.partition_preview(ro, 4, group_offset=np.array([0, 500, 1002], np.uint32))
+    with pytest.raises(hs.HspmmError):
+        hs.partition_preview(ro, 4, group_offset=np.array([0, 1000, 1000, 1001, 1002], np.uint32))
 
 
 def test_partition_balance_on_power_law(hs):

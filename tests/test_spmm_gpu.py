@@ -407,6 +407,74 @@ def test_partition_exported_as_groups_round_trips(torch_cuda, hs, oracle):
     pairs.close()
 
 
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_plans_that_cut_windows_only_where_the_callers_groups_end(torch_cuda, hs, oracle, dtype):
+    """hspmm_set_group_cuts(1): the waves of the gather kernels walk whole groups of the caller's grouped matrix
+    (GBTCF_MTX, reference src/utils/convert.h:245-259) - a heavy window is cut at group ends only, its partial sums
+    are added in group order.  Agrees with the oracle; bit for bit with the plain plan on inputs whose sums are exact."""
+    rng = np.random.default_rng(400 + dtype)
+    rows, cols = 300, 6000
+    A = random_csr(rng, rows, cols, 0.002, dtype, 0.2, (5, 100, 101, 299))
+    bitmap = hs.csr_to_bitmap(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype)
+    grouped = hs.bitmap_to_grouped(bitmap, min_len=7)
+    assert grouped["atomic"].any()
+    hs.configure(producer_warp_group_num=16)            # many short ranges: the heavy windows are cut
+    hs.set_group_cuts(1)
+    if dtype == 1:
+        hs.set_kernel_mode(3)                           # (fp32 storage: by default the LDS-staging kernels, which walk no groups)
+    try:
+        kept = hs.Plan(grouped)
+        hs.set_group_cuts(0)
+        free = hs.Plan(grouped)
+        _run_group_cut_checks(torch_cuda, hs, oracle, rng, A, grouped, kept, free, dtype)
+    finally:
+        hs.set_group_cuts(0)
+        hs.set_kernel_mode(0)
+        hs.configure()
+
+
+def _run_group_cut_checks(torch_cuda, hs, oracle, rng, A, grouped, kept, free, dtype):
+    rows, cols = A["rows"], A["cols"]
+    assert kept.info()["group_cuts_kept"] == 1 and free.info()["group_cuts_kept"] == 0
+    assert kept.info()["n_split_windows"] > 0
+    go = grouped["groupOffset"]
+    assert np.isin(kept.partition()[:, 0], go).all()
+    assert not np.isin(free.partition()[:, 0], go).all()                          # the cost model cuts elsewhere
+    assert np.isin(kept.partition_as_groups()["groupOffset"], go).all()            # what it walks are runs of whole groups
+    for N in (64, 128, 8):
+        B = make_b(rng, cols, N, dtype)
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        got = gpu_spmm(torch_cuda, hs, grouped, B, N, plan=kept)
+        assert_parity(got, ref, mag, dtype, "group cuts N=%d" % N)
+        assert N == 8 or kept.info()["last_kernel_family"] == 2
+    # small integers: every product and sum is exact, so the order of the additions cannot show
+    E = dict(A)
+    E["values"] = encode(rng.integers(-3, 4, A["nnzs"]).astype(np.float32), dtype)
+    eb = hs.csr_to_bitmap(rows, cols, E["row_ptr"], E["col_idx"], E["values"], dtype)
+    eg = hs.bitmap_to_grouped(eb, min_len=7)
+    B = encode(rng.integers(-4, 5, (cols, 64)).astype(np.float32), dtype)
+    hs.set_group_cuts(1)
+    kept_exact = hs.Plan(eg)
+    hs.set_group_cuts(0)
+    assert kept_exact.info()["group_cuts_kept"] == 1
+    got = gpu_spmm(torch_cuda, hs, eg, B, 64, plan=kept_exact)
+    want = gpu_spmm(torch_cuda, hs, convert(hs, E), B, 64)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    for plan in (kept, free, kept_exact):
+        plan.close()
+    # windows merged through equal column lists are not the caller's tiles any more: the cuts are dropped
+    P = random_csr(rng, 64, 64, 1.0, dtype)
+    pg = hs.bitmap_to_grouped(hs.csr_to_bitmap(64, 64, P["row_ptr"], P["col_idx"], P["values"], dtype), min_len=1)
+    hs.set_group_cuts(1)
+    try:
+        merged = hs.Plan(pg)
+    finally:
+        hs.set_group_cuts(0)
+    if merged.info()["n_paired_units"]:
+        assert merged.info()["group_cuts_kept"] == 0
+    merged.close()
+
+
 PANEL_SHAPES = [
     # rows, cols, density, empty-row probability, heavy rows
     (8, 16, 1.0, 0.0, ()),                      # one window, one panel
