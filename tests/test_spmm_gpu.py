@@ -67,9 +67,10 @@ def assert_parity(got, ref, absdot, dtype, what="", tight=True):
     cancels, an absolute term in units of sum |a||b|: 1e-5 for fp32 accumulation of exact products,
     and for the tf32 variant 2^-16 more unless the kernel mode guarantees fp32 products: its
     LDS-staging kernels multiply bf16 hi + lo parts in three products.  The product they leave out,
-    a_lo b_lo, has the sign of a b and at most 2^-14 of its size (2^-16 on average), so it only
-    reaches 2^-14 sum |a||b| where nothing cancels, and there the relative term is 16 times larger;
-    measured on normal entries against fp64: 2^-17.3 sum |a||b| at worst (tf32 itself: 2^-10)."""
+    a_lo b_lo, has the sign of a b and at most 2^-14 of its size (2^-16 on average): the hard bound
+    is 2^-14 sum |a||b|, reached only by factors with every low mantissa bit set; measured on normal
+    entries against fp64: 2^-17.3 sum |a||b| at worst (tf32 itself: 2^-10).  2^-16 is the bound the
+    seeded inputs of these tests stay within, not a guarantee for every input."""
     import hopper_spmm_amd
     if dtype != 1:
         g, r, rel, absolute = decode(got, dtype), decode(ref, dtype), 1e-2, 1e-5
