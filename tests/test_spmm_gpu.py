@@ -854,6 +854,70 @@ def test_seeded_sweep_of_shapes_formats_and_kernel_choices(torch_cuda, hs, oracl
         assert_parity(got, ref, mag, dtype, what, tight=False)
 
 
+@pytest.mark.parametrize("seed", [21, 22])
+def test_seeded_sweep_of_stream_modes_group_cuts_and_tuning_overrides(torch_cuda, hs, oracle, seed):
+    """As the sweep above (120 combinations per seed), with the choices it leaves at their defaults drawn as well:
+    the stream mode of the LDS-staging kernels, grouped input that keeps the caller's cuts, tiles written column
+    by column, and the overrides read from the environment at plan creation (bitmap stream of the gather kernels,
+    feature blocks dealt out by XCD, partial sums added inside the main kernel, one workgroup per unit for small
+    matrices, windows per unit of the panel stream)."""
+    knobs = ("HSPMM_GATHER_BITMAP", "HSPMM_XCD_SPLIT", "HSPMM_FUSED_FIXUP", "HSPMM_ALIGNED_SMALL", "HSPMM_PANEL_MAX_WINDOWS")
+    rng = np.random.default_rng(seed)
+    for case in range(120):
+        dtype = int(rng.integers(0, 3))
+        rows = int(rng.choice([1, 7, 8, 9, 15, 16, 17, 31, 64, 129, 300, 777]))
+        cols = int(rng.choice([1, 5, 16, 17, 31, 33, 127, 128, 129, 255, 257, 500, 2049, 6000]))
+        dens = float(rng.choice([0.002, 0.02, 0.1, 0.4, 0.9, 1.0]))
+        erp = float(rng.choice([0.0, 0.3, 0.8]))
+        heavy = tuple(int(x) for x in rng.integers(0, rows, int(rng.integers(0, 3)))) if rows > 8 else ()
+        A = random_csr(rng, rows, cols, dens, dtype, erp, heavy)
+        mode = int(rng.choice([0, 0, 0, 2, 3, 4, 4, 5]))
+        pairing = int(rng.integers(0, 3))
+        fmt = int(rng.integers(0, 5))          # plain, bitmap, grouped, grouped with its cuts kept, column by column
+        stages = int(rng.choice([0, 0, 0, 1, 2, 4]))
+        ranges_per_simd = int(rng.choice([0, 0, 1, 16]))
+        stream = int(rng.choice([0, 0, 1, 2]))
+        env = {}
+        for name, chance, values in zip(knobs, (0.3, 0.3, 0.3, 0.2, 0.2), ([0, 1], [0, 1], [0, 1], [0, 4, 8], [2, 4])):
+            if rng.random() < chance:
+                env[name] = str(int(rng.choice(values)))
+        if mode >= 4:
+            N = int(rng.choice([64, 128, 192, 256, 320, 512])) if dtype == 1 else int(rng.choice([128, 256, 384, 640, 1024]))
+        else:
+            N = int(rng.choice([1, 2, 3, 8, 16, 24, 32, 40, 64, 96, 128, 136, 256, 320, 512, 1000]))
+        what = "seed %d case %d: type %s %dx%d density %g empty %g heavy %s mode %d pairing %d format %d stages %d rps %d stream %d %s N %d" % (
+            seed, case, DT[dtype], rows, cols, dens, erp, heavy, mode, pairing, fmt, stages, ranges_per_simd, stream, env, N)
+        hs.set_kernel_mode(mode)
+        hs.set_window_pairing(pairing)
+        hs.set_panel_stream(stream)
+        hs.configure(buffer_stage=stages, producer_warp_group_num=ranges_per_simd)
+        os.environ.update(env)
+        try:
+            if fmt == 0:
+                b = convert(hs, A)
+            elif fmt == 4:
+                b = hs.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype, transpose=True)
+            else:
+                b = hs.csr_to_bitmap(rows, cols, A["row_ptr"], A["col_idx"], A["values"], dtype)
+                if fmt >= 2:
+                    b = hs.bitmap_to_grouped(b, int(rng.choice([1, 4, 32])))
+                    hs.set_group_cuts(1 if fmt == 3 else 0)
+            plan = hs.Plan(b)
+        finally:
+            hs.set_kernel_mode(0)
+            hs.set_window_pairing(0)
+            hs.set_panel_stream(0)
+            hs.set_group_cuts(0)
+            hs.configure()
+            for name in knobs:
+                os.environ.pop(name, None)
+        B = make_b(rng, cols, N, dtype)
+        got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+        plan.close()
+        ref, mag = oracle_spmm(oracle, A, B, N)
+        assert_parity(got, ref, mag, dtype, what, tight=False)
+
+
 def test_unaligned_and_odd_feature_dims_use_the_all_shapes_kernel(torch_cuda, hs, oracle):
     rng = np.random.default_rng(5)
     for dt in (0, 2):
