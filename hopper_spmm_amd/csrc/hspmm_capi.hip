@@ -1079,8 +1079,10 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
             return c;
         }
         c.layout = hspmm::kLayoutX4;
-        if (N % 8 == 0 && !(align & 15u) && N > 32) c.V = 4;
-        else if (N % 4 == 0 && !(align & 7u) && N > 16) c.V = 2;
+        // the narrowest block of features (32 V) that covers N: a wave multiplies its whole block whatever N is
+        // (power-law graph, N = 32: 293 -> 225 us with V = 1 instead of 2; N = 48: V = 2 instead of 4)
+        if (N % 8 == 0 && !(align & 15u) && N > 64) c.V = 4;
+        else if (N % 4 == 0 && !(align & 7u) && N > 32) c.V = 2;
         else c.V = 1;
         if (split_features && c.V == 4 && (N == 128 || N == 256 || N == 512)) c.V = 2;
         c.block_feat = 32 * c.V;
@@ -1088,8 +1090,8 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
     }
     if (align & 3u) { c.scalar = true; return c; }
     c.layout = hspmm::kLayoutX4;
-    if (N % 4 == 0 && !(align & 15u) && N > 16) c.V = 4;
-    else if (N % 2 == 0 && !(align & 7u) && N > 8) c.V = 2;
+    if (N % 4 == 0 && !(align & 15u) && N > 32) c.V = 4;         // (as above: blocks of 16 V features)
+    else if (N % 2 == 0 && !(align & 7u) && N > 16) c.V = 2;
     else c.V = 1;
     c.block_feat = 16 * c.V;
     return c;
