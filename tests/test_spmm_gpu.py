@@ -1278,6 +1278,53 @@ def test_benchmark_configurations_full_size(torch_cuda, hs, oracle, index, which
     plan.close()
 
 
+def test_more_than_2_to_24_tiles_and_4_gib_of_tiles_and_of_output(torch_cuda, hs):
+    """Sizes past the 24- and 32-bit marks: 8.4 M windows of two tiles each (16.8 M tiles, 4.3 GB of them) over
+    67 M rows (4.3 GB of C at N = 32).  Small integers, so every sum is exact: the default kernels must agree bit
+    for bit with the all-shapes kernel on every output and with numpy on sampled rows."""
+    torch = torch_cuda
+    W, N, cols = (1 << 23) + 4096, 32, 4096
+    rows = W * 8
+    per_row = np.array([3, 2, 2, 2, 2, 2, 2, 2], np.int64)           # 17 distinct columns per window
+    row_ptr = np.zeros(rows + 1, np.uint32)
+    row_ptr[1:] = np.cumsum(np.tile(per_row, W))
+    nnz = int(row_ptr[-1])
+    rng = np.random.default_rng(1)
+    first = rng.integers(0, cols - 37 * 17, W).astype(np.uint32)
+    order = np.array([0, 8, 16, 1, 9, 2, 10, 3, 11, 4, 12, 5, 13, 6, 14, 7, 15], np.uint32)   # a window's entries row by row
+    col_idx = (first[:, None] + 37 * order[None, :]).astype(np.uint32).reshape(-1)
+    vals = rng.integers(-3, 4, nnz).astype(np.float16)
+    b = hs.csr_to_btcf(rows, cols, row_ptr, col_idx, vals.view(np.uint16), 0)
+    assert b["total_tiles"] > 1 << 24 and b["data"].nbytes > 1 << 32
+    B = rng.integers(-4, 5, (cols, N)).astype(np.float16)
+    dB = torch.from_numpy(B.view(np.int16)).cuda()
+    outs = []
+    for mode in (0, 1):
+        hs.set_kernel_mode(mode)
+        try:
+            plan = hs.Plan(b)
+        finally:
+            hs.set_kernel_mode(0)
+        dC = torch.empty((rows, N), dtype=torch.int16, device="cuda")
+        dC.fill_(0x7E01)
+        plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert plan.info()["last_kernel_family"] == (2 if mode == 0 else 1)
+        plan.close()
+        outs.append(dC)
+    assert outs[0].numel() * 2 > 1 << 32
+    assert torch.equal(outs[0], outs[1])
+    sample = np.unique(np.concatenate([np.arange(64), np.arange(rows - 64, rows), np.arange(rows // 2 - 32, rows // 2 + 32),
+                                       rng.integers(0, rows, 2000)]))
+    got = outs[0][torch.from_numpy(sample).cuda()].cpu().numpy().view(np.float16).astype(np.float32)
+    av, Bf = vals.astype(np.float32), B.astype(np.float32)
+    for i, r in enumerate(sample):
+        lo, hi = int(row_ptr[r]), int(row_ptr[r + 1])
+        assert np.array_equal((av[lo:hi, None] * Bf[col_idx[lo:hi]]).sum(0), got[i]), "row %d" % r
+    del outs, dC, dB
+    torch.cuda.empty_cache()
+
+
 def test_columns_beyond_the_32_bit_offset_range(torch_cuda, hs, oracle):
     """B larger than 4 GiB: the gather uses 64-bit addresses."""
     torch = torch_cuda
