@@ -1325,6 +1325,49 @@ def test_more_than_2_to_24_tiles_and_4_gib_of_tiles_and_of_output(torch_cuda, hs
     torch.cuda.empty_cache()
 
 
+def test_lds_panel_stream_of_more_than_4_gib(torch_cuda, hs):
+    """65536 x 32768 at 10 %, fp32 storage: 3.7 M steps of 2 KB in the stream of the LDS-staging kernels (7.5 GB, past
+    32-bit byte offsets), 19 M tiles from the caller.  Small integers (exact in bf16 parts and in fp32 sums): bit for
+    bit against the all-shapes kernel."""
+    torch = torch_cuda
+    rows, cols, N, mean_gap = 65536, 32768, 64, 10
+    rng = np.random.default_rng(2)
+    per = cols // mean_gap + cols // (mean_gap * 8) + 16
+    counts, chunks = np.zeros(rows + 1, np.int64), []
+    for r0 in range(0, rows, 4096):
+        gaps = rng.integers(1, 2 * mean_gap, (4096, per), dtype=np.int32)         # ascending columns, 10 apart on average
+        gaps[:, 0] = rng.integers(0, mean_gap, 4096)
+        c = np.cumsum(gaps, axis=1, dtype=np.int32)
+        keep = c < cols
+        counts[r0 + 1:r0 + 4097] = keep.sum(1)
+        chunks.append(c[keep].astype(np.uint32))
+    col_idx = np.concatenate(chunks)
+    del chunks
+    row_ptr = np.cumsum(counts).astype(np.uint32)
+    vals = rng.integers(-3, 4, int(row_ptr[-1])).astype(np.float32)
+    b = hs.csr_to_btcf(rows, cols, row_ptr, col_idx, vals, 1)
+    dB = torch.from_numpy(rng.integers(-4, 5, (cols, N)).astype(np.float32)).cuda()
+    outs = []
+    for mode in (0, 1):
+        hs.set_kernel_mode(mode)
+        try:
+            plan = hs.Plan(b)
+        finally:
+            hs.set_kernel_mode(0)
+        dC = torch.full((rows, N), float("nan"), dtype=torch.float32, device="cuda")
+        plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        info = plan.info()
+        assert info["last_kernel_family"] == (3 if mode == 0 else 1)
+        if mode == 0:
+            assert info["n_panel_steps"] * 2048 > 1 << 32
+        plan.close()
+        outs.append(dC)
+    assert torch.equal(outs[0].view(torch.int32), outs[1].view(torch.int32))
+    del outs, dC, dB
+    torch.cuda.empty_cache()
+
+
 def test_columns_beyond_the_32_bit_offset_range(torch_cuda, hs, oracle):
     """B larger than 4 GiB: the gather uses 64-bit addresses."""
     torch = torch_cuda
