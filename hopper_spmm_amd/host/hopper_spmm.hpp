@@ -20,6 +20,7 @@
 #include <cstdlib>
 #include <cmath>
 #include <cstring>
+#include <thread>
 #include <vector>
 
 #include <hip/hip_runtime.h>
@@ -340,6 +341,7 @@ inline void check_shapes(vint a_rows, vint a_cols, const DENSE_MTX &dense_b, con
     }
 }
 inline PERF_RESULT run_plan(hspmm_plan *plan, DENSE_MTX &dense_b, DENSE_MTX &dense_c);
+class PageToucher;
 }  // namespace hspmm_cpp
 
 inline PERF_RESULT hspmm_cpp_spmm(BTCF_MTX_NO_BITMAP &a, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
@@ -397,17 +399,48 @@ inline PERF_RESULT hspmm_cpp_spmm(GBTCF_MTX &a, DENSE_MTX &dense_b, DENSE_MTX &d
     return hspmm_cpp::run_plan(plan, dense_b, dense_c);
 }
 
+// Writes one byte into every page of a buffer on worker threads, so that the pages of a freshly
+// allocated result matrix exist before the copy from the device lands in them (a copy into
+// untouched pages takes its page faults one by one: 78 ms instead of 15 ms for 268 MB).
+class hspmm_cpp::PageToucher {
+public:
+    PageToucher(void *buffer, size_t bytes)
+    {
+        const size_t page = 4096;
+        unsigned n = std::thread::hardware_concurrency();
+        n = n < 1 ? 1 : n > 16 ? 16 : n;
+        if (bytes < (size_t(8) << 20)) return;                 // small results: not worth a thread
+        const size_t per = ((bytes + n - 1) / n + page - 1) / page * page;
+        char *p = static_cast<char *>(buffer);
+        for (unsigned t = 0; t < n; ++t)
+            workers_.emplace_back([=] {
+                for (size_t i = size_t(t) * per; i < bytes && i < size_t(t + 1) * per; i += page)
+                    static_cast<volatile char *>(p)[i] = 0;
+            });
+    }
+    void wait()
+    {
+        for (std::thread &w : workers_) w.join();
+        workers_.clear();
+    }
+    ~PageToucher() { wait(); }
+private:
+    std::vector<std::thread> workers_;
+};
+
 inline PERF_RESULT hspmm_cpp::run_plan(hspmm_plan *plan, DENSE_MTX &dense_b, DENSE_MTX &dense_c)
 {
     PERF_RESULT perf{0.0f, RUNS};
     const size_t b_bytes = size_t(dense_b.rows) * dense_b.cols * sizeof(MAT_VAL_TYPE);
     const size_t c_bytes = size_t(dense_c.rows) * dense_c.cols * sizeof(MAT_VAL_TYPE);
+    hspmm_cpp::PageToucher touch_c(dense_c.values, c_bytes);   // while B goes up and the GPU works
     void *d_b = nullptr, *d_c = nullptr;
     hspmm_cpp::check_hip(hipMalloc(&d_b, b_bytes ? b_bytes : 4), "hipMalloc B");
     hspmm_cpp::check_hip(hipMalloc(&d_c, c_bytes ? c_bytes : 4), "hipMalloc C");
     hspmm_cpp::check_hip(hipMemcpy(d_b, dense_b.values, b_bytes, hipMemcpyHostToDevice), "copy B");
     if (dense_c.cols && hspmm_bench(plan, d_b, d_c, dense_c.cols, WARMUP_RUNS, RUNS, nullptr, &perf.time) != HSPMM_OK)
         hspmm_cpp::die("hspmm_bench");
+    touch_c.wait();
     hspmm_cpp::check_hip(hipMemcpy(dense_c.values, d_c, c_bytes, hipMemcpyDeviceToHost), "copy C");
     hspmm_cpp::check_hip(hipFree(d_b), "hipFree");
     hspmm_cpp::check_hip(hipFree(d_c), "hipFree");
