@@ -752,36 +752,37 @@ void pack_steps(size_t n_steps, bool split, const hspmm_host::ZeroedBuffer<uint3
 }
 
 // The bitmap stream of the gather kernels (Fp16TileDWB in spmm_mfma_kernel.hpp) from the uncompressed 8 x 16 tiles
-// of a 16-bit matrix: per tile the bitmap of the reference's CSR2BTCF (bit 16 r + k for element (r, k), reference
-// src/utils/convert.h:83-101; an element is stored when its bit pattern is not +0) as four 32-bit words, the bit
-// counts of words 0, 0..1 and 0..2 in bytes 1..3 of word 4, and in word 5 the position of the tile's first stored
-// element in `vals` (the reference's nnzOffset), where the stored elements follow tile after tile in bit order.
-void build_gather_bitmap(uint32_t T, const void *data, hspmm_host::ZeroedBuffer<uint32_t> &header, hspmm_host::ZeroedBuffer<uint16_t> &vals)
+// of a 16-bit matrix, made on the device from the tiles already uploaded (p->d_data): per tile the bitmap of the
+// reference's CSR2BTCF (bit 16 r + k for element (r, k), reference src/utils/convert.h:83-101; an element is stored
+// when its bit pattern is not +0) as four 32-bit words, the bit counts of words 0, 0..1 and 0..2 in bytes 1..3 of
+// word 4, and in word 5 the position of the tile's first stored element in `vals` (the reference's nnzOffset),
+// where the stored elements follow tile after tile in bit order.  Leaves p->bm.built false when the positions
+// would not fit 31 bits.  (On the host this took 29 ms for the 257 MB of tiles of the 2^20 power-law graph.)
+int bitmap_from_uploaded_tiles(hspmm_plan *p, uint32_t T)
 {
-    const uint16_t *h = static_cast<const uint16_t *>(data);
-    header = hspmm_host::ZeroedBuffer<uint32_t>(size_t(T) * 8u);
-    std::vector<uint32_t> count(size_t(T) + 1, 0u);
-    hspmm_host::parallel_blocks(T, 4096, [&](size_t tb, size_t te) {
-        for (size_t t = tb; t < te; ++t) {
-            const uint16_t *tile = h + t * 128u;
-            uint32_t *hd = header.data() + t * 8u;
-            for (uint32_t b = 0; b < 128u; ++b) if (tile[b]) hd[b >> 5] |= 1u << (b & 31u);
-            const uint32_t c0 = uint32_t(__builtin_popcount(hd[0])), c1 = c0 + uint32_t(__builtin_popcount(hd[1])),
-                           c2 = c1 + uint32_t(__builtin_popcount(hd[2]));
-            hd[4] = c0 << 8 | c1 << 16 | c2 << 24;
-            count[t + 1] = c2 + uint32_t(__builtin_popcount(hd[3]));
-        }
-    });
-    uint64_t total = 0;
-    for (size_t t = 0; t < T; ++t) { header[t * 8u + 5u] = uint32_t(total); total += count[t + 1]; }
-    vals = hspmm_host::ZeroedBuffer<uint16_t>(size_t(total) + 4u);                // a lane reads 8 bytes from its first element
-    hspmm_host::parallel_blocks(T, 4096, [&](size_t tb, size_t te) {
-        for (size_t t = tb; t < te; ++t) {
-            const uint16_t *tile = h + t * 128u;
-            size_t at = header[t * 8u + 5u];
-            for (uint32_t b = 0; b < 128u; ++b) if (tile[b]) vals[at++] = tile[b];
-        }
-    });
+    const uint32_t n_blocks = hspmm::bitmap_scan_blocks(T);
+    uint64_t *d_sums = nullptr;
+    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->bm.d_header), size_t(T) * 32u));     // (released by hspmm_destroy)
+    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&d_sums), (size_t(n_blocks) + 1u) * sizeof(uint64_t)));
+    auto done = [&](int code) { (void)hipFree(d_sums); return code; };
+    HSPMM_HIP_OR(hspmm::launch_bitmap_header(p->d_data, p->bm.d_header, T, d_sums, nullptr), done);
+    uint64_t stored = 0;
+    HSPMM_HIP_OR(hipMemcpy(&stored, d_sums + n_blocks, sizeof(stored), hipMemcpyDeviceToHost), done);
+    if (stored + 4u >= (uint64_t(1) << 31)) {                   // positions are 32-bit
+        (void)hipFree(p->bm.d_header);
+        p->bm.d_header = nullptr;
+        return done(HSPMM_OK);
+    }
+    uint16_t *dv = nullptr;                                     // (a lane reads 8 bytes from its first element: 4 more)
+    HSPMM_HIP_OR(hipMalloc(reinterpret_cast<void **>(&dv), (size_t(stored) + 4u) * sizeof(uint16_t)), done);
+    p->bm.d_vals = dv;
+    HSPMM_HIP_OR(hipMemset(dv + stored, 0, 4u * sizeof(uint16_t)), done);
+    HSPMM_HIP_OR(hspmm::launch_bitmap_pack(p->d_data, p->bm.d_header, dv, T, d_sums, nullptr), done);
+    HSPMM_HIP_OR(hipStreamSynchronize(nullptr), done);
+    p->bm.stored = stored;
+    p->bm.built = true;
+    p->fixed_bytes += size_t(T) * 32u + (size_t(stored) + 4u) * sizeof(uint16_t);
+    return done(HSPMM_OK);
 }
 
 // Re-tiles the matrix panel by panel for the LDS-panel kernels (spmm_panel_kernel.hpp):
@@ -1495,7 +1496,10 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
         p->n_steps = st.n_steps;
         if ((rc = upload(&p->d_unitOffset, st.unitOffset.data(), st.unitOffset.size(), &p->fixed_bytes))) return bail(rc);
         if ((rc = upload(&p->d_unitRow, st.unitRow.data(), st.unitRow.size(), &p->fixed_bytes))) return bail(rc);
-        {
+        if (dtype != HSPMM_TF32 && st.G == 1) {
+            // single 16-bit windows: the steps are the caller's tiles in the caller's order, their ids these
+            if ((rc = upload(&p->d_ids, clean, n_ids, &p->fixed_bytes))) return bail(rc);
+        } else {
             const hspmm_host::ZeroedBuffer<uint32_t> ids = lane_order_ids(st, dtype, rowOffset, clean);
             if ((rc = upload(&p->d_ids, ids.data(), ids.size(), &p->fixed_bytes))) return bail(rc);
         }
@@ -1534,16 +1538,7 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
             // pays the longer dependent chain: 4096 x 4096 at 1 %, 2.7 MB of tiles: 6.8 -> 7.5 us)
             if (p->cfg.gather_bitmap > 0 ||
                 (stored * 3u < size_t(total_tiles) * 128u && size_t(total_tiles) * 256u >= (size_t(8) << 20))) {
-                hspmm_host::ZeroedBuffer<uint32_t> header;
-                hspmm_host::ZeroedBuffer<uint16_t> vals;
-                try { build_gather_bitmap(total_tiles, data, header, vals); }
-                catch (const std::bad_alloc &) { return bail(fail(HSPMM_ERR_ALLOC, "out of host memory")); }
-                if (vals.size() < (size_t(1) << 31)) {               // positions are 32-bit
-                    uint16_t *dv = nullptr;
-                    if ((rc = upload(&p->bm.d_header, header.data(), header.size(), &p->fixed_bytes))) return bail(rc);
-                    if ((rc = upload(&dv, vals.data(), vals.size(), &p->fixed_bytes))) return bail(rc);
-                    p->bm.d_vals = dv; p->bm.stored = vals.size() - 4u; p->bm.built = true;
-                }
+                if ((rc = bitmap_from_uploaded_tiles(p, total_tiles))) return bail(rc);
             }
         }
         timer.mark("bitmap tiles");

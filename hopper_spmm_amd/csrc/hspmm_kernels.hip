@@ -99,6 +99,152 @@ hipError_t launch_expand_bitmap(const uint32_t *header, const void *vals, void *
     return hipGetLastError();
 }
 
+// Plain 8 x 16 tiles of 16-bit elements -> bitmap tiles, on the device: what hspmm_create does for a matrix of
+// sparse tiles once the plain tiles are uploaded (the reverse of the kernel above; the bitmap is the reference's,
+// src/utils/convert.h:83-101: bit 16 r + k for element (r, k), stored when its bit pattern is not +0).  Three
+// passes: the four mask words, their running bit counts and the tile's count (header words 0..4 and 6); an
+// exclusive sum of the counts over all tiles (header word 5, the reference's nnzOffset); the stored elements
+// written tile after tile in bit order.
+typedef uint32_t bm_u32x4 __attribute__((ext_vector_type(4)));
+constexpr uint32_t kScanTilesPerBlock = 2048;          // 256 threads x 8 tiles
+
+// the 32 elements of word `word` of tile t as a mask (four consecutive lanes take the four words of one tile)
+__device__ __forceinline__ uint32_t tile_word_mask(const uint16_t *tiles, uint32_t t, uint32_t word)
+{
+    const bm_u32x4 *src = reinterpret_cast<const bm_u32x4 *>(tiles + size_t(t) * 128u + word * 32u);
+    uint32_t mask = 0;
+#pragma unroll
+    for (uint32_t q = 0; q < 4; ++q) {
+        const bm_u32x4 v = src[q];
+#pragma unroll
+        for (uint32_t e = 0; e < 4; ++e) {
+            mask |= ((v[e] & 0xFFFFu) ? 1u : 0u) << (q * 8u + 2u * e);
+            mask |= ((v[e] >> 16) ? 1u : 0u) << (q * 8u + 2u * e + 1u);
+        }
+    }
+    return mask;
+}
+
+__global__ __launch_bounds__(256) void bitmap_header_kernel(const uint16_t *__restrict__ tiles, uint32_t *__restrict__ header,
+                                                            uint32_t n_tiles)
+{
+    const uint64_t i = uint64_t(blockIdx.x) * 256u + threadIdx.x;
+    const uint32_t t = uint32_t(i >> 2), word = uint32_t(i & 3u), lane = threadIdx.x & 63u;
+    const bool active = i < uint64_t(n_tiles) * 4u;
+    const uint32_t mask = active ? tile_word_mask(tiles, t, word) : 0u;
+    const uint32_t c = uint32_t(__builtin_popcount(mask)), first = lane & ~3u;
+    const uint32_t c0 = __shfl(c, first), c1 = c0 + __shfl(c, first + 1u), c2 = c1 + __shfl(c, first + 2u),
+                   c3 = c2 + __shfl(c, first + 3u);
+    if (!active) return;
+    uint32_t *hd = header + size_t(t) * 8u;
+    hd[word] = mask;
+    if (word == 0u) { hd[4] = c0 << 8 | c1 << 16 | c2 << 24; hd[6] = c3; hd[7] = 0u; }
+}
+
+// sum of a value over the 256 threads of a workgroup, and the sum over the threads in front of this one
+__device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t v, uint32_t *total)
+{
+    __shared__ uint32_t wave_sum[4];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t x = v;
+#pragma unroll
+    for (uint32_t d = 1; d < 64u; d <<= 1) {
+        const uint32_t y = __shfl_up(x, d);
+        if (lane >= d) x += y;
+    }
+    __syncthreads();                       // (a second call must not overwrite sums still being read)
+    if (lane == 63u) wave_sum[wave] = x;
+    __syncthreads();
+    uint32_t before = 0, all = 0;
+#pragma unroll
+    for (uint32_t w = 0; w < 4u; ++w) { if (w < wave) before += wave_sum[w]; all += wave_sum[w]; }
+    *total = all;
+    return before + x - v;
+}
+
+__global__ __launch_bounds__(256) void bitmap_block_sums_kernel(const uint32_t *__restrict__ header, uint32_t n_tiles,
+                                                                uint64_t *__restrict__ block_sums)
+{
+    const uint64_t t0 = uint64_t(blockIdx.x) * kScanTilesPerBlock + threadIdx.x * 8u;
+    uint32_t s = 0;
+    for (uint32_t k = 0; k < 8u; ++k)
+        if (t0 + k < n_tiles) s += header[(t0 + k) * 8u + 6u];
+    uint32_t total;
+    (void)block_exclusive_sum(s, &total);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+// exclusive sums of block_sums in place (one workgroup; a chunk of 256 block sums is below 2^26), the total behind them
+__global__ __launch_bounds__(256) void bitmap_scan_sums_kernel(uint64_t *block_sums, uint32_t n_blocks)
+{
+    uint64_t carry = 0;
+    for (uint32_t base = 0; base < n_blocks; base += 256u) {
+        const uint32_t i = base + threadIdx.x;
+        const uint32_t v = i < n_blocks ? uint32_t(block_sums[i]) : 0u;
+        uint32_t total;
+        const uint32_t before = block_exclusive_sum(v, &total);
+        if (i < n_blocks) block_sums[i] = carry + before;
+        carry += total;
+    }
+    if (threadIdx.x == 0) block_sums[n_blocks] = carry;
+}
+
+__global__ __launch_bounds__(256) void bitmap_offsets_kernel(uint32_t *__restrict__ header, uint32_t n_tiles,
+                                                             const uint64_t *__restrict__ block_sums)
+{
+    const uint64_t t0 = uint64_t(blockIdx.x) * kScanTilesPerBlock + threadIdx.x * 8u;
+    uint32_t count[8], s = 0;
+    for (uint32_t k = 0; k < 8u; ++k) {
+        count[k] = t0 + k < n_tiles ? header[(t0 + k) * 8u + 6u] : 0u;
+        s += count[k];
+    }
+    uint32_t total;
+    uint64_t at = block_sums[blockIdx.x] + block_exclusive_sum(s, &total);
+    for (uint32_t k = 0; k < 8u; ++k)
+        if (t0 + k < n_tiles) { header[(t0 + k) * 8u + 5u] = uint32_t(at); at += count[k]; }
+}
+
+__global__ __launch_bounds__(256) void bitmap_pack_kernel(const uint16_t *__restrict__ tiles, const uint32_t *__restrict__ header,
+                                                          uint16_t *__restrict__ vals, uint32_t n_tiles)
+{
+    const uint64_t i = uint64_t(blockIdx.x) * 256u + threadIdx.x;
+    if (i >= uint64_t(n_tiles) * 4u) return;
+    const uint32_t t = uint32_t(i >> 2), word = uint32_t(i & 3u);
+    const uint32_t *hd = header + size_t(t) * 8u;
+    uint32_t mask = hd[word];
+    size_t at = size_t(hd[5]) + ((hd[4] >> (8u * word)) & 0xFFu);
+    const uint16_t *src = tiles + size_t(t) * 128u + word * 32u;
+    while (mask) {
+        const uint32_t b = uint32_t(__builtin_ctz(mask));
+        vals[at++] = src[b];
+        mask &= mask - 1u;
+    }
+}
+
+hipError_t launch_bitmap_header(const void *tiles, uint32_t *header, uint32_t n_tiles, uint64_t *block_sums, hipStream_t s)
+{
+    if (!n_tiles) return hipSuccess;
+    const uint32_t word_blocks = uint32_t((uint64_t(n_tiles) * 4u + 255u) / 256u);
+    const uint32_t n_blocks = (n_tiles + kScanTilesPerBlock - 1u) / kScanTilesPerBlock;
+    bitmap_header_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint16_t *>(tiles), header, n_tiles);
+    bitmap_block_sums_kernel<<<dim3(n_blocks), 256, 0, s>>>(header, n_tiles, block_sums);
+    bitmap_scan_sums_kernel<<<dim3(1), 256, 0, s>>>(block_sums, n_blocks);
+    return hipGetLastError();
+}
+
+uint32_t bitmap_scan_blocks(uint32_t n_tiles) { return (n_tiles + kScanTilesPerBlock - 1u) / kScanTilesPerBlock; }
+
+hipError_t launch_bitmap_pack(const void *tiles, uint32_t *header, void *vals, uint32_t n_tiles, const uint64_t *block_sums,
+                              hipStream_t s)
+{
+    if (!n_tiles) return hipSuccess;
+    const uint32_t word_blocks = uint32_t((uint64_t(n_tiles) * 4u + 255u) / 256u);
+    bitmap_offsets_kernel<<<dim3(bitmap_scan_blocks(n_tiles)), 256, 0, s>>>(header, n_tiles, block_sums);
+    bitmap_pack_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint16_t *>(tiles), header,
+                                                        static_cast<uint16_t *>(vals), n_tiles);
+    return hipGetLastError();
+}
+
 #define HSPMM_DECLARE_LAUNCH(name) \
     hipError_t name(int layout, const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, \
                     hipStream_t s, hipEvent_t mid);
