@@ -1,7 +1,8 @@
-// Host-side helper shared by the converters and the plan builder: a loop over
-// [0, n) cut into one contiguous block per worker thread.
+// Host-side helpers shared by the converters and the plan builder: a loop over
+// [0, n) cut into chunks that worker threads take one after the other.
 #pragma once
 #include <algorithm>
+#include <atomic>
 #include <cstddef>
 #include <cstdlib>
 #include <new>
@@ -21,24 +22,42 @@ inline unsigned worker_count(size_t work_items, size_t min_per_worker)
     return unsigned(std::min<size_t>(hw, by_work));
 }
 
-// fn(begin, end) on every block; an exception of a worker (out of memory) is rethrown
-// on the calling thread once all workers are done.
+// fn(begin, end) on chunks of `chunk` items that the workers take off a shared counter until none is left
+// (work spread unevenly over [0, n) - the windows of a power-law graph: the first tenth of them holds half of
+// the entries - still keeps every worker busy to the end).  An exception of a worker (out of memory) is
+// rethrown on the calling thread once all workers are done.
+template <class F>
+void parallel_chunks(size_t n, size_t chunk, F &&fn, unsigned workers = 0)
+{
+    if (chunk < 1) chunk = 1;
+    const unsigned nw = workers ? workers : worker_count(n, chunk);
+    if (nw <= 1) { if (n) fn(size_t(0), n); return; }
+    std::atomic<size_t> next{0};
+    std::vector<std::thread> th;
+    std::vector<std::exception_ptr> err(nw);
+    th.reserve(nw);
+    for (unsigned i = 0; i < nw; ++i)
+        th.emplace_back([&fn, &err, &next, i, n, chunk] {
+            try {
+                for (size_t b = next.fetch_add(chunk); b < n; b = next.fetch_add(chunk)) fn(b, std::min(n, b + chunk));
+            } catch (...) {
+                err[i] = std::current_exception();
+                next.store(n);                        // the others stop at their next chunk
+            }
+        });
+    for (auto &t : th) t.join();
+    for (auto &e : err) if (e) std::rethrow_exception(e);
+}
+
+// A loop over [0, n) for as many workers as have min_per_worker items each: eight chunks per worker, none
+// shorter than min_per_worker.
 template <class F>
 void parallel_blocks(size_t n, size_t min_per_worker, F &&fn)
 {
     const unsigned nw = worker_count(n, min_per_worker);
     if (nw <= 1) { fn(size_t(0), n); return; }
-    std::vector<std::thread> th;
-    std::vector<std::exception_ptr> err(nw);
-    th.reserve(nw);
-    for (unsigned i = 0; i < nw; ++i) {
-        const size_t b = n * i / nw, e = n * (i + 1) / nw;
-        th.emplace_back([&fn, &err, i, b, e] {
-            try { fn(b, e); } catch (...) { err[i] = std::current_exception(); }
-        });
-    }
-    for (auto &t : th) t.join();
-    for (auto &e : err) if (e) std::rethrow_exception(e);
+    const size_t pieces = size_t(nw) * 8u;
+    parallel_chunks(n, std::max<size_t>(min_per_worker, (n + pieces - 1) / pieces), fn, nw);
 }
 
 // n elements that read as zero, without the single-threaded pass a std::vector spends on clearing them

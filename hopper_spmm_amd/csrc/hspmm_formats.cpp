@@ -327,7 +327,7 @@ int hspmm_mtx_load(const char *path, int dtype, hspmm_csr *out)
     for (uint32_t r = 0; r < t.rows; ++r) row_ptr[r + 1] += row_ptr[r];
     std::vector<uint32_t> order(nnz), cursor(row_ptr, row_ptr + t.rows);
     for (size_t i = 0; i < nnz; ++i) order[cursor[t.r[i]]++] = uint32_t(i);
-    parallel_blocks(t.rows, 4096, [&](size_t rb, size_t re) {
+    parallel_chunks(t.rows, 4096, [&](size_t rb, size_t re) {
         for (size_t r = rb; r < re; ++r)
             std::stable_sort(order.begin() + row_ptr[r], order.begin() + row_ptr[r + 1],
                              [&](uint32_t a, uint32_t b) { return t.c[a] < t.c[b]; });
@@ -368,7 +368,7 @@ static uint32_t window_columns(const uint32_t *row_ptr, const uint32_t *col_idx,
     return uint32_t(uniq.size());
 }
 
-// Windows a worker should get at least: what holds about 64 K stored entries (a matrix of few wide
+// Windows a worker takes at a time: what holds about 64 K stored entries (a matrix of few wide
 // windows, like block-clustered weights, still spreads over the cores).
 static size_t windows_per_worker(size_t nwin, size_t nnz)
 {
@@ -383,7 +383,7 @@ static void count_tiles(uint32_t rows, const uint32_t *row_ptr, const uint32_t *
 {
     const size_t nwin = (size_t(rows) + HSPMM_ROW_WINDOW - 1) / HSPMM_ROW_WINDOW;
     tiles.assign(nwin, 0u);
-    parallel_blocks(nwin, windows_per_worker(nwin, row_ptr[rows]), [&](size_t wb, size_t we) {
+    parallel_chunks(nwin, windows_per_worker(nwin, row_ptr[rows]), [&](size_t wb, size_t we) {
         std::vector<uint32_t> uniq;
         for (size_t w = wb; w < we; ++w) {
             const uint32_t r0 = uint32_t(w * HSPMM_ROW_WINDOW);
@@ -441,7 +441,7 @@ int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uin
         set_error("null argument");
         return HSPMM_ERR_INVALID;
     }
-    parallel_blocks(nwin, windows_per_worker(nwin, row_ptr[rows]), [&](size_t wb, size_t we) {
+    parallel_chunks(nwin, windows_per_worker(nwin, row_ptr[rows]), [&](size_t wb, size_t we) {
         std::vector<uint32_t> uniq;
         for (size_t w = wb; w < we; ++w) {
             if (!tiles[w]) continue;
@@ -561,7 +561,7 @@ int hspmm_bitmap_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const u
         }
     };
     if (shared_words) convert_windows(0, nwin);
-    else parallel_blocks(nwin, windows_per_worker(nwin, row_ptr[rows]), convert_windows);
+    else parallel_chunks(nwin, windows_per_worker(nwin, row_ptr[rows]), convert_windows);
     return HSPMM_OK;
 }
 
