@@ -761,27 +761,29 @@ void pack_steps(size_t n_steps, bool split, const hspmm_host::ZeroedBuffer<uint3
 int bitmap_from_uploaded_tiles(hspmm_plan *p, uint32_t T)
 {
     const uint32_t n_blocks = hspmm::bitmap_scan_blocks(T);
+    const size_t header_bytes = size_t(T) * (p->elem == 2u ? 32u : 16u);     // fp32 tiles (8 x 8): two mask words, position, count
+    const size_t spare = 8u / p->elem;                                        // a lane may read 8 bytes from the last element on
     uint64_t *d_sums = nullptr;
-    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->bm.d_header), size_t(T) * 32u));     // (released by hspmm_destroy)
+    HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->bm.d_header), header_bytes));        // (released by hspmm_destroy)
     HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&d_sums), (size_t(n_blocks) + 1u) * sizeof(uint64_t)));
     auto done = [&](int code) { (void)hipFree(d_sums); return code; };
-    HSPMM_HIP_OR(hspmm::launch_bitmap_header(p->d_data, p->bm.d_header, T, d_sums, nullptr), done);
+    HSPMM_HIP_OR(hspmm::launch_bitmap_header(int(p->elem), p->d_data, p->bm.d_header, T, d_sums, nullptr), done);
     uint64_t stored = 0;
     HSPMM_HIP_OR(hipMemcpy(&stored, d_sums + n_blocks, sizeof(stored), hipMemcpyDeviceToHost), done);
-    if (stored + 4u >= (uint64_t(1) << 31)) {                   // positions are 32-bit
+    if (stored + spare >= (uint64_t(1) << 31)) {                // positions are 32-bit
         (void)hipFree(p->bm.d_header);
         p->bm.d_header = nullptr;
         return done(HSPMM_OK);
     }
-    uint16_t *dv = nullptr;                                     // (a lane reads 8 bytes from its first element: 4 more)
-    HSPMM_HIP_OR(hipMalloc(reinterpret_cast<void **>(&dv), (size_t(stored) + 4u) * sizeof(uint16_t)), done);
+    char *dv = nullptr;
+    HSPMM_HIP_OR(hipMalloc(reinterpret_cast<void **>(&dv), (size_t(stored) + spare) * p->elem), done);
     p->bm.d_vals = dv;
-    HSPMM_HIP_OR(hipMemset(dv + stored, 0, 4u * sizeof(uint16_t)), done);
-    HSPMM_HIP_OR(hspmm::launch_bitmap_pack(p->d_data, p->bm.d_header, dv, T, d_sums, nullptr), done);
+    HSPMM_HIP_OR(hipMemset(dv + size_t(stored) * p->elem, 0, spare * p->elem), done);
+    HSPMM_HIP_OR(hspmm::launch_bitmap_pack(int(p->elem), p->d_data, p->bm.d_header, dv, T, d_sums, nullptr), done);
     HSPMM_HIP_OR(hipStreamSynchronize(nullptr), done);
     p->bm.stored = stored;
     p->bm.built = true;
-    p->fixed_bytes += size_t(T) * 32u + (size_t(stored) + 4u) * sizeof(uint16_t);
+    p->fixed_bytes += header_bytes + (size_t(stored) + spare) * p->elem;
     return done(HSPMM_OK);
 }
 
@@ -1094,6 +1096,8 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
     if (N % 4 == 0 && !(align & 15u) && N > 32) c.V = 4;         // (as above: blocks of 16 V features)
     else if (N % 2 == 0 && !(align & 7u) && N > 16) c.V = 2;
     else c.V = 1;
+    // (feature blocks of one 128-byte line with XCDs of their own, what the 16-bit types gain from, lose here:
+    // power-law graph 2^20 in fp32, N = 64: 590 -> 714 us, N = 128: 1191 -> 1337 us)
     c.block_feat = 16 * c.V;
     return c;
 }
@@ -1503,13 +1507,20 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
             const hspmm_host::ZeroedBuffer<uint32_t> ids = lane_order_ids(st, dtype, rowOffset, clean);
             if ((rc = upload(&p->d_ids, ids.data(), ids.size(), &p->fixed_bytes))) return bail(rc);
         }
-        if (dtype != HSPMM_TF32 && st.G == 1) {
-            p->d_tiles = p->d_data;                 // the caller's tile layout already is the lane order
-        } else {
+        // (single fp32 windows: decided below, once it is known whether the gather kernels of this plan read
+        // bitmap tiles - then nothing reads tiles in lane order)
+        const bool lane_tiles_later = dtype == HSPMM_TF32 && st.G == 1;
+        auto upload_lane_order_tiles = [&]() -> int {
             const hspmm_host::ZeroedBuffer<uint32_t> tiles = lane_order_tiles(st, dtype, rowOffset, data);
             uint32_t *dt = nullptr;
-            if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) return bail(rc);
+            const int urc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes);
             p->d_tiles = dt;
+            return urc;
+        };
+        if (dtype != HSPMM_TF32 && st.G == 1) {
+            p->d_tiles = p->d_data;                 // the caller's tile layout already is the lane order
+        } else if (!lane_tiles_later) {
+            if ((rc = upload_lane_order_tiles())) return bail(rc);
         }
         timer.mark("step stream (ids, tiles)");
         // Single 16-bit windows with few stored elements per tile (graphs: 16 of 128): the gather kernels read the
@@ -1525,21 +1536,30 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
                 (void)hipFree(p->bm.d_header); (void)hipFree(p->bm.d_vals);
                 p->bm.d_header = nullptr; p->bm.d_vals = nullptr;
             }
-        } else if (dtype != HSPMM_TF32 && st.G == 1 && p->cfg.gather_bitmap != 0 && total_tiles) {
+        } else if (st.G == 1 && p->cfg.gather_bitmap != 0 && total_tiles) {
+            const size_t n = size_t(total_tiles) * 8u * cw;                 // tile elements
             size_t stored = 0;
             if (p->cfg.gather_bitmap < 0) {
-                const uint16_t *hv = static_cast<const uint16_t *>(data);
-                const size_t n = size_t(total_tiles) * 128u, sample = std::min<size_t>(n, size_t(1) << 22);
-                for (size_t i = 0; i < sample; ++i) stored += hv[i] != 0;
+                const size_t sample = std::min<size_t>(n, size_t(1) << 22);
+                if (elem == 2u) {
+                    const uint16_t *hv = static_cast<const uint16_t *>(data);
+                    for (size_t i = 0; i < sample; ++i) stored += hv[i] != 0;
+                } else {
+                    const uint32_t *wv = static_cast<const uint32_t *>(data);
+                    for (size_t i = 0; i < sample; ++i) stored += wv[i] != 0;
+                }
                 stored = size_t(double(stored) * double(n) / double(sample));
             }
-            // 32 + 2 e bytes against 256 per tile with e stored elements: worth it below about a third full, and
-            // where the tile stream is large enough to be traffic at all (a matrix whose tiles sit in the L2s only
-            // pays the longer dependent chain: 4096 x 4096 at 1 %, 2.7 MB of tiles: 6.8 -> 7.5 us)
+            // 32 + 2 e bytes against 256 per tile with e stored elements (16 + 4 e for fp32): worth it below about a
+            // third full, and where the tile stream is large enough to be traffic at all (a matrix whose tiles sit
+            // in the L2s only pays the longer dependent chain: 4096 x 4096 at 1 %, 2.7 MB of tiles: 6.8 -> 7.5 us)
             if (p->cfg.gather_bitmap > 0 ||
-                (stored * 3u < size_t(total_tiles) * 128u && size_t(total_tiles) * 256u >= (size_t(8) << 20))) {
+                (stored * 3u < n && size_t(total_tiles) * 256u >= (size_t(8) << 20))) {
                 if ((rc = bitmap_from_uploaded_tiles(p, total_tiles))) return bail(rc);
             }
+        }
+        if (lane_tiles_later && !(p->bm.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 3))) {
+            if ((rc = upload_lane_order_tiles())) return bail(rc);
         }
         timer.mark("bitmap tiles");
         p->h_unitOffset = st.unitOffset;
@@ -1976,7 +1996,8 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     }
     ka.unitOffset = p->d_unitOffset; ka.unitRow = p->d_unitRow; ka.ids = p->d_ids; ka.tiles = p->d_tiles;
     int layout = c.layout;
-    if (p->bm.built && c.layout == hspmm::kLayoutDW && (c.V == 2 || c.V == 4) && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 3)) {
+    if (p->bm.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 3) &&
+        (p->dtype == HSPMM_TF32 || (c.layout == hspmm::kLayoutDW && (c.V == 2 || c.V == 4)))) {
         layout = hspmm::kLayoutDWB;                   // tiles as bitmap + stored elements
         ka.tiles = p->bm.d_vals; ka.bm_header = p->bm.d_header;
     }

@@ -98,14 +98,17 @@ hipError_t launch_spmm_panel(int dtype, int G, bool split, bool tall, bool packe
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
 // bitmap tiles (header, stored elements: see KernelArgs::bm_header) -> plain 8 x 16 tiles of 16-bit elements
 hipError_t launch_expand_bitmap(const uint32_t *header, const void *vals, void *tiles, uint32_t n_tiles, hipStream_t s);
-// plain 8 x 16 tiles of 16-bit elements -> bitmap tiles, in two steps with the host in between (it sizes `vals`):
-// launch_bitmap_header writes header words 0..4 and the tiles' counts, and leaves in block_sums
+// plain tiles -> bitmap tiles (8 x 16 tiles of 16-bit elements, elem_bytes = 2: 8 header words per tile, see
+// KernelArgs::bm_header; 8 x 8 tiles of 32-bit elements, elem_bytes = 4: 4 header words - rows 0..3, rows 4..7,
+// position of the first stored element, number of stored elements), in two steps with the host in between (it
+// sizes `vals`): launch_bitmap_header writes the masks and the tiles' counts, and leaves in block_sums
 // (bitmap_scan_blocks(n_tiles) + 1 words of 64 bits) the exclusive sums per 2048 tiles and, last, the number of
-// stored elements; launch_bitmap_pack writes header word 5 and the stored elements.
+// stored elements; launch_bitmap_pack writes the positions and the stored elements.
 uint32_t bitmap_scan_blocks(uint32_t n_tiles);
-hipError_t launch_bitmap_header(const void *tiles, uint32_t *header, uint32_t n_tiles, uint64_t *block_sums, hipStream_t s);
-hipError_t launch_bitmap_pack(const void *tiles, uint32_t *header, void *vals, uint32_t n_tiles, const uint64_t *block_sums,
-                              hipStream_t s);
+hipError_t launch_bitmap_header(int elem_bytes, const void *tiles, uint32_t *header, uint32_t n_tiles, uint64_t *block_sums,
+                                hipStream_t s);
+hipError_t launch_bitmap_pack(int elem_bytes, const void *tiles, uint32_t *header, void *vals, uint32_t n_tiles,
+                              const uint64_t *block_sums, hipStream_t s);
 // Measurement only (gather_rate_kernel in hspmm_kernels.hip): loads part_bytes (128 or 256) of row ids[i] of B for
 // every i < n_ids; parts > 1: `parts` parts of part_bytes each, dealt out by XCD, every part walking all ids.
 hipError_t launch_gather_rate(const uint32_t *ids, uint64_t n_ids, const void *B, uint32_t row_bytes, uint32_t part_bytes,

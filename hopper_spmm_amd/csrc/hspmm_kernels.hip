@@ -162,13 +162,15 @@ __device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t v, uint32_t *to
     return before + x - v;
 }
 
+// (words: header words per tile; at_count / at_first: where a tile's count is and where its position goes)
 __global__ __launch_bounds__(256) void bitmap_block_sums_kernel(const uint32_t *__restrict__ header, uint32_t n_tiles,
-                                                                uint64_t *__restrict__ block_sums)
+                                                                uint64_t *__restrict__ block_sums, uint32_t words,
+                                                                uint32_t at_count)
 {
     const uint64_t t0 = uint64_t(blockIdx.x) * kScanTilesPerBlock + threadIdx.x * 8u;
     uint32_t s = 0;
     for (uint32_t k = 0; k < 8u; ++k)
-        if (t0 + k < n_tiles) s += header[(t0 + k) * 8u + 6u];
+        if (t0 + k < n_tiles) s += header[(t0 + k) * words + at_count];
     uint32_t total;
     (void)block_exclusive_sum(s, &total);
     if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
@@ -190,18 +192,66 @@ __global__ __launch_bounds__(256) void bitmap_scan_sums_kernel(uint64_t *block_s
 }
 
 __global__ __launch_bounds__(256) void bitmap_offsets_kernel(uint32_t *__restrict__ header, uint32_t n_tiles,
-                                                             const uint64_t *__restrict__ block_sums)
+                                                             const uint64_t *__restrict__ block_sums, uint32_t words,
+                                                             uint32_t at_count, uint32_t at_first)
 {
     const uint64_t t0 = uint64_t(blockIdx.x) * kScanTilesPerBlock + threadIdx.x * 8u;
     uint32_t count[8], s = 0;
     for (uint32_t k = 0; k < 8u; ++k) {
-        count[k] = t0 + k < n_tiles ? header[(t0 + k) * 8u + 6u] : 0u;
+        count[k] = t0 + k < n_tiles ? header[(t0 + k) * words + at_count] : 0u;
         s += count[k];
     }
     uint32_t total;
     uint64_t at = block_sums[blockIdx.x] + block_exclusive_sum(s, &total);
     for (uint32_t k = 0; k < 8u; ++k)
-        if (t0 + k < n_tiles) { header[(t0 + k) * 8u + 5u] = uint32_t(at); at += count[k]; }
+        if (t0 + k < n_tiles) { header[(t0 + k) * words + at_first] = uint32_t(at); at += count[k]; }
+}
+
+// The same for 8 x 8 tiles of 32-bit elements (Fp32TileB in spmm_mfma_kernel.hpp): header words {rows 0..3, rows
+// 4..7, position of the first stored element, number of stored elements}; four consecutive lanes take two rows each.
+__global__ __launch_bounds__(256) void bitmap_header32_kernel(const uint32_t *__restrict__ tiles, uint32_t *__restrict__ header,
+                                                              uint32_t n_tiles)
+{
+    const uint64_t i = uint64_t(blockIdx.x) * 256u + threadIdx.x;
+    const uint32_t t = uint32_t(i >> 2), quarter = uint32_t(i & 3u), lane = threadIdx.x & 63u;
+    const bool active = i < uint64_t(n_tiles) * 4u;
+    uint32_t mask = 0;
+    if (active) {
+        const bm_u32x4 *src = reinterpret_cast<const bm_u32x4 *>(tiles + size_t(t) * 64u + quarter * 16u);
+#pragma unroll
+        for (uint32_t q = 0; q < 4; ++q) {
+            const bm_u32x4 v = src[q];
+#pragma unroll
+            for (uint32_t e = 0; e < 4; ++e) mask |= (v[e] ? 1u : 0u) << (q * 4u + e);
+        }
+    }
+    const uint32_t first = lane & ~3u;
+    const uint32_t m0 = __shfl(mask, first), m1 = __shfl(mask, first + 1u), m2 = __shfl(mask, first + 2u),
+                   m3 = __shfl(mask, first + 3u);
+    if (!active || quarter != 0u) return;
+    uint32_t *hd = header + size_t(t) * 4u;
+    const uint32_t lo = m0 | m1 << 16, hi = m2 | m3 << 16;
+    hd[0] = lo; hd[1] = hi; hd[2] = 0u;
+    hd[3] = uint32_t(__builtin_popcount(lo)) + uint32_t(__builtin_popcount(hi));
+}
+
+__global__ __launch_bounds__(256) void bitmap_pack32_kernel(const uint32_t *__restrict__ tiles, const uint32_t *__restrict__ header,
+                                                            uint32_t *__restrict__ vals, uint32_t n_tiles)
+{
+    const uint64_t i = uint64_t(blockIdx.x) * 256u + threadIdx.x;
+    if (i >= uint64_t(n_tiles) * 4u) return;
+    const uint32_t t = uint32_t(i >> 2), quarter = uint32_t(i & 3u);
+    const uint32_t *hd = header + size_t(t) * 4u;
+    const uint32_t w = (quarter & 2u) ? hd[1] : hd[0], sh = 16u * (quarter & 1u);
+    uint32_t mask = (w >> sh) & 0xFFFFu;
+    size_t at = size_t(hd[2]) + ((quarter & 2u) ? uint32_t(__builtin_popcount(hd[0])) : 0u) +
+                uint32_t(__builtin_popcount(w & ((1u << sh) - 1u)));
+    const uint32_t *src = tiles + size_t(t) * 64u + quarter * 16u;
+    while (mask) {
+        const uint32_t b = uint32_t(__builtin_ctz(mask));
+        vals[at++] = src[b];
+        mask &= mask - 1u;
+    }
 }
 
 __global__ __launch_bounds__(256) void bitmap_pack_kernel(const uint16_t *__restrict__ tiles, const uint32_t *__restrict__ header,
@@ -221,27 +271,39 @@ __global__ __launch_bounds__(256) void bitmap_pack_kernel(const uint16_t *__rest
     }
 }
 
-hipError_t launch_bitmap_header(const void *tiles, uint32_t *header, uint32_t n_tiles, uint64_t *block_sums, hipStream_t s)
+hipError_t launch_bitmap_header(int elem_bytes, const void *tiles, uint32_t *header, uint32_t n_tiles, uint64_t *block_sums,
+                                hipStream_t s)
 {
     if (!n_tiles) return hipSuccess;
     const uint32_t word_blocks = uint32_t((uint64_t(n_tiles) * 4u + 255u) / 256u);
     const uint32_t n_blocks = (n_tiles + kScanTilesPerBlock - 1u) / kScanTilesPerBlock;
-    bitmap_header_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint16_t *>(tiles), header, n_tiles);
-    bitmap_block_sums_kernel<<<dim3(n_blocks), 256, 0, s>>>(header, n_tiles, block_sums);
+    if (elem_bytes == 2) {
+        bitmap_header_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint16_t *>(tiles), header, n_tiles);
+        bitmap_block_sums_kernel<<<dim3(n_blocks), 256, 0, s>>>(header, n_tiles, block_sums, 8u, 6u);
+    } else {
+        bitmap_header32_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint32_t *>(tiles), header, n_tiles);
+        bitmap_block_sums_kernel<<<dim3(n_blocks), 256, 0, s>>>(header, n_tiles, block_sums, 4u, 3u);
+    }
     bitmap_scan_sums_kernel<<<dim3(1), 256, 0, s>>>(block_sums, n_blocks);
     return hipGetLastError();
 }
 
 uint32_t bitmap_scan_blocks(uint32_t n_tiles) { return (n_tiles + kScanTilesPerBlock - 1u) / kScanTilesPerBlock; }
 
-hipError_t launch_bitmap_pack(const void *tiles, uint32_t *header, void *vals, uint32_t n_tiles, const uint64_t *block_sums,
-                              hipStream_t s)
+hipError_t launch_bitmap_pack(int elem_bytes, const void *tiles, uint32_t *header, void *vals, uint32_t n_tiles,
+                              const uint64_t *block_sums, hipStream_t s)
 {
     if (!n_tiles) return hipSuccess;
     const uint32_t word_blocks = uint32_t((uint64_t(n_tiles) * 4u + 255u) / 256u);
-    bitmap_offsets_kernel<<<dim3(bitmap_scan_blocks(n_tiles)), 256, 0, s>>>(header, n_tiles, block_sums);
-    bitmap_pack_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint16_t *>(tiles), header,
-                                                        static_cast<uint16_t *>(vals), n_tiles);
+    if (elem_bytes == 2) {
+        bitmap_offsets_kernel<<<dim3(bitmap_scan_blocks(n_tiles)), 256, 0, s>>>(header, n_tiles, block_sums, 8u, 6u, 5u);
+        bitmap_pack_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint16_t *>(tiles), header,
+                                                            static_cast<uint16_t *>(vals), n_tiles);
+    } else {
+        bitmap_offsets_kernel<<<dim3(bitmap_scan_blocks(n_tiles)), 256, 0, s>>>(header, n_tiles, block_sums, 4u, 3u, 2u);
+        bitmap_pack32_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint32_t *>(tiles), header,
+                                                              static_cast<uint32_t *>(vals), n_tiles);
+    }
     return hipGetLastError();
 }
 
@@ -257,12 +319,15 @@ hipError_t launch_mfma_f16_bm(const KernelArgs &ka, int V, int prefetch, bool na
                               hipEvent_t mid);
 hipError_t launch_mfma_bf16_bm(const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, hipStream_t s,
                                hipEvent_t mid);
+hipError_t launch_mfma_f32_bm(const KernelArgs &ka, int V, int prefetch, bool narrow, int waves_per_group, hipStream_t s,
+                              hipEvent_t mid);
 
 hipError_t launch_spmm_mfma(int dtype, int layout, int G, const KernelArgs &ka, int V, int prefetch, bool narrow,
                             int waves_per_group, hipStream_t s, hipEvent_t mid)
 {
     if (layout == kLayoutDWB) {
-        if (G != 1 || dtype == kDtypeF32) return hipErrorInvalidValue;
+        if (G != 1) return hipErrorInvalidValue;
+        if (dtype == kDtypeF32) return launch_mfma_f32_bm(ka, V, prefetch, narrow, waves_per_group, s, mid);
         return dtype == kDtypeBf16 ? launch_mfma_bf16_bm(ka, V, prefetch, narrow, waves_per_group, s, mid)
                                    : launch_mfma_f16_bm(ka, V, prefetch, narrow, waves_per_group, s, mid);
     }

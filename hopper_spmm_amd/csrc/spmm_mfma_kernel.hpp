@@ -562,6 +562,75 @@ struct Fp32Tile {
     }
 };
 
+// fp32 storage, single windows, tiles read as bitmap + stored values (the fp32 form of Fp16TileDWB above; the
+// reference's BTCF_MTX with 8 x 8 tiles, src/utils/class.h:55-67 and src/utils/convert.h:83-101): per tile 64 bits,
+// bit 8 r + k set for a stored element, and the stored elements of all tiles one after the other in ascending bit
+// order.  Lane (g, j) needs a[j % 8][g] and a[j % 8][g + 4]: it counts the tile's bits in front of each, loads the
+// two words from there and keeps those whose bit is set.  A power-law graph stores 8 of a tile's 64 elements:
+// 48 bytes instead of 256.
+//   header per step (uniform, scalar loads): the two bitmap words (rows 0..3, rows 4..7), the position of the
+//   tile's first stored element, the number of its stored elements.
+template <int V_>
+struct Fp32TileB : Fp32Tile<V_, 1> {
+    typedef Fp32Tile<V_, 1> Base;
+    static constexpr int V = V_, G = 1;
+    typedef typename Base::BVec BVec;
+    struct Idx { u32x2 ids; uint32_t lo, hi, first; };
+    struct AVec { uint32_t w0, w1, keep0, keep1; };    // the two words at the lane's positions; all ones where the bit is set
+    struct Lane : Base::Lane {
+        const uint32_t *header;                        // 4 words per step
+        const uint32_t *vals;
+        uint32_t upper, shift, low_mask;               // rows 4..7; the lane's first bit inside its word; the bits below it
+        __device__ __forceinline__ void init(uint32_t lane, const void *values, const uint32_t *ids)
+        {
+            Base::Lane::init(lane, values, ids);
+            vals = static_cast<const uint32_t *>(values);
+            const uint32_t r = this->j & 7u;
+            upper = r >> 2;
+            shift = 8u * (r & 3u) + this->g;
+            low_mask = (1u << shift) - 1u;
+        }
+        __device__ __forceinline__ void bind_bitmap(const uint32_t *h) { header = h; }
+    };
+    __device__ static __forceinline__ Idx load_idx(const Lane &L, uint32_t step)
+    {
+        Idx I;
+        I.ids = *reinterpret_cast<const u32x2 *>(L.idx_src + size_t(step) * 8u);
+        const const_u32_ptr h = as_const(L.header) + size_t(step) * 4u;      // uniform: scalar loads
+        I.lo = h[0]; I.hi = h[1]; I.first = h[2];
+        return I;
+    }
+    template <class GT>
+    __device__ static __forceinline__ void load_tile(const Lane &L, uint32_t, const Idx &I, const GT &gat,
+                                                     BVec &b0, BVec &b1, BVec &, BVec &, AVec &a)
+    {
+        b0 = *reinterpret_cast<const BVec *>(gat.row(I.ids[0]));
+        b1 = *reinterpret_cast<const BVec *>(gat.row(I.ids[1]));
+        const uint32_t w = L.upper ? I.hi : I.lo;
+        const uint32_t before0 = (L.upper ? uint32_t(__builtin_popcount(I.lo)) : 0u) + uint32_t(__builtin_popcount(w & L.low_mask));
+        const uint32_t four = (w >> L.shift) & 31u;                      // bits of columns g .. g + 4
+        const uint32_t before1 = before0 + uint32_t(__builtin_popcount(four & 15u));
+        // (a position behind the tile's last element, for a bit that is not set, still lies inside the array: it
+        // ends with one spare element)
+        const uint32_t *src = L.vals + size_t(I.first);
+        a.w0 = src[before0];
+        a.w1 = src[before1];
+        a.keep0 = ((four & 1u) ? 0xFFFFFFFFu : 0u) & L.a_mask;
+        a.keep1 = ((four & 16u) ? 0xFFFFFFFFu : 0u) & L.a_mask;
+    }
+    __device__ static __forceinline__ void mma(const Lane &, const BVec &b0, const BVec &b1, const BVec &,
+                                               const BVec &, const AVec &a, f32x4 (&acc)[V])
+    {
+        const uint32_t w0 = a.w0 & a.keep0, w1 = a.w1 & a.keep1;
+        const float a0 = __builtin_bit_cast(float, w0), a1 = __builtin_bit_cast(float, w1);
+        Base::template mma_one<0, 0>(a0, b0, acc); Base::template mma_one<0, 1>(a0, b0, acc);
+        Base::template mma_one<0, 2>(a0, b0, acc); Base::template mma_one<0, 3>(a0, b0, acc);
+        Base::template mma_one<0, 0>(a1, b1, acc); Base::template mma_one<0, 1>(a1, b1, acc);
+        Base::template mma_one<0, 2>(a1, b1, acc); Base::template mma_one<0, 3>(a1, b1, acc);
+    }
+};
+template <int V> struct TileTraits<Fp32TileB<V>> { static constexpr bool kBitmap = true; };
+
 // ---------------------------------------------------------------------------
 // Main kernel: one wave per (step range, feature block).
 // ---------------------------------------------------------------------------

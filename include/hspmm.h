@@ -237,7 +237,7 @@ typedef struct {
     uint32_t n_panel_wide_units;    /* of those: units of three or four windows */
     uint32_t last_kernel_family;    /* what the last hspmm_run launched: 0 nothing yet, 1 all-shapes kernel, 2 gather (MFMA) kernels,
                                        3 LDS-staging kernels, 4 clear only (matrix without entries) */
-    uint32_t gather_bitmap;         /* 1: the gather kernels read this plan's tiles as bitmap + stored elements (single 16-bit
+    uint32_t gather_bitmap;         /* 1: the gather kernels read this plan's tiles as bitmap + stored elements (single
                                      * windows with few stored elements per tile), 0: as uncompressed tiles */
     uint32_t bitmap_from_caller;    /* 1: the plan was made from bitmap tiles (hspmm_create_bitmap / _grouped) and uploaded them as they
                                      * came - header words from tcBit and nnzOffset, the stored elements untouched; the plain tiles

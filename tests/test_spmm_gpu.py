@@ -1549,12 +1549,12 @@ def test_lds_staging_hands_every_b_row_to_its_column(torch_cuda, hs, dtype):
 
 
 # ------------------------------------------------------------------ bitmap tiles in the gather kernels
-@pytest.mark.parametrize("dtype", [0, 2])
+@pytest.mark.parametrize("dtype", [0, 1, 2])
 def test_gather_kernels_read_bitmap_tiles(torch_cuda, hs, oracle, dtype):
-    """Single 16-bit windows with few stored elements per tile are kept on the device as the reference's
-    bitmap tiles (128 bits per 8 x 16 tile + the stored elements) and expanded in registers by the gather
-    kernels.  The MFMA inputs are those of the uncompressed tiles, so the results are bit-identical; stored
-    zeros, negative zeros, full tiles and tiles with one element are all in here."""
+    """Single windows with few stored elements per tile are kept on the device as the reference's bitmap
+    tiles (128 bits per 8 x 16 tile, 64 per 8 x 8 tile of fp32 storage, + the stored elements) and expanded in
+    registers by the gather kernels.  The MFMA inputs are those of the uncompressed tiles, so the results are
+    bit-identical; stored zeros, negative zeros, full tiles and tiles with one element are all in here."""
     rng = np.random.default_rng(120 + dtype)
     rows, cols = 530, 1500
     A = random_csr(rng, rows, cols, 0.01, dtype, empty_row_prob=0.1, heavy_rows=(7, 300))
@@ -1563,22 +1563,30 @@ def test_gather_kernels_read_bitmap_tiles(torch_cuda, hs, oracle, dtype):
     v[3::31] = -0.0                                  # negative zeros are
     A["values"] = encode(v, dtype)
     b = convert(hs, A)
-    for N in (64, 128, 256, 512):
+    # (fp32 storage: every width of the lanes' loads - 1, 2, 4 words - has a bitmap form; kernel mode 3 keeps
+    # the plan off the LDS-staging kernels, which fp32 storage prefers from this density on)
+    for N in (64, 128, 256, 512) if dtype != 1 else (8, 16, 24, 32, 64, 128, 256):
         B = make_b(rng, cols, N, dtype)
         ref, mag = oracle_spmm(oracle, A, B, N)
         got = {}
         for use in ("0", "1"):
             os.environ["HSPMM_GATHER_BITMAP"] = use
+            hs.set_kernel_mode(3 if dtype == 1 else 0)
             try:
                 plan = hs.Plan(b)
+                got[use] = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
             finally:
+                hs.set_kernel_mode(0)
                 os.environ.pop("HSPMM_GATHER_BITMAP", None)
-            got[use] = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
             info = plan.info()
             plan.close()
             assert info["last_kernel_family"] == 2 and info["gather_bitmap"] == int(use)
-        assert_parity(got["0"], ref, mag, dtype, "tiles N=%d" % N)
-        assert np.array_equal(got["1"], got["0"]), "bitmap tiles differ at N=%d" % N
+        hs.set_kernel_mode(3 if dtype == 1 else 0)       # (the tolerance of fp32 storage depends on the kernels in use)
+        try:
+            assert_parity(got["0"], ref, mag, dtype, "tiles N=%d" % N)
+        finally:
+            hs.set_kernel_mode(0)
+        assert np.array_equal(got["1"].view(np.uint8), got["0"].view(np.uint8)), "bitmap tiles differ at N=%d" % N
     # dense 8 x 16 tiles (every bit set) next to empty windows, forced through the bitmap path
     D = np.zeros((64, 96))
     D[0:8, 0:16] = rng.integers(1, 4, (8, 16))
