@@ -1371,7 +1371,8 @@ int hspmm_panel_units_preview(int dtype, uint32_t rows, uint32_t cols, uint32_t 
 
 namespace {
 
-// The caller's bitmap tiles (16-bit element types, HSPMM_BITS_PER_TILE words): reference BTCF_MTX, src/utils/class.h:55-67.
+// The caller's bitmap tiles (HSPMM_BITS_PER_TILE words: two per 8 x 16 tile, one per 8 x 8 tile of fp32 storage):
+// reference BTCF_MTX, src/utils/class.h:55-67.
 struct BitmapSource { const uint32_t *nnzOffset; const uint64_t *tcBit; const void *data; };
 // The ends of the caller's groups (groupOffset of the reference's GBTCF_MTX, src/utils/class.h:93-108), n + 1 of them.
 struct GroupCuts { const uint32_t *offsets; uint32_t n_groups; };
@@ -1379,12 +1380,24 @@ constexpr int kNeedsPlainTiles = -1000;     // create_plan with a BitmapSource: 
 
 // Header of the gather kernels' bitmap stream straight from the caller's arrays; returns the first tile whose bit
 // count differs from its nnzOffset span (HSPMM_IDX_MAX: none).
-uint32_t bitmap_header_from_caller(uint32_t T, const BitmapSource &src, hspmm_host::ZeroedBuffer<uint32_t> &header)
+uint32_t bitmap_header_from_caller(uint32_t T, uint32_t elem, const BitmapSource &src, hspmm_host::ZeroedBuffer<uint32_t> &header)
 {
-    header = hspmm_host::ZeroedBuffer<uint32_t>(size_t(T) * 8u);
+    header = hspmm_host::ZeroedBuffer<uint32_t>(size_t(T) * (elem == 2u ? 8u : 4u));
     std::atomic<uint32_t> first_bad{HSPMM_IDX_MAX};
     hspmm_host::parallel_blocks(T, 4096, [&](size_t tb, size_t te) {
         for (size_t t = tb; t < te; ++t) {
+            if (elem == 4u) {
+                // 8 x 8 tiles of 32-bit elements: one 64-bit word per tile; header = rows 0..3, rows 4..7, position, count
+                uint32_t *hd = header.data() + t * 4u;
+                hd[0] = uint32_t(src.tcBit[t]); hd[1] = uint32_t(src.tcBit[t] >> 32);
+                hd[2] = src.nnzOffset[t];
+                hd[3] = uint32_t(__builtin_popcount(hd[0])) + uint32_t(__builtin_popcount(hd[1]));
+                if (src.nnzOffset[t + 1] < src.nnzOffset[t] || src.nnzOffset[t + 1] - src.nnzOffset[t] != hd[3]) {
+                    uint32_t seen = first_bad.load();
+                    while (uint32_t(t) < seen && !first_bad.compare_exchange_weak(seen, uint32_t(t))) {}
+                }
+                continue;
+            }
             uint32_t *hd = header.data() + t * 8u;
             hd[0] = uint32_t(src.tcBit[2 * t]); hd[1] = uint32_t(src.tcBit[2 * t] >> 32);
             hd[2] = uint32_t(src.tcBit[2 * t + 1]); hd[3] = uint32_t(src.tcBit[2 * t + 1] >> 32);
@@ -1401,7 +1414,7 @@ uint32_t bitmap_header_from_caller(uint32_t T, const BitmapSource &src, hspmm_ho
     return first_bad.load();
 }
 
-// hspmm_create; with `bitmap` (16-bit element types, data == nullptr) the tiles come as the caller's bitmap arrays,
+// hspmm_create; with `bitmap` (data == nullptr) the tiles come as the caller's bitmap arrays,
 // which are uploaded as they are, kept as the gather kernels' bitmap stream and expanded on the device for the
 // kernels that read plain tiles.  Returns kNeedsPlainTiles when the plan would need the tiles on the host
 // (windows paired through equal column lists; the caller then expands them).
@@ -1461,21 +1474,21 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
             // the caller's bitmap tiles: header from tcBit / nnzOffset, the stored elements as they are (and four
             // more: a lane of the gather kernels reads 8 bytes from its first element), plain tiles by a kernel
             hspmm_host::ZeroedBuffer<uint32_t> header;
-            const uint32_t bad = bitmap_header_from_caller(total_tiles, *bitmap, header);
+            const uint32_t bad = bitmap_header_from_caller(total_tiles, elem, *bitmap, header);
             if (bad != HSPMM_IDX_MAX)
                 return bail(fail(HSPMM_ERR_INVALID, "tile %u: %s", bad, "the bit count of tcBit differs from the nnzOffset span"));
-            const size_t stored = bitmap->nnzOffset[total_tiles];
-            if (stored + 4u >= (size_t(1) << 31)) return bail(kNeedsPlainTiles);      // positions are 32-bit
+            const size_t stored = bitmap->nnzOffset[total_tiles], spare = 8u / elem;
+            if (stored + spare >= (size_t(1) << 31)) return bail(kNeedsPlainTiles);      // positions are 32-bit
             if ((rc = upload(&p->bm.d_header, header.data(), header.size(), &p->fixed_bytes))) return bail(rc);
-            uint16_t *dv = nullptr;
-            HSPMM_HIP_OR(hipMalloc(reinterpret_cast<void **>(&dv), (stored + 4u) * 2u), bail);
-            p->bm.d_vals = dv; p->bm.stored = stored; p->fixed_bytes += (stored + 4u) * 2u;
-            if (stored) HSPMM_HIP_OR(hipMemcpy(dv, bitmap->data, stored * 2u, hipMemcpyHostToDevice), bail);
-            HSPMM_HIP_OR(hipMemset(dv + stored, 0, 8), bail);
+            char *dv = nullptr;
+            HSPMM_HIP_OR(hipMalloc(reinterpret_cast<void **>(&dv), (stored + spare) * elem), bail);
+            p->bm.d_vals = dv; p->bm.stored = stored; p->fixed_bytes += (stored + spare) * elem;
+            if (stored) HSPMM_HIP_OR(hipMemcpy(dv, bitmap->data, stored * elem, hipMemcpyHostToDevice), bail);
+            HSPMM_HIP_OR(hipMemset(dv + stored * elem, 0, 8), bail);
             uint8_t *dd = nullptr;
             HSPMM_HIP_OR(hipMalloc(reinterpret_cast<void **>(&dd), size_t(total_tiles) * 256u), bail);
             p->d_data = dd; p->fixed_bytes += size_t(total_tiles) * 256u;
-            HSPMM_HIP_OR(hspmm::launch_expand_bitmap(p->bm.d_header, dv, dd, total_tiles, nullptr), bail);
+            HSPMM_HIP_OR(hspmm::launch_expand_bitmap(int(elem), p->bm.d_header, dv, dd, total_tiles, nullptr), bail);
             HSPMM_HIP_OR(hipStreamSynchronize(nullptr), bail);
             p->bm.from_caller = true;
         }
@@ -1510,17 +1523,13 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
         // (single fp32 windows: decided below, once it is known whether the gather kernels of this plan read
         // bitmap tiles - then nothing reads tiles in lane order)
         const bool lane_tiles_later = dtype == HSPMM_TF32 && st.G == 1;
-        auto upload_lane_order_tiles = [&]() -> int {
-            const hspmm_host::ZeroedBuffer<uint32_t> tiles = lane_order_tiles(st, dtype, rowOffset, data);
-            uint32_t *dt = nullptr;
-            const int urc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes);
-            p->d_tiles = dt;
-            return urc;
-        };
         if (dtype != HSPMM_TF32 && st.G == 1) {
             p->d_tiles = p->d_data;                 // the caller's tile layout already is the lane order
         } else if (!lane_tiles_later) {
-            if ((rc = upload_lane_order_tiles())) return bail(rc);
+            const hspmm_host::ZeroedBuffer<uint32_t> tiles = lane_order_tiles(st, dtype, rowOffset, data);
+            uint32_t *dt = nullptr;
+            if ((rc = upload(&dt, tiles.data(), tiles.size(), &p->fixed_bytes))) return bail(rc);
+            p->d_tiles = dt;
         }
         timer.mark("step stream (ids, tiles)");
         // Single 16-bit windows with few stored elements per tile (graphs: 16 of 128): the gather kernels read the
@@ -1531,7 +1540,7 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
             const size_t stored = size_t(p->bm.stored);
             p->bm.built = total_tiles && p->cfg.gather_bitmap != 0 &&
                           (p->cfg.gather_bitmap > 0 ||
-                           (stored * 3u < size_t(total_tiles) * 128u && size_t(total_tiles) * 256u >= (size_t(8) << 20)));
+                           (stored * 3u < size_t(total_tiles) * 8u * cw && size_t(total_tiles) * 256u >= (size_t(8) << 20)));
             if (!p->bm.built) {
                 (void)hipFree(p->bm.d_header); (void)hipFree(p->bm.d_vals);
                 p->bm.d_header = nullptr; p->bm.d_vals = nullptr;
@@ -1558,8 +1567,13 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
                 if ((rc = bitmap_from_uploaded_tiles(p, total_tiles))) return bail(rc);
             }
         }
-        if (lane_tiles_later && !(p->bm.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 3))) {
-            if ((rc = upload_lane_order_tiles())) return bail(rc);
+        if (lane_tiles_later && total_tiles && !(p->bm.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 3))) {
+            // single fp32 windows: steps are the caller's tiles in the caller's order; a kernel re-orders each for the lanes
+            void *dt = nullptr;
+            HSPMM_HIP_OR(hipMalloc(&dt, size_t(total_tiles) * 256u), bail);
+            p->d_tiles = dt; p->fixed_bytes += size_t(total_tiles) * 256u;
+            HSPMM_HIP_OR(hspmm::launch_lane_order32(p->d_data, dt, total_tiles, nullptr), bail);
+            HSPMM_HIP_OR(hipStreamSynchronize(nullptr), bail);
         }
         timer.mark("bitmap tiles");
         p->h_unitOffset = st.unitOffset;
@@ -1737,12 +1751,11 @@ static int create_from_bitmap(hspmm_plan **out, int dtype, uint32_t rows, uint32
     if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16)
         return fail(HSPMM_ERR_INVALID, "unknown dtype %d", dtype);
     if (total_tiles && (!nnzOffset || !tcBit)) return fail(HSPMM_ERR_INVALID, "null nnzOffset or tcBit");
-    // Sparse windows of 16-bit elements (graphs) never need their tiles on the host: the bitmap arrays go to the
-    // device as they are - the gather kernels read them (spmm_mfma_kernel.hpp, Fp16TileDWB) - and a kernel
-    // expands them for the kernels that read plain tiles.  Dense windows (the LDS-panel stream re-tiles them on
-    // the host), paired windows and fp32 storage are expanded here first.
-    if (dtype != HSPMM_TF32 && eff_row_windows && total_tiles && rowOffset && nnzOffset[0] == 0 &&
-        (!nnzOffset[total_tiles] || data)) {
+    // Sparse windows (graphs) never need their tiles on the host: the bitmap arrays go to the device as they are -
+    // the gather kernels read them (spmm_mfma_kernel.hpp, Fp16TileDWB and Fp32TileB) - and kernels expand them
+    // for the kernels that read plain tiles.  Dense windows (the LDS-panel stream re-tiles them on the host) and
+    // paired windows are expanded here first.
+    if (eff_row_windows && total_tiles && rowOffset && nnzOffset[0] == 0 && (!nnzOffset[total_tiles] || data)) {
         int mode;
         { std::lock_guard<std::mutex> lk(g_cfg_mutex); mode = g_cfg.kernel_mode; }
         const double density = double(total_tiles) / (double(eff_row_windows) * double((uint64_t(cols) + 127u) / 128u));

@@ -96,8 +96,12 @@ struct PanelArgs {
 hipError_t launch_spmm_panel(int dtype, int G, bool split, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka,
                              int units, hipStream_t s, hipEvent_t mid);
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
-// bitmap tiles (header, stored elements: see KernelArgs::bm_header) -> plain 8 x 16 tiles of 16-bit elements
-hipError_t launch_expand_bitmap(const uint32_t *header, const void *vals, void *tiles, uint32_t n_tiles, hipStream_t s);
+// bitmap tiles (header, stored elements: see KernelArgs::bm_header and, for 32-bit elements, launch_bitmap_header
+// below) -> plain tiles (8 x 16 of 16-bit elements, 8 x 8 of 32-bit elements)
+hipError_t launch_expand_bitmap(int elem_bytes, const uint32_t *header, const void *vals, void *tiles, uint32_t n_tiles,
+                                hipStream_t s);
+// plain 8 x 8 tiles of 32-bit elements, single windows -> the order the lanes of the fp32 gather kernels read them in
+hipError_t launch_lane_order32(const void *tiles, void *out, uint32_t n_tiles, hipStream_t s);
 // plain tiles -> bitmap tiles (8 x 16 tiles of 16-bit elements, elem_bytes = 2: 8 header words per tile, see
 // KernelArgs::bm_header; 8 x 8 tiles of 32-bit elements, elem_bytes = 4: 4 header words - rows 0..3, rows 4..7,
 // position of the first stored element, number of stored elements), in two steps with the host in between (it

@@ -91,11 +91,50 @@ __global__ __launch_bounds__(256) void expand_bitmap_kernel(const uint32_t *__re
     tiles[size_t(t) * 128u + b] = ((w >> bit) & 1u) ? vals[size_t(h[5]) + before] : uint16_t(0);
 }
 
-hipError_t launch_expand_bitmap(const uint32_t *header, const void *vals, void *tiles, uint32_t n_tiles, hipStream_t s)
+// The same for 8 x 8 tiles of 32-bit elements (header words: rows 0..3, rows 4..7, position of the first stored
+// element, count): one thread per tile element.
+__global__ __launch_bounds__(256) void expand_bitmap32_kernel(const uint32_t *__restrict__ header,
+                                                              const uint32_t *__restrict__ vals,
+                                                              uint32_t *__restrict__ tiles, uint32_t n_tiles)
+{
+    const uint32_t t = blockIdx.x * 4u + (threadIdx.x >> 6), b = threadIdx.x & 63u;
+    if (t >= n_tiles) return;
+    const uint32_t *h = header + size_t(t) * 4u;
+    const uint32_t upper = b >> 5, w = h[upper], bit = b & 31u;
+    const uint32_t before = (upper ? uint32_t(__builtin_popcount(h[0])) : 0u) + uint32_t(__builtin_popcount(w & ((1u << bit) - 1u)));
+    tiles[size_t(t) * 64u + b] = ((w >> bit) & 1u) ? vals[size_t(h[2]) + before] : 0u;
+}
+
+hipError_t launch_expand_bitmap(int elem_bytes, const uint32_t *header, const void *vals, void *tiles, uint32_t n_tiles,
+                                hipStream_t s)
 {
     if (!n_tiles) return hipSuccess;
-    expand_bitmap_kernel<<<dim3((n_tiles + 1u) / 2u), 256, 0, s>>>(header, static_cast<const uint16_t *>(vals),
-                                                                  static_cast<uint16_t *>(tiles), n_tiles);
+    if (elem_bytes == 2)
+        expand_bitmap_kernel<<<dim3((n_tiles + 1u) / 2u), 256, 0, s>>>(header, static_cast<const uint16_t *>(vals),
+                                                                      static_cast<uint16_t *>(tiles), n_tiles);
+    else
+        expand_bitmap32_kernel<<<dim3((n_tiles + 3u) / 4u), 256, 0, s>>>(header, static_cast<const uint32_t *>(vals),
+                                                                        static_cast<uint32_t *>(tiles), n_tiles);
+    return hipGetLastError();
+}
+
+// 8 x 8 tiles of 32-bit elements as the caller holds them ([row r][column k]) -> the order the lanes of the fp32
+// gather kernels read them in, single windows: [row r][g][2] = (a[r][g], a[r][g + 4]) (Fp32Tile in
+// spmm_mfma_kernel.hpp).  One thread per element.
+__global__ __launch_bounds__(256) void lane_order32_kernel(const uint32_t *__restrict__ tiles, uint32_t *__restrict__ out,
+                                                           uint32_t n_tiles)
+{
+    const uint32_t t = blockIdx.x * 4u + (threadIdx.x >> 6), o = threadIdx.x & 63u;
+    if (t >= n_tiles) return;
+    const uint32_t r = o >> 3, g = (o >> 1) & 3u, second = o & 1u;
+    out[size_t(t) * 64u + o] = tiles[size_t(t) * 64u + r * 8u + g + 4u * second];
+}
+
+hipError_t launch_lane_order32(const void *tiles, void *out, uint32_t n_tiles, hipStream_t s)
+{
+    if (!n_tiles) return hipSuccess;
+    lane_order32_kernel<<<dim3((n_tiles + 3u) / 4u), 256, 0, s>>>(static_cast<const uint32_t *>(tiles),
+                                                                 static_cast<uint32_t *>(out), n_tiles);
     return hipGetLastError();
 }
 

@@ -393,10 +393,10 @@ int hspmm_btcf_relayout_fill(int dtype, uint32_t col_window, int transposed, uin
 
 /* Same as hspmm_create for a matrix held as bitmap tiles (row-major bit order,
  * HSPMM_BITS_PER_TILE).  Results are those of hspmm_create on the expanded arrays, bit for bit.
- * Sparse windows of 16-bit elements go to the device as they are: the gather kernels read the
- * caller's tcBit words and stored elements, and a kernel writes the plain tiles other kernels read
- * (hspmm_plan_info.bitmap_from_caller = 1).  Dense windows, windows paired through equal column
- * lists and fp32 storage are expanded on the host first. */
+ * Sparse windows go to the device as they are: the gather kernels read the caller's tcBit words
+ * and stored elements, and a kernel writes the plain tiles other kernels read
+ * (hspmm_plan_info.bitmap_from_caller = 1).  Dense windows and windows paired through equal column
+ * lists are expanded on the host first. */
 int hspmm_create_bitmap(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
                         uint32_t eff_row_windows, uint32_t total_tiles,
                         const uint32_t *rowOffset, const uint32_t *nnzOffset, const uint32_t *tcA2B,

@@ -291,14 +291,14 @@ def test_plans_from_bitmap_and_grouped_formats(torch_cuda, hs, oracle, dtype):
             for name, fmt in (("bitmap", bitmap), ("grouped", grouped), ("grouped-32", hs.bitmap_to_grouped(bitmap))):
                 got = gpu_spmm(torch_cuda, hs, fmt, B, N)
                 assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "%s %dx%d N=%d" % (name, rows, cols, N)
-        # Sparse windows of 16-bit elements: the bitmap arrays go to the device as they are (no expansion on the
+        # Sparse windows: the bitmap arrays go to the device as they are (no expansion on the
         # host); the kernels that read plain tiles (N = 8: the all-shapes kernel) run on what a kernel expanded
         # there, and with the bitmap stream forced the gather kernels read the caller's own words and elements.
         sparse = plain["total_tiles"] < 1.2 * plain["eff_row_windows"] * ((cols + 127) // 128)     # (else: LDS-staging stream, built on the host)
         plan = hs.Plan(bitmap)
-        assert plan.info()["bitmap_from_caller"] == (1 if dtype != 1 and sparse else 0), (rows, cols)
+        assert plan.info()["bitmap_from_caller"] == (1 if sparse else 0), (rows, cols)
         plan.close()
-        if dtype != 1 and sparse:
+        if sparse:
             os.environ["HSPMM_GATHER_BITMAP"] = "1"
             try:
                 forced = hs.Plan(bitmap)
