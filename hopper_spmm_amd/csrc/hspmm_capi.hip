@@ -855,6 +855,10 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     timer.mark("  panel: units of windows");
     const uint32_t U = uint32_t(st.unitRow.size());
     const uint32_t T = rowOffset[W];
+    // Two units per consumer wave (merge_unit_pairs below): the second unit's first step follows whatever step of
+    // the first unit lies in front of it, so it, too, may be at most kMaxJump panels from its predecessor - every
+    // unit of such a stream gets its all-zero steps from panel 0 on, not only behind its first step.
+    const bool tall_stream = rw == 32 && st.G <= 2 && U >= 2 && (p->cfg.panel_tall > 0 || p->cfg.panel_packed > 0);
     const size_t es = p->elem, src_tile_bytes = size_t(8) * cw * es, tile_bytes = size_t(8) * rw * es;
     // Two passes over the windows, both on all cores: the steps every window gets, then the steps.
     std::vector<uint32_t> rt_rowOffset(size_t(W) + 1, 0u), rt_panel;
@@ -874,7 +878,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
             while (i < nreal) {
                 const uint32_t pn = col[i] / KP, a = i;
                 while (i < nreal && col[i] / KP == pn) ++i;
-                while (tiles && pn - last_pn > kMaxJump) { last_pn += kMaxJump; ++tiles; }
+                while ((tiles || tall_stream) && pn - last_pn > kMaxJump) { last_pn += kMaxJump; ++tiles; }
                 tiles += (i - a + rw - 1) / rw;
                 last_pn = pn;
             }
@@ -896,7 +900,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
             while (i < nreal) {
                 const uint32_t pn = col[i] / KP, a = i;
                 while (i < nreal && col[i] / KP == pn) ++i;
-                while (at > rt_rowOffset[w] && pn - last_pn > kMaxJump) {   // all-zero step that only carries the jump
+                while ((at > rt_rowOffset[w] || tall_stream) && pn - last_pn > kMaxJump) {   // all-zero step that only carries the jump
                     last_pn += kMaxJump;
                     rt_panel[at++] = last_pn;
                 }
@@ -1009,7 +1013,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     // (hspmm_set_panel_stream, HSPMM_PANEL_TALL / HSPMM_PANEL_PACKED).
     timer.mark("  panel: tiles in lane order");
     bool tall = false, packed = false;
-    if (rw == 32 && ps.G <= 2 && U >= 2 && (p->cfg.panel_tall > 0 || p->cfg.panel_packed > 0)) {
+    if (tall_stream) {
         tall = true;
         const size_t tile_words = split ? 512u : 256u;
         merge_unit_pairs(U, NP, tile_words, ps.unitOffset, poff, step_panel, ids, tiles);
@@ -1868,7 +1872,8 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     pa.masks = pl.d_masks; pa.vals = pl.d_vals; pa.step_voff = pl.d_step_voff;
     pa.B = dB; pa.C = dC;
     pa.n_units = pl.n_units; pa.rows = p->rows; pa.cols = p->cols; pa.N = N;
-    pa.n_feat_blocks = N / (hspmm::kPanelRowBytes / p->elem);
+    const uint32_t block = hspmm::kPanelRowBytes / p->elem;
+    pa.n_feat_blocks = (N + block - 1u) / block;                   // (the last block may end inside: run_impl says when)
     pa.n_panels = pl.n_panels;
     // The workgroup shape: code 14 / 12 = that many consumer waves and two producers, 13 = 12 consumers and
     // four producers (few enough registers for two workgroups per compute unit, which the 4x4x1 fp32 kernel
@@ -1988,7 +1993,11 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
         // (the producers address a panel of B - up to 256 rows - with 32-bit offsets)
         const bool offsets_fit = uint64_t(N) * p->elem < (uint64_t(1) << 24);
-        if (pays && offsets_fit && N % block_feat == 0 && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
+        // Whole blocks of features, or - the kernels built on the 16-bit MFMA, whose lanes own one feature per
+        // accumulator - any multiple of 16 from one block on (from 16 on for fp32 storage, whose gather kernels
+        // multiply at a sixteenth of the rate): the last block's missing features are zeros in LDS and are not stored.
+        const bool ragged_ok = (p->cw == 16 || p->panel.split) && N % 16u == 0 && (p->dtype == HSPMM_TF32 || N >= block_feat);
+        if (pays && offsets_fit && (N % block_feat == 0 || ragged_ok) && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
     }
     // Feature blocks with XCDs of their own (see spmm_mfma_kernel): pays when B is far larger than an
     // XCD's 4 MB L2, so that what an L2 can keep of it decides the hit rate of the gathers (power-law

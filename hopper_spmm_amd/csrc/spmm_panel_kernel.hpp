@@ -193,11 +193,13 @@ struct Fp16Tr {
     typedef typename HalfOps<BF>::elem_t elem_t;
     struct Lane {
         uint32_t g, j;
+        uint32_t p_valid;                          // accumulators whose feature 16 p + j exists (8 unless N ends inside the block)
         const uint32_t *a_src;
         const uint32_t *idx_src;
         __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
         {
             g = lane >> 4; j = lane & 15u;
+            p_valid = 8u;
             a_src = reinterpret_cast<const uint32_t *>(tiles) + lane * 4u;
             idx_src = ids + (lane >> 2);           // four neighbouring lanes read one word
         }
@@ -215,7 +217,8 @@ struct Fp16Tr {
             if (active && row < rows) {
                 elem_t *dst = reinterpret_cast<elem_t *>(c_lane + size_t(row) * row_bytes);
 #pragma unroll
-                for (int p = 0; p < 8; ++p) stream_store(dst + 16 * p, (elem_t)acc[8 * (W0 >> 1) + p][e]);
+                for (int p = 0; p < 8; ++p)
+                    if (uint32_t(p) < L.p_valid) stream_store(dst + 16 * p, (elem_t)acc[8 * (W0 >> 1) + p][e]);
             }
         }
     }
@@ -226,7 +229,8 @@ struct Fp16Tr {
         for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) {
             elem_t *dst = reinterpret_cast<elem_t *>(c_lane + size_t(r) * row_bytes);
 #pragma unroll
-            for (int p = 0; p < 8; ++p) stream_store(dst + 16 * p, (elem_t)0.f);
+            for (int p = 0; p < 8; ++p)
+                if (uint32_t(p) < L.p_valid) stream_store(dst + 16 * p, (elem_t)0.f);
         }
     }
 };
@@ -339,11 +343,13 @@ struct Fp32Split {
     typedef u32x8 AVec;
     struct Lane {
         uint32_t g, j;
+        uint32_t p_valid;                          // accumulators whose feature 16 p + j exists (4 unless N ends inside the block)
         const uint32_t *a_src;
         const uint32_t *idx_src;
         __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
         {
             g = lane >> 4; j = lane & 15u;
+            p_valid = 4u;
             a_src = reinterpret_cast<const uint32_t *>(tiles) + lane * 8u;
             idx_src = ids + (lane >> 2);           // four neighbouring lanes read one word
         }
@@ -359,7 +365,10 @@ struct Fp32Split {
             if (active && row < rows) {
                 float *dst = reinterpret_cast<float *>(c_lane + size_t(row) * row_bytes);
 #pragma unroll
-                for (int p = 0; p < 4; ++p) { const float v = acc[4 * (W0 >> 1) + p][e]; stream_store(dst + 16 * p, v); }
+                for (int p = 0; p < 4; ++p) {
+                    const float v = acc[4 * (W0 >> 1) + p][e];
+                    if (uint32_t(p) < L.p_valid) stream_store(dst + 16 * p, v);
+                }
             }
         }
     }
@@ -370,7 +379,8 @@ struct Fp32Split {
         for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) {
             float *dst = reinterpret_cast<float *>(c_lane + size_t(r) * row_bytes);
 #pragma unroll
-            for (int p = 0; p < 4; ++p) stream_store(dst + 16 * p, 0.f);
+            for (int p = 0; p < 4; ++p)
+                if (uint32_t(p) < L.p_valid) stream_store(dst + 16 * p, 0.f);
         }
     }
 };
@@ -642,7 +652,10 @@ void spmm_panel_kernel(const PanelArgs pa)
         const uint32_t pt = threadIdx.x - uint32_t(NC) * 64u;       // 0 .. NPW*64-1
         // piece c = pt + i * NPW*64 is bytes [16c, 16c + 16) of the image: row c / 16, 16-byte column c % 16
         const char *b_block = reinterpret_cast<const char *>(pa.B) + size_t(fb) * kPanelRowBytes;
-        const uint32_t piece_row0 = pt >> 4, col_bytes = (pt & 15u) * 16u;
+        // (a feature dimension that ends inside this block: a piece behind a row's end is read from the row's
+        // first piece instead - the features it would feed are never stored, and no load leaves the row)
+        const uint32_t piece_row0 = pt >> 4;
+        const uint32_t col_bytes = size_t(fb) * kPanelRowBytes + (pt & 15u) * 16u < row_bytes ? (pt & 15u) * 16u : 0u;
         // Addresses: the panel's first row (the same in all lanes) plus 32-bit offsets inside the panel
         // (the host checks that a panel of B spans less than 4 GB).  Rows past the matrix are never
         // referenced: their loads are bent to the matrix's last row.
@@ -865,6 +878,7 @@ void spmm_panel_kernel(const PanelArgs pa)
     for (; owed; --owed) panel_barrier();
 
     if (!has_unit) return;
+    set_valid_accumulators<TT>(L, pa.N, fb);        // (here, not at the top: nothing of it lives through the steps)
     // Stores unit `unit` from the sums in `sums` (or leaves them as this chunk's partial sums).
     auto finish = [&](const uint32_t unit, f32x4 (&sums)[Ops::kLive]) __attribute__((always_inline)) {
         Ops::fold(sums);

@@ -64,25 +64,31 @@ def oracle_spmm(oracle, A, B, N):
 
 def assert_parity(got, ref, absdot, dtype, what="", tight=True):
     """fp16 / bf16: 1e-2 relative; fp32-storage ("tf32") variant: 1e-3 relative.  Where the sum
-    cancels, an absolute term in units of sum |a||b|: 1e-5 for fp32 accumulation of exact products,
-    and for the tf32 variant 2^-16 more unless the kernel mode guarantees fp32 products: its
-    LDS-staging kernels multiply bf16 hi + lo parts in three products.  The product they leave out,
-    a_lo b_lo, has the sign of a b and at most 2^-14 of its size (2^-16 on average): the hard bound
-    is 2^-14 sum |a||b|, reached only by factors with every low mantissa bit set; measured on normal
-    entries against fp64: 2^-17.3 sum |a||b| at worst (tf32 itself: 2^-10).  2^-16 is the bound the
-    seeded inputs of these tests stay within, not a guarantee for every input."""
+    cancels, an absolute term in units of sum |a||b|: 1e-5 for fp32 accumulation of exact products.
+    The tf32 variant's LDS-staging kernels multiply bf16 hi + lo parts in three products (unless the
+    kernel mode guarantees fp32 products).  The product they leave out, a_lo b_lo, has the sign of a b
+    and at most 2^-14 of its size (2^-16 on average), so every output must lie within 2^-14 sum |a||b|
+    more - the hard bound, reached only by factors with every low mantissa bit set - and all but one in
+    10^5 of them (one of an array smaller than that) within 2^-16 sum |a||b|: measured on normal entries
+    against fp64 the worst is 2^-17.3 sum |a||b|, and of 10^9 outputs of random inputs five lay beyond
+    2^-16 (tf32 itself: 2^-10)."""
     import hopper_spmm_amd
+    parts = dtype == 1 and hopper_spmm_amd.get_kernel_mode() not in (1, 2, 3, 5)
     if dtype != 1:
         g, r, rel, absolute = decode(got, dtype), decode(ref, dtype), 1e-2, 1e-5
     else:
         g, r, rel = got.astype(np.float64), ref.astype(np.float64), 1e-3
-        absolute = 1e-5 if hopper_spmm_amd.get_kernel_mode() in (1, 2, 3, 5) else 1e-5 + 2.0 ** -16
+        absolute = 1e-5 + 2.0 ** -14 if parts else 1e-5
     assert not np.isnan(g).any(), what + ": unwritten or NaN output"
     err = np.abs(g - r)
     bound = rel * np.abs(r) + absolute * absdot.astype(np.float64)
     bad = err > bound
     assert not bad.any(), "%s: %d of %d outputs outside tolerance, worst %g at %s" % (
         what, int(bad.sum()), bad.size, float((err - bound).max()), np.unravel_index(np.argmax(err - bound), err.shape))
+    if parts:
+        beyond = err > rel * np.abs(r) + (1e-5 + 2.0 ** -16) * absdot.astype(np.float64)
+        assert int(beyond.sum()) <= max(1, beyond.size // 100000), "%s: %d of %d outputs beyond 2^-16 sum |a||b|" % (
+            what, int(beyond.sum()), beyond.size)
     if tight and dtype != 1 and got.size:
         # far tighter in practice (except for long, cancelling sums): one rounding of nearly identical fp32 sums
         ulp = half_ulp_distance(got, ref)
@@ -512,7 +518,10 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
             assert info["n_panels"] == (cols + panel_rows - 1) // panel_rows
             # (adjacent windows with much the same columns may have been given one list: up to four windows per step)
             assert info["n_panel_steps"] >= info["total_tiles"] // (4 * per_step)
-            for N in (block, 2 * block, 5 * block):
+            # whole blocks of features, and - the kernels built on the 16-bit MFMA - a feature dimension that ends
+            # inside the last block at a multiple of 16 (fp32 storage in bf16 parts: also inside the only block)
+            ragged = () if mode == 5 else (block + 16, 3 * block - 16, 16, 48) if dtype == 1 else (block + 16, 3 * block - 48)
+            for N in (block, 2 * block, 5 * block) + ragged:
                 B = make_b(rng, cols, N, dtype)
                 got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
                 ref, mag = oracle_spmm(oracle, A, B, N)
@@ -522,7 +531,7 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
             B = make_b(rng, cols, 24, dtype)
             got = gpu_spmm(torch_cuda, hs, b, B, 24, plan=plan)
             ref, mag = oracle_spmm(oracle, A, B, 24)
-            assert_parity(got, ref, mag, dtype, "panel plan, N=24")
+            assert_parity(got, ref, mag, dtype, "panel plan, N=24", tight=got.size >= 10000)   # (a share of 99.9 % needs that many)
             assert plan.info()["last_kernel_family"] == 2
             plan.close()
         finally:
@@ -601,12 +610,15 @@ def test_long_units_are_walked_by_one_workgroup_each(torch_cuda, hs, oracle, dty
     b = convert(hs, A)
     for pairing in (0, 1):
         hs.set_window_pairing(pairing)
+        if dtype == 1:
+            hs.set_kernel_mode(3)                           # (fp32 storage: the LDS-staging kernels would take N = 16 and 48)
         try:
             plan = hs.Plan(b)
         finally:
             hs.set_window_pairing(0)
+            hs.set_kernel_mode(0)
         assert plan.info()["n_split_windows"] > 0           # the balanced partition cuts units
-        for N in (8, 16, 48, 56 if dtype == 1 else 64):     # (fp32 at N = 64 would go to the LDS-staging kernels)
+        for N in (8, 16, 48, 56 if dtype == 1 else 64):
             Bm = rng.integers(-4, 5, (cols, N))
             got = gpu_spmm(torch, hs, b, encode(Bm, dtype), N, plan=plan)
             assert np.array_equal(got, encode(D @ Bm, dtype)), (pairing, N)
@@ -630,7 +642,8 @@ def test_partial_sums_added_inside_the_main_kernel(torch_cuda, hs, oracle, dtype
     block = 64 if dtype == 1 else 128
     sparse = random_csr(rng, 300, 3000, 0.004, dtype, 0.2, (5, 100, 101, 299))     # heavy windows: cut units
     dense = random_csr(rng, 300, 3000, 0.1, dtype, 0.1)                             # LDS-staging kernels
-    for A, N, family in ((sparse, 48 if dtype == 1 else 64, 2), (dense, block, 3)):   # (fp32, N = 64: LDS-staging kernels)
+    # (fp32 storage: every multiple of 16 goes to the LDS-staging kernels when the plan has them)
+    for A, N, family in ((sparse, 40 if dtype == 1 else 64, 2), (dense, block, 3)):
         b = convert(hs, A)
         B = make_b(rng, 3000, N, dtype)
         hs.configure(producer_warp_group_num=16)
@@ -1504,6 +1517,32 @@ def test_panel_stream_with_two_units_per_wave_and_packed_tiles(torch_cuda, hs, o
             plan.close()
             # (the sums are exact in fp32; the output is their one rounding to the storage type)
             assert np.array_equal(decode(got, dtype), decode(encode(D2 @ Bm, dtype), dtype)), "mode %d" % mode
+        # A wave's second unit whose first step lies more than 15 panels behind the first unit's last one (the
+        # steps count the panels from their predecessor in four bits): single windows, 36 panels, the second
+        # window's only columns in panel 30.
+        rows, cols = 32, 9000
+        D = np.zeros((rows, cols))
+        D[0, 3] = 2; D[1, 200] = -1                     # window 0: panel 0
+        D[8, 7700] = 3; D[9, 7701] = 1                  # window 1: panel 30 only
+        D[16, 5000] = 1; D[17, 8999] = -2               # window 2: panels 19 and 35
+        D[24, 100] = 1                                  # window 3: panel 0 (and an odd man out when units are paired up)
+        rr, cc = np.nonzero(D)
+        rp = np.zeros(rows + 1, np.uint32)
+        rp[1:] = np.cumsum(np.bincount(rr, minlength=rows))
+        Af = dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=cc.astype(np.uint32), values=encode(D[rr, cc].astype(np.float32), dtype))
+        bf = convert(hs, Af)
+        Bm = rng.integers(-4, 5, (cols, N))
+        hs.set_window_pairing(1)                        # (single windows stay single)
+        try:
+            for mode in (0, 1, 2):
+                hs.set_panel_stream(mode)
+                plan = hs.Plan(bf)
+                got = gpu_spmm(torch_cuda, hs, bf, encode(Bm, dtype), N, plan=plan)
+                assert plan.info()["panel_stream_mode"] == mode and plan.info()["last_kernel_family"] == 3
+                plan.close()
+                assert np.array_equal(decode(got, dtype), decode(encode(D @ Bm, dtype), dtype)), "far first step, mode %d" % mode
+        finally:
+            hs.set_window_pairing(0)
     finally:
         hs.set_panel_stream(0)
         hs.set_kernel_mode(0)
