@@ -1994,9 +1994,10 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         // (the producers address a panel of B - up to 256 rows - with 32-bit offsets)
         const bool offsets_fit = uint64_t(N) * p->elem < (uint64_t(1) << 24);
         // Whole blocks of features, or - the kernels built on the 16-bit MFMA, whose lanes own one feature per
-        // accumulator - any multiple of 16 from one block on (from 16 on for fp32 storage, whose gather kernels
-        // multiply at a sixteenth of the rate): the last block's missing features are zeros in LDS and are not stored.
-        const bool ragged_ok = (p->cw == 16 || p->panel.split) && N % 16u == 0 && (p->dtype == HSPMM_TF32 || N >= block_feat);
+        // accumulator - any whole number of 16-byte pieces per row from one block on (from 16 features on for fp32
+        // storage, whose gather kernels multiply at a sixteenth of the rate): what the last block lacks is not stored.
+        const bool ragged_ok = (p->cw == 16 || p->panel.split) && (uint64_t(N) * p->elem) % 16u == 0 &&
+                               (p->dtype == HSPMM_TF32 ? N >= 16u : N >= block_feat);
         if (pays && offsets_fit && (N % block_feat == 0 || ragged_ok) && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
     }
     // Feature blocks with XCDs of their own (see spmm_mfma_kernel): pays when B is far larger than an

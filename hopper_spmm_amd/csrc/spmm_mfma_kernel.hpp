@@ -653,17 +653,17 @@ __device__ __forceinline__ uint32_t unit_windows(const uint32_t row_word)
 }
 
 // Tile classes of the LDS-panel kernels whose lanes own one feature per accumulator (feature 16 p + j of the
-// block) keep in `p_valid` how many of their accumulators lie inside a feature dimension that ends inside the
-// block (N a multiple of 16); other classes have no such member and need whole blocks.
+// block) keep in `f_valid` how many features of their block lie inside a feature dimension that ends inside the
+// block; other classes have no such member and need whole blocks.
 template <class LaneT, class = void> struct HasValidCount { static constexpr bool value = false; };
-template <class LaneT> struct HasValidCount<LaneT, decltype(void(LaneT::p_valid))> { static constexpr bool value = true; };
+template <class LaneT> struct HasValidCount<LaneT, decltype(void(LaneT::f_valid))> { static constexpr bool value = true; };
 template <class TT>
-__device__ __forceinline__ void set_valid_accumulators(typename TT::Lane &L, uint32_t N, uint32_t fb)
+__device__ __forceinline__ void set_valid_features(typename TT::Lane &L, uint32_t N, uint32_t fb)
 {
     if constexpr (HasValidCount<typename TT::Lane>::value) {
         const uint32_t first = fb * uint32_t(TT::kBlockFeat);
         const uint32_t left = N > first ? N - first : 0u;
-        L.p_valid = (left < uint32_t(TT::kBlockFeat) ? left : uint32_t(TT::kBlockFeat)) / 16u;
+        L.f_valid = left < uint32_t(TT::kBlockFeat) ? left : uint32_t(TT::kBlockFeat);
     }
 }
 
@@ -921,7 +921,7 @@ void spmm_fixup_kernel(const KernelArgs ka)
 
     typename TT::Lane L;
     L.init(lane, ka.tiles, ka.ids);
-    set_valid_accumulators<TT>(L, ka.N, fb);
+    set_valid_features<TT>(L, ka.N, fb);
     const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
     const bool active = feat < ka.N;
     const size_t row_bytes = size_t(ka.N) * TT::kElem;

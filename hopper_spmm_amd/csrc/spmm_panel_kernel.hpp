@@ -193,13 +193,13 @@ struct Fp16Tr {
     typedef typename HalfOps<BF>::elem_t elem_t;
     struct Lane {
         uint32_t g, j;
-        uint32_t p_valid;                          // accumulators whose feature 16 p + j exists (8 unless N ends inside the block)
+        uint32_t f_valid;                          // features of the block that exist (128 unless N ends inside the block)
         const uint32_t *a_src;
         const uint32_t *idx_src;
         __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
         {
             g = lane >> 4; j = lane & 15u;
-            p_valid = 8u;
+            f_valid = 128u;
             a_src = reinterpret_cast<const uint32_t *>(tiles) + lane * 4u;
             idx_src = ids + (lane >> 2);           // four neighbouring lanes read one word
         }
@@ -218,7 +218,7 @@ struct Fp16Tr {
                 elem_t *dst = reinterpret_cast<elem_t *>(c_lane + size_t(row) * row_bytes);
 #pragma unroll
                 for (int p = 0; p < 8; ++p)
-                    if (uint32_t(p) < L.p_valid) stream_store(dst + 16 * p, (elem_t)acc[8 * (W0 >> 1) + p][e]);
+                    if (16u * uint32_t(p) + L.j < L.f_valid) stream_store(dst + 16 * p, (elem_t)acc[8 * (W0 >> 1) + p][e]);
             }
         }
     }
@@ -230,7 +230,7 @@ struct Fp16Tr {
             elem_t *dst = reinterpret_cast<elem_t *>(c_lane + size_t(r) * row_bytes);
 #pragma unroll
             for (int p = 0; p < 8; ++p)
-                if (uint32_t(p) < L.p_valid) stream_store(dst + 16 * p, (elem_t)0.f);
+                if (16u * uint32_t(p) + L.j < L.f_valid) stream_store(dst + 16 * p, (elem_t)0.f);
         }
     }
 };
@@ -343,13 +343,13 @@ struct Fp32Split {
     typedef u32x8 AVec;
     struct Lane {
         uint32_t g, j;
-        uint32_t p_valid;                          // accumulators whose feature 16 p + j exists (4 unless N ends inside the block)
+        uint32_t f_valid;                          // features of the block that exist (64 unless N ends inside the block)
         const uint32_t *a_src;
         const uint32_t *idx_src;
         __device__ __forceinline__ void init(uint32_t lane, const void *tiles, const uint32_t *ids)
         {
             g = lane >> 4; j = lane & 15u;
-            p_valid = 4u;
+            f_valid = 64u;
             a_src = reinterpret_cast<const uint32_t *>(tiles) + lane * 8u;
             idx_src = ids + (lane >> 2);           // four neighbouring lanes read one word
         }
@@ -367,7 +367,7 @@ struct Fp32Split {
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
                     const float v = acc[4 * (W0 >> 1) + p][e];
-                    if (uint32_t(p) < L.p_valid) stream_store(dst + 16 * p, v);
+                    if (16u * uint32_t(p) + L.j < L.f_valid) stream_store(dst + 16 * p, v);
                 }
             }
         }
@@ -380,7 +380,7 @@ struct Fp32Split {
             float *dst = reinterpret_cast<float *>(c_lane + size_t(r) * row_bytes);
 #pragma unroll
             for (int p = 0; p < 4; ++p)
-                if (uint32_t(p) < L.p_valid) stream_store(dst + 16 * p, 0.f);
+                if (16u * uint32_t(p) + L.j < L.f_valid) stream_store(dst + 16 * p, 0.f);
         }
     }
 };
@@ -878,7 +878,7 @@ void spmm_panel_kernel(const PanelArgs pa)
     for (; owed; --owed) panel_barrier();
 
     if (!has_unit) return;
-    set_valid_accumulators<TT>(L, pa.N, fb);        // (here, not at the top: nothing of it lives through the steps)
+    set_valid_features<TT>(L, pa.N, fb);        // (here, not at the top: nothing of it lives through the steps)
     // Stores unit `unit` from the sums in `sums` (or leaves them as this chunk's partial sums).
     auto finish = [&](const uint32_t unit, f32x4 (&sums)[Ops::kLive]) __attribute__((always_inline)) {
         Ops::fold(sums);

@@ -154,8 +154,8 @@ void hspmm_get_config(int *buffer_stage, int *consumer_warp_num,
  * for matrices whose windows touch a large share of the columns), 1 = always the
  * scalar all-shapes kernel, 2 = 16-bit MFMA kernel with wide loads only, 3 =
  * 16-bit MFMA kernel with word loads whenever N is a multiple of 32, 4 = the
- * LDS-staging kernels for every matrix (whenever N is a multiple of 16 - from 128
- * on for the 16-bit types - and B and C are 16-byte aligned), 5 = the same
+ * LDS-staging kernels for every matrix (whenever the rows of B are whole 16-byte
+ * pieces, N is 16 at least - 128 for the 16-bit types - and B and C are 16-byte aligned), 5 = the same
  * with fp32 products in the HSPMM_TF32 LDS-staging kernels (N a multiple of 64).  (By default those
  * kernels multiply the bf16 parts hi + lo of every fp32 factor, which keeps 16
  * mantissa bits per factor; the reference's tf32 instruction keeps 10,

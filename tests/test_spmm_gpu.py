@@ -519,8 +519,8 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
             # (adjacent windows with much the same columns may have been given one list: up to four windows per step)
             assert info["n_panel_steps"] >= info["total_tiles"] // (4 * per_step)
             # whole blocks of features, and - the kernels built on the 16-bit MFMA - a feature dimension that ends
-            # inside the last block at a multiple of 16 (fp32 storage in bf16 parts: also inside the only block)
-            ragged = () if mode == 5 else (block + 16, 3 * block - 16, 16, 48) if dtype == 1 else (block + 16, 3 * block - 48)
+            # inside the last block at a whole number of 16-byte pieces (fp32 storage in bf16 parts: also inside the only block)
+            ragged = () if mode == 5 else (block + 16, 3 * block - 16, 16, 48, 20, 68) if dtype == 1 else (block + 16, 3 * block - 48, block + 8, 3 * block - 24)
             for N in (block, 2 * block, 5 * block) + ragged:
                 B = make_b(rng, cols, N, dtype)
                 got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
@@ -528,10 +528,10 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
                 assert_parity(got, ref, mag, dtype, "panel mode %d units %s chunks %s shape %s N=%d" % (mode, units, chunks, shape[:2], N))
                 assert plan.info()["last_kernel_family"] == 3          # the LDS-staging kernels did run
             # a feature dimension the panel kernels do not take falls back to the gather kernels
-            B = make_b(rng, cols, 24, dtype)
-            got = gpu_spmm(torch_cuda, hs, b, B, 24, plan=plan)
-            ref, mag = oracle_spmm(oracle, A, B, 24)
-            assert_parity(got, ref, mag, dtype, "panel plan, N=24", tight=got.size >= 10000)   # (a share of 99.9 % needs that many)
+            B = make_b(rng, cols, 22, dtype)
+            got = gpu_spmm(torch_cuda, hs, b, B, 22, plan=plan)
+            ref, mag = oracle_spmm(oracle, A, B, 22)
+            assert_parity(got, ref, mag, dtype, "panel plan, N=22", tight=got.size >= 10000)   # (a share of 99.9 % needs that many)
             assert plan.info()["last_kernel_family"] == 2
             plan.close()
         finally:
@@ -642,8 +642,8 @@ def test_partial_sums_added_inside_the_main_kernel(torch_cuda, hs, oracle, dtype
     block = 64 if dtype == 1 else 128
     sparse = random_csr(rng, 300, 3000, 0.004, dtype, 0.2, (5, 100, 101, 299))     # heavy windows: cut units
     dense = random_csr(rng, 300, 3000, 0.1, dtype, 0.1)                             # LDS-staging kernels
-    # (fp32 storage: every multiple of 16 goes to the LDS-staging kernels when the plan has them)
-    for A, N, family in ((sparse, 40 if dtype == 1 else 64, 2), (dense, block, 3)):
+    # (fp32 storage: every N of whole 16-byte pieces per row goes to the LDS-staging kernels when the plan has them)
+    for A, N, family in ((sparse, 42 if dtype == 1 else 64, 2), (dense, block, 3)):
         b = convert(hs, A)
         B = make_b(rng, 3000, N, dtype)
         hs.configure(producer_warp_group_num=16)
