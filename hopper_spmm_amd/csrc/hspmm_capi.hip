@@ -1065,11 +1065,12 @@ struct Choice {
 
 // split_features: prefer the load width of one 128-byte line per row and feature block (blocks with XCDs of their own, see
 // spmm_mfma_kernel), where the feature dimension allows it.
-Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32_t N, bool split_features = false)
+// N: features of the launch; ld: elements from one row of B and C to the next (N, or more for a range of the features).
+Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32_t N, uint32_t ld, bool split_features = false)
 {
     Choice c{};
     const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
-    const uint64_t row_bytes = uint64_t(N) * p->elem;
+    const uint64_t row_bytes = uint64_t(ld) * p->elem;
     c.narrow = p->cols < (1u << 24) && row_bytes < (1u << 24) && uint64_t(p->cols) * row_bytes <= (1ull << 32);
     const int mode = p->cfg.kernel_mode;
     if (mode == 1) { c.scalar = true; return c; }
@@ -1947,7 +1948,7 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         ka.unitRow = pl.d_unitRow; ka.ids = pl.d_ids; ka.tiles = pl.d_tiles;
         ka.scratch = pa.scratch;
         ka.C = dC; ka.B = dB;
-        ka.n_split = pl.n_units; ka.n_units = pl.n_units; ka.rows = p->rows; ka.N = N;
+        ka.n_split = pl.n_units; ka.n_units = pl.n_units; ka.rows = p->rows; ka.N = N; ka.ld = N;
         ka.n_feat_blocks = pa.n_feat_blocks;
         ka.uniform_chunks = pa.n_chunks;
     }
@@ -1956,6 +1957,8 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : pl.G, pl.split, pl.tall, pl.packed, pa, ka, units, s, mid));
     return HSPMM_OK;
 }
+
+static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint32_t ld, hipStream_t s, hipEvent_t mid, RunMode mode);
 
 // One launch (or, kPrepare, everything a launch with this N and these pointer alignments would build).
 // mid: when not null, an event recorded between the main kernel and the kernel that adds the partial
@@ -2000,18 +2003,42 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
                                (p->dtype == HSPMM_TF32 ? N >= 16u : N >= block_feat);
         if (pays && offsets_fit && (N % block_feat == 0 || ragged_ok) && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
     }
+    // A feature dimension that no wide load divides (16-bit types: N not a multiple of 8, fp32 storage: of 4) would
+    // run in blocks of 32 resp. 16 features, each block a pass over the tiles and another gather of every row
+    // (power-law graph 2^20, fp16: N = 130 in five passes, 1404 us against 481 us at N = 128).  Two launches
+    // instead: the features up to the last multiple with the wide loads, the few behind it in one narrow block.
+    // (Odd N of a 16-bit type stays with the all-shapes kernel: rows that start on odd halves.)
+    // (Cutting at the last multiple of 64 as well, so that those features run with word loads and bitmap tiles,
+    // measured 1027 -> 895 us at N = 136 and 1175 -> 1259 us at N = 200: not done.)
+    const uint32_t wide = p->elem == 2u ? 8u : 4u;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
+    if (p->cfg.kernel_mode != 1 && N > wide && N % wide != 0 && (p->elem == 4u || N % 2u == 0) && !(align & 3u)) {
+        const uint32_t first = N - N % wide;
+        const int rc = run_gather(p, dB, dC, first, N, s, mid, mode);
+        if (rc) return rc;
+        return run_gather(p, static_cast<const char *>(dB) + size_t(first) * p->elem, static_cast<char *>(dC) + size_t(first) * p->elem,
+                          N - first, N, s, nullptr, mode);
+    }
+    return run_gather(p, dB, dC, N, N, s, mid, mode);
+}
+
+// One launch of the gather kernels (or of the all-shapes kernel) over N features of rows that are ld elements apart.
+static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint32_t ld, hipStream_t s, hipEvent_t mid, RunMode mode)
+{
+    const bool launch = mode != RunMode::kPrepare;
     // Feature blocks with XCDs of their own (see spmm_mfma_kernel): pays when B is far larger than an
     // XCD's 4 MB L2, so that what an L2 can keep of it decides the hit rate of the gathers (power-law
     // graph 2^20, N = 128: 575 -> 535 us; uniform 65536^2: 39.7 -> 35.5 us), and costs a second pass over
     // the tile stream.  Requests below a 128-byte line lose (N = 64 as two blocks of 32: 280 -> 510 us).
     const bool want_split = p->cfg.xcd_split > 0 ||
                              (p->cfg.xcd_split < 0 && uint64_t(p->cols) * N * p->elem >= (uint64_t(8) << 20));
-    const Choice c = choose_kernel(p, dB, dC, N, want_split);
+    const Choice c = choose_kernel(p, dB, dC, N, ld, want_split);
     hspmm::KernelArgs ka{};
     ka.rowOffset = p->d_rowOffset; ka.data = p->d_data; ka.rowIdx = p->d_rowIdx; ka.tcA2B = p->d_a2b_raw;
     ka.B = dB; ka.C = dC;
-    ka.eff_windows = p->W; ka.rows = p->rows; ka.N = N;
+    ka.eff_windows = p->W; ka.rows = p->rows; ka.N = N; ka.ld = ld;
     if (c.scalar) {
+        if (ld != N) return fail(HSPMM_ERR_UNSUPPORTED, "the all-shapes kernel takes whole rows");
         if (!launch) return HSPMM_OK;
         p->last_family.store(1, std::memory_order_relaxed);
         HSPMM_HIP(hspmm::launch_spmm_scalar(p->dtype, ka, s));

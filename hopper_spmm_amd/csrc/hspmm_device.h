@@ -39,6 +39,8 @@ struct KernelArgs {
     const void     *B;           // cols x N
     void           *C;           // rows x N
     uint32_t n_ranges, n_split, eff_windows, n_units, rows, N, n_feat_blocks;
+    uint32_t ld;                 // elements from one row of B (and of C) to the next: N, or more when the launch
+                                 // covers a range of the features only (MFMA kernels; the scalar kernel takes whole rows)
     uint32_t xcd_split;          // != 0 (gather kernels; 2, 4 or 8 feature blocks): every feature block has XCDs of its own
     uint32_t uniform_chunks;     // != 0 (LDS-panel kernels): no split table - entry e is unit e, whose partial sums
                                  // are slots e * uniform_chunks .. + uniform_chunks - 1, in that order

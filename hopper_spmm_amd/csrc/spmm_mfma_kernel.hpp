@@ -720,7 +720,7 @@ void spmm_mfma_kernel(const KernelArgs ka)
     if constexpr (TileTraits<TT>::kBitmap) L.bind_bitmap(ka.bm_header);
     const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
     const bool active = feat < ka.N;
-    const size_t row_bytes = size_t(ka.N) * TT::kElem;
+    const size_t row_bytes = size_t(ka.ld) * TT::kElem;
     char *c_lane = reinterpret_cast<char *>(ka.C) + size_t(feat) * TT::kElem;
     Gather<NARROW> gat;
     gat.base = reinterpret_cast<const char *>(ka.B);
@@ -924,7 +924,7 @@ void spmm_fixup_kernel(const KernelArgs ka)
     set_valid_features<TT>(L, ka.N, fb);
     const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
     const bool active = feat < ka.N;
-    const size_t row_bytes = size_t(ka.N) * TT::kElem;
+    const size_t row_bytes = size_t(ka.ld) * TT::kElem;
     char *c_lane = reinterpret_cast<char *>(ka.C) + size_t(feat) * TT::kElem;
 
     f32x4 acc[NACC];

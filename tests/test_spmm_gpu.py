@@ -185,11 +185,13 @@ def test_random_shapes_and_feature_dims(torch_cuda, hs, oracle, dtype, shape):
         hs.configure()
     if heavy and cols >= 3000:
         assert plan.info()["n_split_windows"] > 0
-    for N in (1, 2, 6, 8, 16, 24, 32, 64, 72, 96, 128, 200, 256, 384):
+    # (10, 30, 100, 130, 250 and, for fp32 storage, 5, 7, 127: feature dimensions that no wide load divides run as two
+    # launches, the features up to the last multiple of 8 resp. 4 and the few behind it)
+    for N in (1, 2, 5, 6, 7, 8, 10, 16, 24, 30, 32, 64, 72, 96, 100, 127, 128, 130, 200, 250, 256, 384):
         B = make_b(rng, cols, N, dtype)
         got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
         ref, mag = oracle_spmm(oracle, A, B, N)
-        assert_parity(got, ref, mag, dtype, "shape %s N=%d" % (shape[:2], N))
+        assert_parity(got, ref, mag, dtype, "shape %s N=%d" % (shape[:2], N), tight=got.size >= 10000)
     plan.close()
 
 
