@@ -1075,6 +1075,12 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
     const int mode = p->cfg.kernel_mode;
     if (mode == 1) { c.scalar = true; return c; }
     if (p->dtype != HSPMM_TF32) {
+        if (N % 2 != 0 && N >= 3) {
+            // rows that start on odd halves: one word per lane, loaded wherever it lies; the lane with the last
+            // feature owns it alone (mark_half_lane in spmm_mfma_kernel.hpp)
+            c.layout = hspmm::kLayoutX4; c.V = 1; c.block_feat = 32;
+            return c;
+        }
         if (N % 2 != 0 || (align & 3u)) { c.scalar = true; return c; }
         // word loads measured equal to or faster than wide loads wherever both apply
         const bool dw_ok = (N % 64 == 0);
@@ -2007,13 +2013,14 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     // run in blocks of 32 resp. 16 features, each block a pass over the tiles and another gather of every row
     // (power-law graph 2^20, fp16: N = 130 in five passes, 1404 us against 481 us at N = 128).  Two launches
     // instead: the features up to the last multiple with the wide loads, the few behind it in one narrow block.
-    // (Odd N of a 16-bit type stays with the all-shapes kernel: rows that start on odd halves.)
+    // (An odd N of a 16-bit type: the narrow block gets nine features rather than one, its last lane reads one half
+    // in front of its feature.)
     // (Cutting at the last multiple of 64 as well, so that those features run with word loads and bitmap tiles,
     // measured 1027 -> 895 us at N = 136 and 1175 -> 1259 us at N = 200: not done.)
     const uint32_t wide = p->elem == 2u ? 8u : 4u;
     const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
-    if (p->cfg.kernel_mode != 1 && N > wide && N % wide != 0 && (p->elem == 4u || N % 2u == 0) && !(align & 3u)) {
-        const uint32_t first = N - N % wide;
+    if (p->cfg.kernel_mode != 1 && N > (p->elem == 2u && N % 2u ? 32u : wide) && N % wide != 0 && !(align & 3u)) {
+        const uint32_t first = N - N % wide - ((p->elem == 2u && N % wide == 1u) ? wide : 0u);
         const int rc = run_gather(p, dB, dC, first, N, s, mid, mode);
         if (rc) return rc;
         return run_gather(p, static_cast<const char *>(dB) + size_t(first) * p->elem, static_cast<char *>(dC) + size_t(first) * p->elem,

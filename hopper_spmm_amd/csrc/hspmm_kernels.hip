@@ -13,7 +13,7 @@ namespace hspmm {
 // All-shapes kernel (any N, any alignment): one workgroup per effective window
 // and 256-feature slab, one thread per feature, plain fp32 multiply-add, reading
 // the format arrays exactly as the caller gave them.  Used when the feature
-// dimension rules out the vector loads above (odd N in fp16), and as an
+// pointers rule out the vector loads above (B or C not 4-byte aligned), for one feature of a 16-bit type, and as an
 // independent second implementation in tests.
 // ---------------------------------------------------------------------------
 template <typename T> __device__ __forceinline__ float to_f32(T v);

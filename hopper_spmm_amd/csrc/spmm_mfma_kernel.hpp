@@ -170,6 +170,7 @@ template <int G>
 struct Fp16Lane {
     typedef typename Vec<2 * G>::type AVec;
     uint32_t g, j;                             // quarter-wave, lane in quarter
+    uint32_t half_shift;                       // 16 for the lane that owns the last feature of an odd N alone (mark_half_lane)
     uint32_t sel_lo, sel_hi;                   // byte selectors for the sparse operand
     const uint32_t *a_src;                     // lane's words inside step 0
     const uint32_t *idx_src;                   // lane's ids inside step 0
@@ -179,6 +180,7 @@ struct Fp16Lane {
     {
         a_base = tiles;
         g = lane >> 4; j = lane & 15u;
+        half_shift = 0u;
         const uint32_t r = j >> 1, parity = j & 1u;
         // v_perm_b32 selectors: bytes 0-3 come from the second source, 0x0c gives 0x00.
         //   even MFMA row: value in the low half  -> {lo: b0 b1 0 0}, {hi: b2 b3 0 0}
@@ -242,13 +244,15 @@ struct Fp16Tile {
     {
         if constexpr (V == 1) return v; else return v[p];
     }
+    // shift: 16 in the lane whose word was loaded one half early (odd N, see mark_half_lane), else 0
     template <int W0, int p>
     __device__ static __forceinline__ void mma_one(const u32x4 av, const BVec &b0, const BVec &b1, const BVec &b2,
-                                                   const BVec &b3, f32x4 (&acc)[G * V])
+                                                   const BVec &b3, f32x4 (&acc)[G * V], uint32_t shift)
     {
         if constexpr (p < V) {
             u32x4 bw;
             bw[0] = word<p>(b0); bw[1] = word<p>(b1); bw[2] = word<p>(b2); bw[3] = word<p>(b3);
+            if constexpr (V == 1) { bw[0] >>= shift; bw[1] >>= shift; bw[2] >>= shift; bw[3] >>= shift; }
             acc[W0 * V + p] = HalfOps<BF>::mfma(av, bw, acc[W0 * V + p]);
         }
     }
@@ -258,8 +262,8 @@ struct Fp16Tile {
     {
         if constexpr (W0 < G) {
             const u32x4 av = L.template sparse_operand<W0>(a);
-            mma_one<W0, 0>(av, b0, b1, b2, b3, acc); mma_one<W0, 1>(av, b0, b1, b2, b3, acc);
-            mma_one<W0, 2>(av, b0, b1, b2, b3, acc); mma_one<W0, 3>(av, b0, b1, b2, b3, acc);
+            mma_one<W0, 0>(av, b0, b1, b2, b3, acc, L.half_shift); mma_one<W0, 1>(av, b0, b1, b2, b3, acc, 0u);
+            mma_one<W0, 2>(av, b0, b1, b2, b3, acc, 0u); mma_one<W0, 3>(av, b0, b1, b2, b3, acc, 0u);
         }
     }
     __device__ static __forceinline__ void mma(const Lane &L, const BVec &b0, const BVec &b1, const BVec &b2,
@@ -279,7 +283,10 @@ struct Fp16Tile {
             uint32_t out[V];
 #pragma unroll
             for (int p = 0; p < V; ++p) out[p] = HalfOps<BF>::pack(acc[W0 * V + p][2 * rr], acc[W0 * V + p][2 * rr + 1]);
-            if (active && row < rows) store_words<V>(c_lane + size_t(row) * row_bytes, out);
+            if (active && row < rows) {
+                if (V == 1 && L.half_shift) stream_store(reinterpret_cast<uint16_t *>(c_lane + size_t(row) * row_bytes), uint16_t(out[0]));
+                else store_words<V>(c_lane + size_t(row) * row_bytes, out);
+            }
         }
     }
     // Zero rows [r_begin, r_end) of this lane's features.
@@ -290,7 +297,10 @@ struct Fp16Tile {
 #pragma unroll
         for (int i = 0; i < V; ++i) z[i] = 0u;
         if (!active) return;
-        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) store_words<V>(c_lane + size_t(r) * row_bytes, z);
+        for (uint32_t r = r_begin + L.g; r < r_end; r += 4u) {
+            if (V == 1 && L.half_shift) stream_store(reinterpret_cast<uint16_t *>(c_lane + size_t(r) * row_bytes), uint16_t(0));
+            else store_words<V>(c_lane + size_t(r) * row_bytes, z);
+        }
     }
 };
 
@@ -667,6 +677,21 @@ __device__ __forceinline__ void set_valid_features(typename TT::Lane &L, uint32_
     }
 }
 
+// An odd feature dimension of a 16-bit type (wide-load layout, one word per lane): the lane whose first feature is
+// the last one owns that feature alone.  It loads its word one half early - the two last features of the row, so
+// that no load leaves the row - and shifts it down, and it stores one half.  Returns the bytes to take off the
+// lane's offset into a row of B.  (The launch covers three features at least.)
+template <class LaneT, class = void> struct HasHalfLane { static constexpr bool value = false; };
+template <class LaneT> struct HasHalfLane<LaneT, decltype(void(LaneT::half_shift))> { static constexpr bool value = true; };
+template <class TT>
+__device__ __forceinline__ uint32_t mark_half_lane(typename TT::Lane &L, uint32_t N, uint32_t feat)
+{
+    if constexpr (HasHalfLane<typename TT::Lane>::value && TT::kLaneFeat == 2) {
+        if ((N & 1u) && feat + 1u == N) { L.half_shift = 16u; return 2u; }
+    }
+    return 0u;
+}
+
 // Stores the windows W0 .. of a unit (window w covers rows row0 + 8 w .. + 7).
 template <class TT, int W0 = 0, int NACC>
 __device__ __forceinline__ void store_unit(const typename TT::Lane &L, const f32x4 (&acc)[NACC], char *c_lane,
@@ -726,6 +751,9 @@ void spmm_mfma_kernel(const KernelArgs ka)
     gat.base = reinterpret_cast<const char *>(ka.B);
     gat.row_bytes = uint32_t(row_bytes);
     gat.lane_off = active ? feat * TT::kElem : 0u;     // lanes past N read (and drop) the row start
+    // (a lane that owns the last feature of an odd N alone reads one half early; the host launches odd N from
+    // three features on, so that lane's first feature is not the launch's first)
+    gat.lane_off -= mark_half_lane<TT>(L, ka.N, feat);
 
     UnitWalk ww;
     ww.u = rd[2];
@@ -924,6 +952,7 @@ void spmm_fixup_kernel(const KernelArgs ka)
     set_valid_features<TT>(L, ka.N, fb);
     const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
     const bool active = feat < ka.N;
+    (void)mark_half_lane<TT>(L, ka.N, feat);
     const size_t row_bytes = size_t(ka.ld) * TT::kElem;
     char *c_lane = reinterpret_cast<char *>(ka.C) + size_t(feat) * TT::kElem;
 

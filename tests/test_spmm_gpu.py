@@ -933,21 +933,40 @@ def test_seeded_sweep_of_stream_modes_group_cuts_and_tuning_overrides(torch_cuda
         assert_parity(got, ref, mag, dtype, what, tight=False)
 
 
-def test_unaligned_and_odd_feature_dims_use_the_all_shapes_kernel(torch_cuda, hs, oracle):
+def test_odd_feature_dims_of_the_16_bit_types(torch_cuda, hs, oracle):
+    """Rows of B and C that start on odd halves.  From three features on the MFMA gather kernels take them: words
+    loaded wherever they lie, the lane with the last feature reading one half early and storing one half, and
+    beyond 32 features two launches (up to the last multiple of 8; the rest - nine features rather than one).
+    Nothing next to C is written.  One feature: the all-shapes kernel."""
+    torch = torch_cuda
     rng = np.random.default_rng(5)
     for dt in (0, 2):
-        A = random_csr(rng, 90, 120, 0.1, dt, 0.2)
-        b = convert(hs, A)
-        plan = hs.Plan(b)
-        for N in (1, 3, 7, 33, 129):
-            B = make_b(rng, 120, N, dt)
-            got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
-            ref, mag = oracle_spmm(oracle, A, B, N)
-            assert_parity(got, ref, mag, dt, "%s odd N=%d" % (DT[dt], N))
-            assert plan.info()["last_kernel_family"] == 1              # the all-shapes kernel
-        got = gpu_spmm(torch_cuda, hs, b, make_b(rng, 120, 34, dt), 34, plan=plan)
-        assert plan.info()["last_kernel_family"] == 2                  # an even N: MFMA kernels again
-        plan.close()
+        for rows, cols, dens, heavy in ((90, 120, 0.1, ()), (300, 3000, 0.004, (5, 100, 299))):
+            A = random_csr(rng, rows, cols, dens, dt, 0.2, heavy)
+            b = convert(hs, A)
+            hs.configure(producer_warp_group_num=16)               # (cut windows: partial sums, second kernel or added inside)
+            try:
+                plan = hs.Plan(b)
+            finally:
+                hs.configure()
+            for N in (1, 3, 5, 7, 9, 31, 33, 41, 127, 129, 257):
+                B = make_b(rng, cols, N, dt)
+                ref, mag = oracle_spmm(oracle, A, B, N)
+                # C inside a larger buffer of a known pattern: the halves around it must survive
+                guard = 64
+                buf = torch.full((rows * N + 2 * guard,), 0x7E01, dtype=torch.int16, device="cuda")
+                dB = torch.from_numpy(np.ascontiguousarray(B, np.uint16).view(np.int16)).cuda()
+                dC = buf[guard:guard + rows * N]
+                plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)
+                torch.cuda.synchronize()
+                out = buf.cpu().numpy()
+                assert (out[:guard] == 0x7E01).all() and (out[-guard:] == 0x7E01).all(), "N=%d: wrote outside C" % N
+                got = out[guard:-guard].reshape(rows, N).view(np.uint16)
+                assert_parity(got, ref, mag, dt, "%s odd N=%d" % (DT[dt], N), tight=False)
+                assert plan.info()["last_kernel_family"] == (1 if N == 1 else 2)
+            got = gpu_spmm(torch_cuda, hs, b, make_b(rng, cols, 34, dt), 34, plan=plan)
+            assert plan.info()["last_kernel_family"] == 2
+            plan.close()
 
 
 @pytest.mark.parametrize("dtype", [0, 1])
