@@ -1075,13 +1075,13 @@ Choice choose_kernel(const hspmm_plan *p, const void *dB, const void *dC, uint32
     const int mode = p->cfg.kernel_mode;
     if (mode == 1) { c.scalar = true; return c; }
     if (p->dtype != HSPMM_TF32) {
-        if (N % 2 != 0 && N >= 3) {
-            // rows that start on odd halves: one word per lane, loaded wherever it lies; the lane with the last
-            // feature owns it alone (mark_half_lane in spmm_mfma_kernel.hpp)
+        if ((N % 2 != 0 && N >= 3) || (N % 2 == 0 && (align & 3u))) {
+            // rows that start on odd halves (an odd N, or B or C itself): one word per lane, loaded wherever it
+            // lies; the lane with the last feature of an odd N owns it alone (mark_half_lane in spmm_mfma_kernel.hpp)
             c.layout = hspmm::kLayoutX4; c.V = 1; c.block_feat = 32;
             return c;
         }
-        if (N % 2 != 0 || (align & 3u)) { c.scalar = true; return c; }
+        if (N % 2 != 0) { c.scalar = true; return c; }
         // word loads measured equal to or faster than wide loads wherever both apply
         const bool dw_ok = (N % 64 == 0);
         if (mode != 2 && (dw_ok || mode == 3) && N % 32 == 0) {

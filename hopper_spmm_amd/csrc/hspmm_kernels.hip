@@ -12,9 +12,9 @@ namespace hspmm {
 // ---------------------------------------------------------------------------
 // All-shapes kernel (any N, any alignment): one workgroup per effective window
 // and 256-feature slab, one thread per feature, plain fp32 multiply-add, reading
-// the format arrays exactly as the caller gave them.  Used when the pointers rule
-// out the vector loads above (B or C not 4-byte aligned), for a single feature of a
-// 16-bit type, and as an independent second implementation in tests.
+// the format arrays exactly as the caller gave them.  Used for a single feature of a
+// 16-bit type, on request (kernel mode 1), and as an independent second implementation
+// in tests.
 // ---------------------------------------------------------------------------
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<_Float16>(_Float16 v) { return (float)v; }

@@ -67,9 +67,11 @@ int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
 
 /* Replaces one launch of fp16_spmm_kernel (reference src/fp16.cu:256): computes
  * all of C = A*B for feature dimension N.  dB (cols x N) and dC (rows x N) are
- * DEVICE pointers, row-major, aligned to the element size (the MFMA kernels want
- * 4 bytes and an even N for the 16-bit types, the LDS-staging kernels 16 bytes;
- * anything else runs through the all-shapes kernel); every element of C is
+ * DEVICE pointers, row-major, aligned to the element size (the LDS-staging kernels
+ * want 16 bytes and rows of whole 16-byte pieces, the widest loads of the other MFMA
+ * kernels 16 bytes and N a multiple of 8 - of 4 for fp32 storage -; everything else
+ * takes narrower loads or two launches, a single feature of a 16-bit type the
+ * all-shapes kernel); every element of C is
  * written (rows without nonzeros become 0).  Asynchronous on `stream` (a
  * hipStream_t, NULL = default stream).
  * Host side: a plan is immutable after hspmm_create except for what the first
