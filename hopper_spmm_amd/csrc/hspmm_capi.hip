@@ -184,6 +184,8 @@ struct hspmm_plan {
     size_t scratch_bytes = 0;
     uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
     size_t arrive_words = 0;
+    uint32_t *d_vector = nullptr;       // a single 16-bit feature widened to words: cols words of B, then rows words of C
+                                        // (made by the first launch with N = 1)
     size_t fixed_bytes = 0;
     // Every real column list strictly ascending and padding only behind a window's last column: what the
     // reference's converters write (reference src/utils/convert.h:166-181).  The gather and all-shapes
@@ -1838,7 +1840,7 @@ void hspmm_destroy(hspmm_plan *p)
     (void)hipFree(p->panel.d_step_panel);
     (void)hipFree(p->panel.d_masks); (void)hipFree(p->panel.d_vals); (void)hipFree(p->panel.d_step_voff);
     (void)hipFree(p->bm.d_header); (void)hipFree(p->bm.d_vals);
-    (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive);
+    (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive); (void)hipFree(p->d_vector);
     for (void *old : p->retired) (void)hipFree(old);
     delete p;
 }
@@ -2017,6 +2019,24 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     // in front of its feature.)
     // (Cutting at the last multiple of 64 as well, so that those features run with word loads and bitmap tiles,
     // measured 1027 -> 895 us at N = 136 and 1175 -> 1259 us at N = 200: not done.)
+    // A single feature of a 16-bit type (matrix times vector): B and C widened to words - the element and a zero -
+    // in a buffer of the plan's, two features through the MFMA kernels, the low halves back (power-law graph 2^20:
+    // 21 ms on the all-shapes kernel).  hspmm_run_static, which allocates nothing, keeps the all-shapes kernel.
+    if (p->elem == 2u && N == 1u && p->cfg.kernel_mode != 1 && mode != RunMode::kStatic) {
+        {
+            std::lock_guard<std::mutex> lk(p->mu);
+            if (!p->d_vector) {
+                HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->d_vector), (size_t(p->cols) + p->rows) * 4u));
+                p->fixed_bytes += (size_t(p->cols) + p->rows) * 4u;
+            }
+        }
+        uint32_t *b2 = p->d_vector, *c2 = p->d_vector + p->cols;
+        if (launch) HSPMM_HIP(hspmm::launch_widen_halves(dB, b2, p->cols, s));
+        const int rc = run_gather(p, b2, c2, 2u, 2u, s, mid, mode);
+        if (rc) return rc;
+        if (launch) HSPMM_HIP(hspmm::launch_narrow_words(c2, dC, p->rows, s));
+        return HSPMM_OK;
+    }
     const uint32_t wide = p->elem == 2u ? 8u : 4u;
     const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
     if (p->cfg.kernel_mode != 1 && N > (p->elem == 2u && N % 2u ? 32u : wide) && N % wide != 0 && !(align & 3u)) {

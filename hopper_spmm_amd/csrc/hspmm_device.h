@@ -102,6 +102,10 @@ hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
 // below) -> plain tiles (8 x 16 of 16-bit elements, 8 x 8 of 32-bit elements)
 hipError_t launch_expand_bitmap(int elem_bytes, const uint32_t *header, const void *vals, void *tiles, uint32_t n_tiles,
                                 hipStream_t s);
+// n 16-bit elements -> n words with the element in the low half (launch_widen_halves), and back (launch_narrow_words):
+// a single feature of a 16-bit type runs as two features, the second all zero
+hipError_t launch_widen_halves(const void *src, void *dst, size_t n, hipStream_t s);
+hipError_t launch_narrow_words(const void *src, void *dst, size_t n, hipStream_t s);
 // plain 8 x 8 tiles of 32-bit elements, single windows -> the order the lanes of the fp32 gather kernels read them in
 hipError_t launch_lane_order32(const void *tiles, void *out, uint32_t n_tiles, hipStream_t s);
 // plain tiles -> bitmap tiles (8 x 16 tiles of 16-bit elements, elem_bytes = 2: 8 header words per tile, see

@@ -5,6 +5,7 @@
 // spmm_panel_<type>.hip).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <algorithm>
 #include "hspmm_device.h"
 
 namespace hspmm {
@@ -12,9 +13,9 @@ namespace hspmm {
 // ---------------------------------------------------------------------------
 // All-shapes kernel (any N, any alignment): one workgroup per effective window
 // and 256-feature slab, one thread per feature, plain fp32 multiply-add, reading
-// the format arrays exactly as the caller gave them.  Used for a single feature of a
-// 16-bit type, on request (kernel mode 1), and as an independent second implementation
-// in tests.
+// the format arrays exactly as the caller gave them.  Used on request (kernel mode 1),
+// for a single feature of a 16-bit type when the caller may not allocate
+// (hspmm_run_static), and as an independent second implementation in tests.
 // ---------------------------------------------------------------------------
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<_Float16>(_Float16 v) { return (float)v; }
@@ -343,6 +344,32 @@ hipError_t launch_bitmap_pack(int elem_bytes, const void *tiles, uint32_t *heade
         bitmap_pack32_kernel<<<dim3(word_blocks), 256, 0, s>>>(static_cast<const uint32_t *>(tiles), header,
                                                               static_cast<uint32_t *>(vals), n_tiles);
     }
+    return hipGetLastError();
+}
+
+// A single feature of a 16-bit type (matrix times vector) runs as two features, the second all zero: the MFMA
+// kernels read whole words.  widen: element i of `src` and a zero to words of `dst`; narrow: the low halves back.
+__global__ __launch_bounds__(256) void widen_halves_kernel(const uint16_t *__restrict__ src, uint32_t *__restrict__ dst, size_t n)
+{
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+__global__ __launch_bounds__(256) void narrow_words_kernel(const uint32_t *__restrict__ src, uint16_t *__restrict__ dst, size_t n)
+{
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = uint16_t(src[i]);
+}
+static uint32_t copy_blocks(size_t n) { return uint32_t(std::min<size_t>((n + 255u) / 256u, 65536u)); }
+hipError_t launch_widen_halves(const void *src, void *dst, size_t n, hipStream_t s)
+{
+    if (!n) return hipSuccess;
+    widen_halves_kernel<<<dim3(copy_blocks(n)), 256, 0, s>>>(static_cast<const uint16_t *>(src), static_cast<uint32_t *>(dst), n);
+    return hipGetLastError();
+}
+hipError_t launch_narrow_words(const void *src, void *dst, size_t n, hipStream_t s)
+{
+    if (!n) return hipSuccess;
+    narrow_words_kernel<<<dim3(copy_blocks(n)), 256, 0, s>>>(static_cast<const uint32_t *>(src), static_cast<uint16_t *>(dst), n);
     return hipGetLastError();
 }
 

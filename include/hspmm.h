@@ -70,8 +70,9 @@ int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
  * DEVICE pointers, row-major, aligned to the element size (the LDS-staging kernels
  * want 16 bytes and rows of whole 16-byte pieces, the widest loads of the other MFMA
  * kernels 16 bytes and N a multiple of 8 - of 4 for fp32 storage -; everything else
- * takes narrower loads or two launches, a single feature of a 16-bit type the
- * all-shapes kernel); every element of C is
+ * takes narrower loads or two launches; a single feature of a 16-bit type goes
+ * through a buffer of cols + rows words that the plan allocates at the first such
+ * launch or at hspmm_prepare(plan, 1)); every element of C is
  * written (rows without nonzeros become 0).  Asynchronous on `stream` (a
  * hipStream_t, NULL = default stream).
  * Host side: a plan is immutable after hspmm_create except for what the first
