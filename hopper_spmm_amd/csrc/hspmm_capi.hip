@@ -2039,7 +2039,13 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     }
     const uint32_t wide = p->elem == 2u ? 8u : 4u;
     const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
-    if (p->cfg.kernel_mode != 1 && N > (p->elem == 2u && N % 2u ? 32u : wide) && N % wide != 0 && !(align & 3u)) {
+    // (not where one block of the narrower loads covers all of N anyway)
+    bool one_block = false;
+    if (p->cfg.kernel_mode != 1) {
+        const Choice whole = choose_kernel(p, dB, dC, N, N);
+        one_block = !whole.scalar && N <= uint32_t(whole.block_feat);
+    }
+    if (p->cfg.kernel_mode != 1 && !one_block && N > wide && N % wide != 0 && !(align & 3u)) {
         const uint32_t first = N - N % wide - ((p->elem == 2u && N % wide == 1u) ? wide : 0u);
         const int rc = run_gather(p, dB, dC, first, N, s, mid, mode);
         if (rc) return rc;
