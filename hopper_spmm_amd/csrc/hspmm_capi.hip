@@ -2004,11 +2004,12 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
         // (the producers address a panel of B - up to 256 rows - with 32-bit offsets)
         const bool offsets_fit = uint64_t(N) * p->elem < (uint64_t(1) << 24);
-        // Whole blocks of features, or - the kernels built on the 16-bit MFMA, whose lanes own one feature per
-        // accumulator - any whole number of 16-byte pieces per row from one block on (from 16 features on for fp32
-        // storage, whose gather kernels multiply at a sixteenth of the rate): what the last block lacks is not stored.
-        const bool ragged_ok = (p->cw == 16 || p->panel.split) && (uint64_t(N) * p->elem) % 16u == 0 &&
-                               (p->dtype == HSPMM_TF32 ? N >= 16u : N >= block_feat);
+        // Whole blocks of features; or any N of one block at least - the last block then moves back to end with
+        // the row (panel_block_first_feature in spmm_mfma_kernel.hpp) -; or, fp32 storage in bf16 parts, whose
+        // gather kernels multiply at a sixteenth of the rate, one partly empty block from 16 features on when the
+        // rows are whole 16-byte pieces (the lanes of that kernel own one feature per accumulator: what the block
+        // lacks is read from the row's first piece and not stored).
+        const bool ragged_ok = N >= block_feat || (p->panel.split && (uint64_t(N) * p->elem) % 16u == 0 && N >= 16u);
         if (pays && offsets_fit && (N % block_feat == 0 || ragged_ok) && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
     }
     // A feature dimension that no wide load divides (16-bit types: N not a multiple of 8, fp32 storage: of 4) would

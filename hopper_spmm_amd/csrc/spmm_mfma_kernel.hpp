@@ -668,13 +668,21 @@ __device__ __forceinline__ uint32_t unit_windows(const uint32_t row_word)
 template <class LaneT, class = void> struct HasValidCount { static constexpr bool value = false; };
 template <class LaneT> struct HasValidCount<LaneT, decltype(void(LaneT::f_valid))> { static constexpr bool value = true; };
 template <class TT>
-__device__ __forceinline__ void set_valid_features(typename TT::Lane &L, uint32_t N, uint32_t fb)
+__device__ __forceinline__ void set_valid_features(typename TT::Lane &L, uint32_t N, uint32_t first)
 {
     if constexpr (HasValidCount<typename TT::Lane>::value) {
-        const uint32_t first = fb * uint32_t(TT::kBlockFeat);
         const uint32_t left = N > first ? N - first : 0u;
         L.f_valid = left < uint32_t(TT::kBlockFeat) ? left : uint32_t(TT::kBlockFeat);
     }
+}
+// First feature of feature block fb of the LDS-panel kernels.  A feature dimension of one block at least that ends
+// inside its last block: that block is moved back to end with the row - features N - block .. N - 1, all of them
+// there, every load inside the row - and computes the features it shares with the block in front of it a second
+// time (same tiles, same rows of B, same order: the same bits).
+__device__ __forceinline__ uint32_t panel_block_first_feature(uint32_t fb, uint32_t block, uint32_t N)
+{
+    const uint32_t first = fb * block;
+    return (first + block > N && N >= block) ? N - block : first;
 }
 
 // An odd feature dimension of a 16-bit type (wide-load layout, one word per lane): the lane whose first feature is
@@ -949,8 +957,10 @@ void spmm_fixup_kernel(const KernelArgs ka)
 
     typename TT::Lane L;
     L.init(lane, ka.tiles, ka.ids);
-    set_valid_features<TT>(L, ka.N, fb);
-    const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
+    // (the sums of the LDS-panel kernels: their last feature block may have been moved back, see above)
+    const uint32_t first = uniform ? panel_block_first_feature(fb, uint32_t(TT::kBlockFeat), ka.N) : fb * uint32_t(TT::kBlockFeat);
+    set_valid_features<TT>(L, ka.N, first);
+    const uint32_t feat = first + L.j * TT::kLaneFeat;
     const bool active = feat < ka.N;
     (void)mark_half_lane<TT>(L, ka.N, feat);
     const size_t row_bytes = size_t(ka.ld) * TT::kElem;

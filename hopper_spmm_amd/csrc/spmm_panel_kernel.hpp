@@ -607,7 +607,9 @@ __device__ __forceinline__ void panel_barrier()
 // panel images to LDS: the consumers' register ring of tile / id loads then never
 // has to wait for a panel load (vector loads return in order, and a wave that had
 // both kinds in flight would drain its ring at every panel).
-template <class TT, int NC, int NPW, bool TALL = false, bool PACKED = false>
+// RAGGED: the feature dimension is no whole number of feature blocks (a build of its own, so that the kernel for
+// whole blocks is exactly the one it was: it is sensitive to every register and instruction around its loop).
+template <class TT, int NC, int NPW, bool TALL = false, bool PACKED = false, bool RAGGED = false>
 __global__ __launch_bounds__((NC + NPW) * 64)
 void spmm_panel_kernel(const PanelArgs pa)
 {
@@ -644,6 +646,8 @@ void spmm_panel_kernel(const PanelArgs pa)
     const uint32_t p_begin = chunk * pa.panels_per_chunk;
     const uint32_t p_end = umin32(p_begin + pa.panels_per_chunk, pa.n_panels);
     const size_t row_bytes = size_t(pa.N) * TT::kElem;
+    // first feature of this block
+    const uint32_t feat0 = RAGGED ? panel_block_first_feature(fb, uint32_t(TT::kBlockFeat), pa.N) : fb * uint32_t(TT::kBlockFeat);
 
     if (wave >= uint32_t(NC)) {
         // ---- producer: panel q goes to buffer q & 1, then the barrier that releases it.
@@ -651,11 +655,11 @@ void spmm_panel_kernel(const PanelArgs pa)
         // the barrier of panel q - 1.
         const uint32_t pt = threadIdx.x - uint32_t(NC) * 64u;       // 0 .. NPW*64-1
         // piece c = pt + i * NPW*64 is bytes [16c, 16c + 16) of the image: row c / 16, 16-byte column c % 16
-        const char *b_block = reinterpret_cast<const char *>(pa.B) + size_t(fb) * kPanelRowBytes;
+        const char *b_block = reinterpret_cast<const char *>(pa.B) + size_t(feat0) * TT::kElem;
         // (a feature dimension that ends inside this block: a piece behind a row's end is read from the row's
         // first piece instead - the features it would feed are never stored, and no load leaves the row)
         const uint32_t piece_row0 = pt >> 4;
-        const uint32_t col_bytes = size_t(fb) * kPanelRowBytes + (pt & 15u) * 16u < row_bytes ? (pt & 15u) * 16u : 0u;
+        const uint32_t col_bytes = (!RAGGED || size_t(feat0) * TT::kElem + (pt & 15u) * 16u < row_bytes) ? (pt & 15u) * 16u : 0u;
         // Addresses: the panel's first row (the same in all lanes) plus 32-bit offsets inside the panel
         // (the host checks that a panel of B spans less than 4 GB).  Rows past the matrix are never
         // referenced: their loads are bent to the matrix's last row.
@@ -720,7 +724,7 @@ void spmm_panel_kernel(const PanelArgs pa)
 
     typename TT::Lane L;
     L.init(lane, pa.tiles, pa.ids);
-    const uint32_t feat = fb * TT::kBlockFeat + L.j * TT::kLaneFeat;
+    const uint32_t feat = feat0 + L.j * TT::kLaneFeat;
     char *c_lane = reinterpret_cast<char *>(pa.C) + size_t(feat) * TT::kElem;
 
     // steps [t0, t1) of the unit lie in this chunk of panels; a wave without a unit has none
@@ -878,7 +882,8 @@ void spmm_panel_kernel(const PanelArgs pa)
     for (; owed; --owed) panel_barrier();
 
     if (!has_unit) return;
-    set_valid_features<TT>(L, pa.N, fb);        // (here, not at the top: nothing of it lives through the steps)
+    // (here, not at the top: nothing of it lives through the steps)
+    if constexpr (RAGGED) set_valid_features<TT>(L, pa.N, feat0);
     // Stores unit `unit` from the sums in `sums` (or leaves them as this chunk's partial sums).
     auto finish = [&](const uint32_t unit, f32x4 (&sums)[Ops::kLive]) __attribute__((always_inline)) {
         Ops::fold(sums);
@@ -949,7 +954,8 @@ static hipError_t launch_panel_tt(const PanelArgs &pa, const KernelArgs &ka, hip
     const uint32_t wave_units = TALL ? (pa.n_units + 1u) / 2u : pa.n_units;     // what one consumer wave takes
     const uint32_t row_blocks = (wave_units + pa.units_per_group - 1u) / pa.units_per_group;
     const dim3 grid(row_blocks * pa.n_feat_blocks * pa.n_chunks), block((NC + NPW) * 64);
-    spmm_panel_kernel<TT, NC, NPW, TALL, PACKED><<<grid, block, 0, s>>>(pa);
+    if (pa.N % uint32_t(TT::kBlockFeat) != 0) spmm_panel_kernel<TT, NC, NPW, TALL, PACKED, true><<<grid, block, 0, s>>>(pa);
+    else spmm_panel_kernel<TT, NC, NPW, TALL, PACKED, false><<<grid, block, 0, s>>>(pa);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || pa.n_chunks == 1u || pa.arrive) return e;
     if (mid && (e = hipEventRecord(mid, s)) != hipSuccess) return e;
