@@ -1998,7 +1998,6 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     if (p->panel.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4)) {
         // LDS-panel kernels: a workgroup covers 256 bytes of every B row with 16-byte accesses
         const uint32_t block_feat = hspmm::kPanelRowBytes / p->elem;
-        const uintptr_t align = reinterpret_cast<uintptr_t>(dB) | reinterpret_cast<uintptr_t>(dC);
         // (a 16-bit matrix near the break-even is served as fast or faster by the gather kernels while
         // one wave of theirs covers all of N)
         const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
@@ -2010,7 +2009,8 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         // rows are whole 16-byte pieces (the lanes of that kernel own one feature per accumulator: what the block
         // lacks is read from the row's first piece and not stored).
         const bool ragged_ok = N >= block_feat || (p->panel.split && (uint64_t(N) * p->elem) % 16u == 0 && N >= 16u);
-        if (pays && offsets_fit && (N % block_feat == 0 || ragged_ok) && !(align & 15u)) return run_panel(p, dB, dC, N, s, mid, mode);
+        // (B and C wherever they start: the producers' 16-byte loads need no alignment, C is stored element by element)
+        if (pays && offsets_fit && (N % block_feat == 0 || ragged_ok)) return run_panel(p, dB, dC, N, s, mid, mode);
     }
     // A feature dimension that no wide load divides (16-bit types: N not a multiple of 8, fp32 storage: of 4) would
     // run in blocks of 32 resp. 16 features, each block a pass over the tiles and another gather of every row

@@ -68,8 +68,8 @@ int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
 /* Replaces one launch of fp16_spmm_kernel (reference src/fp16.cu:256): computes
  * all of C = A*B for feature dimension N.  dB (cols x N) and dC (rows x N) are
  * DEVICE pointers, row-major, aligned to the element size (the LDS-staging kernels
- * want 16 bytes and one block of features - 256 bytes of a row -, the widest loads of the other MFMA
- * kernels 16 bytes and N a multiple of 8 - of 4 for fp32 storage -; everything else
+ * want one block of features - 256 bytes of a row - and take B and C wherever they start, the widest loads
+ * of the other MFMA kernels want 16 bytes and N a multiple of 8 - of 4 for fp32 storage -; everything else
  * takes narrower loads or two launches; a single feature of a 16-bit type goes
  * through a buffer of cols + rows words that the plan allocates at the first such
  * launch or at hspmm_prepare(plan, 1)); every element of C is
@@ -158,7 +158,7 @@ void hspmm_get_config(int *buffer_stage, int *consumer_warp_num,
  * scalar all-shapes kernel, 2 = 16-bit MFMA kernel with wide loads only, 3 =
  * 16-bit MFMA kernel with word loads whenever N is a multiple of 32, 4 = the
  * LDS-staging kernels for every matrix (whenever N is 128 at least - 64 for fp32
- * storage, or 16 with rows of whole 16-byte pieces - and B and C are 16-byte aligned), 5 = the same
+ * storage, or 16 with rows of whole 16-byte pieces), 5 = the same
  * with fp32 products in the HSPMM_TF32 LDS-staging kernels (N 64 at least).  (By default those
  * kernels multiply the bf16 parts hi + lo of every fp32 factor, which keeps 16
  * mantissa bits per factor; the reference's tf32 instruction keeps 10,

@@ -977,9 +977,10 @@ def test_odd_feature_dims_of_the_16_bit_types(torch_cuda, hs, oracle):
 
 @pytest.mark.parametrize("dtype", [0, 1])
 def test_pointer_alignment_selects_the_kernel_family(torch_cuda, hs, oracle, dtype):
-    """B and C need only be aligned to the element size: the LDS-staging kernels want 16 bytes, the
-    MFMA gather kernels take anything (8 and 16 bytes for their wider loads, single words loaded wherever
-    they lie for B or C on an odd half) - with the same result (exact integers) whatever the offsets."""
+    """B and C need only be aligned to the element size: the LDS-staging kernels load their 16-byte pieces
+    wherever they lie and store C element by element, the MFMA gather kernels (kernel mode 3 here) pick their
+    load width by the alignment (single words loaded wherever they lie for B or C on an odd half) - with the
+    same result (exact integers) whatever the offsets."""
     torch = torch_cuda
     rng = np.random.default_rng(61 + dtype)
     rows, cols, N = 96, 1024, 128
@@ -992,17 +993,22 @@ def test_pointer_alignment_selects_the_kernel_family(torch_cuda, hs, oracle, dty
         rp[r + 1] = len(ci)
     A = dict(rows=rows, cols=cols, dtype=dtype, row_ptr=rp, col_idx=np.array(ci, np.uint32),
              values=encode(np.array(vv, np.float32), dtype))
-    plan = hs.Plan(convert(hs, A))
-    assert plan.info()["n_panels"] > 0
+    plans = {3: hs.Plan(convert(hs, A))}
+    assert plans[3].info()["n_panels"] > 0
+    hs.set_kernel_mode(3)
+    try:
+        plans[2] = hs.Plan(convert(hs, A))
+    finally:
+        hs.set_kernel_mode(0)
     Bm = rng.integers(-4, 5, (cols, N))
     want = encode(D @ Bm, dtype)
     es = 4 if dtype == 1 else 2
     tt = torch.float32 if dtype == 1 else torch.int16
     host_b = torch.from_numpy(encode(Bm, dtype) if dtype == 1 else encode(Bm, dtype).view(np.int16))
-    seen = set()
-    for off_b, off_c in ((0, 0), (16, 32), (8, 0), (0, 4), (4, 4), (2, 0), (0, 2), (6, 10)):
+    for want_family, off_b, off_c in [(f, b, c) for f in (3, 2) for b, c in ((0, 0), (16, 32), (8, 0), (0, 4), (4, 4), (2, 0), (0, 2), (6, 10))]:
         if off_b % es or off_c % es:
             continue
+        plan = plans[want_family]
         buf_b = torch.zeros(cols * N + 16, dtype=tt, device="cuda")
         buf_c = torch.full((rows * N + 16,), 7, dtype=tt, device="cuda")
         dB = buf_b[off_b // es: off_b // es + cols * N]
@@ -1017,13 +1023,9 @@ def test_pointer_alignment_selects_the_kernel_family(torch_cuda, hs, oracle, dty
         # nothing outside C was written
         edge = buf_c.cpu().numpy()
         assert (edge[:off_c // es] == 7).all() and (edge[off_c // es + rows * N:] == 7).all()
-        family = plan.info()["last_kernel_family"]
-        seen.add(family)
-        worst = (off_b | off_c) % 16
-        # (B or C on an odd half: the gather kernels still, with one word per lane loaded wherever it lies)
-        assert family == (3 if worst == 0 else 2), (off_b, off_c, family)
-    assert seen == {3, 2}
-    plan.close()
+        assert plan.info()["last_kernel_family"] == want_family, (off_b, off_c)
+    for plan in plans.values():
+        plan.close()
 
 
 def test_matrix_without_entries_gives_zeros(torch_cuda, hs):
