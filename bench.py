@@ -65,6 +65,21 @@ def cpu_baseline(A, B, N, flops_full):
     }
 
 
+def kernel_sources_digest():
+    """sha256 over the kernel and host sources libhspmm.so is built from: the counter figures of
+    profiles/traffic.json carry the digest they were measured with."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "hopper_spmm_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(csrc, "*"))):
+        if path.endswith((".hip", ".hpp", ".h", ".cpp")) or os.path.basename(path) == "Makefile":
+            h.update(os.path.basename(path).encode())
+            with open(path, "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
 def info_family(plan):
     return plan.info()["last_kernel_family"]
 
@@ -194,6 +209,9 @@ def main():
     if os.path.exists(tfile):
         with open(tfile) as f:
             traffic = json.load(f).get("config%d_N%d" % (args.config, N))
+        if traffic is not None:
+            # false: the kernels' sources have changed since the counters were read
+            traffic["measured_with_these_sources"] = traffic.get("kernel_sources_sha256") == kernel_sources_digest()
 
     kernels_ms = main_ms + fix_ms
     out = {
