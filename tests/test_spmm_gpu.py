@@ -28,13 +28,31 @@ def torch_cuda():
     return torch
 
 
-def gpu_spmm(torch, hs, btcf, B, N, plan=None, poison=True):
-    """C = A*B on the device through hspmm_run; B, C as numpy (uint16 bits / float32)."""
+def gpu_spmm(torch, hs, btcf, B, N, plan=None, poison=True, offsets=None):
+    """C = A*B on the device through hspmm_run; B, C as numpy (uint16 bits / float32).
+    offsets = (bytes, bytes): B and C start that far (multiples of the element size, < 64) into their
+    allocations, and the bytes around C must come back untouched."""
     own = plan is None
     if own:
         plan = hs.Plan(btcf)
     dt = btcf["dtype"]
     rows = btcf["rows"]
+    stream = torch.cuda.current_stream().cuda_stream
+    if offsets is not None:
+        off_b, off_c = offsets
+        host_b = np.ascontiguousarray(B, np.float32 if dt == 1 else np.uint16)
+        bytes_b = torch.from_numpy(host_b.view(np.uint8).reshape(-1))
+        raw_b = torch.zeros(bytes_b.numel() + 128, dtype=torch.uint8, device="cuda")
+        raw_b[off_b:off_b + bytes_b.numel()].copy_(bytes_b)
+        size_c = rows * N * host_b.itemsize
+        raw_c = torch.full((size_c + 256,), 0xA5, dtype=torch.uint8, device="cuda")     # (fp32: a NaN pattern too)
+        plan.run(raw_b.data_ptr() + off_b, raw_c.data_ptr() + 64 + off_c, N, stream)
+        torch.cuda.synchronize()
+        host_c = raw_c.cpu().numpy()
+        if own:
+            plan.close()
+        assert (host_c[:64 + off_c] == 0xA5).all() and (host_c[64 + off_c + size_c:] == 0xA5).all(), "bytes next to C written"
+        return host_c[64 + off_c:64 + off_c + size_c].copy().view(host_b.dtype).reshape(rows, N)
     if dt != 1:
         dB = torch.from_numpy(np.ascontiguousarray(B, np.uint16).view(np.int16)).cuda()
         dC = torch.empty((rows, N), dtype=torch.int16, device="cuda")
@@ -45,7 +63,6 @@ def gpu_spmm(torch, hs, btcf, B, N, plan=None, poison=True):
         dC = torch.empty((rows, N), dtype=torch.float32, device="cuda")
         if poison:
             dC.fill_(float("nan"))
-    stream = torch.cuda.current_stream().cuda_stream
     plan.run(dB.data_ptr(), dC.data_ptr(), N, stream)
     torch.cuda.synchronize()
     out = dC.cpu().numpy()
@@ -873,13 +890,14 @@ def test_seeded_sweep_of_shapes_formats_and_kernel_choices(torch_cuda, hs, oracl
         assert_parity(got, ref, mag, dtype, what, tight=False)
 
 
-@pytest.mark.parametrize("seed", [21, 22])
+@pytest.mark.parametrize("seed", [21, 22, 23])
 def test_seeded_sweep_of_stream_modes_group_cuts_and_tuning_overrides(torch_cuda, hs, oracle, seed):
     """As the sweep above (120 combinations per seed), with the choices it leaves at their defaults drawn as well:
     the stream mode of the LDS-staging kernels, grouped input that keeps the caller's cuts, tiles written column
     by column, and the overrides read from the environment at plan creation (bitmap stream of the gather kernels,
     feature blocks dealt out by XCD, partial sums added inside the main kernel, one workgroup per unit for small
-    matrices, windows per unit of the panel stream)."""
+    matrices, windows per unit of the panel stream), feature dimensions that end inside a block of features or
+    are odd, and B and C that start anywhere on an element (nothing around C may be written)."""
     knobs = ("HSPMM_GATHER_BITMAP", "HSPMM_XCD_SPLIT", "HSPMM_FUSED_FIXUP", "HSPMM_ALIGNED_SMALL", "HSPMM_PANEL_MAX_WINDOWS")
     rng = np.random.default_rng(seed)
     for case in range(120):
@@ -900,12 +918,16 @@ def test_seeded_sweep_of_stream_modes_group_cuts_and_tuning_overrides(torch_cuda
         for name, chance, values in zip(knobs, (0.3, 0.3, 0.3, 0.2, 0.2), ([0, 1], [0, 1], [0, 1], [0, 4, 8], [2, 4])):
             if rng.random() < chance:
                 env[name] = str(int(rng.choice(values)))
-        if mode >= 4:
-            N = int(rng.choice([64, 128, 192, 256, 320, 512])) if dtype == 1 else int(rng.choice([128, 256, 384, 640, 1024]))
+        if mode >= 4 and dtype == 1:
+            N = int(rng.choice([16, 20, 48, 64, 65, 67, 68, 80, 100, 127, 128, 130, 144, 192, 250, 256, 320, 512]))
+        elif mode >= 4:
+            N = int(rng.choice([128, 129, 130, 136, 144, 200, 208, 250, 255, 256, 384, 400, 640, 1000, 1001, 1024]))
         else:
-            N = int(rng.choice([1, 2, 3, 8, 16, 24, 32, 40, 64, 96, 128, 136, 256, 320, 512, 1000]))
-        what = "seed %d case %d: type %s %dx%d density %g empty %g heavy %s mode %d pairing %d format %d stages %d rps %d stream %d %s N %d" % (
-            seed, case, DT[dtype], rows, cols, dens, erp, heavy, mode, pairing, fmt, stages, ranges_per_simd, stream, env, N)
+            N = int(rng.choice([1, 2, 3, 6, 7, 8, 10, 16, 24, 30, 32, 40, 64, 96, 100, 127, 128, 130, 136, 250, 256, 320, 512, 1000, 1002]))
+        element = 4 if dtype == 1 else 2
+        offsets = tuple(int(rng.choice([0, 0, 1, 2, 3, 4, 5, 8])) * element if rng.random() < 0.5 else 0 for _ in range(2))
+        what = "seed %d case %d: type %s %dx%d density %g empty %g heavy %s mode %d pairing %d format %d stages %d rps %d stream %d %s N %d B, C %s bytes in" % (
+            seed, case, DT[dtype], rows, cols, dens, erp, heavy, mode, pairing, fmt, stages, ranges_per_simd, stream, env, N, offsets)
         hs.set_kernel_mode(mode)
         hs.set_window_pairing(pairing)
         hs.set_panel_stream(stream)
@@ -931,7 +953,7 @@ def test_seeded_sweep_of_stream_modes_group_cuts_and_tuning_overrides(torch_cuda
             for name in knobs:
                 os.environ.pop(name, None)
         B = make_b(rng, cols, N, dtype)
-        got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan)
+        got = gpu_spmm(torch_cuda, hs, b, B, N, plan=plan, offsets=offsets)
         plan.close()
         ref, mag = oracle_spmm(oracle, A, B, N)
         assert_parity(got, ref, mag, dtype, what, tight=False)
