@@ -1594,10 +1594,13 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     // measured 1027 -> 895 us at N = 136 and 1175 -> 1259 us at N = 200: not done.)
     // A single feature of a 16-bit type (matrix times vector): B and C widened to words - the element and a zero -
     // in a buffer of the plan's, two features through the MFMA kernels, the low halves back (power-law graph 2^20:
-    // 21 ms on the all-shapes kernel).  hspmm_run_static, which allocates nothing, keeps the all-shapes kernel.
-    if (p->elem == 2u && N == 1u && p->cfg.kernel_mode != 1 && mode != RunMode::kStatic) {
+    // 21 ms on the all-shapes kernel).  hspmm_run_static, which allocates nothing, wants the buffer made already.
+    if (p->elem == 2u && N == 1u && p->cfg.kernel_mode != 1) {
         {
             std::lock_guard<std::mutex> lk(p->mu);
+            if (!p->d_vector && mode == RunMode::kStatic)
+                return fail(HSPMM_ERR_UNSUPPORTED, "hspmm_run_static: a single feature of a 16-bit type goes through a buffer "
+                            "of the plan's that does not exist yet (call hspmm_prepare(plan, 1) or hspmm_run with N = 1 first)");
             if (!p->d_vector) {
                 HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->d_vector), (size_t(p->cols) + p->rows) * 4u));
                 p->fixed_bytes += (size_t(p->cols) + p->rows) * 4u;

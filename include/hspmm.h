@@ -100,7 +100,8 @@ int hspmm_prepare(hspmm_plan *plan, uint32_t N);
  * array of device memory that the library holds on every device it is loaded
  * on (HSPMM_STATIC_SCRATCH_BYTES, from library load until the process ends)
  * instead of the plan's own buffer.  It calls no hipMalloc / hipFree and builds
- * nothing: the work partition for this N must exist already (hspmm_prepare, or
+ * nothing: the work partition for this N (and, for a single feature of a 16-bit
+ * type, the plan's buffer of cols + rows words) must exist already (hspmm_prepare, or
  * one hspmm_run with this N), else HSPMM_ERR_UNSUPPORTED; so does a launch whose
  * partial sums exceed the array (the message says how much it needs).  Results
  * are bit-identical to hspmm_run.  All calls on one device share the one array

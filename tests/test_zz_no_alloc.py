@@ -88,6 +88,41 @@ def test_static_scratch_entry_point_matches_hspmm_run(torch_cuda, hs, oracle, dt
         plan.close()
 
 
+def test_static_scratch_entry_point_with_a_single_feature(torch_cuda, hs, oracle):
+    """Matrix times vector in a 16-bit type goes through a buffer of the plan's (B and C widened to words): the
+    entry point refuses until hspmm_prepare(plan, 1) has made it, then gives the bits of hspmm_run."""
+    torch = torch_cuda
+    stream = torch.cuda.current_stream().cuda_stream
+    rng = np.random.default_rng(78)
+    A = random_csr(rng, 300, 3000, 0.004, 0, 0.2, (5, 100, 299))
+    b = convert(hs, A)
+    hs.configure(producer_warp_group_num=16)                        # (cut windows: partial sums in the fixed array)
+    try:
+        plan = hs.Plan(b)
+    finally:
+        hs.configure()
+    B = make_b(rng, A["cols"], 1, 0)
+    dB, dC = _device_buffers(torch, B, A["rows"], 1, 0)
+    with pytest.raises(hs.HspmmError) as e:
+        plan.run_static(dB.data_ptr(), dC.data_ptr(), 1, stream)
+    assert "hspmm_prepare" in str(e.value)
+    plan.prepare(1)
+    before = plan.info()["device_bytes"]
+    for _ in range(2):
+        _poison(dC, 0)
+        plan.run_static(dB.data_ptr(), dC.data_ptr(), 1, stream)
+        torch.cuda.synchronize()
+        got = _result(dC, 0)
+        assert plan.info()["last_kernel_family"] == 2 and plan.info()["device_bytes"] == before
+    _poison(dC, 0)
+    plan.run(dB.data_ptr(), dC.data_ptr(), 1, stream)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.view(np.uint8), _result(dC, 0).view(np.uint8))
+    ref, mag = oracle_spmm(oracle, A, B, 1)
+    assert_parity(got, ref, mag, 0, "single feature")
+    plan.close()
+
+
 def test_static_scratch_entry_point_rejects_what_does_not_fit(torch_cuda, hs):
     """A launch whose partial sums exceed the fixed array is refused with a message that says so."""
     torch = torch_cuda
