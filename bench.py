@@ -223,8 +223,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 in, f32 accumulate" if dt == hs.FP16 else "f32 (tf32 variant)",
         "data": "synthetic",
-        # seeded generators of hopper_spmm_amd/generators.py: bit-stable for a given numpy version
-        "data_generator": "numpy %s Philox" % np.__version__,
+        # seeded generators of hopper_spmm_amd/generators.py: raw words of Philox 4x64-10 (numpy's bit generator, a
+        # stream numpy keeps stable) through the module's own transforms (Box-Muller normals)
+        "data_generator": "Philox 4x64-10 raw words, own transforms (numpy %s)" % np.__version__,
         "config": {"workload": "configs[%d]: %s, N=%d" % (args.config, cfg["name"], N),
                    "rows": A["rows"], "cols": A["cols"], "nnz": nnz, "tiles": int(b["total_tiles"]),
                    "eff_row_windows": int(b["eff_row_windows"]), "ranges": info["n_ranges"],
