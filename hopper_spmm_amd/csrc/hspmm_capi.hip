@@ -181,12 +181,21 @@ struct hspmm_plan {
         uint64_t stored = 0;
         bool from_caller = false;     // header and elements are the caller's tcBit / nnzOffset / data, uploaded as they came
     } bm;
-    float *d_scratch = nullptr;
-    size_t scratch_bytes = 0;
-    uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
-    size_t arrive_words = 0;
-    uint32_t *d_vector = nullptr;       // a single 16-bit feature widened to words: cols words of B, then rows words of C
-                                        // (made by the first launch with N = 1)
+    // What launches write besides C, one set per stream that has launched this plan (launches on different
+    // streams may overlap in time): the first stream seen gets set 0, every other stream a set of its own at its
+    // first launch - except a stream that is being captured (no allocation under capture) and streams beyond
+    // kMaxStreamBuffers, which share set 0.
+    struct StreamBuffers {
+        hipStream_t stream = nullptr;
+        float *d_scratch = nullptr;         // partial sums of cut units
+        size_t scratch_bytes = 0;
+        uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
+        size_t arrive_words = 0;
+        uint32_t *d_vector = nullptr;       // a single 16-bit feature widened to words: cols words of B, then rows words
+                                            // of C (made by the first launch with N = 1, or by hspmm_prepare(plan, 1))
+    };
+    static constexpr size_t kMaxStreamBuffers = 16;
+    std::vector<StreamBuffers> buffers;
     size_t fixed_bytes = 0;
     // Every real column list strictly ascending and padding only behind a window's last column: what the
     // reference's converters write (reference src/utils/convert.h:166-181).  The gather and all-shapes
@@ -716,27 +725,62 @@ int static_scratch_address(int device, float **out)
     return HSPMM_OK;
 }
 
-// Arrival counters of the in-kernel reduction (an experiment switch, never used by hspmm_run_static).
-// Called with the plan's mutex held.
-int ensure_arrive(hspmm_plan *p, size_t words, uint32_t **out)
+// The set of buffers a launch on stream s uses (see hspmm_plan::StreamBuffers); create = false (hspmm_run_static,
+// which allocates nothing): the stream's own set if it has one, else set 0, null if there is none yet.
+// Called with the plan's mutex held; the reference is good until the mutex is released.
+hspmm_plan::StreamBuffers *buffers_for(hspmm_plan *p, hipStream_t s, bool create)
 {
-    if (words > p->arrive_words) {
-        uint32_t *fresh = nullptr;
-        HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&fresh), words * 4));
-        HSPMM_HIP(hipMemset(fresh, 0, words * 4));
-        HSPMM_HIP(hipStreamSynchronize(nullptr));   // the launch that follows may be on a stream that does not wait for this one
-        if (p->d_arrive) p->retired.push_back(p->d_arrive);
-        p->d_arrive = fresh;
-        p->arrive_words = words;
+    for (auto &b : p->buffers)
+        if (b.stream == s) return &b;
+    if (!create) return p->buffers.empty() ? nullptr : &p->buffers[0];
+    bool own_set = p->buffers.size() < hspmm_plan::kMaxStreamBuffers;
+    if (own_set && !p->buffers.empty() && s != nullptr) {
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &status) != hipSuccess || status != hipStreamCaptureStatusNone) own_set = false;
     }
-    *out = p->d_arrive;
+    if (!own_set && !p->buffers.empty()) return &p->buffers[0];
+    p->buffers.emplace_back();
+    p->buffers.back().stream = s;
+    return &p->buffers.back();
+}
+
+// The sets of buffers a call fills: that of the stream; hspmm_prepare (no stream, nothing launched): every set
+// there is, set 0 made if there is none.  Called with the plan's mutex held.
+std::vector<hspmm_plan::StreamBuffers *> sets_for(hspmm_plan *p, hipStream_t s, RunMode mode)
+{
+    std::vector<hspmm_plan::StreamBuffers *> sets;
+    if (mode != RunMode::kPrepare) {
+        sets.push_back(buffers_for(p, s, true));
+        return sets;
+    }
+    if (p->buffers.empty()) p->buffers.emplace_back();
+    for (auto &b : p->buffers) sets.push_back(&b);
+    return sets;
+}
+
+// Arrival counters of the in-kernel reduction (never used by hspmm_run_static).
+// Called with the plan's mutex held.
+int ensure_arrive(hspmm_plan *p, hipStream_t s, size_t words, RunMode mode, uint32_t **out)
+{
+    for (hspmm_plan::StreamBuffers *b : sets_for(p, s, mode)) {
+        if (words > b->arrive_words) {
+            uint32_t *fresh = nullptr;
+            HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&fresh), words * 4));
+            HSPMM_HIP(hipMemset(fresh, 0, words * 4));
+            HSPMM_HIP(hipStreamSynchronize(nullptr));   // the launch that follows may be on a stream that does not wait for this one
+            if (b->d_arrive) p->retired.push_back(b->d_arrive);
+            b->d_arrive = fresh;
+            b->arrive_words = words;
+        }
+        *out = b->d_arrive;
+    }
     return HSPMM_OK;
 }
 
 // The buffer for `bytes` of partial sums.  kStatic: the device's fixed array (bytes must fit).  Else the
-// plan's buffer, grown when too small (sizes are powers of two, so the superseded buffers, which stay
+// buffer of the stream's set, grown when too small (sizes are powers of two, so the superseded buffers, which stay
 // allocated until hspmm_destroy, never add up to more than the current one).  Called with the plan's mutex held.
-int scratch_for(hspmm_plan *p, size_t bytes, RunMode mode, float **out)
+int scratch_for(hspmm_plan *p, hipStream_t s, size_t bytes, RunMode mode, float **out)
 {
     if (mode == RunMode::kStatic) {
         if (bytes > kStaticScratchBytes)
@@ -745,16 +789,18 @@ int scratch_for(hspmm_plan *p, size_t bytes, RunMode mode, float **out)
                         "(use hspmm_run)", bytes, kStaticScratchBytes);
         return static_scratch_address(p->device, out);
     }
-    if (bytes > p->scratch_bytes) {
-        size_t cap = size_t(1) << 16;
-        while (cap < bytes) cap <<= 1;
-        float *fresh = nullptr;
-        HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&fresh), cap));
-        if (p->d_scratch) p->retired.push_back(p->d_scratch);
-        p->d_scratch = fresh;
-        p->scratch_bytes = cap;
+    for (hspmm_plan::StreamBuffers *b : sets_for(p, s, mode)) {
+        if (bytes > b->scratch_bytes) {
+            size_t cap = size_t(1) << 16;
+            while (cap < bytes) cap <<= 1;
+            float *fresh = nullptr;
+            HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&fresh), cap));
+            if (b->d_scratch) p->retired.push_back(b->d_scratch);
+            b->d_scratch = fresh;
+            b->scratch_bytes = cap;
+        }
+        *out = b->d_scratch;
     }
-    *out = p->d_scratch;
     return HSPMM_OK;
 }
 
@@ -1412,7 +1458,7 @@ void hspmm_destroy(hspmm_plan *p)
     (void)hipFree(p->panel.d_step_panel);
     (void)hipFree(p->panel.d_masks); (void)hipFree(p->panel.d_vals); (void)hipFree(p->panel.d_step_voff);
     (void)hipFree(p->bm.d_header); (void)hipFree(p->bm.d_vals);
-    (void)hipFree(p->d_scratch); (void)hipFree(p->d_arrive); (void)hipFree(p->d_vector);
+    for (auto &b : p->buffers) { (void)hipFree(b.d_scratch); (void)hipFree(b.d_arrive); (void)hipFree(b.d_vector); }
     for (void *old : p->retired) (void)hipFree(old);
     delete p;
 }
@@ -1515,13 +1561,13 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
             return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many partial sums", N);
         {
             std::lock_guard<std::mutex> lk(p->mu);
-            int rc = scratch_for(p, need, mode, &pa.scratch);
+            int rc = scratch_for(p, s, need, mode, &pa.scratch);
             if (rc) return rc;
             // As in the gather kernels, the wave that brings a unit's last chunk adds the chunk sums itself
             // (16-byte device-scope accesses; block-clustered configuration at N = 512: 56.0 + 8.1 us in two
             // launches, 60.3 us in one).  It addresses a unit's chunk sums with 32-bit offsets.
             if (p->cfg.fused_fixup != 0 && mode != RunMode::kStatic && uint64_t(pa.n_chunks) * pa.n_feat_blocks * nacc * 1024u < (1ull << 31) &&
-                (rc = ensure_arrive(p, size_t(pl.n_units) * pa.n_feat_blocks, &pa.arrive)))
+                (rc = ensure_arrive(p, s, size_t(pl.n_units) * pa.n_feat_blocks, mode, &pa.arrive)))
                 return rc;
         }
         // the chunk sums of unit u are slots u * chunks .. + chunks - 1: no table
@@ -1596,17 +1642,26 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     // in a buffer of the plan's, two features through the MFMA kernels, the low halves back (power-law graph 2^20:
     // 21 ms on the all-shapes kernel).  hspmm_run_static, which allocates nothing, wants the buffer made already.
     if (p->elem == 2u && N == 1u && p->cfg.kernel_mode != 1) {
+        uint32_t *b2 = nullptr;
         {
             std::lock_guard<std::mutex> lk(p->mu);
-            if (!p->d_vector && mode == RunMode::kStatic)
-                return fail(HSPMM_ERR_UNSUPPORTED, "hspmm_run_static: a single feature of a 16-bit type goes through a buffer "
-                            "of the plan's that does not exist yet (call hspmm_prepare(plan, 1) or hspmm_run with N = 1 first)");
-            if (!p->d_vector) {
-                HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&p->d_vector), (size_t(p->cols) + p->rows) * 4u));
-                p->fixed_bytes += (size_t(p->cols) + p->rows) * 4u;
+            if (mode == RunMode::kStatic) {
+                hspmm_plan::StreamBuffers *b = buffers_for(p, s, false);
+                if (!b || !b->d_vector)
+                    return fail(HSPMM_ERR_UNSUPPORTED, "hspmm_run_static: a single feature of a 16-bit type goes through a buffer "
+                                "of the plan's that does not exist yet (call hspmm_prepare(plan, 1) or hspmm_run with N = 1 first)");
+                b2 = b->d_vector;
+            } else {
+                for (hspmm_plan::StreamBuffers *b : sets_for(p, s, mode)) {
+                    if (!b->d_vector) {
+                        HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&b->d_vector), (size_t(p->cols) + p->rows) * 4u));
+                        p->fixed_bytes += (size_t(p->cols) + p->rows) * 4u;
+                    }
+                    b2 = b->d_vector;
+                }
             }
         }
-        uint32_t *b2 = p->d_vector, *c2 = p->d_vector + p->cols;
+        uint32_t *c2 = b2 + p->cols;
         if (launch) HSPMM_HIP(hspmm::launch_widen_halves(dB, b2, p->cols, s));
         const int rc = run_gather(p, b2, c2, 2u, 2u, s, mid, mode);
         if (rc) return rc;
@@ -1708,9 +1763,9 @@ static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint3
         if (uint64_t(ka.n_ranges) * ka.n_feat_blocks > 0x7FFFFFFFull)
             return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many work items", N);
         const size_t need = size_t(dp.part.n_slots) * ka.n_feat_blocks * size_t(c.V) * size_t(p->G) * 64u * 16u;
-        int rc = scratch_for(p, need, mode, &ka.scratch);
+        int rc = scratch_for(p, s, need, mode, &ka.scratch);
         if (rc) return rc;
-        if (fused && ka.n_split && (rc = ensure_arrive(p, size_t(ka.n_split) * ka.n_feat_blocks, &ka.arrive))) return rc;
+        if (fused && ka.n_split && (rc = ensure_arrive(p, s, size_t(ka.n_split) * ka.n_feat_blocks, mode, &ka.arrive))) return rc;
     }
     ka.ranges = dp.d_ranges; ka.split = dp.d_split; ka.fix_slots = dp.d_fix_slots;
     if (!launch) return HSPMM_OK;
@@ -1843,7 +1898,11 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->compute_units = uint32_t(p->compute_units);
     info->n_units = p->n_units;
     info->n_paired_units = p->n_paired;
-    info->device_bytes = uint64_t(p->fixed_bytes) + uint64_t(p->scratch_bytes);
+    info->device_bytes = uint64_t(p->fixed_bytes);
+    {
+        std::lock_guard<std::mutex> lk(const_cast<hspmm_plan *>(p)->mu);
+        for (const auto &b : p->buffers) info->device_bytes += uint64_t(b.scratch_bytes);
+    }
     info->n_panels = p->panel.built ? p->panel.n_panels : 0u;
     info->n_panel_steps = p->panel.built ? p->panel.n_steps : 0u;
     info->n_panel_units = p->panel.built ? p->panel.n_units : 0u;

@@ -76,22 +76,31 @@ int hspmm_create(hspmm_plan **plan, int dtype, uint32_t rows, uint32_t cols,
  * written (rows without nonzeros become 0).  Asynchronous on `stream` (a
  * hipStream_t, NULL = default stream).
  * Host side: a plan is immutable after hspmm_create except for what the first
- * launch with a new N may add under the plan's own mutex - a work partition for
- * that width and a larger buffer for partial sums (older buffers stay allocated
- * until hspmm_destroy, so launches recorded earlier, e.g. in a HIP graph, stay
- * valid whatever N is run afterwards).  hspmm_run may therefore be called from
- * several threads; after hspmm_prepare(plan, N), or one earlier call with that
- * N, it only launches kernels (no allocation, memset or copy) and can be
+ * launch with a new N, or on a new stream, may add under the plan's own mutex -
+ * a work partition for that width and buffers for what a launch writes besides C
+ * (partial sums of cut windows, their arrival counters; older buffers stay
+ * allocated until hspmm_destroy, so launches recorded earlier, e.g. in a HIP
+ * graph, stay valid whatever N is run afterwards).  hspmm_run may therefore be
+ * called from several threads; after one earlier call with that N on that
+ * stream it only launches kernels (no allocation, memset or copy) and can be
  * captured in a HIP graph.
- * Device side: launches of one plan share its partial-sum buffer, so two
- * launches of one plan must not overlap in time (one stream per plan, or an
- * event between them); different plans may run concurrently. */
+ * Device side: every stream that launches a plan gets buffers of its own at its
+ * first launch, so launches of one plan on different streams may overlap in time
+ * (as may different plans); launches on one stream are ordered anyway.  Two
+ * exceptions share the buffers of the first stream the plan saw, and must then
+ * not overlap with its launches: a stream that is being captured when it first
+ * launches the plan (nothing is allocated under capture: launch once on that
+ * stream before the capture, or call hspmm_prepare(plan, N) first and keep the
+ * graph's replays apart from launches on the plan's first stream), and streams
+ * beyond the sixteenth. */
 int hspmm_run(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stream);
 
 /* No reference counterpart (the reference allocates inside every call,
  * src/fp16.cu:236-249): builds now what the first hspmm_run with feature
- * dimension N would build - the work partition for that width and the buffer
- * for partial sums, for every alignment of B and C - and launches nothing. */
+ * dimension N would build - the work partition for that width and, for every
+ * stream that has launched the plan so far (for the set that the first stream
+ * and streams under capture use, if none has), the buffers a launch writes
+ * besides C, for every alignment of B and C - and launches nothing. */
 int hspmm_prepare(hspmm_plan *plan, uint32_t N);
 
 /* No reference counterpart; for callers that must not allocate device memory

@@ -1121,6 +1121,48 @@ def test_plans_on_different_streams_do_not_disturb_each_other(torch_cuda, hs, or
         plan.close()
 
 
+@pytest.mark.parametrize("dtype,density,heavy,N", [(0, 0.003, (3, 200, 777), 64), (2, 0.1, (), 256), (1, 0.1, (), 64), (0, 0.02, (5,), 1)])
+def test_one_plan_on_several_streams_at_once(torch_cuda, hs, oracle, dtype, density, heavy, N):
+    """Launches of one plan on different streams may overlap in time: every stream that launches a plan gets
+    partial-sum buffers, arrival counters and (a single feature of a 16-bit type) a vector buffer of its own.
+    Three streams, each with its own B and C, launched round robin without waiting; every output must be
+    bit-identical to what the plan gives for that B alone, and the plan's device memory grows with the streams."""
+    torch = torch_cuda
+    rng = np.random.default_rng(31)
+    rows, cols = 1600, 8000
+    A = random_csr(rng, rows, cols, density, dtype, 0.1, heavy)
+    b = convert(hs, A)
+    hs.configure(producer_warp_group_num=16)                        # (many ranges: units cut across waves)
+    try:
+        plan = hs.Plan(b)
+    finally:
+        hs.configure()
+    tt = torch.float32 if dtype == 1 else torch.int16
+    lanes = []
+    for k in range(3):
+        B = make_b(rng, cols, N, dtype)
+        alone = gpu_spmm(torch, hs, b, B, N, plan=plan)
+        if k == 0:
+            ref, mag = oracle_spmm(oracle, A, B, N)
+            assert_parity(alone, ref, mag, dtype, "alone")
+            assert plan.info()["n_split_windows"] > 0 or plan.info()["n_panels"] > 0    # (something uses the buffers)
+        dB = torch.from_numpy(B if dtype == 1 else B.view(np.int16)).cuda()
+        dC = torch.empty((rows, N), dtype=tt, device="cuda")
+        lanes.append((dB, dC, alone, torch.cuda.Stream()))
+    torch.cuda.synchronize()
+    one_stream = plan.info()["device_bytes"]
+    for _ in range(30):
+        for dB, dC, _, stream in lanes:
+            plan.run(dB.data_ptr(), dC.data_ptr(), N, stream.cuda_stream)
+    torch.cuda.synchronize()
+    assert plan.info()["device_bytes"] > one_stream
+    for k, (dB, dC, alone, _) in enumerate(lanes):
+        got = dC.cpu().numpy()
+        got = got if dtype == 1 else got.view(np.uint16)
+        assert np.array_equal(got, alone), "stream %d" % k
+    plan.close()
+
+
 def test_run_captured_in_a_hip_graph_replays_correctly(torch_cuda, hs, oracle):
     """After one eager call (which sizes the plan's scratch memory) hspmm_run only
     launches kernels, so a stream capture records it; every replay, with eager work
