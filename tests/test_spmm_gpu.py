@@ -1217,6 +1217,51 @@ def test_run_captured_in_a_hip_graph_replays_correctly(torch_cuda, hs, oracle):
         plan.close()
 
 
+def test_capture_right_after_prepare_on_a_stream_the_plan_has_not_seen(torch_cuda, hs, oracle):
+    """hspmm_prepare(plan, N) makes the buffers a stream under capture uses (nothing may be allocated then): the
+    first launch of the plan at all may be the one recorded, on a stream of its own, after eager launches on
+    another stream as well."""
+    torch = torch_cuda
+    rng = np.random.default_rng(17)
+    for dtype, density, heavy, N, eager_first in ((0, 0.003, (3, 200), 64, False), (1, 0.1, (), 128, False), (2, 0.1, (), 256, True)):
+        A = random_csr(rng, 400, 4000, density, dtype, 0.1, heavy)
+        b = convert(hs, A)
+        hs.configure(producer_warp_group_num=16)
+        try:
+            plan = hs.Plan(b)
+        finally:
+            hs.configure()
+        B = make_b(rng, 4000, N, dtype)
+        tt = torch.float32 if dtype == 1 else torch.int16
+        dB = torch.from_numpy(B if dtype == 1 else B.view(np.int16)).cuda()
+        dC = torch.empty((400, N), dtype=tt, device="cuda")
+        plan.prepare(N)
+        if eager_first:
+            gpu_spmm(torch, hs, b, B, N, plan=plan)             # (the default stream becomes the plan's first stream)
+        before = plan.info()["device_bytes"]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)
+        assert plan.info()["device_bytes"] == before            # nothing allocated under capture
+        want = None
+        for rep in range(3):
+            dC.fill_(0x7E01 if dtype != 1 else float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = dC.cpu().numpy()
+            got = got if dtype == 1 else got.view(np.uint16)
+            if want is None:
+                want = gpu_spmm(torch, hs, b, B, N, plan=plan)
+                ref, mag = oracle_spmm(oracle, A, B, N)
+                assert_parity(got, ref, mag, dtype, "recorded launch")
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "replay %d" % rep
+        del graph
+        plan.close()
+
+
 def test_graph_captured_at_one_width_survives_launches_at_another(torch_cuda, hs, oracle):
     """A launch recorded in a HIP graph carries the addresses of the plan's partial-sum buffer and
     tables.  Running the same plan eagerly at a wider N afterwards (more partial sums, another number
