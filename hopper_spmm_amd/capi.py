@@ -17,8 +17,7 @@ IDX_MAX = 0xFFFFFFFF
 ROW_WINDOW = 8
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# HSPMM_LIBRARY: another build of the library to load instead (the measurement builds of `make measure`)
-_LIB = os.environ.get("HSPMM_LIBRARY") or os.path.join(_HERE, "libhspmm.so")
+_LIB = os.path.join(_HERE, "libhspmm.so")
 _lib = None
 
 
@@ -32,9 +31,12 @@ def library_path():
     return _LIB
 
 
-def build_library(force=True):
-    """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU)."""
+def build_library(force=True, experimental=False):
+    """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU).  experimental: also the kernel
+    variants that no automatic plan selects (EXPERIMENTAL=1 of csrc/Makefile)."""
     cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j8"]
+    if experimental:
+        cmd.append("EXPERIMENTAL=1")
     if force:
         cmd.insert(1, "-B")
     subprocess.check_call(cmd, stdout=subprocess.DEVNULL)
@@ -109,6 +111,7 @@ def load_library():
     L.hspmm_set_kernel_mode.argtypes = [i]
     L.hspmm_set_window_pairing.argtypes = [i]
     L.hspmm_set_panel_stream.argtypes = [i]
+    L.hspmm_has_experimental.argtypes = []
     L.hspmm_set_group_cuts.argtypes = [i]
     L.hspmm_get_plan_info.argtypes = [vp, C.POINTER(PlanInfo)]
     L.hspmm_get_partition.argtypes = [vp, vp, u32]
@@ -198,6 +201,11 @@ def set_group_cuts(mode):
     """1: plans made from groups (GBTCF_MTX) cut a window only where the caller's groups end; 0 (default): where
     the plan's cost model puts the cuts.  Read by the next plan creation."""
     _check(load_library().hspmm_set_group_cuts(mode))
+
+
+def has_experimental():
+    """True when the library holds the kernel variants no automatic plan selects (built with EXPERIMENTAL=1)."""
+    return bool(load_library().hspmm_has_experimental())
 
 
 def set_panel_stream(mode):

@@ -74,38 +74,37 @@ struct Config {
     int group_cuts = 0;                 // 1: plans of hspmm_create_grouped cut a window only where the caller's groups end
     // Tuning overrides from the environment (HSPMM_*), read once by hspmm_create: a plan's behaviour does
     // not change with the environment afterwards and the launch path reads no variable.
-    double window_cost = 1.5, slack = 0.35, whole_window_margin = 32.0;     // cost model of partition.hpp
-    double aligned_four_from = 2.5;     // ways the balanced partition must cut every unit before one workgroup walks it
-    double panel_wide_cost = 1.25;      // a step of three or four windows, in steps of two
-    int panel_units = 0;                // workgroup shape of the LDS-panel kernels: 12, 13, 14 (0: by tile type)
-    int panel_units_per_group = 0;      // consumer waves of a workgroup that get a unit (0: searched per N)
     int panel_chunks = 0;               // chunks of panels (0: searched per N)
     int panel_max_windows = 0;          // 2 or 4: windows per unit of the panel stream (0: by matrix size)
-    int panel_tall = 0;                 // LDS-panel waves with two units each (1: whenever the stream allows)
-    int panel_packed = 0;               // ... and their tiles stored without zeros (1: whenever the stream allows)
     int aligned_small = -1;             // small matrices: waves per unit of the one-workgroup-per-unit partition (-1: by size; 0, 4, 8)
     int gather_bitmap = -1;             // gather kernels read single 16-bit windows as bitmap + stored elements (-1: by fill)
     int xcd_split = -1;                 // gather kernels: two feature blocks dealt out by XCD half (-1: by matrix, 0 never, 1 always)
+    // (set through hspmm_set_panel_stream; builds with HSPMM_EXPERIMENTAL only)
+    int panel_tall = 0;                 // LDS-panel waves with two units each
+    int panel_packed = 0;               // ... and their tiles stored without zeros
+    int panel_units_per_group = 0;      // consumer waves of a workgroup that get a unit (0: searched per N)
+    // (builds with HSPMM_EXPERIMENTAL only)
+    int panel_units = 0;                // workgroup shape of the fp32-MFMA LDS-panel kernels: 12, 13, 14 (0: by tile type)
 
     void read_environment()
     {
         if (const char *e = std::getenv("HSPMM_FUSED_FIXUP")) fused_fixup = std::atoi(e) != 0;
-        if (const char *e = std::getenv("HSPMM_WINDOW_COST")) window_cost = std::atof(e);
-        if (const char *e = std::getenv("HSPMM_SLACK")) slack = std::atof(e);
-        if (const char *e = std::getenv("HSPMM_WHOLE_WINDOW_MARGIN")) whole_window_margin = std::atof(e);
-        if (const char *e = std::getenv("HSPMM_ALIGNED_FOUR_FROM")) aligned_four_from = std::atof(e);
-        if (const char *e = std::getenv("HSPMM_PANEL_WIDE_COST")) panel_wide_cost = std::atof(e);
-        if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) panel_units = std::atoi(e) == 14 ? 14 : std::atoi(e) == 13 ? 13 : 12;
-        if (const char *e = std::getenv("HSPMM_PANEL_UNITS_PER_GROUP")) panel_units_per_group = std::max(1, std::atoi(e));
         if (const char *e = std::getenv("HSPMM_PANEL_CHUNKS")) panel_chunks = std::max(1, std::atoi(e));
         if (const char *e = std::getenv("HSPMM_PANEL_MAX_WINDOWS")) panel_max_windows = std::atoi(e) >= 4 ? 4 : 2;
         if (const char *e = std::getenv("HSPMM_XCD_SPLIT")) xcd_split = std::atoi(e) != 0;
         if (const char *e = std::getenv("HSPMM_GATHER_BITMAP")) gather_bitmap = std::atoi(e) != 0;
         if (const char *e = std::getenv("HSPMM_ALIGNED_SMALL")) { const int v = std::atoi(e); aligned_small = v == 4 || v == 8 ? v : 0; }
-        if (const char *e = std::getenv("HSPMM_PANEL_TALL")) panel_tall = std::atoi(e) != 0;
-        if (const char *e = std::getenv("HSPMM_PANEL_PACKED")) panel_packed = std::atoi(e) != 0;
+        if (const char *e = std::getenv("HSPMM_PANEL_UNITS_PER_GROUP")) panel_units_per_group = std::max(1, std::atoi(e));
+#ifdef HSPMM_EXPERIMENTAL
+        if (const char *e = std::getenv("HSPMM_PANEL_UNITS")) panel_units = std::atoi(e) == 14 ? 14 : std::atoi(e) == 13 ? 13 : 12;
+#endif
     }
 };
+// cost model of partition.hpp (a range costs its steps + 1.5 per unit; a cut within 35 % of a mean range of a unit
+// boundary snaps onto it; units up to a mean range + 32 steps are never cut)
+constexpr double kWindowCost = 1.5, kSlack = 0.35, kWholeWindowMargin = 32.0;
+constexpr double kAlignedFourFrom = 2.5;   // ways the balanced partition must cut every unit before one workgroup walks it
+constexpr double kPanelWideCost = 1.25;    // a step of three or four windows, in steps of two
 std::mutex g_cfg_mutex;
 Config g_cfg;
 
@@ -148,6 +147,8 @@ struct hspmm_plan {
     int aligned_group = 0;              // waves of the workgroup that walks one unit in [4]; 0: units too short for it
     std::vector<uint32_t> h_unitOffset;
     std::vector<uint32_t> h_unitRow;       // first row of every unit | its windows less one (for hspmm_partition_as_groups)
+    std::vector<uint32_t> h_winOffset, h_winRow;   // plans whose units merge windows: the caller's rowOffset and rowIdx
+                                                   // (hspmm_partition_as_groups writes groups of the caller's tiles)
     std::vector<uint32_t> caller_cuts;     // hspmm_create_grouped with hspmm_set_group_cuts(1): the ends of the caller's groups,
                                            // the only places where the gather kernels' partition cuts a window
     // LDS-panel kernels (matrices whose windows touch a large share of the columns):
@@ -187,6 +188,7 @@ struct hspmm_plan {
     // kMaxStreamBuffers, which share set 0.
     struct StreamBuffers {
         hipStream_t stream = nullptr;
+        bool unowned = false;               // made by hspmm_prepare before any launch: the first stream to launch takes it
         float *d_scratch = nullptr;         // partial sums of cut units
         size_t scratch_bytes = 0;
         uint32_t *d_arrive = nullptr;       // arrival counters of cut units, zero between launches
@@ -207,6 +209,7 @@ struct hspmm_plan {
     // Superseded scratch buffers stay allocated until hspmm_destroy: launches recorded earlier (HIP
     // graphs) carry their addresses.
     std::vector<void *> retired;
+    size_t retired_bytes = 0;               // partial-sum buffers among them (counters are part of fixed_bytes)
     std::atomic<uint32_t> last_family{0};   // kernel family of the last hspmm_run: 0 none yet, 1 all-shapes, 2 gather, 3 LDS-panel, 4 clear
 };
 
@@ -305,7 +308,7 @@ int build_and_upload_partition(hspmm_plan *p, int level, uint32_t group = 1, boo
 {
     hspmm_plan::DevPartition &dp = p->parts[aligned ? 4 : group > 1 ? 3 : level];
     if (dp.built || p->W == 0) return HSPMM_OK;
-    const double window_cost = p->cfg.window_cost, slack = p->cfg.slack, margin = p->cfg.whole_window_margin;
+    const double window_cost = kWindowCost, slack = kSlack, margin = kWholeWindowMargin;
     uint32_t target = uint32_t(choose_ranges(p)) >> level;
     const uint32_t floor_ranges = uint32_t(p->compute_units) * 4u;       // at least one range per SIMD
     if (target < floor_ranges) target = std::min<uint32_t>(floor_ranges, uint32_t(choose_ranges(p)));
@@ -410,12 +413,18 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
         // 8192 and 11008 rows: 0.93 - 1.1 x up to N = 512, 1.2 - 1.3 x only from N = 2048 on), and for
         // fp32 storage in bf16 parts, with twice the MFMAs per LDS read, they gain nothing (0.82 - 1.2 x).
         // Pairing mode 2 takes them wherever windows qualify.
-        const double wide_cost = p->cfg.panel_wide_cost;
+        const double wide_cost = kPanelWideCost;
         uint32_t max_windows = (p->cfg.pairing == 2 || cw == 16) ? 4u : 2u;
+#ifndef HSPMM_EXPERIMENTAL
+        if (split) max_windows = 2u;            // (units of four windows in bf16 parts measured 0.82 - 1.2 x: not built)
+#endif
         size_t min_wide_units = p->cfg.pairing == 2 ? 0u : size_t(p->compute_units) * 3u / 2u;
         if (p->cfg.panel_max_windows) {                                                           // tuning override
             max_windows = uint32_t(p->cfg.panel_max_windows);
             min_wide_units = 0;
+#ifndef HSPMM_EXPERIMENTAL
+            if (split) max_windows = 2u;
+#endif
         }
         std::vector<uint32_t> first, count;
         group_windows(W, cw, uint32_t(p->elem), KP, rw, max_windows, wide_cost, min_wide_units, rowOffset, tcA2B, data,
@@ -487,29 +496,34 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
                     last_pn += kMaxJump;
                     rt_panel[at++] = last_pn;
                 }
-                const uint32_t nt = (i - a + rw - 1) / rw;
+                const uint32_t cnt = i - a, nt = (cnt + rw - 1) / rw;
+                // The columns of every step.  16-bit MFMA forms: one LDS instruction reads, in each block of 16
+                // lanes, the rows of four columns of the step (block g, instruction h: columns 8g + 4h .. + 3), the
+                // LDS serves two blocks (g = 0, 1 or g = 2, 3) at a time, and rows whose numbers differ mod 8 lie
+                // in different banks.  So a step should hold every remainder mod 8 at most four times, dealt out over
+                // the four sets of eight columns that are read together.  Any choice of columns makes a step: the
+                // window's columns in this panel, ordered by remainder (stable), are dealt out over the panel's
+                // steps in turn - a step then holds floor or ceil of every remainder's share (pruned weights at 10 %:
+                // about 26 of 32 rows per remainder and 7 steps; consecutive columns per step gave five or six of one
+                // remainder in most steps, one conflict cycle per LDS read) and the steps are equally full.
+                uint32_t perm[hspmm::kPanelRowsWide];
+                if (rw == 32) {
+                    uint32_t m = 0;
+                    for (uint32_t res = 0; res < 8; ++res)
+                        for (uint32_t k = a; k < i; ++k)
+                            if (((col[k] - pn * KP) & 7u) == res) perm[m++] = k;
+                }
                 for (uint32_t tl = 0; tl < nt; ++tl, ++at) {
                     rt_panel[at] = pn;
-                    // The columns of the step.  16-bit types: one LDS instruction reads, in each block of 16
-                    // lanes, the rows of four consecutive columns of the step (block g, instruction h: columns
-                    // 8g + 4h .. + 3), the LDS serves two blocks (g = 0, 1 or g = 2, 3) at a time, and rows
-                    // whose numbers differ mod 8 lie in different banks: columns ordered by row number mod 8
-                    // (stable) and dealt out over the four sets of eight that are read together put
-                    // different remainders into a set wherever the step has them.
-                    const uint32_t first_col = a + tl * rw, n = std::min(rw, i - first_col);
+                    // n columns: rw == 32: perm[tl], perm[tl + nt], ... (in remainder order); else consecutive ones
+                    const uint32_t n = rw == 32 ? (cnt - tl + nt - 1) / nt : std::min(rw, cnt - tl * rw);
+                    auto source = [&](uint32_t k) { return rw == 32 ? perm[tl + k * nt] : a + tl * rw + k; };
                     uint32_t order[32];
                     if (rw == 32) {
-                        uint32_t sorted[32], m = 0;
-                        for (uint32_t res = 0; res < 8; ++res)
-                            for (uint32_t k = 0; k < rw; ++k) {
-                                // padding takes the row of the last real column (its tile column stays zero)
-                                const uint32_t c = col[first_col + std::min(k, n - 1)] - pn * KP;
-                                if ((c & 7u) == res) sorted[m++] = k;
-                            }
                         for (uint32_t k = 0; k < rw; ++k) {
                             const uint32_t set = k % 4, e = k / 4;          // set = 2 * (g / 2) + h
                             const uint32_t g = 2 * (set / 2) + e / 4, h = set % 2;
-                            order[8 * g + 4 * h + e % 4] = sorted[k];
+                            order[8 * g + 4 * h + e % 4] = k;
                         }
                     } else {
                         for (uint32_t k = 0; k < rw; ++k) order[k] = k;
@@ -517,7 +531,8 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
                     uint8_t *dt_tile = rt_data.data() + at * tile_bytes;
                     for (uint32_t k = 0; k < rw; ++k) {
                         const uint32_t from = order[k];
-                        const uint32_t srci = first_col + std::min(from, n - 1);
+                        // padding takes the row of the step's last real column (its tile column stays zero)
+                        const uint32_t srci = source(std::min(from, n - 1));
                         rt_ids[at * rw + k] = col[srci] - pn * KP;      // row inside the panel
                         if (from >= n) continue;
                         const uint8_t *st_tile = src_data + size_t(t0 + srci / cw) * src_tile_bytes;
@@ -731,7 +746,13 @@ int static_scratch_address(int device, float **out)
 hspmm_plan::StreamBuffers *buffers_for(hspmm_plan *p, hipStream_t s, bool create)
 {
     for (auto &b : p->buffers)
-        if (b.stream == s) return &b;
+        if (b.stream == s && !b.unowned) return &b;
+    // the set hspmm_prepare made before any launch goes to the first stream that launches (also one under capture)
+    if (!p->buffers.empty() && p->buffers[0].unowned) {
+        p->buffers[0].stream = s;
+        p->buffers[0].unowned = false;
+        return &p->buffers[0];
+    }
     if (!create) return p->buffers.empty() ? nullptr : &p->buffers[0];
     bool own_set = p->buffers.size() < hspmm_plan::kMaxStreamBuffers;
     if (own_set && !p->buffers.empty() && s != nullptr) {
@@ -753,7 +774,10 @@ std::vector<hspmm_plan::StreamBuffers *> sets_for(hspmm_plan *p, hipStream_t s, 
         sets.push_back(buffers_for(p, s, true));
         return sets;
     }
-    if (p->buffers.empty()) p->buffers.emplace_back();
+    if (p->buffers.empty()) {
+        p->buffers.emplace_back();
+        p->buffers.back().unowned = true;
+    }
     for (auto &b : p->buffers) sets.push_back(&b);
     return sets;
 }
@@ -766,11 +790,18 @@ int ensure_arrive(hspmm_plan *p, hipStream_t s, size_t words, RunMode mode, uint
         if (words > b->arrive_words) {
             uint32_t *fresh = nullptr;
             HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&fresh), words * 4));
-            HSPMM_HIP(hipMemset(fresh, 0, words * 4));
-            HSPMM_HIP(hipStreamSynchronize(nullptr));   // the launch that follows may be on a stream that does not wait for this one
+            if (mode == RunMode::kPrepare) {
+                // no stream yet: cleared now, and waited for, so that any stream may launch afterwards
+                HSPMM_HIP(hipMemset(fresh, 0, words * 4));
+                HSPMM_HIP(hipStreamSynchronize(nullptr));
+            } else {
+                // cleared by a kernel on the launching stream, in front of the launch that counts in it
+                HSPMM_HIP(hspmm::launch_fill_zero(fresh, words * 4, s));
+            }
             if (b->d_arrive) p->retired.push_back(b->d_arrive);
             b->d_arrive = fresh;
             b->arrive_words = words;
+            p->fixed_bytes += words * 4;
         }
         *out = b->d_arrive;
     }
@@ -795,7 +826,7 @@ int scratch_for(hspmm_plan *p, hipStream_t s, size_t bytes, RunMode mode, float 
             while (cap < bytes) cap <<= 1;
             float *fresh = nullptr;
             HSPMM_HIP(hipMalloc(reinterpret_cast<void **>(&fresh), cap));
-            if (b->d_scratch) p->retired.push_back(b->d_scratch);
+            if (b->d_scratch) { p->retired.push_back(b->d_scratch); p->retired_bytes += b->scratch_bytes; }
             b->d_scratch = fresh;
             b->scratch_bytes = cap;
         }
@@ -814,8 +845,13 @@ const char *hspmm_last_error(void) { return g_last_error.c_str(); }
 
 int hspmm_configure(int buffer_stage, int consumer_warp_num, int producer_warp_group_num, int sm_num)
 {
+#ifdef HSPMM_EXPERIMENTAL
     if (buffer_stage < 0 || buffer_stage > 8 || buffer_stage == 5 || buffer_stage == 7)
         return fail(HSPMM_ERR_INVALID, "buffer_stage %d: supported depths are 1, 2, 3, 4, 6, 8 (0 = default)", buffer_stage);
+#else
+    if (buffer_stage != 0 && (buffer_stage < 2 || buffer_stage > 4))
+        return fail(HSPMM_ERR_INVALID, "buffer_stage %d: supported depths are 2, 3, 4 (0 = default)", buffer_stage);
+#endif
     if (consumer_warp_num < 0 || consumer_warp_num > hspmm::kMaxWavesPerGroup)
         return fail(HSPMM_ERR_INVALID, "consumer_warp_num %d outside 0..%d", consumer_warp_num, hspmm::kMaxWavesPerGroup);
     if (producer_warp_group_num < 0 || producer_warp_group_num > 16)
@@ -862,9 +898,23 @@ int hspmm_set_group_cuts(int mode)
     return HSPMM_OK;
 }
 
+int hspmm_has_experimental(void)
+{
+#ifdef HSPMM_EXPERIMENTAL
+    return 1;
+#else
+    return 0;
+#endif
+}
+
 int hspmm_set_panel_stream(int mode)
 {
     if (mode < 0 || mode > 2) return fail(HSPMM_ERR_INVALID, "panel stream mode %d outside 0..2", mode);
+#ifndef HSPMM_EXPERIMENTAL
+    if (mode != 0)
+        return fail(HSPMM_ERR_UNSUPPORTED, "panel stream mode %d needs a library built with EXPERIMENTAL=1 (the default "
+                    "stream measured faster)", mode);
+#endif
     std::lock_guard<std::mutex> lk(g_cfg_mutex);
     g_cfg.panel_tall = mode >= 1;
     g_cfg.panel_packed = mode == 2;
@@ -883,7 +933,7 @@ static int partition_preview(uint32_t eff_row_windows, const uint32_t *rowOffset
         if (rowOffset[w + 1] <= rowOffset[w] || rowOffset[0] != 0)
             return fail(HSPMM_ERR_INVALID, "rowOffset must start at 0 and increase strictly");
     const hspmm::Partition part =
-        hspmm::build_partition(eff_row_windows, rowOffset, target_ranges, 1.5, 0.35, 32.0, group, allowed_cuts);
+        hspmm::build_partition(eff_row_windows, rowOffset, target_ranges, kWindowCost, kSlack, kWholeWindowMargin, group, allowed_cuts);
     if (n_ranges) *n_ranges = uint32_t(part.ranges.size());
     if (n_split_windows) *n_split_windows = uint32_t(part.split.size());
     if (n_partial_slots) *n_partial_slots = part.n_slots;
@@ -980,7 +1030,7 @@ int hspmm_panel_units_preview(int dtype, uint32_t rows, uint32_t cols, uint32_t 
     const void *d = data;
     try {
         // column lists that do not ascend strictly, or with padding inside a window, are never merged
-        group_windows(W, cw, elem, hspmm::kPanelRowsWide, 32u, canonical ? max_windows : 1u, 1.25, 0, rowOffset, tcA2B, d,
+        group_windows(W, cw, elem, hspmm::kPanelRowsWide, 32u, canonical ? max_windows : 1u, kPanelWideCost, 0, rowOffset, tcA2B, d,
                       rowIdx, un, first, count);
     } catch (const std::bad_alloc &) { return fail(HSPMM_ERR_ALLOC, "out of host memory"); }
     const uint32_t T = W ? rowOffset[W] : 0u;
@@ -1209,6 +1259,10 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
         timer.mark("bitmap tiles");
         p->h_unitOffset = st.unitOffset;
         p->h_unitRow = st.unitRow;
+        if (st.G != 1) {
+            p->h_winOffset.assign(rowOffset, rowOffset + size_t(p->W) + 1u);
+            p->h_winRow.assign(rowIdx, rowIdx + size_t(p->W));
+        }
         // single windows walked tile by tile: the caller's tile numbers are the stream's, its cuts can be kept
         if (cuts && p->cfg.group_cuts && st.G == 1) p->caller_cuts.assign(cuts->offsets, cuts->offsets + size_t(cuts->n_groups) + 1u);
         if ((rc = build_and_upload_partition(p, 0))) return bail(rc);
@@ -1221,7 +1275,7 @@ int create_plan(hspmm_plan **out, int dtype, uint32_t rows, uint32_t cols, uint3
                 shortest = std::min(shortest, st.unitOffset[u + 1] - st.unitOffset[u]);
             const double steps_per_range = double(p->n_steps) / double(p->parts[0].part.ranges.size());
             const double ways = double(p->n_steps) / double(p->n_units) / steps_per_range;
-            const double four_from = p->cfg.aligned_four_from;
+            const double four_from = kAlignedFourFrom;
             const int group = ways >= 8.0 ? hspmm::kAlignedGroupWaves : ways >= four_from ? hspmm::kMaxWavesPerGroup : 0;
             if (group && shortest >= 8u * uint32_t(group) && uint64_t(p->n_units) * group <= (1u << 24)) p->aligned_group = group;
             // A matrix too small to fill the waves of the GPU with ranges of useful length: what its launch takes
@@ -1475,9 +1529,12 @@ int hspmm_run_static(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *
 
 int hspmm_prepare(hspmm_plan *p, uint32_t N)
 {
-    // B and C at the three alignments that select different load widths (and so different partitions and
-    // amounts of partial sums); nothing is launched and the pointers are never dereferenced
-    for (uintptr_t align : {uintptr_t(16), uintptr_t(8), uintptr_t(4)}) {
+    // B and C at the alignments that select different load widths (and so different partitions and amounts of
+    // partial sums; 2: a 16-bit B or C that starts on an odd half); nothing is launched and the pointers are
+    // never dereferenced
+    if (!p) return fail(HSPMM_ERR_INVALID, "null plan");
+    for (uintptr_t align : {uintptr_t(16), uintptr_t(8), uintptr_t(4), uintptr_t(2)}) {
+        if (align < p->elem) continue;
         const int rc = run_impl(p, reinterpret_cast<const void *>(align), reinterpret_cast<void *>(align), N, nullptr,
                                 nullptr, RunMode::kPrepare);
         if (rc) return rc;
@@ -1770,10 +1827,11 @@ static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint3
     ka.ranges = dp.d_ranges; ka.split = dp.d_split; ka.fix_slots = dp.d_fix_slots;
     if (!launch) return HSPMM_OK;
     p->last_family.store(2, std::memory_order_relaxed);
-    // default depth: what fits 128 registers per lane without spilling
-    const int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage
-                         : p->dtype == HSPMM_TF32 ? (p->G == 2 && c.V == 4 ? 3 : 4)
-                         : (p->G == 2 && c.V == 4 ? 2 : 3);
+    const int default_depth = hspmm::default_prefetch(int(p->elem), p->G, c.V);
+    int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage : default_depth;
+#ifndef HSPMM_EXPERIMENTAL
+    if (!c.narrow) prefetch = default_depth;      // (64-bit gather offsets are built for the default depth only)
+#endif
     HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, layout, p->G, ka, c.V, prefetch, c.narrow, wpg, s, mid));
     return HSPMM_OK;
 }
@@ -1898,9 +1956,10 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->compute_units = uint32_t(p->compute_units);
     info->n_units = p->n_units;
     info->n_paired_units = p->n_paired;
-    info->device_bytes = uint64_t(p->fixed_bytes);
     {
+        // everything the plan holds on the device: its arrays, the buffers of every stream, superseded buffers
         std::lock_guard<std::mutex> lk(const_cast<hspmm_plan *>(p)->mu);
+        info->device_bytes = uint64_t(p->fixed_bytes) + uint64_t(p->retired_bytes);
         for (const auto &b : p->buffers) info->device_bytes += uint64_t(b.scratch_bytes);
     }
     info->n_panels = p->panel.built ? p->panel.n_panels : 0u;
@@ -1932,10 +1991,21 @@ int hspmm_partition_as_groups(const hspmm_plan *p, uint32_t capacity_groups, uin
                               uint32_t *groupRowIdx, uint8_t *atomic)
 {
     if (!p || !total_groups) return fail(HSPMM_ERR_INVALID, "null argument");
-    if (p->W && p->G != 1)
-        return fail(HSPMM_ERR_UNSUPPORTED, "the plan walks pairs of windows: its ranges are not groups of the caller's tiles");
-    const std::vector<hspmm::Range> &ranges = p->parts[0].part.ranges;
-    const std::vector<uint32_t> &first_tile = p->h_unitOffset;       // single windows: a step is a tile
+    // A plan that walks pairs of windows has steps the caller never had: the groups then come from the balanced
+    // partition of the caller's single windows, built here with the plan's cost model.
+    hspmm::Partition own;
+    if (p->W && p->G != 1) {
+        const uint64_t waves = uint64_t(p->compute_units) * 4u * uint64_t(p->cfg.producer_warp_group_num > 0 ? p->cfg.producer_warp_group_num : 4);
+        const uint64_t cap = (uint64_t(p->T) + kMinTilesPerRange - 1) / kMinTilesPerRange;
+        const uint32_t target = uint32_t(std::max<uint64_t>(1, std::min(waves, cap)));
+        try {
+            own = hspmm::build_partition(p->W, p->h_winOffset.data(), target, kWindowCost, kSlack, kWholeWindowMargin, 1, nullptr);
+        } catch (const std::bad_alloc &) { return fail(HSPMM_ERR_ALLOC, "out of host memory"); }
+    }
+    const bool merged = p->W && p->G != 1;
+    const std::vector<hspmm::Range> &ranges = merged ? own.ranges : p->parts[0].part.ranges;
+    const std::vector<uint32_t> &first_tile = merged ? p->h_winOffset : p->h_unitOffset;     // single windows: a step is a tile
+    const std::vector<uint32_t> &first_row = merged ? p->h_winRow : p->h_unitRow;
     const bool write = groupOffset && groupRowIdx && atomic;
     uint32_t n = 0;
     for (const hspmm::Range &r : ranges) {
@@ -1944,7 +2014,7 @@ int hspmm_partition_as_groups(const hspmm_plan *p, uint32_t capacity_groups, uin
             const uint32_t end = std::min(r.tile_end, first_tile[w + 1]);
             if (write && n < capacity_groups) {
                 groupOffset[n] = t;
-                groupRowIdx[n] = p->h_unitRow[w] & ~7u;
+                groupRowIdx[n] = first_row[w] & ~7u;
                 atomic[n] = (t > first_tile[w] || end < first_tile[w + 1]) ? 1 : 0;     // the window continues in another group
             }
             ++n;

@@ -53,6 +53,13 @@ struct KernelArgs {
 constexpr int kLayoutX4 = 0, kLayoutDW = 1, kLayoutDWB = 2;   // DWB: word loads, tiles as bitmap + stored elements (16-bit, G = 1)
 // element types, numbered as HSPMM_FP16 / HSPMM_TF32 / HSPMM_BF16 of the public header
 constexpr int kDtypeF16 = 0, kDtypeF32 = 1, kDtypeBf16 = 2;
+// The gather kernels' prefetch depth (steps of loads in flight per wave) when the caller sets none: what fits 128
+// registers per lane without spilling.  Workgroups of eight waves and 64-bit gather offsets are built for this depth
+// only; depths 2, 3 and 4 exist for the rest (1, 6 and 8 in builds with HSPMM_EXPERIMENTAL).
+constexpr int default_prefetch(int elem_bytes, int G, int V)
+{
+    return elem_bytes == 4 ? (G == 2 && V == 4 ? 3 : 4) : (G == 2 && V == 4 ? 2 : 3);
+}
 // narrow: B < 4 GiB and cols < 2^24 (32-bit gather offsets).
 // mid: optional event recorded between the main kernel and the partial-sum kernel.
 // G: windows per unit in the step stream (1, or 2 when the plan paired windows).

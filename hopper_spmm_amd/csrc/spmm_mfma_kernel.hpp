@@ -839,6 +839,7 @@ void spmm_mfma_kernel(const KernelArgs ka)
                         if (lane == 0)
                             old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         old = __builtin_amdgcn_readfirstlane(old);
+                        asm volatile("" ::: "memory");      // the loads below stay behind the count they depend on
                         const uint32_t sb = fx[1], sc = fx[2];
                         if (old + 1u == sc) {
 #pragma unroll
@@ -989,23 +990,34 @@ void spmm_fixup_kernel(const KernelArgs ka)
 template <class TT, bool NARROW>
 static hipError_t launch_main_p(const KernelArgs &ka, int prefetch, dim3 grid, dim3 block, hipStream_t s)
 {
+    constexpr int kDefault = default_prefetch(TT::kElem, TT::G, TT::V);
     if (block.x > 64u * kMaxWavesPerGroup) {
-        // workgroups of kAlignedGroupWaves waves (aligned partition): built for the default depths only
-        switch (prefetch) {
-        case 2: spmm_mfma_kernel<TT, 2, NARROW, kAlignedGroupWaves><<<grid, block, 0, s>>>(ka); break;
-        case 3: spmm_mfma_kernel<TT, 3, NARROW, kAlignedGroupWaves><<<grid, block, 0, s>>>(ka); break;
-        case 4: spmm_mfma_kernel<TT, 4, NARROW, kAlignedGroupWaves><<<grid, block, 0, s>>>(ka); break;
-        default: return hipErrorInvalidValue;
+        // workgroups of kAlignedGroupWaves waves (aligned partition): 32-bit offsets, the default depth
+        if constexpr (NARROW) {
+            if (prefetch != kDefault) return hipErrorInvalidValue;
+            spmm_mfma_kernel<TT, kDefault, true, kAlignedGroupWaves><<<grid, block, 0, s>>>(ka);
+            return hipGetLastError();
         }
+        return hipErrorInvalidValue;
+    }
+#ifndef HSPMM_EXPERIMENTAL
+    if constexpr (!NARROW) {
+        // 64-bit gather offsets (a B of 4 GiB or more): the default depth
+        if (prefetch != kDefault) return hipErrorInvalidValue;
+        spmm_mfma_kernel<TT, kDefault, false><<<grid, block, 0, s>>>(ka);
         return hipGetLastError();
     }
+#endif
     switch (prefetch) {
-    case 1: spmm_mfma_kernel<TT, 1, NARROW><<<grid, block, 0, s>>>(ka); break;
     case 2: spmm_mfma_kernel<TT, 2, NARROW><<<grid, block, 0, s>>>(ka); break;
+    case 3: spmm_mfma_kernel<TT, 3, NARROW><<<grid, block, 0, s>>>(ka); break;
     case 4: spmm_mfma_kernel<TT, 4, NARROW><<<grid, block, 0, s>>>(ka); break;
+#ifdef HSPMM_EXPERIMENTAL
+    case 1: spmm_mfma_kernel<TT, 1, NARROW><<<grid, block, 0, s>>>(ka); break;
     case 6: spmm_mfma_kernel<TT, 6, NARROW><<<grid, block, 0, s>>>(ka); break;
     case 8: spmm_mfma_kernel<TT, 8, NARROW><<<grid, block, 0, s>>>(ka); break;
-    default: spmm_mfma_kernel<TT, 3, NARROW><<<grid, block, 0, s>>>(ka); break;
+#endif
+    default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }

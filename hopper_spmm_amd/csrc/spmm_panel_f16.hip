@@ -11,7 +11,11 @@ hipError_t launch_panel_f16_tall(int G, bool packed, const PanelArgs &pa, const 
 hipError_t launch_panel_f16(int G, bool tall, bool packed, const PanelArgs &pa, const KernelArgs &ka, int waves, hipStream_t s,
                            hipEvent_t mid)
 {
+#ifdef HSPMM_EXPERIMENTAL
     if (tall) return launch_panel_f16_tall(G, packed, pa, ka, s, mid);
+#else
+    if (tall || packed) return hipErrorInvalidValue;
+#endif
     if (G == 4) return launch_panel_nw<PanelTile<4>>(pa, ka, waves, s, mid);
     return G == 2 ? launch_panel_nw<PanelTile<2>>(pa, ka, waves, s, mid)
                   : launch_panel_nw<PanelTile<1>>(pa, ka, waves, s, mid);

@@ -29,19 +29,7 @@
 #include <type_traits>
 #include "spmm_mfma_kernel.hpp"
 
-// Measurement builds (make measure): HSPMM_MEASURE_SKIP is a mask of work that the kernels built on the
-// 16-bit MFMA leave out, to see what the rest of a launch costs.  The results of such a build are wrong.
-//   1: the consumers' MFMAs            2: the consumers' LDS reads
-//   4: the producers' copy to LDS      8: the producers' loads of B
-//  16: the consumers' loads of tiles and ids behind the first ring
-//  32: the producers' split of fp32 rows of B into bf16 parts (the words are copied as they are)
-#ifndef HSPMM_MEASURE_SKIP
-#define HSPMM_MEASURE_SKIP 0
-#endif
-
 namespace hspmm {
-
-constexpr int kMeasureSkip = HSPMM_MEASURE_SKIP;
 
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
 
@@ -291,10 +279,6 @@ struct PanelOps<Fp16Tr<G_, BF>> {
         Half<H> B;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            if constexpr (kMeasureSkip & 2) {
-                B.b[p] = u32x4{I, uint32_t(p), I, 0u};
-                continue;
-            }
             const tr16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a0 + 32 * (4 * H + p)));
             const tr16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(a1 + 32 * (4 * H + p)));
             const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
@@ -308,10 +292,6 @@ struct PanelOps<Fp16Tr<G_, BF>> {
     {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            if constexpr (kMeasureSkip & 1) {
-                asm volatile("" :: "v"(B.b[p]), "v"(A.r[0]));
-                continue;
-            }
             acc[4 * H + p] = HalfOps<BF>::mfma(A.r[0], B.b[p], acc[4 * H + p]);
             if constexpr (kFour) acc[8 + 4 * H + p] = HalfOps<BF>::mfma(A.r[1], B.b[p], acc[8 + 4 * H + p]);
         }
@@ -409,12 +389,6 @@ struct PanelOps<Fp32Split<G_>> {
     __device__ static __forceinline__ void write_piece(char *row, uint32_t c, const u32x4 x)
     {
         u32x2 hi, lo;
-        if constexpr (kMeasureSkip & 32) {
-            hi[0] = x[0]; hi[1] = x[1]; lo[0] = x[2]; lo[1] = x[3];
-            *reinterpret_cast<u32x2 *>(row + c * 8u) = hi;
-            *reinterpret_cast<u32x2 *>(row + 128u + c * 8u) = lo;
-            return;
-        }
         hi[0] = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);       // the upper halves
         hi[1] = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
         lo[0] = pack_bf16_rn(split_rest(x[0]), split_rest(x[1]));
@@ -482,10 +456,6 @@ struct PanelOps<Fp32Split<G_>> {
         Half<H> B;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            if constexpr (kMeasureSkip & 2) {
-                B.hi[p] = u32x4{I, uint32_t(p), I, 0u}; B.lo[p] = u32x4{I, 1u, I, uint32_t(p)};
-                continue;
-            }
             B.hi[p] = operand(a0, a1, 32 * (2 * H + p));
             B.lo[p] = operand(a0, a1, 128 + 32 * (2 * H + p));
         }
@@ -505,10 +475,6 @@ struct PanelOps<Fp32Split<G_>> {
         for (int p = 0; p < 2; ++p) {
 #pragma unroll
             for (int h = 0; h < kRowSets; ++h) {
-                if constexpr (kMeasureSkip & 1) {
-                    asm volatile("" :: "v"(B.hi[p]), "v"(B.lo[p]), "v"(a_hi[h]), "v"(a_lo[h]));
-                    continue;
-                }
                 // small terms first; a_lo * b_lo (below 2^-14 |a||b|, 2^-16 on average) is left out
                 const int q = 4 * h + 2 * H + p;
                 f32x4 c = HalfOps<true>::mfma(a_lo[h], B.hi[p], acc[q]);
@@ -682,8 +648,7 @@ void spmm_panel_kernel(const PanelArgs pa)
         // measured no faster.)
         u32x4 X[kPieces];
         auto copy_piece = [&](char *row, const u32x4 &x) __attribute__((always_inline)) {
-            if constexpr (kMeasureSkip & 4) asm volatile("" :: "v"(x));
-            else Ops::write_piece(row, pt & 15u, x);
+            Ops::write_piece(row, pt & 15u, x);
         };
         {
             const char *panel = panel_base(p_begin);
@@ -702,7 +667,7 @@ void spmm_panel_kernel(const PanelArgs pa)
 #pragma unroll
                 for (int i = 0; i < kPieces; ++i) {
                     copy_piece(img + uint32_t(i) * (NPW * 4) * kPitch, X[i]);
-                    if constexpr (!(kMeasureSkip & 8)) X[i] = load_piece(panel, last_off, i);
+                    X[i] = load_piece(panel, last_off, i);
                     __builtin_amdgcn_sched_barrier(0);              // in the order the loads return
                 }
             } else {
@@ -783,14 +748,10 @@ void spmm_panel_kernel(const PanelArgs pa)
 #define HSPMM_HEADER(k) ((k##u & 1u) ? H1 : H0)
 #define HSPMM_OTHER_HEADER(k) ((k##u & 1u) ? H0 : H1)
     // (two sets of accumulators leave registers for fewer steps in flight; packed tiles: see Ops::kPackedRing)
-#ifdef HSPMM_PANEL_RING
-    constexpr uint32_t kRing = HSPMM_PANEL_RING;                    // (measurement builds)
-#else
     constexpr uint32_t kRing = [] {
         if constexpr (PACKED) return Ops::kPackedRing;
         else return Ops::kRing;
     }();
-#endif
     static_assert(kRing >= 1 && kRing <= 6, "ring slots are named variables");
     static_assert(!PACKED || kRing % 2u == 0u, "the two headers alternate with the ring slots");
     // (PACKED: the header of a step is requested one slot ahead of the loads that need it)
@@ -861,7 +822,7 @@ void spmm_panel_kernel(const PanelArgs pa)
 #define HSPMM_PANEL_STEADY(k, kn) if constexpr (kRing > k) { \
         step(I##k, A##k, HSPMM_NEXT_IDX(k, kn), Ops::jump(HSPMM_NEXT_IDX(k, kn))); \
         request(HSPMM_OTHER_HEADER(k), t + k##u + kRing + 1u); \
-        if constexpr (!(kMeasureSkip & 16)) { I##k = ring_idx(t + k##u + kRing); A##k = ring_a(HSPMM_HEADER(k), t + k##u + kRing); } }
+        I##k = ring_idx(t + k##u + kRing); A##k = ring_a(HSPMM_HEADER(k), t + k##u + kRing); }
         HSPMM_RING2(HSPMM_PANEL_STEADY)
 #undef HSPMM_PANEL_STEADY
     }
@@ -915,6 +876,7 @@ void spmm_panel_kernel(const PanelArgs pa)
             uint32_t old = 0;
             if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             old = __builtin_amdgcn_readfirstlane(old);
+            asm volatile("" ::: "memory");                  // the loads below stay behind the count they depend on
             if (old + 1u == pa.n_chunks) {
 #pragma unroll
                 for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -970,12 +932,19 @@ static hipError_t launch_panel_nw(const PanelArgs &pa, const KernelArgs &ka, int
     // panels of 256 rows need four producer waves to hold one in registers
     if constexpr (PanelOps<TT>::kRows > 128u) return launch_panel_tt<TT, PanelOps<TT>::kConsumers, 4>(pa, ka, s, mid);
     else {
+#ifdef HSPMM_EXPERIMENTAL
         if (units == 14) return launch_panel_tt<TT, 14, 2>(pa, ka, s, mid);
         if (units == 13) return launch_panel_tt<TT, 12, 4>(pa, ka, s, mid);      // 12 units, four producer waves
         return launch_panel_tt<TT, 12, 2>(pa, ka, s, mid);
+#else
+        // the shapes the plans choose: 12 + 4 waves for the 4x4x1 instruction, 14 + 2 for pairs of windows
+        if constexpr (std::is_same<TT, Fp32Quad>::value) return units == 13 ? launch_panel_tt<TT, 12, 4>(pa, ka, s, mid) : hipErrorInvalidValue;
+        else return units == 14 ? launch_panel_tt<TT, 14, 2>(pa, ka, s, mid) : hipErrorInvalidValue;
+#endif
     }
 }
 
+#ifdef HSPMM_EXPERIMENTAL
 // Waves with two units each (kernels built on the 16-bit MFMA, units of one or two windows); packed: the
 // stream holds the tiles without their zeros.
 template <class TT>
@@ -988,5 +957,6 @@ static hipError_t launch_panel_tall(const PanelArgs &pa, const KernelArgs &ka, b
     return packed ? launch_panel_tt<TT, kTallConsumers, 4, true, true>(pa, ka, s, mid)
                   : launch_panel_tt<TT, kTallConsumers, 4, true, false>(pa, ka, s, mid);
 }
+#endif  // HSPMM_EXPERIMENTAL
 
 }  // namespace hspmm

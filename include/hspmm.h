@@ -99,7 +99,8 @@ int hspmm_run(hspmm_plan *plan, const void *dB, void *dC, uint32_t N, void *stre
  * src/fp16.cu:236-249): builds now what the first hspmm_run with feature
  * dimension N would build - the work partition for that width and, for every
  * stream that has launched the plan so far (for the set that the first stream
- * and streams under capture use, if none has), the buffers a launch writes
+ * and streams under capture use, if none has; the first stream that launches
+ * the plan afterwards takes that set over), the buffers a launch writes
  * besides C, for every alignment of B and C - and launches nothing. */
 int hspmm_prepare(hspmm_plan *plan, uint32_t N);
 
@@ -152,7 +153,9 @@ const char *hspmm_last_error(void);
 
 /* Replaces Scheduler::configure (reference src/scheduler.h:33-38).  Values are
  * read by the next hspmm_create on any thread; 0 keeps the built-in default.
- *   buffer_stage             tiles each wave keeps in flight (prefetch depth): 1, 2, 3, 4, 6 or 8
+ *   buffer_stage             tiles each wave keeps in flight (prefetch depth): 2, 3 or 4 (builds with
+ *                            EXPERIMENTAL=1 also 1, 6 and 8); launches with 64-bit gather offsets (a B of
+ *                            4 GiB or more) and workgroups of eight waves use the default depth
  *   consumer_warp_num        waves per workgroup, 1..4
  *   producer_warp_group_num  tile ranges (waves) per SIMD the partition aims at, 1..16
  *   sm_num                   compute units to balance over (default: the device's) */
@@ -161,6 +164,13 @@ int hspmm_configure(int buffer_stage, int consumer_warp_num,
 /* Getter side of the same singleton (reference src/scheduler.h:26-30, 41). */
 void hspmm_get_config(int *buffer_stage, int *consumer_warp_num,
                       int *producer_warp_group_num, int *sm_num);
+
+/* No reference counterpart.  1 when the library was built with EXPERIMENTAL=1 (csrc/Makefile): it then also
+ * holds the kernel variants that no automatic plan selects - prefetch depths 1, 6 and 8, the stream modes 1 and 2
+ * of hspmm_set_panel_stream, units of four windows for fp32 storage in bf16 parts, the other workgroup shapes of
+ * the fp32-MFMA LDS-staging kernels - which were measured against the defaults and lost.  0: those requests fail
+ * with HSPMM_ERR_INVALID / HSPMM_ERR_UNSUPPORTED. */
+int hspmm_has_experimental(void);
 
 /* Kernel selection, read by the next hspmm_create: 0 = automatic (MFMA kernels
  * whenever the feature dimension allows; the kernels that stage B through LDS
@@ -198,7 +208,8 @@ int hspmm_set_window_pairing(int mode);
  * bit-identical in all three modes.  Both cut the bytes a launch moves (measured: a
  * third and 60 % fewer 128-byte lines into the compute units) and neither makes it
  * faster on the configurations measured: these kernels are bound by the LDS reads and
- * MFMAs of a step, not by their traffic; hence the default. */
+ * MFMAs of a step, not by their traffic; hence the default.  Modes 1 and 2 exist in builds with
+ * EXPERIMENTAL=1 only (hspmm_has_experimental); elsewhere they return HSPMM_ERR_UNSUPPORTED. */
 int hspmm_set_panel_stream(int mode);
 
 /* No reference counterpart (the reference defines the grouped format, src/utils/class.h:93-108
@@ -274,8 +285,9 @@ int hspmm_get_partition(const hspmm_plan *plan, uint32_t *ranges, uint32_t capac
  * length instead): one group per piece of a window that one wave walks, groupOffset[g] its first tile in the
  * caller's tile arrays (groupOffset[total] = total_tiles), groupRowIdx[g] the window's first row, atomic[g] = 1
  * where the window continues in another group.  Together with the tile arrays the plan was made from this is a
- * GBTCF_MTX that hspmm_create_grouped takes back.  First call with the arrays NULL for *total_groups.  Plans
- * that walk pairs of windows have no such form (HSPMM_ERR_UNSUPPORTED).  Host only. */
+ * GBTCF_MTX that hspmm_create_grouped takes back.  First call with the arrays NULL for *total_groups.  A plan
+ * that walks pairs of windows (equal column lists merged: its steps are not the caller's tiles) writes the balanced
+ * partition of the caller's single windows instead, built with the same cost model.  Host only. */
 int hspmm_partition_as_groups(const hspmm_plan *plan, uint32_t capacity_groups, uint32_t *total_groups,
                               uint32_t *groupOffset, uint32_t *groupRowIdx, uint8_t *atomic);
 

@@ -62,3 +62,27 @@ def test_cli_end_to_end_with_verification(hs, tmp_path):
         assert "verification passed" in r.stdout
         assert "SpMM timed runs: 5" in r.stdout                      # RUNS, src/common.h:49
         assert "stored entries: %d" % nnz in r.stdout
+
+
+@pytest.mark.gpu
+def test_cli_balanced_groups_of_a_block_clustered_matrix(hs, tmp_path):
+    """--format balanced on a matrix whose adjacent windows share their column lists (16 x 16 blocks): the plan
+    behind BTCF2GBTCF_balanced pairs those windows, and still hands out groups of the caller's tiles."""
+    rng = np.random.default_rng(9)
+    rows, cols = 256, 640
+    p = tmp_path / "blocks.mtx"
+    entries = []
+    for bi in range(0, rows, 16):
+        for bj in range(0, cols, 16):
+            if rng.random() < 0.5:
+                for r in range(16):
+                    for c in range(16):
+                        entries.append((bi + r + 1, bj + c + 1, rng.normal()))
+    with open(p, "w") as f:
+        f.write("%%MatrixMarket matrix coordinate real general\n%d %d %d\n" % (rows, cols, len(entries)))
+        for r, c, v in entries:
+            f.write("%d %d %.6g\n" % (r, c, v))
+    for name in ("fp16_test", "tf32_test"):
+        r = run(hs, name, str(p), "64", "--seed", "7", "--verify", "--format", "balanced")
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert "verification passed" in r.stdout and "total groups" in r.stdout

@@ -14,7 +14,7 @@ import os
 import numpy as np
 import pytest
 
-from util import csr_to_dense64, decode, encode, half_ulp_distance, random_csr
+from util import built_depth, csr_to_dense64, decode, encode, half_ulp_distance, random_csr
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -214,8 +214,10 @@ def test_random_shapes_and_feature_dims(torch_cuda, hs, oracle, dtype, shape):
 
 @pytest.mark.parametrize("dtype", [0, 1, 2])
 @pytest.mark.parametrize("mode", [1, 2, 3])
-@pytest.mark.parametrize("stages", [1, 2, 4, 6, 8])
+@pytest.mark.parametrize("stages", [1, 2, 3, 4, 6, 8])
 def test_kernel_variants_agree_with_oracle(torch_cuda, hs, oracle, dtype, mode, stages):
+    if stages not in (2, 3, 4) and not hs.has_experimental():
+        pytest.skip("prefetch depth %d exists in libraries built with EXPERIMENTAL=1 only" % stages)
     rng = np.random.default_rng(77)
     A = random_csr(rng, 260, 2000, 0.01, dtype, 0.2, (17, 130))
     b = convert(hs, A)
@@ -271,7 +273,7 @@ def test_windows_with_one_column_list_share_their_gather(torch_cuda, hs, oracle,
     else:
         A = _block_matrix(rng, 203, 500, 16, 8, 0.6, dtype)          # rows % 16 != 0: last pair is ragged
     b = convert(hs, A)
-    for pairing, stages in ((0, 0), (2, 0), (2, 1), (2, 4), (1, 0)):
+    for pairing, stages in ((0, 0), (2, 0), (2, 1 if hs.has_experimental() else 3), (2, 4), (1, 0)):
         hs.set_window_pairing(pairing)
         hs.configure(buffer_stage=stages, producer_warp_group_num=16)
         try:
@@ -424,13 +426,31 @@ def test_partition_exported_as_groups_round_trips(torch_cuda, hs, oracle):
         B = make_b(rng, 3000, N, 0)
         want = gpu_spmm(torch_cuda, hs, plain, B, N)
         assert np.array_equal(gpu_spmm(torch_cuda, hs, grouped, B, N), want)
-    # plans that walk pairs of windows have no such form
-    P = random_csr(rng, 64, 64, 1.0, 0)                                                 # every window has the same columns
-    pairs = hs.Plan(convert(hs, P))
-    if pairs.info()["n_paired_units"]:
-        with pytest.raises(hs.HspmmError):
-            pairs.partition_as_groups()
+    # A plan that walks pairs of windows (equal column lists merged) exports the balanced partition of the caller's
+    # single windows: groups of the caller's tiles again, which hspmm_create_grouped takes back.
+    P = _block_matrix(rng, 256, 1200, 16, 16, 0.5, 0)                                   # block-clustered: windows pair up
+    pplain = convert(hs, P)
+    pbitmap = hs.csr_to_bitmap(256, 1200, P["row_ptr"], P["col_idx"], P["values"], 0)
+    hs.configure(producer_warp_group_num=16)
+    try:
+        pairs = hs.Plan(pplain)
+    finally:
+        hs.configure()
+    assert pairs.info()["n_paired_units"] > 0
+    g = pairs.partition_as_groups()
     pairs.close()
+    go = g["groupOffset"].astype(np.int64)
+    assert go[0] == 0 and go[-1] == pplain["total_tiles"] and (np.diff(go) > 0).all()
+    assert set(pplain["rowOffset"].tolist()) <= set(go.tolist())
+    window_of_group = np.searchsorted(pplain["rowOffset"], go[:-1], side="right") - 1
+    assert np.array_equal(g["rowIdx"], pplain["rowIdx"][window_of_group])
+    groups_per_window = np.bincount(window_of_group, minlength=pplain["eff_row_windows"])
+    assert np.array_equal(g["atomic"].astype(bool), groups_per_window[window_of_group] > 1)
+    pgrouped = {k: pbitmap[k] for k in ("rows", "cols", "nnzs", "dtype", "cw", "nnzOffset", "tcA2B", "tcBit", "data")}
+    pgrouped.update(g, tgl=0, total_row_windows=g["total_groups"] + 1, eff_row_windows=g["total_groups"] + 1)
+    B = make_b(rng, 1200, 64, 0)
+    ref, mag = oracle_spmm(oracle, P, B, 64)
+    assert_parity(gpu_spmm(torch_cuda, hs, pgrouped, B, 64), ref, mag, 0, "groups of a plan that pairs windows")
 
 
 @pytest.mark.parametrize("dtype", [0, 1, 2])
@@ -519,12 +539,13 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
     A = random_csr(rng, rows, cols, dens, dtype, erp, heavy)
     b = convert(hs, A)
     block = 64 if dtype == 1 else 128
-    cases = [(4, u, c) for u, c in (("", ""), ("12", ""), ("14", ""), ("13", "2"), ("12", "1"), ("14", "3"), ("12", "1000"))]
+    # units: consumer waves of a workgroup that get a unit (HSPMM_PANEL_UNITS_PER_GROUP; the kernels have 8, 12 or 14)
+    cases = [(4, u, c) for u, c in (("", ""), ("12", ""), ("5", ""), ("7", "2"), ("1", "1"), ("14", "3"), ("3", "1000"))]
     if dtype == 1:                              # fp32 products: the 4x4x1 / 16x16x4 MFMA forms
-        cases += [(5, "", ""), (5, "12", "2"), (5, "13", "3"), (5, "14", "1")]
+        cases += [(5, "", ""), (5, "12", "2"), (5, "6", "3"), (5, "14", "1")]
     for mode, units, chunks in cases:
         if units:
-            os.environ["HSPMM_PANEL_UNITS"] = units
+            os.environ["HSPMM_PANEL_UNITS_PER_GROUP"] = units
         if chunks:
             os.environ["HSPMM_PANEL_CHUNKS"] = chunks
         hs.set_kernel_mode(mode)
@@ -559,7 +580,7 @@ def test_lds_panel_kernels_on_every_shape(torch_cuda, hs, oracle, dtype, shape):
             plan.close()
         finally:
             hs.set_kernel_mode(0)
-            os.environ.pop("HSPMM_PANEL_UNITS", None)
+            os.environ.pop("HSPMM_PANEL_UNITS_PER_GROUP", None)
             os.environ.pop("HSPMM_PANEL_CHUNKS", None)
 
 
@@ -795,8 +816,10 @@ def test_adjacent_windows_with_overlapping_columns_share_units(torch_cuda, hs, o
             if grouped:
                 assert info["n_panels"] > 0
                 assert (info["n_panel_paired_units"] > 0) == (pairing != 1), (mode, pairing, info)
-                assert (info["n_panel_wide_units"] > 0) == (pairing == 2), (mode, pairing, info)
-                if pairing == 2:        # 8, 7 and 8 windows between the gaps: two fours, a four and a three, two fours
+                # (fp32 storage in bf16 parts has units of three and four windows in builds with EXPERIMENTAL=1 only)
+                wide = pairing == 2 and (dtype != 1 or hs.has_experimental())
+                assert (info["n_panel_wide_units"] > 0) == wide, (mode, pairing, info)
+                if wide:                # 8, 7 and 8 windows between the gaps: two fours, a four and a three, two fours
                     assert info["n_panel_units"] == 6 and info["n_panel_wide_units"] == 6, info
             for chunks in (None, "2") if grouped else (None,):
                 if chunks:
@@ -858,7 +881,7 @@ def test_seeded_sweep_of_shapes_formats_and_kernel_choices(torch_cuda, hs, oracl
         mode = int(rng.choice([0, 0, 2, 3, 4, 4, 5]))
         pairing = int(rng.integers(0, 3))
         fmt = int(rng.integers(0, 3))
-        stages = int(rng.choice([0, 0, 1, 2, 4]))
+        stages = built_depth(hs, int(rng.choice([0, 0, 1, 2, 4])))
         ranges_per_simd = int(rng.choice([0, 0, 1, 16]))
         if mode >= 4 and large:
             N = int(rng.choice([64, 128, 320, 512])) if dtype == 1 else int(rng.choice([128, 256, 640, 1024]))
@@ -911,9 +934,11 @@ def test_seeded_sweep_of_stream_modes_group_cuts_and_tuning_overrides(torch_cuda
         mode = int(rng.choice([0, 0, 0, 2, 3, 4, 4, 5]))
         pairing = int(rng.integers(0, 3))
         fmt = int(rng.integers(0, 5))          # plain, bitmap, grouped, grouped with its cuts kept, column by column
-        stages = int(rng.choice([0, 0, 0, 1, 2, 4]))
+        stages = built_depth(hs, int(rng.choice([0, 0, 0, 1, 2, 4])))
         ranges_per_simd = int(rng.choice([0, 0, 1, 16]))
         stream = int(rng.choice([0, 0, 1, 2]))
+        if not hs.has_experimental():
+            stream = 0                         # (stream modes 1 and 2 are built with EXPERIMENTAL=1 only)
         env = {}
         for name, chance, values in zip(knobs, (0.3, 0.3, 0.3, 0.2, 0.2), ([0, 1], [0, 1], [0, 1], [0, 4, 8], [2, 4])):
             if rng.random() < chance:
@@ -1600,6 +1625,11 @@ def test_panel_stream_with_two_units_per_wave_and_packed_tiles(torch_cuda, hs, o
     2 = also the tiles of the steps without their zeros (masks + stored values, expanded in
     registers).  The MFMA inputs are the same in all three modes, so with the same split into
     chunks of panels the results are bit-identical; and exact-integer inputs are exact."""
+    if not hs.has_experimental():
+        with pytest.raises(hs.HspmmError) as e:            # refused with a message, not ignored
+            hs.set_panel_stream(1)
+        assert e.value.code == 5 and "EXPERIMENTAL" in str(e.value)
+        pytest.skip("stream modes 1 and 2 of the LDS-staging kernels exist in libraries built with EXPERIMENTAL=1 only")
     rng = np.random.default_rng(70 + dtype)
     feature_dims = (64, 128) if dtype == 1 else (128, 384)
     cases = [

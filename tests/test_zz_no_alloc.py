@@ -62,12 +62,17 @@ def test_static_scratch_entry_point_matches_hspmm_run(torch_cuda, hs, oracle, dt
                 plan.run_static(dB.data_ptr(), dC.data_ptr(), N, stream)
             assert "hspmm_prepare" in str(e.value)
         plan.prepare(N)
-        before = torch.cuda.memory_allocated(), plan.info()["device_bytes"]
         _poison(dC, dtype)
+        torch.cuda.synchronize()
+        # the device allocator itself: free memory of the device before and after the call (the plan's own
+        # accounting, which also counts arrival counters and superseded buffers, must agree)
+        before = torch.cuda.mem_get_info()[0], plan.info()["device_bytes"]
         plan.run_static(dB.data_ptr(), dC.data_ptr(), N, stream)
         torch.cuda.synchronize()
+        after = torch.cuda.mem_get_info()[0], plan.info()["device_bytes"]
         got = _result(dC, dtype)
-        assert plan.info()["device_bytes"] == before[1], name + ": the plan's device memory changed"
+        assert after[1] == before[1], name + ": the plan's device memory changed"
+        assert after[0] >= before[0], name + ": %d bytes of device memory were allocated by the call" % (before[0] - after[0])
         # the existing entry point, same plan, same inputs
         _poison(dC, dtype)
         plan.run(dB.data_ptr(), dC.data_ptr(), N, stream)
@@ -148,4 +153,67 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(torch_cuda, hs):
     plan.run(dB.data_ptr(), dC.data_ptr(), N, torch.cuda.current_stream().cuda_stream)   # the allocating entry point serves it
     torch.cuda.synchronize()
     assert not dC.any().item()
+    plan.close()
+
+
+def test_prepare_covers_rows_that_start_on_odd_halves(torch_cuda, hs, oracle):
+    """hspmm_prepare builds for every alignment of B and C, also a 16-bit B or C that starts on an odd half: that
+    launch takes one-word loads in blocks of 32 features, i.e. several feature blocks, another partition and another
+    amount of partial sums than the aligned launches.  hspmm_run_static, which builds nothing, must then run it."""
+    torch = torch_cuda
+    stream = torch.cuda.current_stream().cuda_stream
+    rng = np.random.default_rng(79)
+    A = random_csr(rng, 64, 6000, 0.3, 0, 0.0, (3, 40))            # every unit far longer than a range
+    b = convert(hs, A)
+    hs.set_kernel_mode(3)                                           # (gather kernels, whatever the density)
+    try:
+        plan = hs.Plan(b)
+    finally:
+        hs.set_kernel_mode(0)
+    N = 256
+    B = make_b(rng, A["cols"], N, 0)
+    flatB = torch.zeros(A["cols"] * N + 1, dtype=torch.int16, device="cuda")
+    flatC = torch.zeros(A["rows"] * N + 1, dtype=torch.int16, device="cuda")
+    flatB[1:] = torch.from_numpy(np.ascontiguousarray(B, np.uint16).view(np.int16).ravel()).cuda()
+    pB, pC = flatB.data_ptr() + 2, flatC.data_ptr() + 2             # one half into their allocations
+    plan.prepare(N)
+    torch.cuda.synchronize()
+    before = torch.cuda.mem_get_info()[0], plan.info()["device_bytes"]
+    plan.run_static(pB, pC, N, stream)
+    torch.cuda.synchronize()
+    assert plan.info()["device_bytes"] == before[1] and torch.cuda.mem_get_info()[0] >= before[0]
+    got = flatC[1:].cpu().numpy().view(np.uint16).reshape(A["rows"], N)
+    ref, mag = oracle_spmm(oracle, A, B, N)
+    assert_parity(got, ref, mag, 0, "B and C on odd halves")
+    assert int(flatC[0].item()) == 0                                # nothing in front of C was written
+    plan.close()
+
+
+def test_first_launch_after_prepare_takes_the_prepared_buffers(torch_cuda, hs, oracle):
+    """hspmm_prepare on a plan that has not launched yet makes one set of buffers; the first stream that launches
+    the plan - here a stream of its own, not the default one - takes that set instead of allocating another."""
+    torch = torch_cuda
+    rng = np.random.default_rng(80)
+    A = random_csr(rng, 300, 3000, 0.004, 0, 0.2, (5, 100, 299))
+    b = convert(hs, A)
+    hs.configure(producer_warp_group_num=16)                        # (cut windows: partial sums and counters)
+    try:
+        plan = hs.Plan(b)
+    finally:
+        hs.configure()
+    N = 128
+    B = make_b(rng, A["cols"], N, 0)
+    dB, dC = _device_buffers(torch, B, A["rows"], N, 0)
+    plan.prepare(N)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        dC.zero_()                      # (the runtime's own memory for a new stream's first launch exists after this)
+    torch.cuda.synchronize()
+    before = torch.cuda.mem_get_info()[0], plan.info()["device_bytes"]
+    plan.run(dB.data_ptr(), dC.data_ptr(), N, side.cuda_stream)
+    side.synchronize()
+    assert plan.info()["device_bytes"] == before[1], "the first launch allocated buffers of its own"
+    assert torch.cuda.mem_get_info()[0] >= before[0]
+    ref, mag = oracle_spmm(oracle, A, B, N)
+    assert_parity(_result(dC, 0), ref, mag, 0, "first launch after prepare")
     plan.close()

@@ -98,3 +98,9 @@ def half_ulp_distance(a_bits, b_bits):
         x = x.astype(np.int32)
         return np.where(x & 0x8000, -(x & 0x7FFF), x & 0x7FFF)
     return np.abs(key(a_bits) - key(b_bits))
+
+
+def built_depth(hs, stages):
+    """The prefetch depth a test asks for, or the default-build depth 3 in its place when the library holds
+    depths 2, 3 and 4 only (1, 6 and 8 are built with EXPERIMENTAL=1)."""
+    return stages if stages in (0, 2, 3, 4) or hs.has_experimental() else 3
