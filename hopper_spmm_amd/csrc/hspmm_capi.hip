@@ -531,8 +531,13 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
                     uint8_t *dt_tile = rt_data.data() + at * tile_bytes;
                     for (uint32_t k = 0; k < rw; ++k) {
                         const uint32_t from = order[k];
-                        // padding takes the row of the step's last real column (its tile column stays zero)
-                        const uint32_t srci = source(std::min(from, n - 1));
+                        // Padding (its tile column stays zero) takes the row of a real column that is read together
+                        // with it - entries four apart are in one set - so that it asks for no bank of its own: lanes
+                        // that read one address are served together.
+                        uint32_t real = from;
+                        while (real >= n && real >= 4u) real -= 4u;
+                        if (real >= n) real = n - 1;
+                        const uint32_t srci = source(real);
                         rt_ids[at * rw + k] = col[srci] - pn * KP;      // row inside the panel
                         if (from >= n) continue;
                         const uint8_t *st_tile = src_data + size_t(t0 + srci / cw) * src_tile_bytes;
