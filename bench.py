@@ -21,7 +21,95 @@ for p in (ROOT, os.path.join(ROOT, "oracle")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
-MFMA_PEAK_TFLOPS = {0: 2500.0, 1: 157.3}   # dense fp16 / fp32 matrix
+# dense peak of the matrix instruction a kernel issues (hspmm_plan_info.last_mfma_kind)
+MFMA = {1: ("v_mfma_f32_16x16x32_f16", 2500.0), 2: ("v_mfma_f32_16x16x32_bf16", 2500.0),
+        3: ("v_mfma_f32_16x16x4_f32", 157.3), 4: ("v_mfma_f32_4x4x1_16B_f32", 157.3)}
+# which roofline binds each configuration by its compulsory bytes and padded flops: the pruned fp32 weight and the
+# block-clustered weight at N = 512 are bound by the matrix cores, the rest by HBM
+BOUND = {(3, 256): "mfma", (4, 512): "mfma"}
+KERNELS = {1: "spmm_scalar_kernel", 2: "spmm_mfma_kernel", 3: "spmm_panel_kernel"}
+
+
+def mfma_report(info, useful_flops, kernel_ms):
+    """Matrix-core use of the last launch: flops issued (zero padding of tiles and rows included) and useful
+    (2 * nnz * N), both against the dense peak of the instruction the kernel issues."""
+    kind = info["last_mfma_kind"]
+    if kind not in MFMA or kernel_ms <= 0:
+        return None
+    name, peak = MFMA[kind]
+    issued = float(info["last_mfma_instructions"]) * info["last_mfma_flops"]
+    t = kernel_ms * 1e-3
+    return {"instruction": name, "peak_tflops": peak, "instructions_per_launch": int(info["last_mfma_instructions"]),
+            "issued_tflops": issued / t / 1e12, "issued_frac": issued / t / 1e12 / peak,
+            "useful_tflops": useful_flops / t / 1e12, "useful_frac": useful_flops / t / 1e12 / peak}
+
+
+def device_buffers(torch, np, hs, A, B, N):
+    if A["dtype"] == hs.FP16:
+        return (torch.from_numpy(B.view(np.int16)).cuda(),
+                torch.empty((A["rows"], N), dtype=torch.int16, device="cuda"))
+    return torch.from_numpy(B).cuda(), torch.empty((A["rows"], N), dtype=torch.float32, device="cuda")
+
+
+def measure_config(torch, np, hs, G, index, N, steps, warmup, mode=0, matrix=None):
+    """One configuration through hspmm_run, timed with device events on the launch stream (the reference's
+    convention, src/common.h:48-58: warm-up launches, then timed launches back to back)."""
+    cfg = matrix or G.make_config(index, 1)
+    A = cfg["A"]
+    b = cfg.get("btcf") or hs.csr_to_btcf(A["rows"], A["cols"], A["row_ptr"], A["col_idx"], A["values"], A["dtype"])
+    cfg["btcf"] = b
+    B = G.dense_b(A["cols"], N, cfg["b_seed"], A["dtype"])
+    hs.set_kernel_mode(mode)
+    try:
+        plan = hs.Plan(b)
+    finally:
+        hs.set_kernel_mode(0)
+    dB, dC = device_buffers(torch, np, hs, A, B, N)
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(warmup):
+        plan.run(dB.data_ptr(), dC.data_ptr(), N, stream)
+    main_ms, fix_ms = plan.profile(dB.data_ptr(), dC.data_ptr(), N, runs=steps, stream=stream)
+    main_ms /= steps
+    fix_ms /= steps
+    info = plan.info()
+    flops = 2.0 * int(A["nnzs"]) * N
+    bytes_alg = G.algorithmic_bytes(b, N)
+    t = (main_ms + fix_ms) * 1e-3
+    out = {"workload": "configs[%d]: %s, N=%d" % (index, cfg["name"], N),
+           "dtype": "f16 in, f32 accumulate" if A["dtype"] == hs.FP16 else "f32 (tf32 variant)",
+           "kernel": KERNELS.get(info["last_kernel_family"], "none"),
+           "kernel_ms": main_ms, "fixup_kernel_ms": fix_ms,
+           "tflops": flops / t / 1e12, "algorithmic_bytes": bytes_alg,
+           "bound": BOUND.get((index, N), "hbm"),
+           "hbm_gbps": bytes_alg / t / 1e9, "hbm_frac": bytes_alg / t / 1e9 / HBM_PEAK_GBPS,
+           "mfma": mfma_report(info, flops, main_ms)}
+    out["frac"] = out["mfma"]["useful_frac"] if out["bound"] == "mfma" and out["mfma"] else out["hbm_frac"]
+    if info["last_kernel_family"] == 2 and (N * (2 if A["dtype"] != 1 else 4)) % 128 == 0:
+        g_ms, _ = plan.measure_gather(dB.data_ptr(), N, runs=5, stream=stream)
+        out["gather_only_ms"] = g_ms
+    plan.close()
+    del dB, dC
+    return out, cfg
+
+
+def all_configs(torch, np, hs, G, steps, warmup):
+    """The other benchmark configurations, one line each: the configuration the CPU check path is quoted on, the
+    uniform 65536^2 matrix, the pruned fp32 weight in both arithmetic forms of the tf32 variant (bf16 hi / lo
+    parts in three products, the default; fp32 MFMA products, kernel mode 5) and the block-clustered weight at
+    N = 16, 64 and 512."""
+    rows = []
+    for index, n_list in ((0, (64,)), (1, (128,)), (3, (256,)), (4, (16, 64, 512))):
+        cfg = None
+        for N in n_list:
+            r, cfg = measure_config(torch, np, hs, G, index, N, steps, warmup, matrix=cfg)
+            if index == 3:
+                r["arithmetic"] = "bf16 hi / lo parts of every fp32 factor, three products (a_lo * b_lo left out)"
+            rows.append(r)
+            if index == 3:
+                r5, cfg = measure_config(torch, np, hs, G, index, N, steps, warmup, mode=5, matrix=cfg)
+                r5["arithmetic"] = "fp32 MFMA products (hspmm_set_kernel_mode(5))"
+                rows.append(r5)
+    return rows
 
 
 def cpu_baseline(A, B, N, flops_full):
@@ -101,6 +189,8 @@ def main():
                     help="stream of the LDS-panel kernels (hspmm_set_panel_stream): 0 tiles, 1 two units per wave, 2 packed tiles")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain device copy of 1 GiB (reference point for traffic counters)")
+    ap.add_argument("--no-all-configs", action="store_true",
+                    help="leave out the lines for the other benchmark configurations (all_configs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this operator runs on a single MI355X and nothing here uses a "
@@ -232,17 +322,16 @@ def main():
                    "split_windows": info["n_split_windows"]},
         "effective_gbps": bytes_alg / (ms_per_step * 1e-3) / 1e9,
         # achieved: algorithmic bytes of one launch / (main kernel + partial-sum kernel), device events
-        "roofline": {"bound": "hbm", "achieved": bytes_alg / (kernels_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": BOUND.get((args.config, N), "hbm"), "achieved": bytes_alg / (kernels_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": bytes_alg / (kernels_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      # counter figures stored with the rocprofv3 summary they come from (not measured in this run)
                      "traffic": traffic,
-                     "kernel": {1: "spmm_scalar_kernel", 2: "spmm_mfma_kernel", 3: "spmm_panel_kernel"}.get(
-                         plan.info()["last_kernel_family"], "none"),
+                     "kernel": KERNELS.get(info["last_kernel_family"], "none"),
                      "kernel_ms": main_ms, "fixup_kernel_ms": fix_ms,
                      "algorithmic_bytes": bytes_alg, "gather_bytes": bytes_gather,
                      # every gathered B row counted every time it is gathered, for comparison with the HBM peak
                      "gathered_gbps": bytes_gather / (kernels_ms * 1e-3) / 1e9,
-                     "mfma_frac_of_peak_useful_flops": flops / (main_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[dt]},
+                     "mfma": mfma_report(info, flops, main_ms)},
         "reference_convention_ms": ref_conv_ms,
         # one call of the host-buffer interface (fp16_spmm): plan + upload, one launch, download of C
         "host_buffer_call": {"upload_and_plan_ms": t_h2d * 1e3, "download_ms": t_d2h * 1e3,
@@ -261,6 +350,9 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(A, B, N, flops)
     plan.close()
+    if args.config == 2 and not args.n and not args.no_all_configs and args.mode == 0:
+        del dB, dC
+        out["all_configs"] = all_configs(torch, np, hs, G, args.steps, args.warmup)
     print(json.dumps(out))
 
 

@@ -70,7 +70,8 @@ class PlanInfo(C.Structure):
                 ("n_panel_units", C.c_uint32), ("n_panel_paired_units", C.c_uint32),
                 ("n_panel_wide_units", C.c_uint32), ("last_kernel_family", C.c_uint32),
                 ("gather_bitmap", C.c_uint32), ("bitmap_from_caller", C.c_uint32), ("panel_stream_mode", C.c_uint32),
-                ("group_cuts_kept", C.c_uint32)]
+                ("group_cuts_kept", C.c_uint32), ("last_mfma_kind", C.c_uint32), ("last_mfma_flops", C.c_uint32),
+                ("last_mfma_instructions", C.c_uint64)]
 
 
 def load_library():

@@ -211,6 +211,15 @@ struct hspmm_plan {
     std::vector<void *> retired;
     size_t retired_bytes = 0;               // partial-sum buffers among them (counters are part of fixed_bytes)
     std::atomic<uint32_t> last_family{0};   // kernel family of the last hspmm_run: 0 none yet, 1 all-shapes, 2 gather, 3 LDS-panel, 4 clear
+    // matrix instructions of the last launch's main kernel: kind (hspmm_plan_info::last_mfma_kind) and count
+    std::atomic<uint32_t> last_mfma_kind{0};
+    std::atomic<uint64_t> last_mfma_count{0};
+    void note_launch(uint32_t family, uint32_t kind, uint64_t count)
+    {
+        last_family.store(family, std::memory_order_relaxed);
+        last_mfma_kind.store(kind, std::memory_order_relaxed);
+        last_mfma_count.store(count, std::memory_order_relaxed);
+    }
 };
 
 namespace {
@@ -1641,7 +1650,13 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         ka.uniform_chunks = pa.n_chunks;
     }
     if (mode == RunMode::kPrepare) return HSPMM_OK;
-    p->last_family.store(3, std::memory_order_relaxed);
+    {
+        // matrix instructions per step and feature block (PanelOps<...>::mma_half in spmm_panel_kernel.hpp)
+        const uint64_t wide_rows = pl.G == 4 ? 2u : 1u;
+        const uint32_t kind = pl.quad ? 4u : (p->dtype == HSPMM_TF32 && !pl.split) ? 3u : (p->dtype == HSPMM_FP16 ? 1u : 2u);
+        const uint64_t per_step = pl.quad ? 16u : pl.split ? 12u * wide_rows : p->dtype != HSPMM_TF32 ? 8u * wide_rows : 8u * uint64_t(pl.G);
+        p->note_launch(3, kind, uint64_t(pl.n_steps) * pa.n_feat_blocks * per_step);
+    }
     HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : pl.G, pl.split, pl.tall, pl.packed, pa, ka, units, s, mid));
     return HSPMM_OK;
 }
@@ -1671,7 +1686,7 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (p->W == 0) {
         if (!launch) return HSPMM_OK;
-        p->last_family.store(4, std::memory_order_relaxed);
+        p->note_launch(4, 0, 0);
         HSPMM_HIP(hspmm::launch_fill_zero(dC, size_t(p->rows) * N * p->elem, s));
         return HSPMM_OK;
     }
@@ -1766,7 +1781,7 @@ static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint3
     if (c.scalar) {
         if (ld != N) return fail(HSPMM_ERR_UNSUPPORTED, "the all-shapes kernel takes whole rows");
         if (!launch) return HSPMM_OK;
-        p->last_family.store(1, std::memory_order_relaxed);
+        p->note_launch(1, 0, 0);
         HSPMM_HIP(hspmm::launch_spmm_scalar(p->dtype, ka, s));
         return HSPMM_OK;
     }
@@ -1831,7 +1846,9 @@ static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint3
     }
     ka.ranges = dp.d_ranges; ka.split = dp.d_split; ka.fix_slots = dp.d_fix_slots;
     if (!launch) return HSPMM_OK;
-    p->last_family.store(2, std::memory_order_relaxed);
+    // (per step and feature block: G * V instructions of 16 x 16 x 32, or 2 G V of 16 x 16 x 4 for 32-bit elements)
+    p->note_launch(2, p->dtype == HSPMM_TF32 ? 3u : p->dtype == HSPMM_FP16 ? 1u : 2u,
+                   uint64_t(p->n_steps) * ka.n_feat_blocks * uint64_t(p->G) * uint64_t(c.V) * (p->dtype == HSPMM_TF32 ? 2u : 1u));
     const int default_depth = hspmm::default_prefetch(int(p->elem), p->G, c.V);
     int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage : default_depth;
 #ifndef HSPMM_EXPERIMENTAL
@@ -1973,6 +1990,10 @@ int hspmm_get_plan_info(const hspmm_plan *p, hspmm_plan_info *info)
     info->n_panel_paired_units = p->panel.built ? p->panel.n_paired : 0u;
     info->n_panel_wide_units = p->panel.built ? p->panel.n_wide : 0u;
     info->last_kernel_family = p->last_family.load(std::memory_order_relaxed);
+    info->last_mfma_kind = p->last_mfma_kind.load(std::memory_order_relaxed);
+    static const uint32_t kMfmaFlops[5] = {0u, 16384u, 16384u, 2048u, 512u};
+    info->last_mfma_flops = kMfmaFlops[info->last_mfma_kind];
+    info->last_mfma_instructions = p->last_mfma_count.load(std::memory_order_relaxed);
     info->gather_bitmap = p->bm.built ? 1u : 0u;
     info->bitmap_from_caller = p->bm.from_caller ? 1u : 0u;
     info->group_cuts_kept = p->caller_cuts.empty() ? 0u : 1u;

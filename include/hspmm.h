@@ -269,6 +269,11 @@ typedef struct {
     uint32_t panel_stream_mode;     /* the LDS-staging stream as built (hspmm_set_panel_stream): 0 uncompressed tiles, 1 two units
                                      * per consumer wave, 2 also tiles without their zeros; 0 when the plan has no such stream */
     uint32_t group_cuts_kept;       /* 1: the plan cuts a window only where the caller's groups end (hspmm_set_group_cuts) */
+    uint32_t last_mfma_kind;        /* matrix instruction of the last hspmm_run's main kernel: 0 none (all-shapes kernel, clear),
+                                     * 1 v_mfma_f32_16x16x32_f16, 2 v_mfma_f32_16x16x32_bf16, 3 v_mfma_f32_16x16x4_f32,
+                                     * 4 v_mfma_f32_4x4x1_16B_f32 */
+    uint32_t last_mfma_flops;       /* floating-point operations of one such instruction (16384, 16384, 2048, 512) */
+    uint64_t last_mfma_instructions;    /* how many of them that launch issued (zero padding of tiles and rows included) */
 } hspmm_plan_info;
 
 /* No reference counterpart (the reference prints its statistics from main,
