@@ -763,18 +763,6 @@ void spmm_mfma_kernel(const KernelArgs ka)
     // three features on, so that lane's first feature is not the launch's first)
     gat.lane_off -= mark_half_lane<TT>(L, ka.N, feat);
 
-    UnitWalk ww;
-    ww.u = rd[2];
-    ww.ustart = unitOffset[ww.u];
-    ww.uend = unitOffset[ww.u + 1u];
-    ww.row = unitRow[ww.u];
-    ww.next_row = (ww.u + 1u < U) ? (unitRow[ww.u + 1u] & ~7u) : rows;
-    ww.seg_start = t0;
-    ww.seg_end = umin32(ww.uend, t1);
-
-    // Rows before the first effective window belong to the wave that starts at step 0.
-    if (t0 == 0u) TT::zero_rows(L, c_lane, row_bytes, 0u, unitRow[0] & ~7u, active);
-
     f32x4 acc[NACC];
 #pragma unroll
     for (int p = 0; p < NACC; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -797,7 +785,21 @@ void spmm_mfma_kernel(const KernelArgs ka)
     // loop), hence the scheduling barriers.
     HSPMM_FOR_STAGES(HSPMM_PRO_IDX)
     __builtin_amdgcn_sched_barrier(0);
+    // The unit the range starts in: looked up while the first ids are on their way (they depend on the range's
+    // bounds alone; in front of them these lookups were one more trip to memory before the first gather).
+    UnitWalk ww;
+    ww.u = rd[2];
+    ww.ustart = unitOffset[ww.u];
+    ww.uend = unitOffset[ww.u + 1u];
+    ww.row = unitRow[ww.u];
+    ww.next_row = (ww.u + 1u < U) ? (unitRow[ww.u + 1u] & ~7u) : rows;
+    ww.seg_start = t0;
+    ww.seg_end = umin32(ww.uend, t1);
+    const uint32_t first_row = unitRow[0] & ~7u;
+    __builtin_amdgcn_sched_barrier(0);
     HSPMM_FOR_STAGES(HSPMM_PRO_TILE)
+    // Rows before the first effective window belong to the wave that starts at step 0.
+    if (t0 == 0u) TT::zero_rows(L, c_lane, row_bytes, 0u, first_row, active);
 
     // MFMAs of `step` from its registers, then the unit bookkeeping.
     auto compute = [&](const BVec &b0, const BVec &b1, const BVec &b2, const BVec &b3, const AVec &a,
