@@ -45,13 +45,15 @@ def build_library(force=True, experimental=False):
     cli = ["make", "-C", os.path.join(_HERE, "host")]
     if force:
         subprocess.check_call(cli + ["clean"], stdout=subprocess.DEVNULL)
-    subprocess.check_call(cli + ["-j4", "fp16_test", "bf16_test", "tf32_test", "fp16_transposed_test"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(cli + ["-j4", "fp16_test", "bf16_test", "tf32_test", "fp16_transposed_test", "tf32_k4_test"],
+                          stdout=subprocess.DEVNULL)
     return _LIB
 
 
 def cli_path(name):
     """Path of a built command-line driver: 'fp16_test', 'bf16_test', 'tf32_test', or
-    'fp16_transposed_test' (fp16_test built with -DSPARSE_A_TRANSPOSE)."""
+    'fp16_transposed_test' (fp16_test built with -DSPARSE_A_TRANSPOSE), 'tf32_k4_test' (tf32_test built with
+    -DMMA_M16N8K4: 8 x 4 tiles)."""
     return os.path.join(_HERE, "host", name)
 
 
@@ -129,6 +131,8 @@ def load_library():
     L.hspmm_csr_free.restype = None
     L.hspmm_btcf_sizes.argtypes = [i, u32, vp, vp, C.POINTER(u32), C.POINTER(u32)]
     L.hspmm_btcf_fill.argtypes = [i, u32, vp, vp, vp, i, vp, vp, vp, vp]
+    L.hspmm_btcf_sizes_cw.argtypes = [i, u32, u32, vp, vp, C.POINTER(u32), C.POINTER(u32)]
+    L.hspmm_btcf_fill_cw.argtypes = [i, u32, u32, vp, vp, vp, i, vp, vp, vp, vp]
     L.hspmm_bitmap_sizes.argtypes = [i, u32, vp, vp, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]
     L.hspmm_bitmap_fill.argtypes = [i, u32, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp]
     L.hspmm_bitmap_expand.argtypes = [i, u32, vp, vp, vp, vp]
@@ -232,26 +236,27 @@ def mtx_load(path, dtype):
         L.hspmm_csr_free(C.byref(m))
 
 
-def csr_to_btcf(rows, cols, row_ptr, col_idx, values, dtype, transpose=False):
+def csr_to_btcf(rows, cols, row_ptr, col_idx, values, dtype, transpose=False, cw=None):
     """CSR2BTCFNOBITMAP of the reference (src/utils/convert.h:146): returns the
-    BTCF_MTX_NO_BITMAP fields (src/utils/class.h:74-85) as a dict of numpy arrays."""
+    BTCF_MTX_NO_BITMAP fields (src/utils/class.h:74-85) as a dict of numpy arrays.  cw: tile width, the
+    element type's default or 4 for TF32 (the reference's -DMMA_M16N8K4 build, src/common.h:28-35)."""
     L = load_library()
     vt = _val_dtype(dtype)
-    cw = 8 if dtype == TF32 else 16
+    cw = cw or (8 if dtype == TF32 else 16)
     row_ptr = np.ascontiguousarray(row_ptr, np.uint32)
     col_idx = np.ascontiguousarray(col_idx, np.uint32)
     values = np.ascontiguousarray(values, vt)
     if row_ptr.size != rows + 1:
         raise ValueError("row_ptr must have rows + 1 entries")
     W, T = C.c_uint32(), C.c_uint32()
-    _check(L.hspmm_btcf_sizes(dtype, rows, _p(row_ptr), _p(col_idx), C.byref(W), C.byref(T)))
+    _check(L.hspmm_btcf_sizes_cw(dtype, cw, rows, _p(row_ptr), _p(col_idx), C.byref(W), C.byref(T)))
     W, T = W.value, T.value
     rowOffset = np.zeros(W + 1, np.uint32)
     tcA2B = np.empty(T * cw, np.uint32)
     data = np.empty(T * ROW_WINDOW * cw, vt)
     rowIdx = np.empty(W, np.uint32)
-    _check(L.hspmm_btcf_fill(dtype, rows, _p(row_ptr), _p(col_idx), _p(values), int(transpose),
-                             _p(rowOffset), _p(tcA2B), _p(data), _p(rowIdx)))
+    _check(L.hspmm_btcf_fill_cw(dtype, cw, rows, _p(row_ptr), _p(col_idx), _p(values), int(transpose),
+                                _p(rowOffset), _p(tcA2B), _p(data), _p(rowIdx)))
     return dict(rows=rows, cols=cols, nnzs=int(col_idx.size), dtype=dtype, cw=cw, transposed=bool(transpose),
                 total_row_windows=(rows + ROW_WINDOW - 1) // ROW_WINDOW, eff_row_windows=W,
                 total_tiles=T, rowOffset=rowOffset, tcA2B=tcA2B, data=data, rowIdx=rowIdx)

@@ -1558,21 +1558,29 @@ int hspmm_prepare(hspmm_plan *p, uint32_t N)
 
 }  // extern "C"
 
-// Launch through the LDS-panel kernels.  Grid = row blocks x feature blocks x chunks of
-// panels; the chunk count is what it takes to have about two workgroups per compute unit.
-// The launch shape is a function of the plan and N alone.
-static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStream_t s, hipEvent_t mid, RunMode mode)
+// ---------------------------------------------------------------------------
+// A launch in three steps: choose (a function of the plan, N and the pointers' alignment alone: kernel
+// family, load layout, launch shape), acquire (what the choice needs beyond the plan's fixed arrays - a work
+// partition, partial sums, arrival counters - under the plan's mutex), launch.  hspmm_prepare stops after the
+// second step; hspmm_run_static fails in the second when something would have to be built.
+// ---------------------------------------------------------------------------
+
+// Shape of a launch of the LDS-panel kernels: grid = row blocks x feature blocks x chunks of panels.
+struct PanelShape {
+    int units = 0;                      // workgroup shape code (launch_spmm_panel)
+    uint32_t units_per_group = 0;       // consumer waves of a workgroup that get a unit
+    uint32_t n_feat_blocks = 0, n_chunks = 0, panels_per_chunk = 0;
+    size_t acc_per_unit = 0;            // accumulator registers (of four floats per lane) a unit's chunk sums take
+    uint32_t mfma_kind = 0;
+    uint64_t mfma_count = 0;
+};
+
+static int choose_panel_shape(const hspmm_plan *p, uint32_t N, PanelShape *out)
 {
     const hspmm_plan::Panel &pl = p->panel;
-    hspmm::PanelArgs pa{};
-    pa.unitRow = pl.d_unitRow; pa.poff = pl.d_poff; pa.step_panel = pl.d_step_panel; pa.ids = pl.d_ids;
-    pa.tiles = pl.d_tiles; pa.n_steps = pl.n_steps;
-    pa.masks = pl.d_masks; pa.vals = pl.d_vals; pa.step_voff = pl.d_step_voff;
-    pa.B = dB; pa.C = dC;
-    pa.n_units = pl.n_units; pa.rows = p->rows; pa.cols = p->cols; pa.N = N;
+    PanelShape sh;
     const uint32_t block = hspmm::kPanelRowBytes / p->elem;
-    pa.n_feat_blocks = (N + block - 1u) / block;                   // (the last block may end inside: run_impl says when)
-    pa.n_panels = pl.n_panels;
+    sh.n_feat_blocks = (N + block - 1u) / block;                   // (the last block may end inside: panel_serves says when)
     // The workgroup shape: code 14 / 12 = that many consumer waves and two producers, 13 = 12 consumers and
     // four producers (few enough registers for two workgroups per compute unit, which the 4x4x1 fp32 kernel
     // needs to keep its short MFMAs fed).  Of the consumer waves any number may be given a unit.
@@ -1595,13 +1603,12 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
     const uint64_t slots = uint64_t(p->compute_units) * (pl.quad ? 2u : 1u);     // workgroups resident at a time
     // Units per workgroup and chunks of panels: the workgroups should fill the compute units in whole
     // rounds.  Cost of a shape = rounds x panels per chunk x (units + 3: a panel costs its LDS reads and
-    // MFMAs, which go with the units, plus its copy and barrier), plus the second launch when there are
-    // chunk sums.
+    // MFMAs, which go with the units, plus its copy and barrier), plus what chunk sums cost.
     uint64_t chunks = 1;
     int best_units = max_units;
     double best_cost = 0.0;
     for (int nc = forced_units ? forced_units : std::max(4, max_units / 2); nc <= (forced_units ? forced_units : max_units); ++nc) {
-        const uint64_t rbs = (uint64_t(wave_units) + nc - 1) / nc, base = rbs * pa.n_feat_blocks;
+        const uint64_t rbs = (uint64_t(wave_units) + nc - 1) / nc, base = rbs * sh.n_feat_blocks;
         uint64_t ch = base >= slots ? 1 : std::min<uint64_t>(slots / base, pl.n_panels);
         const uint64_t ppc = (pl.n_panels + ch - 1) / ch;
         ch = (pl.n_panels + ppc - 1) / ppc;
@@ -1613,23 +1620,47 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
                                     : double(rounds) * double(ppc) * (double(nc) + 3.0) + (ch > 1 ? 80.0 : 0.0);
         if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best_units = nc; chunks = ch; }
     }
-    pa.units_per_group = uint32_t(best_units);
+    sh.units = units;
+    sh.units_per_group = uint32_t(best_units);
     const uint64_t row_blocks = (uint64_t(wave_units) + best_units - 1) / best_units;
-    const uint64_t base = row_blocks * pa.n_feat_blocks;
+    const uint64_t base = row_blocks * sh.n_feat_blocks;
     if (p->cfg.panel_chunks) chunks = uint64_t(p->cfg.panel_chunks);
     if (chunks < 1) chunks = 1;
     if (chunks > pl.n_panels) chunks = pl.n_panels;
-    pa.panels_per_chunk = uint32_t((pl.n_panels + chunks - 1) / chunks);
-    pa.n_chunks = (pl.n_panels + pa.panels_per_chunk - 1) / pa.panels_per_chunk;
-    if (base * pa.n_chunks > 0x7FFFFFFFull)
+    sh.panels_per_chunk = uint32_t((pl.n_panels + chunks - 1) / chunks);
+    sh.n_chunks = (pl.n_panels + sh.panels_per_chunk - 1) / sh.panels_per_chunk;
+    if (base * sh.n_chunks > 0x7FFFFFFFull)
         return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many workgroups", N);
+    if (uint64_t(pl.n_units) * sh.n_chunks > 0xFFFFFFFFull)
+        return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many partial sums", N);
+    const size_t wide_rows = pl.G == 4 ? 2u : 1u;
+    sh.acc_per_unit = pl.quad ? 2u : pl.split ? 4u * wide_rows : p->dtype != HSPMM_TF32 ? 8u * wide_rows : 4u * size_t(pl.G);
+    // matrix instructions per step and feature block (PanelOps<...>::mma_half in spmm_panel_kernel.hpp)
+    sh.mfma_kind = pl.quad ? 4u : (p->dtype == HSPMM_TF32 && !pl.split) ? 3u : (p->dtype == HSPMM_FP16 ? 1u : 2u);
+    const uint64_t per_step = pl.quad ? 16u : pl.split ? 12u * wide_rows : p->dtype != HSPMM_TF32 ? 8u * wide_rows : 8u * uint64_t(pl.G);
+    sh.mfma_count = uint64_t(pl.n_steps) * sh.n_feat_blocks * per_step;
+    *out = sh;
+    return HSPMM_OK;
+}
+
+// Launch through the LDS-panel kernels.  The launch shape is a function of the plan and N alone.
+static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStream_t s, hipEvent_t mid, RunMode mode)
+{
+    PanelShape sh;
+    if (int rc = choose_panel_shape(p, N, &sh)) return rc;
+    const hspmm_plan::Panel &pl = p->panel;
+    hspmm::PanelArgs pa{};
+    pa.unitRow = pl.d_unitRow; pa.poff = pl.d_poff; pa.step_panel = pl.d_step_panel; pa.ids = pl.d_ids;
+    pa.tiles = pl.d_tiles; pa.n_steps = pl.n_steps;
+    pa.masks = pl.d_masks; pa.vals = pl.d_vals; pa.step_voff = pl.d_step_voff;
+    pa.B = dB; pa.C = dC;
+    pa.n_units = pl.n_units; pa.rows = p->rows; pa.cols = p->cols; pa.N = N;
+    pa.n_feat_blocks = sh.n_feat_blocks; pa.n_panels = pl.n_panels;
+    pa.units_per_group = sh.units_per_group; pa.n_chunks = sh.n_chunks; pa.panels_per_chunk = sh.panels_per_chunk;
     hspmm::KernelArgs ka{};
-    if (pa.n_chunks > 1) {
-        const size_t wide_acc = pl.G == 4 ? 2u : 1u;
-        const size_t nacc = pl.quad ? 2u : pl.split ? 4u * wide_acc : p->dtype != HSPMM_TF32 ? 8u * wide_acc : 4u * size_t(pl.G);
-        const size_t need = size_t(pl.n_units) * pa.n_chunks * pa.n_feat_blocks * nacc * 64u * 16u;
-        if (uint64_t(pl.n_units) * pa.n_chunks > 0xFFFFFFFFull)
-            return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many partial sums", N);
+    if (sh.n_chunks > 1) {
+        // acquire: the chunk sums and, where the last wave to arrive adds them, the arrival counters
+        const size_t need = size_t(pl.n_units) * sh.n_chunks * sh.n_feat_blocks * sh.acc_per_unit * 64u * 16u;
         {
             std::lock_guard<std::mutex> lk(p->mu);
             int rc = scratch_for(p, s, need, mode, &pa.scratch);
@@ -1637,8 +1668,9 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
             // As in the gather kernels, the wave that brings a unit's last chunk adds the chunk sums itself
             // (16-byte device-scope accesses; block-clustered configuration at N = 512: 56.0 + 8.1 us in two
             // launches, 60.3 us in one).  It addresses a unit's chunk sums with 32-bit offsets.
-            if (p->cfg.fused_fixup != 0 && mode != RunMode::kStatic && uint64_t(pa.n_chunks) * pa.n_feat_blocks * nacc * 1024u < (1ull << 31) &&
-                (rc = ensure_arrive(p, s, size_t(pl.n_units) * pa.n_feat_blocks, mode, &pa.arrive)))
+            if (p->cfg.fused_fixup != 0 && mode != RunMode::kStatic &&
+                uint64_t(sh.n_chunks) * sh.n_feat_blocks * sh.acc_per_unit * 1024u < (1ull << 31) &&
+                (rc = ensure_arrive(p, s, size_t(pl.n_units) * sh.n_feat_blocks, mode, &pa.arrive)))
                 return rc;
         }
         // the chunk sums of unit u are slots u * chunks .. + chunks - 1: no table
@@ -1646,24 +1678,40 @@ static int run_panel(hspmm_plan *p, const void *dB, void *dC, uint32_t N, hipStr
         ka.scratch = pa.scratch;
         ka.C = dC; ka.B = dB;
         ka.n_split = pl.n_units; ka.n_units = pl.n_units; ka.rows = p->rows; ka.N = N; ka.ld = N;
-        ka.n_feat_blocks = pa.n_feat_blocks;
-        ka.uniform_chunks = pa.n_chunks;
+        ka.n_feat_blocks = sh.n_feat_blocks;
+        ka.uniform_chunks = sh.n_chunks;
     }
     if (mode == RunMode::kPrepare) return HSPMM_OK;
-    {
-        // matrix instructions per step and feature block (PanelOps<...>::mma_half in spmm_panel_kernel.hpp)
-        const uint64_t wide_rows = pl.G == 4 ? 2u : 1u;
-        const uint32_t kind = pl.quad ? 4u : (p->dtype == HSPMM_TF32 && !pl.split) ? 3u : (p->dtype == HSPMM_FP16 ? 1u : 2u);
-        const uint64_t per_step = pl.quad ? 16u : pl.split ? 12u * wide_rows : p->dtype != HSPMM_TF32 ? 8u * wide_rows : 8u * uint64_t(pl.G);
-        p->note_launch(3, kind, uint64_t(pl.n_steps) * pa.n_feat_blocks * per_step);
-    }
-    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : pl.G, pl.split, pl.tall, pl.packed, pa, ka, units, s, mid));
+    p->note_launch(3, sh.mfma_kind, sh.mfma_count);
+    HSPMM_HIP(hspmm::launch_spmm_panel(p->dtype, pl.quad ? 0 : pl.G, pl.split, pl.tall, pl.packed, pa, ka, sh.units, s, mid));
     return HSPMM_OK;
+}
+
+// Whether the LDS-panel kernels serve feature dimension N (a workgroup covers 256 bytes of every B row with
+// 16-byte accesses).
+static bool panel_serves(const hspmm_plan *p, uint32_t N)
+{
+    if (!p->panel.built || !(p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4)) return false;
+    const uint32_t block_feat = hspmm::kPanelRowBytes / p->elem;
+    // (a 16-bit matrix near the break-even is served as fast or faster by the gather kernels while
+    // one wave of theirs covers all of N)
+    const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
+    // (the producers address a panel of B - up to 256 rows - with 32-bit offsets)
+    const bool offsets_fit = uint64_t(N) * p->elem < (uint64_t(1) << 24);
+    // Whole blocks of features; or any N of one block at least - the last block then moves back to end with
+    // the row (panel_block_first_feature in spmm_mfma_kernel.hpp) -; or, fp32 storage in bf16 parts, whose
+    // gather kernels multiply at a sixteenth of the rate, one partly empty block from 16 features on when the
+    // rows are whole 16-byte pieces (the lanes of that kernel own one feature per accumulator: what the block
+    // lacks is read from the row's first piece and not stored).
+    const bool ragged_ok = N >= block_feat || (p->panel.split && (uint64_t(N) * p->elem) % 16u == 0 && N >= 16u);
+    // (B and C wherever they start: the producers' 16-byte loads need no alignment, C is stored element by element)
+    return pays && offsets_fit && (N % block_feat == 0 || ragged_ok);
 }
 
 static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint32_t ld, hipStream_t s, hipEvent_t mid, RunMode mode);
 
-// One launch (or, kPrepare, everything a launch with this N and these pointer alignments would build).
+// One launch (or, kPrepare, everything a launch with this N and these pointer alignments would build): which
+// kernel family serves N, and in how many pieces.
 // mid: when not null, an event recorded between the main kernel and the kernel that adds the partial
 // sums of split windows.
 static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *stream, hipEvent_t mid, RunMode mode)
@@ -1690,23 +1738,7 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
         HSPMM_HIP(hspmm::launch_fill_zero(dC, size_t(p->rows) * N * p->elem, s));
         return HSPMM_OK;
     }
-    if (p->panel.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode >= 4)) {
-        // LDS-panel kernels: a workgroup covers 256 bytes of every B row with 16-byte accesses
-        const uint32_t block_feat = hspmm::kPanelRowBytes / p->elem;
-        // (a 16-bit matrix near the break-even is served as fast or faster by the gather kernels while
-        // one wave of theirs covers all of N)
-        const bool pays = p->cfg.kernel_mode >= 4 || p->cw != 16 || p->panel.density >= 2.2 || N >= 256u;
-        // (the producers address a panel of B - up to 256 rows - with 32-bit offsets)
-        const bool offsets_fit = uint64_t(N) * p->elem < (uint64_t(1) << 24);
-        // Whole blocks of features; or any N of one block at least - the last block then moves back to end with
-        // the row (panel_block_first_feature in spmm_mfma_kernel.hpp) -; or, fp32 storage in bf16 parts, whose
-        // gather kernels multiply at a sixteenth of the rate, one partly empty block from 16 features on when the
-        // rows are whole 16-byte pieces (the lanes of that kernel own one feature per accumulator: what the block
-        // lacks is read from the row's first piece and not stored).
-        const bool ragged_ok = N >= block_feat || (p->panel.split && (uint64_t(N) * p->elem) % 16u == 0 && N >= 16u);
-        // (B and C wherever they start: the producers' 16-byte loads need no alignment, C is stored element by element)
-        if (pays && offsets_fit && (N % block_feat == 0 || ragged_ok)) return run_panel(p, dB, dC, N, s, mid, mode);
-    }
+    if (panel_serves(p, N)) return run_panel(p, dB, dC, N, s, mid, mode);
     // A feature dimension that no wide load divides (16-bit types: N not a multiple of 8, fp32 storage: of 4) would
     // run in blocks of 32 resp. 16 features, each block a pass over the tiles and another gather of every row
     // (power-law graph 2^20, fp16: N = 130 in five passes, 1404 us against 481 us at N = 128).  Two launches
@@ -1763,17 +1795,71 @@ static int run_impl(hspmm_plan *p, const void *dB, void *dC, uint32_t N, void *s
     return run_gather(p, dB, dC, N, N, s, mid, mode);
 }
 
-// One launch of the gather kernels (or of the all-shapes kernel) over N features of rows that are ld elements apart.
-static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint32_t ld, hipStream_t s, hipEvent_t mid, RunMode mode)
+// What a launch of the gather kernels (or of the all-shapes kernel) over N features looks like: a function of the
+// plan, N, the row pitch and the alignment of B and C.
+struct GatherShape {
+    Choice c{};
+    int layout = 0;                     // c.layout, or the bitmap form of it
+    uint32_t n_feat_blocks = 0, xcd_split = 0;
+    int level = 0;                      // which partition: fewer, longer ranges for more feature blocks
+    int wpg = 0;                        // waves per workgroup
+    bool combine = false;               // the waves of a workgroup add the sums of one unit among themselves
+    bool aligned = false;               // every unit is cut into the ranges of one workgroup, which stores it
+    int prefetch = 0;
+    int partition_index() const { return aligned ? 4 : combine ? 3 : level; }
+};
+
+static GatherShape choose_gather_shape(const hspmm_plan *p, const void *dB, const void *dC, uint32_t N, uint32_t ld)
 {
-    const bool launch = mode != RunMode::kPrepare;
+    GatherShape g;
     // Feature blocks with XCDs of their own (see spmm_mfma_kernel): pays when B is far larger than an
     // XCD's 4 MB L2, so that what an L2 can keep of it decides the hit rate of the gathers (power-law
     // graph 2^20, N = 128: 575 -> 535 us; uniform 65536^2: 39.7 -> 35.5 us), and costs a second pass over
     // the tile stream.  Requests below a 128-byte line lose (N = 64 as two blocks of 32: 280 -> 510 us).
     const bool want_split = p->cfg.xcd_split > 0 ||
                              (p->cfg.xcd_split < 0 && uint64_t(p->cols) * N * p->elem >= (uint64_t(8) << 20));
-    const Choice c = choose_kernel(p, dB, dC, N, ld, want_split);
+    g.c = choose_kernel(p, dB, dC, N, ld, want_split);
+    if (g.c.scalar) return g;
+    const Choice &c = g.c;
+    g.layout = c.layout;
+    if (p->bm.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 3) &&
+        (p->dtype == HSPMM_TF32 || (c.layout == hspmm::kLayoutDW && (c.V == 2 || c.V == 4))))
+        g.layout = hspmm::kLayoutDWB;                 // tiles as bitmap + stored elements
+    g.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
+    g.xcd_split = (want_split && (g.n_feat_blocks == 2u || g.n_feat_blocks == 4u || g.n_feat_blocks == 8u)) ? 1u : 0u;
+    // Several feature blocks give several waves per range; fewer, longer ranges then keep
+    // the number of waves, and pay off where units are long enough to be cut into many
+    // pieces (each piece of a cut unit costs a partial sum).
+    const double steps_per_unit = double(p->n_steps) / double(p->n_units);
+    const double steps_per_range = double(p->n_steps) / double(p->parts[0].part.ranges.size());
+    if (steps_per_unit >= 8.0 * steps_per_range) g.level = g.n_feat_blocks >= 4 ? 2 : g.n_feat_blocks >= 2 ? 1 : 0;
+    // One feature block: the waves of a workgroup walk consecutive ranges and add the partial sums of
+    // one unit among themselves.
+    g.wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
+    g.combine = g.level == 0 && g.n_feat_blocks == 1 && g.wpg > 1 && p->cfg.fused_fixup <= 0;
+    // Units that are all long (block-clustered, pruned or dense-ish random matrices at a small N): every
+    // unit is cut into the ranges of one workgroup of four or eight waves, which stores it itself - no
+    // partial sums leave the chip and there is no second launch (block-clustered 4096 x 14336, N = 16:
+    // 18.9 + 6.4 us -> 19 us; random 8192 x 8192 at 2 %, N = 128: 26.8 + 7.1 -> 22.8 us).  With the default
+    // knobs only: the eight-wave kernels exist for the default depth.
+    g.aligned = g.combine && p->aligned_group && c.narrow && p->cfg.consumer_warp_num == 0 &&
+                (p->cfg.buffer_stage == 0 || p->aligned_group == hspmm::kMaxWavesPerGroup) &&
+                p->cfg.producer_warp_group_num == 0;
+    if (g.aligned) g.wpg = p->aligned_group;
+    const int default_depth = hspmm::default_prefetch(int(p->elem), p->G, c.V);
+    g.prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage : default_depth;
+#ifndef HSPMM_EXPERIMENTAL
+    if (!c.narrow) g.prefetch = default_depth;    // (64-bit gather offsets are built for the default depth only)
+#endif
+    return g;
+}
+
+// One launch of the gather kernels (or of the all-shapes kernel) over N features of rows that are ld elements apart.
+static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint32_t ld, hipStream_t s, hipEvent_t mid, RunMode mode)
+{
+    const bool launch = mode != RunMode::kPrepare;
+    const GatherShape g = choose_gather_shape(p, dB, dC, N, ld);
+    const Choice &c = g.c;
     hspmm::KernelArgs ka{};
     ka.rowOffset = p->d_rowOffset; ka.data = p->d_data; ka.rowIdx = p->d_rowIdx; ka.tcA2B = p->d_a2b_raw;
     ka.B = dB; ka.C = dC;
@@ -1786,39 +1872,12 @@ static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint3
         return HSPMM_OK;
     }
     ka.unitOffset = p->d_unitOffset; ka.unitRow = p->d_unitRow; ka.ids = p->d_ids; ka.tiles = p->d_tiles;
-    int layout = c.layout;
-    if (p->bm.built && (p->cfg.kernel_mode == 0 || p->cfg.kernel_mode == 3) &&
-        (p->dtype == HSPMM_TF32 || (c.layout == hspmm::kLayoutDW && (c.V == 2 || c.V == 4)))) {
-        layout = hspmm::kLayoutDWB;                   // tiles as bitmap + stored elements
-        ka.tiles = p->bm.d_vals; ka.bm_header = p->bm.d_header;
-    }
+    if (g.layout == hspmm::kLayoutDWB) { ka.tiles = p->bm.d_vals; ka.bm_header = p->bm.d_header; }
     ka.n_units = p->n_units;
-    ka.n_feat_blocks = (N + uint32_t(c.block_feat) - 1u) / uint32_t(c.block_feat);
-    ka.xcd_split = (want_split && (ka.n_feat_blocks == 2u || ka.n_feat_blocks == 4u || ka.n_feat_blocks == 8u)) ? 1u : 0u;
-    // Several feature blocks give several waves per range; fewer, longer ranges then keep
-    // the number of waves, and pay off where units are long enough to be cut into many
-    // pieces (each piece of a cut unit costs a partial sum).
-    int level = 0;
-    {
-        const double steps_per_unit = double(p->n_steps) / double(p->n_units);
-        const double steps_per_range = double(p->n_steps) / double(p->parts[0].part.ranges.size());
-        if (steps_per_unit >= 8.0 * steps_per_range) level = ka.n_feat_blocks >= 4 ? 2 : ka.n_feat_blocks >= 2 ? 1 : 0;
-    }
-    // One feature block: the waves of a workgroup walk consecutive ranges and add the partial sums of
-    // one unit among themselves.
-    int wpg = p->cfg.consumer_warp_num > 0 ? p->cfg.consumer_warp_num : hspmm::kMaxWavesPerGroup;
-    const bool combine = level == 0 && ka.n_feat_blocks == 1 && wpg > 1 && p->cfg.fused_fixup <= 0;
-    // Units that are all long (block-clustered, pruned or dense-ish random matrices at a small N): every
-    // unit is cut into the ranges of one workgroup of four or eight waves, which stores it itself - no
-    // partial sums leave the chip and there is no second launch (block-clustered 4096 x 14336, N = 16:
-    // 18.9 + 6.4 us -> 19 us; random 8192 x 8192 at 2 %, N = 128: 26.8 + 7.1 -> 22.8 us).  With the default
-    // knobs only: the eight-wave kernels exist for the default depths.
-    bool fused = false;
-    const bool aligned = combine && p->aligned_group && c.narrow && p->cfg.consumer_warp_num == 0 &&
-                         (p->cfg.buffer_stage == 0 || p->aligned_group == hspmm::kMaxWavesPerGroup) &&
-                         p->cfg.producer_warp_group_num == 0;
-    if (aligned) wpg = p->aligned_group;
-    hspmm_plan::DevPartition &dp = p->parts[aligned ? 4 : combine ? 3 : level];
+    ka.n_feat_blocks = g.n_feat_blocks;
+    ka.xcd_split = g.xcd_split;
+    // acquire: the partition this shape walks, the partial sums of its cut units, their arrival counters
+    hspmm_plan::DevPartition &dp = p->parts[g.partition_index()];
     {
         std::lock_guard<std::mutex> lk(p->mu);
         if (!dp.built) {
@@ -1826,7 +1885,7 @@ static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint3
                 return fail(HSPMM_ERR_UNSUPPORTED,
                             "hspmm_run_static: the work partition for N = %u is not built yet; call hspmm_prepare(plan, N) "
                             "or hspmm_run once with this N first", N);
-            const int rc = build_and_upload_partition(p, level, combine ? uint32_t(wpg) : 1u, aligned);
+            const int rc = build_and_upload_partition(p, g.level, g.combine ? uint32_t(g.wpg) : 1u, g.aligned);
             if (rc) return rc;
         }
         ka.n_ranges = uint32_t(dp.part.ranges.size());
@@ -1835,8 +1894,8 @@ static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint3
         // kernel would): worth it where few units are cut and the second launch is most of what they cost
         // (power-law graph, 382 of 110 746 units: 540.6 + 9.4 -> 541.1 us); where every unit is cut the
         // device-scope traffic costs more than the launch (block-clustered: 30 -> 129 us).
-        fused = mode != RunMode::kStatic && !combine &&
-                (p->cfg.fused_fixup > 0 || (p->cfg.fused_fixup < 0 && ka.n_split && uint64_t(ka.n_split) * 32u <= p->n_units));
+        const bool fused = mode != RunMode::kStatic && !g.combine &&
+                           (p->cfg.fused_fixup > 0 || (p->cfg.fused_fixup < 0 && ka.n_split && uint64_t(ka.n_split) * 32u <= p->n_units));
         if (uint64_t(ka.n_ranges) * ka.n_feat_blocks > 0x7FFFFFFFull)
             return fail(HSPMM_ERR_UNSUPPORTED, "feature dimension %u needs too many work items", N);
         const size_t need = size_t(dp.part.n_slots) * ka.n_feat_blocks * size_t(c.V) * size_t(p->G) * 64u * 16u;
@@ -1849,12 +1908,7 @@ static int run_gather(hspmm_plan *p, const void *dB, void *dC, uint32_t N, uint3
     // (per step and feature block: G * V instructions of 16 x 16 x 32, or 2 G V of 16 x 16 x 4 for 32-bit elements)
     p->note_launch(2, p->dtype == HSPMM_TF32 ? 3u : p->dtype == HSPMM_FP16 ? 1u : 2u,
                    uint64_t(p->n_steps) * ka.n_feat_blocks * uint64_t(p->G) * uint64_t(c.V) * (p->dtype == HSPMM_TF32 ? 2u : 1u));
-    const int default_depth = hspmm::default_prefetch(int(p->elem), p->G, c.V);
-    int prefetch = p->cfg.buffer_stage > 0 ? p->cfg.buffer_stage : default_depth;
-#ifndef HSPMM_EXPERIMENTAL
-    if (!c.narrow) prefetch = default_depth;      // (64-bit gather offsets are built for the default depth only)
-#endif
-    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, layout, p->G, ka, c.V, prefetch, c.narrow, wpg, s, mid));
+    HSPMM_HIP(hspmm::launch_spmm_mfma(p->dtype, g.layout, p->G, ka, c.V, g.prefetch, c.narrow, g.wpg, s, mid));
     return HSPMM_OK;
 }
 

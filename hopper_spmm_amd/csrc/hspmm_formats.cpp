@@ -399,15 +399,27 @@ static void count_tiles(uint32_t rows, const uint32_t *row_ptr, const uint32_t *
 
 extern "C" {
 
-int hspmm_btcf_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
-                     uint32_t *eff_row_windows, uint32_t *total_tiles)
+// Tile width for an element type: the default (16 for the 16-bit types, 8 for fp32 storage) or, for fp32
+// storage, the 4 of the reference's -DMMA_M16N8K4 build (src/common.h:28-35).  0 on a bad request.
+static uint32_t tile_width(int dtype, uint32_t col_window)
 {
-    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16) { set_error("unknown dtype"); return 0; }
+    const uint32_t dflt = dtype == HSPMM_TF32 ? 8u : 16u;
+    if (col_window == 0 || col_window == dflt) return dflt;
+    if (dtype == HSPMM_TF32 && col_window == 4u) return 4u;
+    set_error("col_window: the element type's default (16 / 8), or 4 for HSPMM_TF32");
+    return 0;
+}
+
+int hspmm_btcf_sizes_cw(int dtype, uint32_t col_window, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                        uint32_t *eff_row_windows, uint32_t *total_tiles)
+{
+    const uint32_t cw = tile_width(dtype, col_window);
+    if (!cw) return HSPMM_ERR_INVALID;
     if (!row_ptr || !eff_row_windows || !total_tiles || (!col_idx && row_ptr[rows])) {
         set_error("null argument");
         return HSPMM_ERR_INVALID;
     }
-    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
     std::vector<uint32_t> tiles;
     count_tiles(rows, row_ptr, col_idx, cw, tiles);
     uint64_t W = 0, T = 0;
@@ -418,13 +430,26 @@ int hspmm_btcf_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const ui
     return HSPMM_OK;
 }
 
+int hspmm_btcf_sizes(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                     uint32_t *eff_row_windows, uint32_t *total_tiles)
+{
+    return hspmm_btcf_sizes_cw(dtype, 0, rows, row_ptr, col_idx, eff_row_windows, total_tiles);
+}
+
 int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
                     const void *values, int transpose, uint32_t *rowOffset, uint32_t *tcA2B, void *data,
                     uint32_t *rowIdx)
 {
-    if (dtype != HSPMM_FP16 && dtype != HSPMM_TF32 && dtype != HSPMM_BF16) { set_error("unknown dtype"); return HSPMM_ERR_INVALID; }
+    return hspmm_btcf_fill_cw(dtype, 0, rows, row_ptr, col_idx, values, transpose, rowOffset, tcA2B, data, rowIdx);
+}
+
+int hspmm_btcf_fill_cw(int dtype, uint32_t col_window, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                       const void *values, int transpose, uint32_t *rowOffset, uint32_t *tcA2B, void *data,
+                       uint32_t *rowIdx)
+{
+    const uint32_t cw = tile_width(dtype, col_window);
+    if (!cw) return HSPMM_ERR_INVALID;
     if (!row_ptr || !rowOffset) { set_error("null argument"); return HSPMM_ERR_INVALID; }
-    const uint32_t cw = dtype == HSPMM_TF32 ? 8u : 16u;
     const size_t es = dtype == HSPMM_TF32 ? 4 : 2;
     const size_t tile_elems = size_t(HSPMM_ROW_WINDOW) * cw;
     std::vector<uint32_t> tiles;

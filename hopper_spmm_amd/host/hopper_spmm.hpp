@@ -47,7 +47,11 @@
 #define HSPMM_BUILD_DTYPE HSPMM_BF16
 #else
 #define MAT_VAL_TYPE float
+#ifdef MMA_M16N8K4
+#define COL_WINDOW 4            // reference src/common.h:28-35: 8 x 4 tiles
+#else
 #define COL_WINDOW 8
+#endif
 #define HSPMM_BUILD_DTYPE HSPMM_TF32
 #endif
 
@@ -165,7 +169,7 @@ inline void CSR2BTCFNOBITMAP(const CSR_MTX &csr, BTCF_MTX_NO_BITMAP &btcf)
     uint32_t W = 0, T = 0;
     static const MAT_PTR_TYPE zero_ptr[1] = {0};
     const MAT_PTR_TYPE *rp = csr.row_ptr ? csr.row_ptr : zero_ptr;
-    if (hspmm_btcf_sizes(HSPMM_BUILD_DTYPE, csr.rows, rp, csr.col_idx, &W, &T) != HSPMM_OK)
+    if (hspmm_btcf_sizes_cw(HSPMM_BUILD_DTYPE, COL_WINDOW, csr.rows, rp, csr.col_idx, &W, &T) != HSPMM_OK)
         hspmm_cpp::die("CSR2BTCFNOBITMAP");
     btcf.rowOffset.assign(size_t(W) + 1, 0);
     btcf.tcA2B.assign(size_t(T) * COL_WINDOW, 0);
@@ -176,8 +180,8 @@ inline void CSR2BTCFNOBITMAP(const CSR_MTX &csr, BTCF_MTX_NO_BITMAP &btcf)
 #else
     const int transpose = 0;
 #endif
-    if (hspmm_btcf_fill(HSPMM_BUILD_DTYPE, csr.rows, rp, csr.col_idx, csr.values, transpose, btcf.rowOffset.data(),
-                        btcf.tcA2B.data(), btcf.data.data(), btcf.rowIdx.data()) != HSPMM_OK)
+    if (hspmm_btcf_fill_cw(HSPMM_BUILD_DTYPE, COL_WINDOW, csr.rows, rp, csr.col_idx, csr.values, transpose,
+                           btcf.rowOffset.data(), btcf.tcA2B.data(), btcf.data.data(), btcf.rowIdx.data()) != HSPMM_OK)
         hspmm_cpp::die("CSR2BTCFNOBITMAP");
     btcf.eff_row_windows = W;
     btcf.total_tiles = T;
@@ -187,6 +191,11 @@ inline void CSR2BTCFNOBITMAP(const CSR_MTX &csr, BTCF_MTX_NO_BITMAP &btcf)
 // CSR2BTCF of the reference (src/utils/convert.h:22-139).
 inline void CSR2BTCF(const CSR_MTX &csr, BTCF_MTX &btcf)
 {
+#ifdef MMA_M16N8K4
+    // (the library's bitmap tiles are 8 x 8 words of 64 bits; the 32-bit words of 8 x 4 tiles have no kernel)
+    std::fprintf(stderr, "CSR2BTCF: bitmap tiles of 8 x 4 (-DMMA_M16N8K4) are not supported; use CSR2BTCFNOBITMAP\n");
+    std::exit(EXIT_FAILURE);
+#endif
     btcf.rows = csr.rows; btcf.cols = csr.cols; btcf.nnzs = csr.nnzs;
     btcf.total_row_windows = (csr.rows + ROW_WINDOW - 1) / ROW_WINDOW;
     uint32_t W = 0, T = 0, S = 0;

@@ -360,6 +360,15 @@ int hspmm_btcf_fill(int dtype, uint32_t rows, const uint32_t *row_ptr, const uin
                     const void *values, int transpose,
                     uint32_t *rowOffset, uint32_t *tcA2B, void *data, uint32_t *rowIdx);
 
+/* The same converter with the tile width given: col_window 0 or the element type's default (16 / 8), or 4 for
+ * HSPMM_TF32 - the 8 x 4 tiles of the reference's -DMMA_M16N8K4 build (src/common.h:28-35: COL_WINDOW 4), which
+ * hspmm_create_layout takes. */
+int hspmm_btcf_sizes_cw(int dtype, uint32_t col_window, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                        uint32_t *eff_row_windows, uint32_t *total_tiles);
+int hspmm_btcf_fill_cw(int dtype, uint32_t col_window, uint32_t rows, const uint32_t *row_ptr, const uint32_t *col_idx,
+                       const void *values, int transpose,
+                       uint32_t *rowOffset, uint32_t *tcA2B, void *data, uint32_t *rowIdx);
+
 /* ---- bitmap-compressed and grouped formats ------------------------------ */
 
 /* Words of tcBit per tile: one 64-bit word for 8 x 8 tiles (HSPMM_TF32), two

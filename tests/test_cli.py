@@ -56,7 +56,9 @@ def test_cli_end_to_end_with_verification(hs, tmp_path):
                          ("tf32_test", "32", "grouped"), ("bf16_test", "64", "grouped"),
                          ("fp16_test", "64", "balanced"), ("tf32_test", "16", "balanced"),
                          # tiles written column by column (-DSPARSE_A_TRANSPOSE)
-                         ("fp16_transposed_test", "128", "tiles"), ("fp16_transposed_test", "40", "bitmap")):
+                         ("fp16_transposed_test", "128", "tiles"), ("fp16_transposed_test", "40", "bitmap"),
+                         # the tf32 variant with 8 x 4 tiles (-DMMA_M16N8K4, reference src/common.h:28-35)
+                         ("tf32_k4_test", "64", "tiles"), ("tf32_k4_test", "7", "tiles")):
         r = run(hs, name, str(p), n, "--seed", "42", "--verify", "--format", fmt)
         assert r.returncode == 0, r.stdout + r.stderr
         assert "verification passed" in r.stdout

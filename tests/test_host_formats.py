@@ -176,6 +176,27 @@ def test_converter_equals_oracle(hs, oracle, dtype):
             _same_btcf(a, o)
 
 
+def test_converter_writes_the_8_by_4_tiles_of_the_m16n8k4_build(hs, oracle):
+    """CSR2BTCFNOBITMAP with COL_WINDOW 4 (the reference's -DMMA_M16N8K4 build of the tf32 variant,
+    src/common.h:28-35), row by row and column by column: the library's converter against the oracle's,
+    bit for bit; the width is refused for the 16-bit types."""
+    rng = np.random.default_rng(270)
+    shapes = [(1, 1, 1.0, 0.0), (8, 4, 1.0, 0.0), (9, 5, 0.5, 0.0), (27, 12, 0.1, 0.7), (64, 500, 0.05, 0.3),
+              (203, 77, 0.3, 0.1), (1000, 1000, 0.004, 0.5), (16, 4000, 0.6, 0.0)]
+    for rows, cols, dens, erp in shapes:
+        A = random_csr(rng, rows, cols, dens, 1, erp)
+        for tr in (False, True):
+            a = hs.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], 1, transpose=tr, cw=4)
+            o = oracle.csr_to_btcf(rows, cols, A["row_ptr"], A["col_idx"], A["values"], "tf32", transpose=tr, cw=4)
+            assert a["cw"] == 4 and a["tcA2B"].size == 4 * a["total_tiles"] and a["data"].size == 32 * a["total_tiles"]
+            _same_btcf(a, o)
+    A = random_csr(rng, 16, 40, 0.3, 0)
+    with pytest.raises(hs.HspmmError):
+        hs.csr_to_btcf(16, 40, A["row_ptr"], A["col_idx"], A["values"], 0, cw=4)
+    with pytest.raises(hs.HspmmError):
+        hs.csr_to_btcf(16, 40, A["row_ptr"], A["col_idx"], A["values"].astype(np.float32), 1, cw=16)
+
+
 @pytest.mark.parametrize("dtype", [0, 1, 2])
 def test_relayout_of_the_build_switch_formats_gives_the_default_tiles(hs, oracle, dtype):
     """Tiles written with -DSPARSE_A_TRANSPOSE (convert.h:207-209) and, for fp32 storage, the

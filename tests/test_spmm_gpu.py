@@ -359,8 +359,8 @@ def test_plans_from_transposed_tiles_and_from_tiles_four_columns_wide(torch_cuda
     """The tile layouts of the reference's two optional build switches describe the same matrix:
     tiles written column by column (-DSPARSE_A_TRANSPOSE, src/utils/convert.h:207-209), by the
     library's converter and by the oracle's, and for fp32 storage the 8 x 4 tiles of -DMMA_M16N8K4
-    (src/common.h:28-35), which only the oracle's converter writes.  Their plans give bit for bit
-    what the plan of the default layout gives, and that agrees with the oracle."""
+    (src/common.h:28-35), by both converters as well.  Their plans give bit for bit what the plan of the
+    default layout gives, and that agrees with the oracle."""
     rng = np.random.default_rng(190 + dtype)
     for rows, cols, dens, erp, heavy in [(27, 100, 0.1, 0.5, ()), (300, 3000, 0.004, 0.2, (5, 100, 101, 299)),
                                          (1000, 700, 0.01, 0.6, (512,)), (64, 64, 1.0, 0.0, ())]:
@@ -369,6 +369,10 @@ def test_plans_from_transposed_tiles_and_from_tiles_four_columns_wide(torch_cuda
         csr = (rows, cols, A["row_ptr"], A["col_idx"], A["values"])
         layouts = [("transposed", hs.csr_to_btcf(*csr, dtype, transpose=True))]
         assert layouts[0][1]["transposed"] and not np.array_equal(layouts[0][1]["data"], plain["data"])
+        if dtype == 1:
+            layouts += [("library 8x4", hs.csr_to_btcf(*csr, dtype, cw=4)),
+                        ("library 8x4 transposed", hs.csr_to_btcf(*csr, dtype, transpose=True, cw=4))]
+            assert layouts[1][1]["cw"] == 4 and layouts[1][1]["total_tiles"] >= plain["total_tiles"]
         for name, kw in (("oracle transposed", dict(transpose=True)), ("8x4", dict(cw=4)),
                          ("8x4 transposed", dict(cw=4, transpose=True))):
             if "cw" in kw and dtype != 1:
