@@ -13,8 +13,9 @@
  * Parity status of each function (what pins it):
  *   orc_f32_to_f16 / orc_f16_to_f32  exhaustive comparison with numpy float16
  *   orc_f32_to_bf16 / orc_bf16_to_f32 comparison with torch.bfloat16 (CPU), all 65536 patterns back
- *   orc_mtx_read                     reference-produced golden vectors (tiny.mtx,
- *                                    gap.mtx), scipy COO->CSR cross-check
+ *   orc_mtx_read                     golden vectors (tiny.mtx, gap.mtx: definition cases small
+ *                                    enough to re-derive by hand from the reference's source
+ *                                    text), scipy COO->CSR cross-check
  *   orc_btcf_count / orc_btcf_fill   the same golden vectors, round-trip to CSR,
  *                                    brute force on small dense matrices
  *   orc_bitmap_fill                  golden nnzOffset / packed data / as-written tcBit

@@ -1,5 +1,5 @@
 """The product's host format functions (hspmm_mtx_load, hspmm_btcf_sizes/fill in
-libhspmm.so) against the pinned oracle and the reference-produced golden vectors.
+libhspmm.so) against the pinned oracle and the golden vectors (hand-checkable definition cases of the reference converters).
 Bit-exact: this is integer / byte work."""
 import json
 import os
