@@ -4,14 +4,20 @@
 // tf32_test / bf16_test.
 // B is filled with rand() / RAND_MAX as in the reference (src/fp16.cu:303-309);
 // --seed calls srand first (the reference never seeds, i.e. seed 1).  --verify
-// repeats the product with the library's scalar all-shapes kernel, a second
-// implementation on the GPU, and compares the two results element by element
-// (1e-2 relative, 1e-3 for tf32_test, plus a term in sum |a||b| for sums that cancel).
+// fills in the reference's empty "verify" step (src/fp16.cu:317) with the check its
+// test programs make (src/test_fp16.cu:284-315, src/tf32.cu:11-82): the product again
+// on the host, C[i][j] += float(a) * float(b) in fp32 over the stored entries of row i
+// in column order, compared element by element (1e-2 relative, 1e-3 for tf32_test,
+// plus a term in sum |a||b| for sums that cancel).  The check only reads what the GPU
+// wrote; nothing of it is ever returned as a result.
 // --format hands the matrix to the operator as uncompressed tiles (the reference's
 // only path, the default), as bitmap tiles (CSR2BTCF), as groups of the reference's
 // fixed length (BTCF2GBTCF) or as the groups of the library's balanced partition.
+#include <algorithm>
 #include <cstring>
 #include <string>
+#include <thread>
+#include <vector>
 
 #include "hopper_spmm.hpp"
 
@@ -82,30 +88,44 @@ int main(int argc, char *argv[])
 
     int rc = 0;
     if (verify) {
-        DENSE_MTX second{btcf.rows, feature_dim, new MAT_VAL_TYPE[size_t(btcf.rows) * feature_dim]};
-        if (hspmm_set_kernel_mode(1) != HSPMM_OK) hspmm_cpp::die("hspmm_set_kernel_mode");
-        hspmm_cpp_spmm(btcf, dense_b, second);
-        hspmm_set_kernel_mode(0);
+        // the reference's check arithmetic on the host, rows dealt out over worker threads; with it
         // sum |a||b| per element: the scale of what the two results may differ by where a sum cancels
         // (fp32 accumulation in another order; for tf32_test also the products of bf16 parts)
+        DENSE_MTX expected{btcf.rows, feature_dim, new MAT_VAL_TYPE[size_t(btcf.rows) * feature_dim]};
         std::vector<double> sum_abs(size_t(btcf.rows) * feature_dim, 0.0);
-        for (vint r = 0; r < csr.rows; ++r)
-            for (MAT_PTR_TYPE i = csr.row_ptr[r]; i < csr.row_ptr[r + 1]; ++i) {
-                const double a = std::fabs(double(csr.values[i]));
-                const MAT_VAL_TYPE *brow = dense_b.values + size_t(csr.col_idx[i]) * feature_dim;
-                double *srow = sum_abs.data() + size_t(r) * feature_dim;
-                for (vint j = 0; j < feature_dim; ++j) srow[j] += a * std::fabs(double(brow[j]));
-            }
+        unsigned workers = std::thread::hardware_concurrency();
+        workers = workers < 1 ? 1 : workers > 16 ? 16 : workers;
+        std::vector<std::thread> pool;
+        for (unsigned w = 0; w < workers; ++w)
+            pool.emplace_back([&, w] {
+                std::vector<float> acc(feature_dim);
+                for (vint r = w; r < csr.rows; r += workers) {
+                    std::fill(acc.begin(), acc.end(), 0.0f);
+                    double *srow = sum_abs.data() + size_t(r) * feature_dim;
+                    for (MAT_PTR_TYPE i = csr.row_ptr[r]; i < csr.row_ptr[r + 1]; ++i) {
+                        const float a = float(csr.values[i]);
+                        const MAT_VAL_TYPE *brow = dense_b.values + size_t(csr.col_idx[i]) * feature_dim;
+                        for (vint j = 0; j < feature_dim; ++j) {
+                            const float b = float(brow[j]);
+                            acc[j] += a * b;                                     // src/test_fp16.cu:292-297
+                            srow[j] += std::fabs(double(a)) * std::fabs(double(b));
+                        }
+                    }
+                    MAT_VAL_TYPE *erow = expected.values + size_t(r) * feature_dim;
+                    for (vint j = 0; j < feature_dim; ++j) erow[j] = MAT_VAL_TYPE(acc[j]);
+                }
+            });
+        for (std::thread &t : pool) t.join();
 #if defined(USE_TF32)
         // the tf32 bound: 1e-3 relative; products of bf16 parts: 2^-16 of sum |a||b| more where a sum cancels
         const double rel_tol = 1e-3, abs_tol = 1e-5 + 1.0 / 65536.0;
 #else
         const double rel_tol = 1e-2, abs_tol = 1e-5;
 #endif
-        const bool ok = verify_dense_matrix(&dense_c, &second, rel_tol, sum_abs.data(), abs_tol);
+        const bool ok = verify_dense_matrix(&dense_c, &expected, rel_tol, sum_abs.data(), abs_tol);
         std::printf(ok ? "verification passed\n" : "verification FAILED\n");
         rc = ok ? 0 : 2;
-        delete[] second.values;
+        delete[] expected.values;
     }
     delete[] dense_b.values;
     delete[] dense_c.values;
