@@ -158,8 +158,8 @@ struct Gather {
 // ---------------------------------------------------------------------------
 // Element-type traits: how one step is loaded, multiplied and stored.
 // V = 32-bit words of a B row a lane owns, G = windows per unit (1 or 2).
-// The plan stores the tiles of a step in lane order (hspmm_capi.hip,
-// build_lane_order): what one lane needs of a step is one contiguous load.
+// The plan stores the tiles of a step in lane order (step_stream.hpp,
+// lane_order_tiles): what one lane needs of a step is one contiguous load.
 // ---------------------------------------------------------------------------
 
 // Common part of the two fp16 layouts: the sparse operand.

@@ -158,7 +158,7 @@ struct PanelOps {
 //     (g, j): unit row 4g + e, feature 16 p + j.
 // The rows of the LDS image are 288 bytes apart and the LDS serves two blocks of lanes at a
 // time: the eight rows they read lie in different banks when their numbers differ mod 8,
-// and the plan orders the columns of a step accordingly (hspmm_capi.hip, build_panel_stream).
+// and the plan orders the columns of a step accordingly (hspmm_create.hip, build_panel_stream).
 // Units of three and four windows (G = 4; the third and fourth in a second KB of the step's
 // tile copy) run every second operand against two first operands: half the LDS reads per
 // row, which is what binds these kernels, with eight consumer waves of twice the

@@ -1,7 +1,7 @@
 // The step streams a plan is built from: units (windows, or groups of adjacent windows) and, per step, the column
 // ids and tiles in the order the lanes of the MFMA kernels read them; groups of windows that carry the union of
 // their column lists for the LDS-panel kernels; steps stored without their zeros.  Host code only, no device
-// calls: hspmm_capi.hip uploads what these functions return.
+// calls: hspmm_create.hip uploads what these functions return.
 #pragma once
 #include <stdint.h>
 #include <stddef.h>

@@ -24,6 +24,14 @@ def test_every_declared_symbol_is_exported(hs):
         assert hasattr(lib, n), n
 
 
+def test_nothing_but_the_declared_c_abi_is_exported(hs):
+    # the dynamic symbol table of the library, defined symbols only
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", hs.library_path()], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+    assert exported == declared_symbols()
+
+
 def test_no_torch_types_in_the_header():
     text = open(os.path.join(ROOT, "include", "hspmm.h")).read()
     assert "torch" not in text and "at::" not in text and 'extern "C"' in text
@@ -124,7 +132,7 @@ def test_static_scratch_array_is_a_visible_symbol_of_the_device_code(hs):
     import subprocess
     import tempfile
     tools = "/opt/rocm/llvm/bin"
-    obj = os.path.join(ROOT, "hopper_spmm_amd", "csrc", "build", "hspmm_capi.hip.o")
+    obj = os.path.join(ROOT, "hopper_spmm_amd", "csrc", "build", "hspmm_run.hip.o")
     if not (os.path.exists(obj) and shutil.which(os.path.join(tools, "clang-offload-bundler"))):
         pytest.skip("needs the object file of the last build and the ROCm llvm tools")
     with tempfile.TemporaryDirectory() as d:
