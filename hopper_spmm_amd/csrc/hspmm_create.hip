@@ -34,16 +34,30 @@ int validate_format(uint32_t rows, uint32_t cols, uint32_t W, uint32_t T, uint32
     }
     if (rowOffset[W] != T)
         return fail(HSPMM_ERR_INVALID, "rowOffset[%u] = %u differs from total_tiles = %u", W, rowOffset[W], T);
-    for (uint32_t t = 0; t < T; ++t) {
+    // every tile's ids: real columns below `cols`, padding only behind them.  Checked on all cores; the message
+    // names the first tile that fails.
+    auto tile_error = [&](uint32_t t, bool report) -> bool {
         const uint32_t *ids = tcA2B + size_t(t) * cw;
-        if (ids[0] == HSPMM_IDX_MAX) return fail(HSPMM_ERR_INVALID, "tile %u starts with a padding column", t);
+        if (ids[0] == HSPMM_IDX_MAX) { if (report) fail(HSPMM_ERR_INVALID, "tile %u starts with a padding column", t); return true; }
         bool pad = false;
         for (uint32_t k = 0; k < cw; ++k) {
             if (ids[k] == HSPMM_IDX_MAX) { pad = true; continue; }
-            if (pad) return fail(HSPMM_ERR_INVALID, "tile %u: column id after padding", t);
-            if (ids[k] >= cols) return fail(HSPMM_ERR_INVALID, "tile %u: column id %u >= cols %u", t, ids[k], cols);
+            if (pad) { if (report) fail(HSPMM_ERR_INVALID, "tile %u: column id after padding", t); return true; }
+            if (ids[k] >= cols) { if (report) fail(HSPMM_ERR_INVALID, "tile %u: column id %u >= cols %u", t, ids[k], cols); return true; }
         }
-    }
+        return false;
+    };
+    std::atomic<uint32_t> first_bad{T};
+    hspmm_host::parallel_blocks(T, 65536, [&](size_t tb, size_t te) {
+        if (tb >= first_bad.load(std::memory_order_relaxed)) return;
+        for (size_t t = tb; t < te; ++t)
+            if (tile_error(uint32_t(t), false)) {
+                uint32_t seen = first_bad.load(std::memory_order_relaxed);
+                while (uint32_t(t) < seen && !first_bad.compare_exchange_weak(seen, uint32_t(t), std::memory_order_relaxed)) {}
+                return;
+            }
+    });
+    if (first_bad.load() < T) { tile_error(first_bad.load(), true); return HSPMM_ERR_INVALID; }
     if (canonical) {
         std::atomic<bool> ok{true};
         hspmm_host::parallel_blocks(W, 4096, [&](size_t wb, size_t we) {

@@ -82,6 +82,21 @@ def test_create_rejects_malformed_formats_before_touching_the_device(hs):
     assert b"dtype" in L.hspmm_last_error() and not h.value
 
 
+def test_validation_on_all_cores_names_the_first_bad_tile(hs):
+    # 200 000 tiles (the check runs on worker threads from 65 536 tiles per worker on): two bad tiles planted
+    W, per = 25000, 8
+    T = W * per
+    ids = np.tile(np.arange(per * 16, dtype=np.uint32), W)
+    ids[150000 * 16 + 3] = 5000                             # column id >= cols
+    ids[70000 * 16 + 1] = 0xFFFFFFFF                        # a real id behind padding
+    fmt = dict(rows=W * 8, cols=per * 16, dtype=0, eff_row_windows=W, total_tiles=T,
+               rowOffset=(np.arange(W + 1) * per).astype(np.uint32), rowIdx=(np.arange(W) * 8).astype(np.uint32),
+               tcA2B=ids, data=np.zeros(T * 128, np.uint16))
+    with pytest.raises(hs.HspmmError) as e:
+        hs.Plan(fmt)
+    assert e.value.code == 1 and "tile 70000:" in str(e.value), str(e.value)
+
+
 def test_bitmap_and_grouped_plans_reject_malformed_arrays_before_touching_the_device(hs):
     from util import random_csr
     rng = np.random.default_rng(21)
