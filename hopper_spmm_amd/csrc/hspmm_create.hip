@@ -400,7 +400,7 @@ bool build_panel_stream(hspmm_plan *p, const StepStream &gather_st, const uint32
     // twice the rows; a packed step is its stored values and 64 bytes of masks).  Measured, the lines go down
     // by a third and by 60 % and the time does not: what binds these kernels is the LDS reads and MFMAs of a
     // step, which a SIMD runs one after the other.  Both are therefore taken on request only
-    // (hspmm_set_panel_stream, HSPMM_PANEL_TALL / HSPMM_PANEL_PACKED).
+    // (hspmm_set_panel_stream, libraries built with EXPERIMENTAL=1).
     timer.mark("  panel: tiles in lane order");
     bool tall = false, packed = false;
     if (tall_stream) {
